@@ -1,0 +1,364 @@
+// TensorEngine (kernel caches, multi-kernel capture, non-contraction front-ends) and the KernelExecutor base
+// class with its policy registry.  Call order and asserts follow the reference's kernel/TensorEngine.cpp:70-95,
+// 290-336,538-767 and exec/KernelExecutor.cpp:12-131.
+#include <map>
+
+#include "TensorEngine.hpp"
+
+namespace acro
+{
+
+// -------------------------------------------------------------------------------------- KernelExecutor
+
+KernelExecutor *CreateHipExecutor(DimensionedMultiKernel *multi_kernel);  // hip_executor.cpp
+
+namespace
+{
+std::map<std::string, KernelExecutor::Creator> &registry()
+{
+    static std::map<std::string, KernelExecutor::Creator> table = {{"HIP", &CreateHipExecutor}};
+    return table;
+}
+}  // namespace
+
+KernelExecutor::KernelExecutor(DimensionedMultiKernel *multi_kernel)
+    : MultiKernel(multi_kernel), FirstKernel(multi_kernel->Kernels.empty() ? nullptr : multi_kernel->Kernels[0])
+{
+}
+
+KernelExecutor::~KernelExecutor()
+{
+    for (size_t ki = 0; ki < SubExecutors.size(); ++ki)
+    {
+        delete SubExecutors[ki];
+        delete SubKernels[ki];
+    }
+}
+
+void KernelExecutor::Register(const std::string &exec_type, Creator creator)
+{
+    registry()[exec_type] = creator;
+}
+
+bool KernelExecutor::IsRegistered(const std::string &exec_type)
+{
+    return registry().count(exec_type) > 0;
+}
+
+KernelExecutor *KernelExecutor::Create(std::string exec_type, DimensionedMultiKernel *multi_kernel)
+{
+    auto it = registry().find(exec_type);
+    ACROBATIC_ASSERT(it != registry().end(), "Executor type does not exist:  " + exec_type);
+    return it->second(multi_kernel);
+}
+
+void KernelExecutor::MoveTensorsFromGPU(Tensor *output, std::vector<Tensor *> &inputs)
+{
+    output->MoveFromGPU();
+    for (Tensor *t : inputs) t->MoveFromGPU();
+}
+
+void KernelExecutor::MoveTensorsToGPU(Tensor *output, std::vector<Tensor *> &inputs)
+{
+    // MoveToGPU maps on demand and copies only when the host side holds the current data.
+    output->MoveToGPU();
+    for (Tensor *t : inputs) t->MoveToGPU();
+}
+
+void KernelExecutor::MoveTensorsToOutputLocation(Tensor *output, std::vector<Tensor *> &inputs)
+{
+    if (output->IsOnGPU())
+        MoveTensorsToGPU(output, inputs);
+    else
+        MoveTensorsFromGPU(output, inputs);
+}
+
+void KernelExecutor::ExecuteMulti(std::vector<Tensor *> &output, std::vector<std::vector<Tensor *>> &inputs)
+{
+    const size_t nk = MultiKernel->Kernels.size();
+    if (SubExecutors.size() != nk)
+    {
+        SubKernels.assign(nk, nullptr);
+        SubExecutors.assign(nk, nullptr);
+        for (size_t ki = 0; ki < nk; ++ki)
+        {
+            SubKernels[ki] = new DimensionedMultiKernel(MultiKernel->Kernels[ki]);
+            SubExecutors[ki] = KernelExecutor::Create(GetExecType(), SubKernels[ki]);
+        }
+    }
+    for (size_t ki = 0; ki < nk; ++ki) SubExecutors[ki]->ExecuteSingle(output[ki], inputs[ki]);
+}
+
+// ---------------------------------------------------------------------------------------- TensorEngine
+
+TensorEngine::TensorEngine() : Ops(nullptr), IsMultiKernelLaunch(false), LastExecutor(nullptr) {}
+
+TensorEngine::TensorEngine(const char *bare_exec_type) : TensorEngine()
+{
+    SetExecutorType(std::string(bare_exec_type));
+}
+
+TensorEngine::TensorEngine(const std::string &exec_type) : TensorEngine()
+{
+    SetExecutorType(exec_type);
+}
+
+TensorEngine::~TensorEngine()
+{
+    Clear();
+}
+
+void TensorEngine::SetExecutorType(const char *bare_exec_type)
+{
+    SetExecutorType(std::string(bare_exec_type));
+}
+
+void TensorEngine::SetExecutorType(const std::string &exec_type)
+{
+    ACROBATIC_ASSERT(exec_type != "CPUInterpreted" || KernelExecutor::IsRegistered(exec_type),
+                     "Executor type CPUInterpreted is not part of this library: it only provides the \"HIP\" "
+                     "policy and never computes on the host.");
+    ACROBATIC_ASSERT(KernelExecutor::IsRegistered(exec_type), "Unknown Executor type:  " + exec_type);
+    // No device work happens here: kernels can be generated and compiled without a device, and the first
+    // operation that needs one fails with the HIP error if none is usable.
+
+    Clear();
+    ExecutorType = exec_type;
+    if (ExecutorType == "HIP")
+    {
+        ComputeLocation = "GPU";
+        Ops = new HipGPUOps();
+    }
+    else
+    {
+        ComputeLocation = "CPU";  // a registered host policy brings no non-contraction ops with it
+    }
+}
+
+void TensorEngine::ResetCapture()
+{
+    MKLKernels.clear();
+    MKLOutputT.clear();
+    MKLInputT.clear();
+}
+
+void TensorEngine::operator()(const std::string &kernel_str, Tensor *output, std::vector<Tensor *> &inputs)
+{
+    ACROBATIC_ASSERT(!ExecutorType.empty(), "No executor type has been set on this TensorEngine.");
+    ACROBATIC_ASSERT(output->IsInitialized(), "Output variable not initilized in:  " + kernel_str);
+    for (Tensor *in : inputs)
+    {
+        ACROBATIC_ASSERT(in->IsInitialized(), "Input variable not initilized in:  " + kernel_str);
+    }
+
+    if (!IsMultiKernelLaunch) ResetCapture();
+    TensorKernel *kernel = GetAddTensorKernel(kernel_str);
+    MKLKernels.push_back(GetAddDimensionedKernel(kernel, output, inputs));
+    MKLOutputT.push_back(output);
+    MKLInputT.push_back(inputs);
+
+    if (!IsMultiKernelLaunch)
+    {
+        LastExecutor = GetAddKernelExecutor();
+        LastExecutor->ExecuteSingle(output, inputs);
+    }
+}
+
+void TensorEngine::BeginMultiKernelLaunch()
+{
+    ACROBATIC_ASSERT(!IsMultiKernelLaunch, "Trying to BeginMultiKernelLaunch twice.");
+    IsMultiKernelLaunch = true;
+    ResetCapture();
+}
+
+void TensorEngine::EndMultiKernelLaunch()
+{
+    ACROBATIC_ASSERT(IsMultiKernelLaunch, "Found and EndMultiKernelLaunch before a BeginMultiKernelLaunch!");
+    IsMultiKernelLaunch = false;
+    if (MKLKernels.empty()) return;
+    LastExecutor = GetAddKernelExecutor();
+    LastExecutor->ExecuteMulti(MKLOutputT, MKLInputT);
+}
+
+std::string TensorEngine::GetImplementation(const std::string &kernel_str, Tensor *output,
+                                            std::vector<Tensor *> &inputs)
+{
+    ACROBATIC_ASSERT(!IsMultiKernelLaunch, "GetImplementation not currently supported for multi kernel launch.");
+    ResetCapture();
+    TensorKernel *kernel = GetAddTensorKernel(kernel_str);
+    MKLKernels.push_back(GetAddDimensionedKernel(kernel, output, inputs));
+    MKLOutputT.push_back(output);
+    MKLInputT.push_back(inputs);
+    return GetAddKernelExecutor()->GetImplementation(MKLOutputT, MKLInputT);
+}
+
+std::string TensorEngine::EndMultiKernelLaunchGetImplementation()
+{
+    ACROBATIC_ASSERT(IsMultiKernelLaunch, "Found and EndMultiKernelLaunch before a BeginMultiKernelLaunch!");
+    IsMultiKernelLaunch = false;
+    if (MKLKernels.empty()) return "";
+    return GetAddKernelExecutor()->GetImplementation(MKLOutputT, MKLInputT);
+}
+
+std::string TensorEngine::GetLastImplementation()
+{
+    return LastExecutor ? LastExecutor->GetImplementation() : std::string();
+}
+
+TensorKernel *TensorEngine::GetAddTensorKernel(const std::string &kernel_str)
+{
+    auto it = KernelMap.find(kernel_str);
+    if (it != KernelMap.end()) return it->second;
+    TensorKernel *kernel = new TensorKernel(kernel_str);
+    KernelMap[kernel_str] = kernel;
+    return kernel;
+}
+
+DimensionedKernel *TensorEngine::GetAddDimensionedKernel(TensorKernel *kernel, Tensor *output,
+                                                         std::vector<Tensor *> &inputs)
+{
+    // Rank and extent checks happen inside GetLoopIdxSizes, before anything is cached.
+    std::string key = kernel->GetDimensionedNameString(output, inputs);
+    auto it = DimensionedKernelMap.find(key);
+    if (it != DimensionedKernelMap.end()) return it->second;
+    DimensionedKernel *dk = new DimensionedKernel(kernel, output, inputs);
+    DimensionedKernelMap[key] = dk;
+    return dk;
+}
+
+KernelExecutor *TensorEngine::GetAddKernelExecutor()
+{
+    std::string key;
+    for (DimensionedKernel *k : MKLKernels) key += k->GetDimensionedNameString() + ";";
+    auto it = ExecutorMap.find(key);
+    if (it != ExecutorMap.end()) return it->second;
+
+    DimensionedMultiKernel *mk = new DimensionedMultiKernel(MKLKernels);
+    OwnedMultiKernels.push_back(mk);
+    KernelExecutor *executor = KernelExecutor::Create(ExecutorType, mk);
+    ExecutorMap[key] = executor;
+    return executor;
+}
+
+namespace
+{
+void checkInverseShapes(Tensor &Ainv, Tensor &A)
+{
+    const int rank = A.GetRank();
+    ACROBATIC_ASSERT(rank >= 2, "Can't BatchMatrixInverse a tensor of rank < 2.");
+    ACROBATIC_ASSERT(rank == Ainv.GetRank(), "Can't BatchMatrixInverse with mismatched ranks for Ainv and A.");
+    for (int d = 0; d < rank; ++d)
+    {
+        ACROBATIC_ASSERT(Ainv.GetDim(d) == A.GetDim(d), "Can't BatchMatrixInverse with mismatched dims for Ainv and A.");
+    }
+    ACROBATIC_ASSERT(A.GetDim(rank - 1) == A.GetDim(rank - 2), "Can't BatchMatrixInverse with mismatched dims for m,n.");
+    ACROBATIC_ASSERT(A.GetDim(rank - 1) <= 3, "Can't BatchMatrixInverse with matrix dims > 3.");
+}
+
+void checkDetShapes(Tensor &Adet, Tensor &A)
+{
+    const int rank = A.GetRank();
+    ACROBATIC_ASSERT(rank >= 3, "Can't BatchMatrixDet a tensor of rank < 3.");
+    ACROBATIC_ASSERT(Adet.GetRank() == rank - 2, "Can't BatchMatrixDet with mismatched ranks for Adet and A.");
+    for (int d = 0; d < rank - 2; ++d)
+    {
+        ACROBATIC_ASSERT(Adet.GetDim(d) == A.GetDim(d), "Can't BatchMatrixDet with mismatched dims for Adet and A.");
+    }
+    ACROBATIC_ASSERT(A.GetDim(rank - 1) == A.GetDim(rank - 2), "Can't BatchMatrixDet with mismatched dims for m,n in the matrix.");
+    ACROBATIC_ASSERT(A.GetDim(rank - 1) <= 3, "Can't BatchMatrixDet with matrix dims > 3.");
+}
+}  // namespace
+
+void TensorEngine::BatchMatrixInverse(Tensor &Ainv, Tensor &A)
+{
+    ACROBATIC_ASSERT(Ops != nullptr, "The executor type of this engine provides no non-contraction ops.");
+    checkInverseShapes(Ainv, A);
+    SwitchToComputeLocation(Ainv);
+    MoveToComputeLocation(A);
+    Ops->BatchMatrixInverse(Ainv, A);
+}
+
+void TensorEngine::BatchMatrixDet(Tensor &Adet, Tensor &A)
+{
+    ACROBATIC_ASSERT(Ops != nullptr, "The executor type of this engine provides no non-contraction ops.");
+    checkDetShapes(Adet, A);
+    SwitchToComputeLocation(Adet);
+    MoveToComputeLocation(A);
+    Ops->BatchMatrixDet(Adet, A);
+}
+
+void TensorEngine::BatchMatrixInvDet(Tensor &Ainv, Tensor &Adet, Tensor &A)
+{
+    ACROBATIC_ASSERT(Ops != nullptr, "The executor type of this engine provides no non-contraction ops.");
+    checkInverseShapes(Ainv, A);
+    checkDetShapes(Adet, A);
+    SwitchToComputeLocation(Ainv);
+    SwitchToComputeLocation(Adet);
+    MoveToComputeLocation(A);
+    Ops->BatchMatrixInvDet(Ainv, Adet, A);
+}
+
+void TensorEngine::FlatIndexedScatter(Tensor &Aout, Tensor &Ain, IndexMapping &M)
+{
+    ACROBATIC_ASSERT(Ops != nullptr, "The executor type of this engine provides no non-contraction ops.");
+    ACROBATIC_ASSERT(Aout.GetSize() == M.GetRangeSize(), "IndexMapping RangeSize does not match the output Tensor size.");
+    ACROBATIC_ASSERT(Ain.GetSize() == M.GetDomainSize(), "IndexMapping DomainSize does not match the input Tensor size.");
+    SwitchToComputeLocation(Aout);
+    MoveToComputeLocation(Ain);
+    MoveToComputeLocation(M);
+    Ops->FlatIndexedScatter(Aout, Ain, M);
+}
+
+void TensorEngine::FlatIndexedSumGather(Tensor &Aout, Tensor &Ain, IndexMapping &M)
+{
+    ACROBATIC_ASSERT(Ops != nullptr, "The executor type of this engine provides no non-contraction ops.");
+    ACROBATIC_ASSERT(Aout.GetSize() == M.GetDomainSize(), "IndexMapping DomainSize does not match the output Tensor size.");
+    ACROBATIC_ASSERT(Ain.GetSize() == M.GetRangeSize(), "IndexMapping RangeSize does not match the input Tensor size.");
+    if (!M.IsInverseComputed()) M.ComputeInverse();
+    SwitchToComputeLocation(Aout);
+    MoveToComputeLocation(Ain);
+    MoveToComputeLocation(M);
+    Ops->FlatIndexedSumGather(Aout, Ain, M);
+}
+
+void TensorEngine::Clear()
+{
+    for (auto &e : ExecutorMap) delete e.second;
+    ExecutorMap.clear();
+    for (DimensionedMultiKernel *mk : OwnedMultiKernels) delete mk;
+    OwnedMultiKernels.clear();
+    for (auto &k : DimensionedKernelMap) delete k.second;
+    DimensionedKernelMap.clear();
+    for (auto &k : KernelMap) delete k.second;
+    KernelMap.clear();
+    delete Ops;
+    Ops = nullptr;
+    LastExecutor = nullptr;
+    ResetCapture();
+}
+
+void TensorEngine::MoveToComputeLocation(Tensor &T)
+{
+    if (ComputeLocation == "GPU")
+        T.MoveToGPU();
+    else
+        T.MoveFromGPU();
+}
+
+void TensorEngine::SwitchToComputeLocation(Tensor &T)
+{
+    if (ComputeLocation == "GPU")
+        T.SwitchToGPU();
+    else
+        T.SwitchFromGPU();
+}
+
+void TensorEngine::MoveToComputeLocation(IndexMapping &M)
+{
+    if (ComputeLocation == "GPU")
+        M.MoveToGPU();
+    else
+        M.MoveFromGPU();
+}
+
+}  // namespace acro

@@ -1,0 +1,1043 @@
+// Generator: DimensionedMultiKernel -> HIP C++ source (see hip_codegen.hpp for the schedule in words).
+// The reference's generator (exec/CudaExecutor.cpp:111-702) maps one CUDA thread to one output entry and loops
+// over the contraction reading shared memory twice per multiply-add; this one maps a lane to a pencil of outputs,
+// keeps operands in registers / SGPRs and batches several elements per workgroup.
+#include "hip_codegen.hpp"
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdlib>
+#include <map>
+#include <set>
+#include <sstream>
+
+#include "Error.hpp"
+
+namespace acro
+{
+
+namespace
+{
+
+// One occurrence of a variable in a kernel.
+struct VarRef
+{
+    int uvar = -1;
+    std::vector<int> idx;     // loop id of every dimension
+    std::vector<int> ext;     // extent of every dimension
+    std::vector<int> stride;  // row-major element stride of every dimension
+    int size = 1;
+    bool repeated = false;    // some index occurs in two dimensions
+};
+
+struct Sub
+{
+    std::string text;
+    VarRef out;
+    std::vector<VarRef> in;
+    char op = '=';            // '=', '+' or '-'
+    std::vector<int> outIdx;  // distinct loop ids of the output
+    std::vector<int> contr;   // contraction loop ids, first-appearance order
+    // schedule
+    std::vector<int> lane;    // loop ids enumerated by the work items (last one fastest)
+    std::vector<int> tile;    // loop ids kept in registers by one work item
+    bool loopMode = false;    // contraction as counted loops instead of unrolled code
+    bool fusedWithPrev = false;
+    int forwardedInput = -1;  // input occurrence served from the previous kernel's registers
+    long laneCount = 1, tileCount = 1, contrCount = 1;
+};
+
+struct UVarInfo
+{
+    std::string name;
+    std::vector<int> dims;
+    int size = 0;
+    bool written = false;
+    bool read = false;
+    int firstWrite = -1;
+    int lastUse = -1;
+    bool consistent = true;       // same shape and batch positions in every occurrence
+    std::vector<int> batchDims;   // dimensions carrying the batch index
+    bool anyRepeated = false;
+    // LDS residency of the per-batch-entry tile
+    bool wantLds = false;
+    bool inLds = false;
+    int tileSize = 0;             // doubles per batch entry
+    std::vector<int> ldsStride;   // per dimension (0 for batch dimensions)
+    int ldsOffset = 0;            // in doubles, start of the NB tiles
+    int liveFrom = 0, liveTo = 0;
+    bool elide = false;           // no store to device memory
+};
+
+long product(const std::vector<int> &ids, const std::vector<int> &extent)
+{
+    long p = 1;
+    for (int i : ids) p *= extent[i];
+    return p;
+}
+
+bool has(const std::vector<int> &v, int x)
+{
+    return std::find(v.begin(), v.end(), x) != v.end();
+}
+
+std::string str(long v)
+{
+    return std::to_string(v);
+}
+
+uint64_t hashString(const std::string &s)
+{
+    uint64_t h = 1469598103934665603ull;
+    for (unsigned char c : s)
+    {
+        h ^= c;
+        h *= 1099511628211ull;
+    }
+    return h;
+}
+
+int envInt(const char *name)
+{
+    const char *v = std::getenv(name);
+    return v ? std::atoi(v) : 0;
+}
+
+class Generator
+{
+  public:
+    Generator(const DimensionedMultiKernel &mk_, const HipCodegenOptions &opt_) : mk(mk_), opt(opt_) {}
+
+    HipKernelPlan Run()
+    {
+        HipKernelPlan plan;
+        BuildModel();
+        std::string why;
+        if (!CheckFusable(why))
+        {
+            plan.fusable = false;
+            plan.why_not = why;
+            return plan;
+        }
+        ChooseTiles();
+        PlanFusion();
+        ChooseBatching();
+        Emit(plan);
+        plan.fusable = true;
+        return plan;
+    }
+
+  private:
+    const DimensionedMultiKernel &mk;
+    const HipCodegenOptions &opt;
+
+    int nidx = 0;
+    std::vector<std::string> idxName;
+    std::vector<int> extent;
+    std::vector<Sub> subs;
+    std::vector<UVarInfo> uvars;
+    int batch = -1;
+    long E = 1;
+    int NB = 1, NT = 128;
+    int ldsDoubles = 0;
+    bool extentsConsistent = true;
+
+    // ------------------------------------------------------------------------------------------ model
+    // Operand numbering: unique variables by name, or one operand per occurrence in positional mode.
+    bool Positional() const { return opt.positional && mk.GetNumKernels() == 1; }
+    int NumOperands() const { return Positional() ? mk.Kernels[0]->GetNumVars() : mk.GetNumUVars(); }
+    int OperandOf(int ki, int vari) const { return Positional() ? vari + 1 : mk.GetUVari(ki, vari); }
+    std::pair<int, int> FirstOccurrence(int u) const
+    {
+        return Positional() ? std::make_pair(0, u - 1) : mk.GetFirstKiVariForUVari(u);
+    }
+
+    void BuildModel()
+    {
+        nidx = static_cast<int>(mk.LoopIndices.size());
+        idxName = mk.LoopIndices;
+        extent.assign(nidx, 1);
+        for (int i = 0; i < nidx; ++i) extent[i] = mk.GetLoopDim(i);
+
+        uvars.resize(NumOperands());
+        const int K = mk.GetNumKernels();
+        subs.resize(K);
+        for (int ki = 0; ki < K; ++ki)
+        {
+            DimensionedKernel *k = mk.Kernels[ki];
+            Sub &s = subs[ki];
+            s.text = k->KernelStr;
+            s.op = k->EqOperator[0] == '=' ? '=' : k->EqOperator[0];
+            auto makeRef = [&](int vari) {
+                VarRef r;
+                r.uvar = OperandOf(ki, vari);
+                const KernelVar &kv = k->GetVar(vari);
+                const int rank = static_cast<int>(kv.IndexNames.size());
+                r.idx.resize(rank);
+                r.ext.resize(rank);
+                r.stride.assign(rank, 1);
+                for (int d = 0; d < rank; ++d)
+                {
+                    r.idx[d] = mk.GetIndexLoopNum(kv.IndexNames[d]);
+                    r.ext[d] = k->GetLoopDim(kv.IndexNames[d]);
+                    if (r.ext[d] != extent[r.idx[d]]) extentsConsistent = false;
+                }
+                for (int d = rank - 2; d >= 0; --d) r.stride[d] = r.stride[d + 1] * r.ext[d + 1];
+                r.size = 1;
+                for (int d = 0; d < rank; ++d) r.size *= r.ext[d];
+                std::set<int> distinct(r.idx.begin(), r.idx.end());
+                r.repeated = static_cast<int>(distinct.size()) != rank;
+                return r;
+            };
+            s.out = makeRef(-1);
+            for (int vari = 0; vari < k->GetNumInputVars(); ++vari) s.in.push_back(makeRef(vari));
+            for (int id : s.out.idx)
+            {
+                if (!has(s.outIdx, id)) s.outIdx.push_back(id);
+            }
+            for (const auto &name : k->ContractionIndexNames) s.contr.push_back(mk.GetIndexLoopNum(name));
+            s.contrCount = product(s.contr, extent);
+        }
+
+        if (!mk.SharedOuterIndexNames.empty())
+        {
+            batch = mk.GetIndexLoopNum(mk.SharedOuterIndexNames[0]);
+            E = extent[batch];
+        }
+
+        // Unique-variable facts, in program order (a kernel reads its inputs before it writes its output).
+        for (int ki = 0; ki < K; ++ki)
+        {
+            const Sub &s = subs[ki];
+            auto note = [&](const VarRef &r, bool is_write) {
+                UVarInfo &u = uvars[r.uvar];
+                std::vector<int> bd;
+                for (size_t d = 0; d < r.idx.size(); ++d)
+                {
+                    if (r.idx[d] == batch) bd.push_back(static_cast<int>(d));
+                }
+                if (u.lastUse < 0 && u.dims.empty())
+                {
+                    u.dims = r.ext;
+                    u.size = r.size;
+                    u.batchDims = bd;
+                }
+                else if (u.dims != r.ext || u.batchDims != bd)
+                {
+                    u.consistent = false;
+                }
+                u.anyRepeated = u.anyRepeated || r.repeated;
+                u.lastUse = ki;
+                if (is_write)
+                {
+                    if (!u.written) u.firstWrite = ki;
+                    u.written = true;
+                }
+                else
+                {
+                    u.read = true;
+                }
+            };
+            for (const auto &r : s.in) note(r, false);
+            if (s.op != '=') note(s.out, false);
+            note(s.out, true);
+        }
+        for (int u = 0; u < NumOperands(); ++u)
+        {
+            auto first = FirstOccurrence(u);
+            uvars[u].name = mk.Kernels[first.first]->GetVarName(first.second);
+        }
+    }
+
+    bool CheckFusable(std::string &why)
+    {
+        if (mk.GetNumKernels() == 1) return true;  // a single kernel always has a private batch index
+        if (batch < 0)
+        {
+            why = "the kernels share no outer index";
+            return false;
+        }
+        if (!extentsConsistent)
+        {
+            why = "an index name has different extents in different kernels";
+            return false;
+        }
+        for (const auto &u : uvars)
+        {
+            if (u.written && !u.consistent)
+            {
+                why = "variable " + u.name + " is written and used with different shapes or element positions";
+                return false;
+            }
+        }
+        return true;
+    }
+
+    // --------------------------------------------------------------------------------------- schedule
+    bool IsPureInput(int uvar) const { return !uvars[uvar].written; }
+
+    // Operand can be read with scalar loads: never written here, no aliasing, small, and its address does not
+    // depend on the lane (only on tile / contraction indices, which are literals or uniform loop counters).
+    bool IsUniform(const Sub &s, const VarRef &r, const std::vector<int> &tile) const
+    {
+        if (!opt.noalias || !IsPureInput(r.uvar) || r.size > 4096) return false;
+        for (int id : r.idx)
+        {
+            if (id == batch) return false;
+            if (!has(tile, id) && !has(s.contr, id)) return false;
+        }
+        return true;
+    }
+
+    long LoadsPerItem(const Sub &s, const std::vector<int> &tile) const
+    {
+        long loads = 0;
+        for (const auto &r : s.in)
+        {
+            if (IsUniform(s, r, tile)) continue;
+            std::set<int> seen;
+            long n = 1;
+            for (int id : r.idx)
+            {
+                if ((has(tile, id) || has(s.contr, id)) && seen.insert(id).second) n *= extent[id];
+            }
+            loads += n;
+        }
+        return loads;
+    }
+
+    static constexpr long kUnrollBudget = 8192;   // multiply-adds emitted per work item
+    static constexpr long kMaxTile = 32;
+    static constexpr long kMaxLiveValues = 160;   // loaded operands + accumulators held by one lane
+
+    void ChooseTiles()
+    {
+        for (auto &s : subs)
+        {
+            std::vector<int> mid;
+            for (int id : s.outIdx)
+            {
+                if (id != batch) mid.push_back(id);
+            }
+            const long nin = static_cast<long>(s.in.size());
+            if (s.contrCount * nin > kUnrollBudget)
+            {
+                s.loopMode = true;
+                s.tile.clear();
+            }
+            else
+            {
+                std::vector<std::vector<int>> candidates(1);  // the empty tile
+                for (size_t a = 0; a < mid.size(); ++a)
+                {
+                    candidates.push_back({mid[a]});
+                    for (size_t b = a + 1; b < mid.size(); ++b) candidates.push_back({mid[a], mid[b]});
+                }
+                double bestScore = 1e300;
+                std::vector<int> best;
+                for (const auto &t : candidates)
+                {
+                    const long tc = product(t, extent);
+                    if (tc > kMaxTile || tc * s.contrCount * nin > kUnrollBudget) continue;
+                    const long loads = LoadsPerItem(s, t);
+                    if (loads + tc > kMaxLiveValues && !t.empty()) continue;
+                    // loads per produced output; a small bias keeps the tile short when nothing is gained
+                    double score = static_cast<double>(loads) / tc + 1e-3 * t.size() + 1e-6 * tc;
+                    if (score < bestScore)
+                    {
+                        bestScore = score;
+                        best = t;
+                    }
+                }
+                s.tile = best;
+            }
+            SetLanes(s);
+        }
+    }
+
+    void SetLanes(Sub &s)
+    {
+        s.lane.clear();
+        // Lane order follows the dimension order of the tensor that should see unit-stride lanes: the output
+        // when it is stored to device memory, otherwise the largest operand read from device memory.
+        const VarRef *order = &s.out;
+        const UVarInfo &uo = uvars[s.out.uvar];
+        const bool out_stays_on_chip = opt.transient.size() > static_cast<size_t>(s.out.uvar) &&
+                                       opt.transient[s.out.uvar] && uo.lastUse > uo.firstWrite;
+        if (out_stays_on_chip)
+        {
+            const VarRef *big = nullptr;
+            for (const auto &r : s.in)
+            {
+                if (!IsPureInput(r.uvar) || !has(r.idx, batch)) continue;
+                if (big == nullptr || r.size > big->size) big = &r;
+            }
+            if (big != nullptr) order = big;
+        }
+        auto consider = [&](int id) {
+            if (id == batch || has(s.tile, id) || has(s.lane, id) || !has(s.outIdx, id)) return;
+            s.lane.push_back(id);
+        };
+        for (int id : order->idx) consider(id);
+        // Output indices that the ordering tensor does not carry go in front (slowest).
+        std::vector<int> front;
+        for (int id : s.outIdx)
+        {
+            if (id != batch && !has(s.tile, id) && !has(s.lane, id)) front.push_back(id);
+        }
+        s.lane.insert(s.lane.begin(), front.begin(), front.end());
+        s.laneCount = product(s.lane, extent);
+        s.tileCount = product(s.tile, extent);
+    }
+
+    void PlanFusion()
+    {
+        const int K = static_cast<int>(subs.size());
+        for (int k = 1; k < K; ++k)
+        {
+            Sub &s = subs[k];
+            const Sub &p = subs[k - 1];
+            if (!s.contr.empty() || p.loopMode || p.out.repeated || s.out.repeated) continue;
+            std::set<int> a(s.outIdx.begin(), s.outIdx.end()), b(p.outIdx.begin(), p.outIdx.end());
+            if (a != b) continue;
+            int fwd = -1;
+            for (size_t v = 0; v < s.in.size(); ++v)
+            {
+                if (s.in[v].uvar == p.out.uvar && s.in[v].idx == p.out.idx) fwd = static_cast<int>(v);
+            }
+            if (fwd < 0) continue;
+            // Every other use of the producer's variable in this kernel would need the stored copy.
+            bool other_use = (s.out.uvar == p.out.uvar);
+            for (size_t v = 0; v < s.in.size(); ++v)
+            {
+                if (static_cast<int>(v) != fwd && s.in[v].uvar == p.out.uvar) other_use = true;
+            }
+            if (other_use) continue;
+            s.fusedWithPrev = true;
+            s.forwardedInput = fwd;
+            s.tile = p.tile;
+            s.lane = p.lane;
+            s.laneCount = p.laneCount;
+            s.tileCount = p.tileCount;
+            s.loopMode = false;
+        }
+    }
+
+    void ComputeLdsWishes()
+    {
+        const int K = static_cast<int>(subs.size());
+        for (auto &u : uvars)
+        {
+            u.wantLds = false;
+            u.inLds = false;
+        }
+        if (batch < 0) return;
+        for (size_t ui = 0; ui < uvars.size(); ++ui)
+        {
+            UVarInfo &u = uvars[ui];
+            if (!u.written || !u.consistent || u.anyRepeated || u.batchDims.size() != 1) continue;
+            // Readers after the first write that are not served from registers.
+            int lastReader = -1;
+            for (int k = u.firstWrite + 1; k < K; ++k)
+            {
+                const Sub &s = subs[k];
+                for (size_t v = 0; v < s.in.size(); ++v)
+                {
+                    if (s.in[v].uvar != static_cast<int>(ui)) continue;
+                    if (s.fusedWithPrev && s.forwardedInput == static_cast<int>(v)) continue;
+                    lastReader = k;
+                }
+                if (s.out.uvar == static_cast<int>(ui) && s.op != '=') lastReader = k;
+            }
+            if (lastReader < 0) continue;
+            u.wantLds = true;
+            u.liveFrom = u.firstWrite;
+            u.liveTo = lastReader;
+            u.tileSize = u.size / u.dims[u.batchDims[0]];
+            u.ldsStride.assign(u.dims.size(), 0);
+            int st = 1;
+            for (int d = static_cast<int>(u.dims.size()) - 1; d >= 0; --d)
+            {
+                if (d == u.batchDims[0]) continue;
+                u.ldsStride[d] = st;
+                st *= u.dims[d];
+            }
+        }
+    }
+
+    // First-fit placement of the tiles that are live at the same time; returns doubles needed for nb entries.
+    int PlaceLds(int nb)
+    {
+        std::vector<int> order;
+        for (size_t ui = 0; ui < uvars.size(); ++ui)
+        {
+            if (uvars[ui].wantLds && uvars[ui].inLds) order.push_back(static_cast<int>(ui));
+        }
+        std::sort(order.begin(), order.end(), [&](int a, int b) {
+            if (uvars[a].liveFrom != uvars[b].liveFrom) return uvars[a].liveFrom < uvars[b].liveFrom;
+            return a < b;
+        });
+        int total = 0;
+        std::vector<int> placed;
+        for (int ui : order)
+        {
+            UVarInfo &u = uvars[ui];
+            const int need = u.tileSize * nb;
+            int offset = 0;
+            bool moved = true;
+            while (moved)
+            {
+                moved = false;
+                for (int pj : placed)
+                {
+                    const UVarInfo &p = uvars[pj];
+                    const bool timeOverlap = !(p.liveTo < u.liveFrom || u.liveTo < p.liveFrom);
+                    const int pneed = p.tileSize * nb;
+                    const bool spaceOverlap = !(p.ldsOffset + pneed <= offset || offset + need <= p.ldsOffset);
+                    if (timeOverlap && spaceOverlap)
+                    {
+                        offset = p.ldsOffset + pneed;
+                        moved = true;
+                    }
+                }
+            }
+            u.ldsOffset = offset;
+            placed.push_back(ui);
+            total = std::max(total, offset + need);
+        }
+        return total;
+    }
+
+    void ChooseBatching()
+    {
+        ComputeLdsWishes();
+        long maxLane = 1;
+        for (const auto &s : subs) maxLane = std::max(maxLane, s.laneCount);
+
+        NT = opt.force_nt > 0 ? opt.force_nt : envInt("ACRO_HIP_NT");
+        if (NT <= 0) NT = maxLane > 128 ? 256 : 128;
+        NB = opt.force_nb > 0 ? opt.force_nb : envInt("ACRO_HIP_NB");
+        if (NB <= 0)
+        {
+            // As many batch entries as fit in one pass of the widest kernel, rounded down to a power of two.
+            long fit = std::max<long>(1, NT / maxLane);
+            NB = 1;
+            while (NB * 2 <= fit) NB *= 2;
+        }
+        if (batch < 0) NB = 1;
+        NB = static_cast<int>(std::min<long>(NB, E));
+
+        // Everything that wants LDS gets it while the workgroup stays within the budget; otherwise shrink the
+        // batch, and finally leave the largest tiles in device memory.
+        const int budgetDoubles = 48 * 1024 / 8;
+        for (auto &u : uvars) u.inLds = u.wantLds;
+        while (true)
+        {
+            ldsDoubles = PlaceLds(NB);
+            if (ldsDoubles <= budgetDoubles) break;
+            if (NB > 1 && opt.force_nb <= 0)
+            {
+                NB /= 2;
+                continue;
+            }
+            int biggest = -1;
+            for (size_t ui = 0; ui < uvars.size(); ++ui)
+            {
+                if (uvars[ui].inLds && (biggest < 0 || uvars[ui].tileSize > uvars[biggest].tileSize))
+                    biggest = static_cast<int>(ui);
+            }
+            if (biggest < 0) break;
+            uvars[biggest].inLds = false;
+        }
+
+        // Stores to device memory that may be dropped: transient, produced by a plain assignment before any
+        // read, and every later read is served on chip.
+        for (size_t ui = 0; ui < uvars.size(); ++ui)
+        {
+            UVarInfo &u = uvars[ui];
+            u.elide = false;
+            if (ui >= opt.transient.size() || !opt.transient[ui] || !u.written) continue;
+            bool ok = subs[u.firstWrite].op == '=';
+            bool laterRead = false;
+            for (int k = 0; k < static_cast<int>(subs.size()); ++k)
+            {
+                const Sub &s = subs[k];
+                for (size_t v = 0; v < s.in.size(); ++v)
+                {
+                    if (s.in[v].uvar != static_cast<int>(ui)) continue;
+                    if (k <= u.firstWrite) ok = false;  // read before (or while) first produced
+                    laterRead = true;
+                    const bool fromRegs = s.fusedWithPrev && s.forwardedInput == static_cast<int>(v);
+                    if (!fromRegs && !u.inLds) ok = false;
+                }
+                if (s.out.uvar == static_cast<int>(ui) && s.op != '=' && !u.inLds) ok = false;
+            }
+            u.elide = ok && laterRead;
+        }
+    }
+
+    // --------------------------------------------------------------------------------------- emission
+    std::ostringstream out;
+
+    std::string PtrName(int uvar) const { return "T" + str(uvar); }
+    std::string ConstPtrName(int uvar) const { return "C" + str(uvar); }
+    std::string IdxVar(int id) const { return "i_" + idxName[id]; }
+
+    // Offset of an occurrence split into a run-time part (batch entry + lane indices) and, for a given
+    // assignment of tile / contraction indices, a literal part.
+    std::string RuntimeOffset(const VarRef &r, const Sub &s, bool lds) const
+    {
+        const UVarInfo &u = uvars[r.uvar];
+        std::string expr;
+        auto add = [&](const std::string &term) { expr += (expr.empty() ? "" : " + ") + term; };
+        if (lds) add(str(u.ldsOffset) + " + b * " + str(u.tileSize));
+        for (size_t d = 0; d < r.idx.size(); ++d)
+        {
+            const int id = r.idx[d];
+            const long st = lds ? u.ldsStride[d] : r.stride[d];
+            if (id == batch)
+            {
+                if (!lds) add("e * " + str(st));
+            }
+            else if (has(s.lane, id))
+            {
+                add(IdxVar(id) + " * " + str(st));
+            }
+        }
+        return expr.empty() ? "0" : expr;
+    }
+
+    long LiteralOffset(const VarRef &r, const Sub &s, bool lds, const std::vector<int> &value) const
+    {
+        const UVarInfo &u = uvars[r.uvar];
+        long off = 0;
+        for (size_t d = 0; d < r.idx.size(); ++d)
+        {
+            const int id = r.idx[d];
+            if (id == batch || has(s.lane, id)) continue;
+            off += static_cast<long>(value[id]) * (lds ? u.ldsStride[d] : r.stride[d]);
+        }
+        return off;
+    }
+
+    // Where an input occurrence of kernel k is read from.
+    enum Source
+    {
+        kFromRegisters,
+        kFromConstant,
+        kFromLds,
+        kFromGlobal
+    };
+    Source SourceOf(int k, int v) const
+    {
+        const Sub &s = subs[k];
+        const VarRef &r = s.in[v];
+        if (s.fusedWithPrev && s.forwardedInput == v) return kFromRegisters;
+        const UVarInfo &u = uvars[r.uvar];
+        if (u.inLds && u.written && u.firstWrite < k) return kFromLds;
+        if (IsUniform(s, r, s.tile)) return kFromConstant;
+        return kFromGlobal;
+    }
+
+    struct Body
+    {
+        std::vector<std::string> bases;    // run-time base offsets
+        std::vector<std::string> loads;    // operand loads
+        std::vector<std::string> compute;  // partial sums and outputs
+        std::vector<std::string> stores;
+        std::map<std::string, std::string> loadMemo;
+        std::map<std::string, std::string> sumMemo;
+        int counter = 0;
+    };
+
+    std::string OperandExpr(int k, int v, const std::vector<int> &value, Body &body,
+                            const std::map<long, std::string> &forwarded)
+    {
+        const Sub &s = subs[k];
+        const VarRef &r = s.in[v];
+        const Source src = SourceOf(k, v);
+        const std::string tag = "k" + str(k) + "v" + str(v);
+        if (src == kFromRegisters)
+        {
+            // Same index names in the same order as the producer's output: its literal offset names the value.
+            return forwarded.at(LiteralOffset(subs[k - 1].out, subs[k - 1], false, value));
+        }
+        if (src == kFromConstant)
+        {
+            return ConstPtrName(r.uvar) + "[" + str(LiteralOffset(r, s, false, value)) + "]";
+        }
+        const bool lds = (src == kFromLds);
+        const long off = LiteralOffset(r, s, lds, value);
+        const std::string key = tag + ":" + str(off);
+        auto it = body.loadMemo.find(key);
+        if (it != body.loadMemo.end()) return it->second;
+        const std::string name = "x" + str(k) + "_" + str(body.counter++);
+        const std::string base = "o_" + tag;
+        if (lds)
+            body.loads.push_back("const double " + name + " = lds[" + base + " + " + str(off) + "];");
+        else
+            body.loads.push_back("const double " + name + " = " + PtrName(r.uvar) + "[" + base + " + " + str(off) + "];");
+        body.loadMemo[key] = name;
+        return name;
+    }
+
+    // Sum over the contraction indices deeper than `depth`, of the product of the factors that close at those
+    // levels.  Returns the name of a temporary, or "" when the remaining sum is exactly one.
+    std::string PartialSum(int k, int depth, std::vector<int> &value, Body &body, const std::vector<int> &level,
+                           const std::map<long, std::string> &forwarded)
+    {
+        const Sub &s = subs[k];
+        const int n = static_cast<int>(s.contr.size());
+        if (depth == n) return "";
+
+        // The value depends on the already assigned indices only through the deeper factors.
+        std::set<int> relevant;
+        for (size_t v = 0; v < s.in.size(); ++v)
+        {
+            if (level[v] > depth)
+            {
+                for (int id : s.in[v].idx)
+                {
+                    if (id != batch && !has(s.lane, id)) relevant.insert(id);
+                }
+            }
+        }
+        std::string key = "d" + str(depth);
+        for (int id : relevant)
+        {
+            bool assigned = has(s.tile, id);
+            for (int j = 0; j < depth; ++j) assigned = assigned || s.contr[j] == id;
+            if (assigned) key += "," + str(id) + "=" + str(value[id]);
+        }
+        auto it = body.sumMemo.find(key);
+        if (it != body.sumMemo.end()) return it->second;
+
+        const int cid = s.contr[depth];
+        std::vector<std::string> terms;
+        for (int x = 0; x < extent[cid]; ++x)
+        {
+            value[cid] = x;
+            std::string prod;
+            for (size_t v = 0; v < s.in.size(); ++v)
+            {
+                if (level[v] != depth + 1) continue;
+                const std::string opnd = OperandExpr(k, static_cast<int>(v), value, body, forwarded);
+                prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
+            }
+            const std::string rest = PartialSum(k, depth + 1, value, body, level, forwarded);
+            std::string term;
+            if (prod.empty() && rest.empty())
+                term = "1.0";
+            else if (prod.empty())
+                term = rest;
+            else if (rest.empty())
+                term = prod;
+            else
+                term = prod + " * " + rest;
+            terms.push_back(term);
+        }
+        value[cid] = 0;
+        const std::string name = "s" + str(k) + "_" + str(body.counter++);
+        body.compute.push_back("double " + name + " = " + terms[0] + ";");
+        for (size_t t = 1; t < terms.size(); ++t) body.compute.push_back(name + " += " + terms[t] + ";");
+        body.sumMemo[key] = name;
+        return name;
+    }
+
+    void EmitBases(int k, Body &body)
+    {
+        const Sub &s = subs[k];
+        for (size_t v = 0; v < s.in.size(); ++v)
+        {
+            const Source src = SourceOf(k, static_cast<int>(v));
+            if (src == kFromRegisters || src == kFromConstant) continue;
+            body.bases.push_back("const int o_k" + str(k) + "v" + str(v) + " = " +
+                                 RuntimeOffset(s.in[v], s, src == kFromLds) + ";");
+        }
+        body.bases.push_back("const int o_k" + str(k) + "g = " + RuntimeOffset(s.out, s, false) + ";");
+        if (uvars[s.out.uvar].inLds)
+            body.bases.push_back("const int o_k" + str(k) + "l = " + RuntimeOffset(s.out, s, true) + ";");
+    }
+
+    // Is the output variable's tile already on chip before kernel k (needed by += and -=)?
+    bool OldValueInLds(int k) const
+    {
+        const UVarInfo &u = uvars[subs[k].out.uvar];
+        return u.inLds && u.firstWrite < k;
+    }
+
+    bool NeedsLdsCopy(int k) const
+    {
+        const UVarInfo &u = uvars[subs[k].out.uvar];
+        return u.inLds && u.liveTo > k;
+    }
+
+    // Unrolled body of kernel k for one work item.  `forwarded` maps the literal output offsets of the previous
+    // kernel to the registers holding them; on return it describes this kernel's outputs.
+    void EmitUnrolledBody(int k, std::map<long, std::string> &forwarded, std::vector<std::string> &lines)
+    {
+        const Sub &s = subs[k];
+        Body body;
+        EmitBases(k, body);
+
+        const int n = static_cast<int>(s.contr.size());
+        std::vector<int> level(s.in.size(), 0);
+        for (size_t v = 0; v < s.in.size(); ++v)
+        {
+            for (int j = 0; j < n; ++j)
+            {
+                if (has(s.in[v].idx, s.contr[j])) level[v] = j + 1;
+            }
+        }
+
+        std::map<long, std::string> produced;
+        std::vector<int> value(nidx, 0);
+        const long tc = s.tileCount;
+        for (long t = 0; t < tc; ++t)
+        {
+            long rem = t;
+            for (int j = static_cast<int>(s.tile.size()) - 1; j >= 0; --j)
+            {
+                value[s.tile[j]] = static_cast<int>(rem % extent[s.tile[j]]);
+                rem /= extent[s.tile[j]];
+            }
+            std::string prod;
+            for (size_t v = 0; v < s.in.size(); ++v)
+            {
+                if (level[v] != 0) continue;
+                const std::string opnd = OperandExpr(k, static_cast<int>(v), value, body, forwarded);
+                prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
+            }
+            const std::string rest = PartialSum(k, 0, value, body, level, forwarded);
+            std::string rhs;
+            if (prod.empty() && rest.empty())
+                rhs = "1.0";
+            else if (prod.empty())
+                rhs = rest;
+            else if (rest.empty())
+                rhs = prod;
+            else
+                rhs = prod + " * " + rest;
+
+            const long goff = LiteralOffset(s.out, s, false, value);
+            const long loff = uvars[s.out.uvar].inLds ? LiteralOffset(s.out, s, true, value) : 0;
+            const std::string gaddr = PtrName(s.out.uvar) + "[o_k" + str(k) + "g + " + str(goff) + "]";
+            const std::string laddr = "lds[o_k" + str(k) + "l + " + str(loff) + "]";
+            const std::string name = "r" + str(k) + "_" + str(t);
+            if (s.op == '=')
+            {
+                body.compute.push_back("const double " + name + " = " + rhs + ";");
+            }
+            else
+            {
+                const std::string old = OldValueInLds(k) ? laddr : gaddr;
+                body.compute.push_back("const double " + name + " = " + old + (s.op == '+' ? " + " : " - ") + rhs + ";");
+            }
+            if (NeedsLdsCopy(k)) body.stores.push_back(laddr + " = " + name + ";");
+            if (!uvars[s.out.uvar].elide) body.stores.push_back(gaddr + " = " + name + ";");
+            produced[goff] = name;
+        }
+
+        lines.push_back("// " + s.text);
+        for (const auto &l : body.bases) lines.push_back(l);
+        for (const auto &l : body.loads) lines.push_back(l);
+        for (const auto &l : body.compute) lines.push_back(l);
+        for (const auto &l : body.stores) lines.push_back(l);
+        forwarded.swap(produced);
+    }
+
+    // Counted-loop body (long contractions): one output per work item, no tile.
+    void EmitLoopBody(int k, std::vector<std::string> &lines)
+    {
+        const Sub &s = subs[k];
+        Body body;
+        EmitBases(k, body);
+        lines.push_back("// " + s.text + "   (contraction as counted loops)");
+        for (const auto &l : body.bases) lines.push_back(l);
+        lines.push_back("double sum = 0.0;");
+        std::string indent;
+        for (size_t j = 0; j < s.contr.size(); ++j)
+        {
+            const std::string c = IdxVar(s.contr[j]);
+            if (j + 1 == s.contr.size()) lines.push_back(indent + "#pragma unroll 4");
+            lines.push_back(indent + "for (int " + c + " = 0; " + c + " < " + str(extent[s.contr[j]]) + "; ++" + c + ")");
+            lines.push_back(indent + "{");
+            indent += "    ";
+        }
+        std::string prod;
+        for (size_t v = 0; v < s.in.size(); ++v)
+        {
+            const VarRef &r = s.in[v];
+            const Source src = SourceOf(k, static_cast<int>(v));
+            const bool lds = (src == kFromLds);
+            std::string off;
+            for (size_t d = 0; d < r.idx.size(); ++d)
+            {
+                const int id = r.idx[d];
+                if (!has(s.contr, id)) continue;
+                const long st = lds ? uvars[r.uvar].ldsStride[d] : r.stride[d];
+                off += (off.empty() ? "" : " + ") + IdxVar(id) + " * " + str(st);
+            }
+            if (off.empty()) off = "0";
+            std::string opnd;
+            if (src == kFromConstant)
+                opnd = ConstPtrName(r.uvar) + "[" + off + "]";
+            else if (lds)
+                opnd = "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
+            else
+                opnd = PtrName(r.uvar) + "[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
+            prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
+        }
+        lines.push_back(indent + "sum += " + prod + ";");
+        for (size_t j = 0; j < s.contr.size(); ++j)
+        {
+            indent.resize(indent.size() - 4);
+            lines.push_back(indent + "}");
+        }
+        const std::string gaddr = PtrName(s.out.uvar) + "[o_k" + str(k) + "g]";
+        const std::string laddr = "lds[o_k" + str(k) + "l]";
+        if (s.op == '=')
+            lines.push_back("const double r = sum;");
+        else
+            lines.push_back(std::string("const double r = ") + (OldValueInLds(k) ? laddr : gaddr) +
+                            (s.op == '+' ? " + sum;" : " - sum;"));
+        if (NeedsLdsCopy(k)) lines.push_back(laddr + " = r;");
+        if (!uvars[s.out.uvar].elide) lines.push_back(gaddr + " = r;");
+    }
+
+    void Emit(HipKernelPlan &plan)
+    {
+        const int K = static_cast<int>(subs.size());
+        const int U = static_cast<int>(uvars.size());
+        const std::string dimName = mk.GetDimensionedNameString();
+        std::string variant = str(NB) + "/" + str(NT) + "/" + (opt.noalias ? "n" : "a") + (Positional() ? "p" : "u");
+        for (int u = 0; u < U; ++u) variant += uvars[u].elide ? "e" : (uvars[u].inLds ? "l" : "g");
+        char hex[32];
+        std::snprintf(hex, sizeof(hex), "%016llx", static_cast<unsigned long long>(hashString(dimName + variant)));
+        plan.function_name = std::string("acro_mk_") + hex;
+
+        std::ostringstream sched;
+        sched << "batch index " << (batch >= 0 ? idxName[batch] : std::string("(none)")) << " extent " << E << ", " << NB
+              << " per workgroup of " << NT << " lanes, LDS " << ldsDoubles * 8 << " bytes\n";
+        for (int k = 0; k < K; ++k)
+        {
+            const Sub &s = subs[k];
+            sched << "  [" << k << "] " << s.text << " : lanes(";
+            for (size_t j = 0; j < s.lane.size(); ++j) sched << (j ? "," : "") << idxName[s.lane[j]];
+            sched << ")=" << s.laneCount << " tile(";
+            for (size_t j = 0; j < s.tile.size(); ++j) sched << (j ? "," : "") << idxName[s.tile[j]];
+            sched << ")=" << s.tileCount << " contraction=" << s.contrCount << (s.loopMode ? " looped" : " unrolled")
+                  << (s.fusedWithPrev ? " in-register after previous" : "") << "; operands:";
+            for (size_t v = 0; v < s.in.size(); ++v)
+            {
+                static const char *const names[] = {"registers", "scalar", "lds", "global"};
+                sched << " " << uvars[s.in[v].uvar].name << "<-" << names[SourceOf(k, static_cast<int>(v))];
+            }
+            const UVarInfo &uo = uvars[s.out.uvar];
+            sched << "; " << uo.name << "->" << (NeedsLdsCopy(k) ? "lds" : "") << (uo.elide ? "" : (NeedsLdsCopy(k) ? "+global" : "global"))
+                  << "\n";
+        }
+        plan.schedule = sched.str();
+
+        out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
+        {
+            std::istringstream lines(plan.schedule);
+            std::string l;
+            while (std::getline(lines, l)) out << "// " << l << "\n";
+        }
+        out << "typedef const __attribute__((address_space(4))) double *acro_scalar_ptr;\n\n";
+        out << "extern \"C\" __global__ __launch_bounds__(" << NT << ") void " << plan.function_name << "(";
+        for (int u = 0; u < U; ++u)
+        {
+            const bool constant = !uvars[u].written;
+            out << (u ? ", " : "") << (constant ? "const double *" : "double *") << (opt.noalias ? "__restrict__ " : "")
+                << PtrName(u);
+        }
+        out << ")\n{\n";
+        if (ldsDoubles > 0) out << "    __shared__ double lds[" << ldsDoubles << "];\n";
+        std::set<int> scalarVars;
+        for (int k = 0; k < K; ++k)
+        {
+            for (size_t v = 0; v < subs[k].in.size(); ++v)
+            {
+                if (SourceOf(k, static_cast<int>(v)) == kFromConstant) scalarVars.insert(subs[k].in[v].uvar);
+            }
+        }
+        for (int u : scalarVars)
+            out << "    const acro_scalar_ptr " << ConstPtrName(u) << " = (acro_scalar_ptr)" << PtrName(u) << ";\n";
+        out << "    const int tid = threadIdx.x;\n";
+        out << "    const int e0 = blockIdx.x * " << NB << ";\n";
+
+        const bool guardBatch = (E % NB) != 0;
+        int k = 0;
+        bool first = true;
+        while (k < K)
+        {
+            int last = k;
+            while (last + 1 < K && subs[last + 1].fusedWithPrev) ++last;
+            const Sub &s = subs[k];
+            if (!first) out << "    __syncthreads();\n";
+            first = false;
+            const long W = static_cast<long>(NB) * s.laneCount;
+            out << "    for (int w = tid; w < " << W << "; w += " << NT << ")\n    {\n";
+            out << "        const int b = w / " << s.laneCount << ";\n";
+            out << "        const int e = e0 + b;\n";
+            if (guardBatch) out << "        if (e >= " << E << ") break;\n";
+            if (!s.lane.empty())
+            {
+                out << "        const int r_ = w - b * " << s.laneCount << ";\n";
+                long st = s.laneCount;
+                for (size_t j = 0; j < s.lane.size(); ++j)
+                {
+                    const int id = s.lane[j];
+                    st /= extent[id];
+                    out << "        const int " << IdxVar(id) << " = ";
+                    if (j == 0)
+                        out << "r_ / " << st << ";\n";
+                    else
+                        out << "(r_ / " << st << ") % " << extent[id] << ";\n";
+                }
+            }
+            std::map<long, std::string> forwarded;
+            for (int kk = k; kk <= last; ++kk)
+            {
+                std::vector<std::string> lines;
+                if (subs[kk].loopMode)
+                    EmitLoopBody(kk, lines);
+                else
+                    EmitUnrolledBody(kk, forwarded, lines);
+                // Scopes nest (closed after the group) so that a kernel applied in registers sees the values
+                // of its producer.
+                out << "        {\n";
+                for (const auto &l : lines) out << "            " << l << "\n";
+            }
+            for (int kk = k; kk <= last; ++kk) out << "        }\n";
+            out << "    }\n";
+            k = last + 1;
+        }
+        out << "}\n";
+
+        plan.source = out.str();
+        plan.grid = static_cast<unsigned>((E + NB - 1) / NB);
+        plan.block = static_cast<unsigned>(NT);
+        plan.nb = NB;
+        plan.lds_bytes = ldsDoubles * 8;
+        plan.param_occurrence.resize(U);
+        plan.stored.assign(U, false);
+        for (int u = 0; u < U; ++u)
+        {
+            plan.param_occurrence[u] = FirstOccurrence(u);
+            plan.stored[u] = uvars[u].written && !uvars[u].elide;
+        }
+    }
+};
+
+}  // namespace
+
+HipKernelPlan GenerateHipKernel(const DimensionedMultiKernel &mk, const HipCodegenOptions &options)
+{
+    Generator g(mk, options);
+    return g.Run();
+}
+
+}  // namespace acro

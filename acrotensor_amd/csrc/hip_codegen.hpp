@@ -1,0 +1,64 @@
+// Kernel code generator of the "HIP" policy: DimensionedMultiKernel -> fixed-size HIP C++ source for gfx950.
+// Replaces the reference's CUDA text generator (exec/CudaExecutor.cpp:111-702) with a different schedule,
+// designed for 64-wide wavefronts and HBM-bound finite-element chains:
+//
+//  * One workgroup owns NB consecutive values of the batch index (the largest index shared as an outer index by
+//    every kernel of the group - the "element" index) and runs every kernel of the group on them, separated by
+//    workgroup barriers.  Nothing is exchanged between workgroups.
+//  * Inside a kernel a lane owns one "pencil": fixed values of the lane indices and ALL values of the tile
+//    indices.  Contraction and tile loops are fully unrolled; every operand entry is loaded once per pencil and
+//    partial sums that do not depend on an inner index are hoisted (sum factorisation inside the lane).
+//  * Small operands that do not vary with the lane (basis matrices) are read through the constant address space,
+//    i.e. with scalar loads into SGPRs, and feed the FMAs as scalar operands.
+//  * An output that a later kernel of the group consumes stays in LDS (one tile per batch entry); its store to
+//    device memory is skipped when the tensor is marked transient.  A kernel without contraction whose operand
+//    was just produced with the same index set is applied in registers (no LDS round trip).
+//  * Contractions too long to unroll fall back to counted loops with the same lane mapping.
+#ifndef ACRO_HIP_CODEGEN_HPP
+#define ACRO_HIP_CODEGEN_HPP
+
+#include <string>
+#include <utility>
+#include <vector>
+#include "DimensionedMultiKernel.hpp"
+
+namespace acro
+{
+
+struct HipCodegenOptions
+{
+    // Per unique variable: the executor allows the store to device memory to be dropped (transient tensor).
+    std::vector<bool> transient;
+    // False when two unique variables overlap in device memory and one of them is written: pointers are then
+    // not declared restrict and nothing is read through the constant address space.
+    bool noalias = true;
+    // Single kernels only: every variable occurrence is a separate operand even when two occurrences share a
+    // name (the caller bound them to different tensors).  transient is then indexed by occurrence: output, then
+    // inputs in order.
+    bool positional = false;
+    int force_nb = 0;  // 0 = choose
+    int force_nt = 0;  // 0 = choose
+};
+
+struct HipKernelPlan
+{
+    bool fusable = false;        // false: the group must be run as one launch per kernel
+    std::string why_not;         // reason when !fusable
+    std::string function_name;
+    std::string source;
+    unsigned grid = 0;
+    unsigned block = 0;
+    // Kernel parameter i is the device pointer of the tensor bound to this (kernel number, variable number)
+    // occurrence; variable number -1 is that kernel's output.
+    std::vector<std::pair<int, int>> param_occurrence;
+    std::vector<bool> stored;      // per parameter: the kernel writes it to device memory
+    int lds_bytes = 0;
+    int nb = 0;
+    std::string schedule;          // human readable schedule summary (also a comment in the source)
+};
+
+HipKernelPlan GenerateHipKernel(const DimensionedMultiKernel &mk, const HipCodegenOptions &options);
+
+}  // namespace acro
+
+#endif

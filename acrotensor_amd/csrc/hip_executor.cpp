@@ -1,0 +1,195 @@
+// HipExecutor — the "HIP" execution policy: generates, compiles and launches one fused kernel per
+// DimensionedMultiKernel.  Takes the place of the reference's CudaExecutor launch glue
+// (exec/CudaExecutor.cpp:17-108: constructor JIT, ExecuteSingle / ExecuteMulti pointer packing, GetImplementation).
+//
+// Differences that matter to callers:
+//  * kernels are generated lazily (first execution or GetImplementation) and per "binding variant": which
+//    tensors are transient (their stores may be dropped) and whether any two variables overlap in device memory;
+//  * a group that cannot be fused safely (no common outer index, a variable used with different shapes, or
+//    overlapping variables of which one is written) is executed as one launch per kernel, in stream order;
+//  * everything is enqueued on the library's stream and never synchronised here.
+#include <map>
+#include <memory>
+
+#include "HipRuntime.hpp"
+#include "KernelExecutor.hpp"
+#include "hip_codegen.hpp"
+#include "hip_kernel.hpp"
+
+namespace acro
+{
+
+class HipExecutor : public KernelExecutor
+{
+  public:
+    explicit HipExecutor(DimensionedMultiKernel *multi_kernel) : KernelExecutor(multi_kernel) {}
+    ~HipExecutor() override {}
+
+    std::string GetExecType() override { return "HIP"; }
+
+    std::string GetImplementation() override
+    {
+        if (LastVariant != nullptr) return Describe(*LastVariant);
+        HipCodegenOptions options;
+        options.transient.assign(MultiKernel->GetNumUVars(), false);
+        return Describe(GetVariant(options));
+    }
+
+    std::string GetImplementation(std::vector<Tensor *> &outputs, std::vector<std::vector<Tensor *>> &inputs) override
+    {
+        HipCodegenOptions options;
+        bool fallback = false;
+        Bind(outputs, inputs, options, fallback);
+        if (fallback) return "// not fused (overlapping or re-bound variables): one launch per kernel\n";
+        return Describe(GetVariant(options));
+    }
+
+    void ExecuteSingle(Tensor *output, std::vector<Tensor *> &inputs) override
+    {
+        std::vector<Tensor *> outs(1, output);
+        std::vector<std::vector<Tensor *>> ins(1, inputs);
+        Execute(outs, ins);
+    }
+
+    void ExecuteMulti(std::vector<Tensor *> &output, std::vector<std::vector<Tensor *>> &inputs) override
+    {
+        Execute(output, inputs);
+    }
+
+  private:
+    struct Variant
+    {
+        HipKernelPlan plan;
+        std::unique_ptr<HipKernel> kernel;  // null when the group is not fusable
+    };
+
+    std::string Describe(const Variant &v)
+    {
+        if (v.plan.fusable) return v.plan.source;
+        return "// not fused (" + v.plan.why_not + "): one launch per kernel\n";
+    }
+
+    Variant &GetVariant(const HipCodegenOptions &options)
+    {
+        std::string key = std::string(options.noalias ? "n" : "a") + (options.positional ? "p" : "u");
+        for (bool t : options.transient) key += t ? '1' : '0';
+        auto it = Variants.find(key);
+        if (it == Variants.end())
+        {
+            std::unique_ptr<Variant> v(new Variant);
+            v->plan = GenerateHipKernel(*MultiKernel, options);
+            if (v->plan.fusable) v->kernel.reset(new HipKernel(v->plan.function_name, v->plan.source));
+            it = Variants.emplace(key, std::move(v)).first;
+        }
+        LastVariant = it->second.get();
+        return *LastVariant;
+    }
+
+    // Decides how the tensors of this call bind to kernel operands.  Variables are identified by name, as in the
+    // reference's exec/CudaExecutor.cpp:83-99; when one name is bound to two different tensors a group falls back
+    // to one launch per kernel and a single kernel switches to one operand per occurrence.  Also the aliasing
+    // analysis: two different operands that overlap in memory, one of them written, forbid restrict / scalar
+    // reads (single kernel) or fusion (group).  Host buffers mirror device buffers one to one, so the analysis
+    // works before anything is mapped to the device.
+    void Bind(std::vector<Tensor *> &outputs, std::vector<std::vector<Tensor *>> &inputs, HipCodegenOptions &options,
+              bool &fallback)
+    {
+        const int K = MultiKernel->GetNumKernels();
+        ACROBATIC_ASSERT(static_cast<int>(outputs.size()) == K && static_cast<int>(inputs.size()) == K,
+                         "Number of tensor lists does not match the number of kernels.");
+        auto tensorAt = [&](int ki, int vari) { return vari < 0 ? outputs[ki] : inputs[ki][vari]; };
+        auto sameStorage = [](const Tensor *a, const Tensor *b) {
+            return a == b || (a->GetData() == b->GetData() && a->GetSize() == b->GetSize());
+        };
+
+        bool rebound = false;
+        for (int ki = 0; ki < K; ++ki)
+        {
+            for (int vari = -1; vari < MultiKernel->Kernels[ki]->GetNumInputVars(); ++vari)
+            {
+                auto first = MultiKernel->GetFirstKiVariForUVari(MultiKernel->GetUVari(ki, vari));
+                if (!sameStorage(tensorAt(ki, vari), tensorAt(first.first, first.second))) rebound = true;
+            }
+        }
+        options.positional = (K == 1 && rebound);
+
+        std::vector<Tensor *> operand;
+        std::vector<bool> written;
+        if (options.positional)
+        {
+            for (int vari = -1; vari < MultiKernel->Kernels[0]->GetNumInputVars(); ++vari)
+            {
+                operand.push_back(tensorAt(0, vari));
+                written.push_back(vari < 0);
+            }
+        }
+        else
+        {
+            for (int u = 0; u < MultiKernel->GetNumUVars(); ++u)
+            {
+                auto first = MultiKernel->GetFirstKiVariForUVari(u);
+                operand.push_back(tensorAt(first.first, first.second));
+                written.push_back(MultiKernel->IsOutputUVar(u));
+            }
+        }
+        options.transient.assign(operand.size(), false);
+        bool hazard = false;
+        for (size_t a = 0; a < operand.size(); ++a)
+        {
+            options.transient[a] = operand[a]->IsTransient();
+            for (size_t b = a + 1; b < operand.size(); ++b)
+            {
+                const double *pa = operand[a]->GetData(), *pb = operand[b]->GetData();
+                const bool overlap = pa < pb + operand[b]->GetSize() && pb < pa + operand[a]->GetSize();
+                if (overlap && (written[a] || written[b])) hazard = true;
+            }
+        }
+        fallback = K > 1 && (hazard || rebound);
+        options.noalias = !hazard;
+    }
+
+    void Execute(std::vector<Tensor *> &outputs, std::vector<std::vector<Tensor *>> &inputs)
+    {
+        const int K = MultiKernel->GetNumKernels();
+        ACROBATIC_ASSERT(static_cast<int>(outputs.size()) == K && static_cast<int>(inputs.size()) == K,
+                         "Number of tensor lists does not match the number of kernels.");
+        for (int ki = 0; ki < K; ++ki) MoveTensorsToGPU(outputs[ki], inputs[ki]);
+
+        HipCodegenOptions options;
+        bool fallback = false;
+        Bind(outputs, inputs, options, fallback);
+        if (fallback)
+        {
+            KernelExecutor::ExecuteMulti(outputs, inputs);
+            return;
+        }
+        Variant &v = GetVariant(options);
+        if (!v.plan.fusable)
+        {
+            ACROBATIC_ASSERT(K > 1, "Internal error: a single kernel must always be executable.");
+            KernelExecutor::ExecuteMulti(outputs, inputs);
+            return;
+        }
+        const size_t nparam = v.plan.param_occurrence.size();
+        std::vector<double *> ptr(nparam);
+        std::vector<void *> args(nparam);
+        for (size_t i = 0; i < nparam; ++i)
+        {
+            const auto &occ = v.plan.param_occurrence[i];
+            ptr[i] = (occ.second < 0 ? outputs[occ.first] : inputs[occ.first][occ.second])->GetDeviceData();
+            ACROBATIC_ASSERT(ptr[i] != nullptr, "Tensor has no device memory.");
+            args[i] = &ptr[i];
+        }
+        v.kernel->Launch(v.plan.grid, v.plan.block, args.data());
+    }
+
+    std::map<std::string, std::unique_ptr<Variant>> Variants;
+    Variant *LastVariant = nullptr;
+};
+
+KernelExecutor *CreateHipExecutor(DimensionedMultiKernel *multi_kernel)
+{
+    return new HipExecutor(multi_kernel);
+}
+
+}  // namespace acro

@@ -1,0 +1,182 @@
+#include "hip_kernel.hpp"
+
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <iostream>
+
+#include "HipRuntime.hpp"
+
+namespace acro
+{
+
+namespace
+{
+
+const char *const kCompileOptions[] = {
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+};
+constexpr int kNumCompileOptions = sizeof(kCompileOptions) / sizeof(kCompileOptions[0]);
+
+uint64_t fnv1a(const std::string &s, uint64_t h = 1469598103934665603ull)
+{
+    for (unsigned char c : s)
+    {
+        h ^= c;
+        h *= 1099511628211ull;
+    }
+    return h;
+}
+
+std::string cacheDir()
+{
+    const char *env = std::getenv("ACRO_HIP_CACHE_DIR");
+    if (env != nullptr)
+    {
+        if (std::string(env) == "off" || std::string(env).empty()) return "";
+        return env;
+    }
+    const char *home = std::getenv("HOME");
+    if (home == nullptr || *home == '\0') return "";
+    return std::string(home) + "/.cache/acrotensor_hip";
+}
+
+bool makeDirs(const std::string &path)
+{
+    std::string partial;
+    for (size_t i = 0; i <= path.size(); ++i)
+    {
+        if (i == path.size() || path[i] == '/')
+        {
+            if (!partial.empty() && ::mkdir(partial.c_str(), 0755) != 0 && errno != EEXIST) return false;
+        }
+        if (i < path.size()) partial += path[i];
+    }
+    return true;
+}
+
+std::string cachePath(const std::string &name, const std::string &source)
+{
+    std::string dir = cacheDir();
+    if (dir.empty()) return "";
+    int major = 0, minor = 0;
+    hiprtcVersion(&major, &minor);
+    std::string salt = std::to_string(major) + "." + std::to_string(minor);
+    for (int i = 0; i < kNumCompileOptions; ++i) salt += std::string(" ") + kCompileOptions[i];
+    uint64_t h = fnv1a(source, fnv1a(salt + name));
+    char hex[32];
+    std::snprintf(hex, sizeof(hex), "%016llx", static_cast<unsigned long long>(h));
+    return dir + "/" + hex + ".hsaco";
+}
+
+void rtcCheck(hiprtcResult r, const char *what)
+{
+    if (r != HIPRTC_SUCCESS)
+    {
+        throw_error(std::string("hipRTC failure in ") + what + ": " + hiprtcGetErrorString(r));
+    }
+}
+
+}  // namespace
+
+HipKernel::HipKernel(const std::string &function_name, const std::string &source)
+    : FunctionName(function_name), Source(source), CacheHit(false), Module(nullptr), Function(nullptr)
+{
+    Compile();
+}
+
+HipKernel::~HipKernel()
+{
+    if (Module != nullptr) (void)hipModuleUnload(static_cast<hipModule_t>(Module));
+}
+
+void HipKernel::Compile()
+{
+    const std::string path = cachePath(FunctionName, Source);
+    if (!path.empty())
+    {
+        std::ifstream in(path, std::ios::binary | std::ios::ate);
+        if (in)
+        {
+            std::streamsize n = in.tellg();
+            in.seekg(0);
+            CodeObject.resize(static_cast<size_t>(n));
+            if (n > 0 && in.read(CodeObject.data(), n))
+            {
+                CacheHit = true;
+                return;
+            }
+            CodeObject.clear();
+        }
+    }
+
+    hiprtcProgram prog;
+    rtcCheck(hiprtcCreateProgram(&prog, Source.c_str(), (FunctionName + ".hip").c_str(), 0, nullptr, nullptr),
+             "hiprtcCreateProgram");
+    hiprtcResult result = hiprtcCompileProgram(prog, kNumCompileOptions, const_cast<const char **>(kCompileOptions));
+    if (result != HIPRTC_SUCCESS)
+    {
+        size_t log_size = 0;
+        hiprtcGetProgramLogSize(prog, &log_size);
+        std::string log(log_size, '\0');
+        if (log_size > 0) hiprtcGetProgramLog(prog, &log[0]);
+        hiprtcDestroyProgram(&prog);
+        std::cerr << "---- generated kernel that failed to compile ----\n"
+                  << Source << "\n---- compiler log ----\n"
+                  << log << std::endl;
+        throw_error("hipRTC compilation of " + FunctionName + " failed:\n" + log);
+    }
+    size_t code_size = 0;
+    rtcCheck(hiprtcGetCodeSize(prog, &code_size), "hiprtcGetCodeSize");
+    CodeObject.resize(code_size);
+    rtcCheck(hiprtcGetCode(prog, CodeObject.data()), "hiprtcGetCode");
+    hiprtcDestroyProgram(&prog);
+
+    if (!path.empty() && makeDirs(cacheDir()))
+    {
+        // Write to a private name first so that a concurrent reader never sees a partial file.
+        std::string tmp = path + ".tmp" + std::to_string(static_cast<long>(::getpid()));
+        std::ofstream out(tmp, std::ios::binary);
+        if (out && out.write(CodeObject.data(), static_cast<std::streamsize>(CodeObject.size())))
+        {
+            out.close();
+            if (std::rename(tmp.c_str(), path.c_str()) != 0) std::remove(tmp.c_str());
+        }
+    }
+}
+
+void HipKernel::EnsureLoaded()
+{
+    if (Function != nullptr) return;
+    hipModule_t module;
+    ACRO_HIP_CHECK(hipModuleLoadData(&module, CodeObject.data()));
+    Module = module;
+    hipFunction_t function;
+    ACRO_HIP_CHECK(hipModuleGetFunction(&function, module, FunctionName.c_str()));
+    Function = function;
+}
+
+void HipKernel::Launch(unsigned grid, unsigned block, void **args)
+{
+    EnsureLoaded();
+    ACRO_HIP_CHECK(hipModuleLaunchKernel(static_cast<hipFunction_t>(Function), grid, 1, 1, block, 1, 1, 0,
+                                         static_cast<hipStream_t>(hip::Stream()), args, nullptr));
+}
+
+void HipKernel::WriteCodeToFile(const std::string &path) const
+{
+    std::ofstream out(path);
+    ACROBATIC_ASSERT(static_cast<bool>(out), "Can't open " + path + " for writing.");
+    out << Source;
+}
+
+}  // namespace acro

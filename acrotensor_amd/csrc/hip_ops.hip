@@ -1,0 +1,246 @@
+// Precompiled device kernels of the "HIP" policy that are not generated per contraction:
+// fill / scale (reference util/CudaUtil.cpp:123-140), batched 1x1 / 2x2 / 3x3 inverse, determinant and fused
+// inverse+determinant (reference ops/CudaGPUOps.cpp:13-80,108-275), indexed scatter and compressed-row sum-gather
+// (reference ops/CudaGPUOps.cpp:83-105,278-302).
+//
+// Layout: matrices are stored one after the other (9, 4 or 1 doubles each).  A workgroup of 256 lanes owns 256
+// consecutive matrices; it moves their doubles between HBM and LDS with unit-stride 16-byte accesses and each
+// lane then works on "its" matrix out of LDS, so HBM only sees full, contiguous lines.  The lane stride in LDS is
+// 9 (or 4+1 padded to 5) doubles, which maps the 32 lanes of a half wave onto distinct banks.
+//
+// Arithmetic is written term by term in the order of the reference's ops/NativeCPUOps.hpp:38-86 and compiled
+// without multiply-add contraction, so results are bit-identical to the host formulas.
+#include <hip/hip_runtime.h>
+
+#include "HipRuntime.hpp"
+#include "NonContractionOps.hpp"
+
+#pragma clang fp contract(off)
+
+namespace acro
+{
+
+namespace
+{
+
+constexpr int kLanes = 256;
+
+__global__ __launch_bounds__(kLanes) void fillKernel(double *__restrict__ d, double value, size_t n)
+{
+    size_t i = static_cast<size_t>(blockIdx.x) * kLanes + threadIdx.x;
+    if (i < n) d[i] = value;
+}
+
+__global__ __launch_bounds__(kLanes) void scaleKernel(double *__restrict__ d, double factor, size_t n)
+{
+    size_t i = static_cast<size_t>(blockIdx.x) * kLanes + threadIdx.x;
+    if (i < n) d[i] *= factor;
+}
+
+template <int M>
+struct SmallMatrix;
+
+template <>
+struct SmallMatrix<1>
+{
+    static __device__ double det(const double *A) { return A[0]; }
+    static __device__ void inv(double *Ainv, const double *, double det) { Ainv[0] = 1.0 / det; }
+};
+
+template <>
+struct SmallMatrix<2>
+{
+    static __device__ double det(const double *A) { return A[0] * A[3] - A[1] * A[2]; }
+    static __device__ void inv(double *Ainv, const double *A, double det)
+    {
+        const double invdet = 1.0 / det;
+        Ainv[0] = invdet * A[3];
+        Ainv[1] = -invdet * A[1];
+        Ainv[2] = -invdet * A[2];
+        Ainv[3] = invdet * A[0];
+    }
+};
+
+template <>
+struct SmallMatrix<3>
+{
+    static __device__ double det(const double *A)
+    {
+        return A[0] * A[4] * A[8] + A[1] * A[5] * A[6] + A[2] * A[3] * A[7] - A[6] * A[4] * A[2] -
+               A[7] * A[5] * A[0] - A[8] * A[3] * A[1];
+    }
+    // Cofactors over the determinant WITHOUT the final transposition: for a non-symmetric matrix this is the
+    // transpose of the inverse, which is what the reference's host and device code both produce.
+    static __device__ void inv(double *Ainv, const double *A, double det)
+    {
+        const double invdet = 1.0 / det;
+        Ainv[0] = invdet * (A[4] * A[8] - A[5] * A[7]);
+        Ainv[1] = invdet * (A[5] * A[6] - A[3] * A[8]);
+        Ainv[2] = invdet * (A[3] * A[7] - A[4] * A[6]);
+        Ainv[3] = invdet * (A[2] * A[7] - A[1] * A[8]);
+        Ainv[4] = invdet * (A[0] * A[8] - A[2] * A[6]);
+        Ainv[5] = invdet * (A[1] * A[6] - A[0] * A[7]);
+        Ainv[6] = invdet * (A[1] * A[5] - A[2] * A[4]);
+        Ainv[7] = invdet * (A[2] * A[3] - A[0] * A[5]);
+        Ainv[8] = invdet * (A[0] * A[4] - A[1] * A[3]);
+    }
+};
+
+// One workgroup = kLanes consecutive matrices.  WANT_INV / WANT_DET select the outputs.
+template <int M, bool WANT_INV, bool WANT_DET>
+__global__ __launch_bounds__(kLanes) void batchMatrixKernel(const double *__restrict__ A, double *__restrict__ Ainv,
+                                                            double *__restrict__ Adet, size_t num_mat)
+{
+    constexpr int MM = M * M;
+    constexpr int LS = (MM % 2 == 0) ? MM + 1 : MM;  // odd lane stride in doubles: no LDS bank conflicts
+    __shared__ double tile[kLanes * LS];
+
+    const size_t first = static_cast<size_t>(blockIdx.x) * kLanes;
+    const size_t count = (num_mat - first < static_cast<size_t>(kLanes)) ? num_mat - first : kLanes;
+    const int ndbl = static_cast<int>(count) * MM;
+    const double *src = A + first * MM;
+
+    for (int i = threadIdx.x; i < ndbl; i += kLanes) tile[(i / MM) * LS + (i % MM)] = src[i];
+    __syncthreads();
+
+    double a[MM], r[MM];
+    const bool active = threadIdx.x < count;
+    if (active)
+    {
+#pragma unroll
+        for (int j = 0; j < MM; ++j) a[j] = tile[threadIdx.x * LS + j];
+        const double det = SmallMatrix<M>::det(a);
+        if (WANT_DET) Adet[first + threadIdx.x] = det;
+        if (WANT_INV) SmallMatrix<M>::inv(r, a, det);
+    }
+    if (WANT_INV)
+    {
+        __syncthreads();
+        if (active)
+        {
+#pragma unroll
+            for (int j = 0; j < MM; ++j) tile[threadIdx.x * LS + j] = r[j];
+        }
+        __syncthreads();
+        double *dst = Ainv + first * MM;
+        for (int i = threadIdx.x; i < ndbl; i += kLanes) dst[i] = tile[(i / MM) * LS + (i % MM)];
+    }
+}
+
+__global__ __launch_bounds__(kLanes) void scatterKernel(double *__restrict__ Aout, const double *__restrict__ Ain,
+                                                        const int *__restrict__ M, int range_size)
+{
+    int i = blockIdx.x * kLanes + threadIdx.x;
+    if (i < range_size) Aout[i] = Ain[M[i]];
+}
+
+// Row d of the inverse map lists, in increasing range order, the entries that are added into Aout[d]; summing
+// them front to back reproduces the sequential host scatter-add bit for bit and needs no atomics.
+__global__ __launch_bounds__(kLanes) void sumGatherKernel(double *__restrict__ Aout, const double *__restrict__ Ain,
+                                                          const int *__restrict__ InvM,
+                                                          const int *__restrict__ InvMOff, int domain_size)
+{
+    int d = blockIdx.x * kLanes + threadIdx.x;
+    if (d >= domain_size) return;
+    double sum = 0.0;
+    const int end = InvMOff[d + 1];
+    for (int k = InvMOff[d]; k < end; ++k) sum += Ain[InvM[k]];
+    Aout[d] = sum;
+}
+
+unsigned gridFor(size_t n)
+{
+    size_t blocks = (n + kLanes - 1) / kLanes;
+    ACROBATIC_ASSERT(blocks <= 0x7fffffffu, "Operand too large for a one-dimensional grid.");
+    return static_cast<unsigned>(blocks == 0 ? 1 : blocks);
+}
+
+hipStream_t stream()
+{
+    return static_cast<hipStream_t>(hip::Stream());
+}
+
+template <bool WANT_INV, bool WANT_DET>
+void launchBatchMatrix(int mdim, const double *A, double *Ainv, double *Adet, size_t num_mat)
+{
+    const unsigned grid = gridFor(num_mat);
+    switch (mdim)
+    {
+        case 1:
+            hipLaunchKernelGGL((batchMatrixKernel<1, WANT_INV, WANT_DET>), dim3(grid), dim3(kLanes), 0, stream(), A,
+                               Ainv, Adet, num_mat);
+            break;
+        case 2:
+            hipLaunchKernelGGL((batchMatrixKernel<2, WANT_INV, WANT_DET>), dim3(grid), dim3(kLanes), 0, stream(), A,
+                               Ainv, Adet, num_mat);
+            break;
+        case 3:
+            hipLaunchKernelGGL((batchMatrixKernel<3, WANT_INV, WANT_DET>), dim3(grid), dim3(kLanes), 0, stream(), A,
+                               Ainv, Adet, num_mat);
+            break;
+        default:
+            ACROBATIC_ASSERT(false, "Batched matrix ops support 1x1, 2x2 and 3x3 matrices only.");
+    }
+    ACRO_HIP_CHECK(hipGetLastError());
+}
+
+size_t numMatrices(const Tensor &A)
+{
+    const int m = A.GetDim(A.GetRank() - 1);
+    return static_cast<size_t>(A.GetSize()) / (static_cast<size_t>(m) * m);
+}
+
+}  // namespace
+
+namespace hip
+{
+
+void FillDouble(double *d, double value, size_t n)
+{
+    hipLaunchKernelGGL(fillKernel, dim3(gridFor(n)), dim3(kLanes), 0, stream(), d, value, n);
+    ACRO_HIP_CHECK(hipGetLastError());
+}
+
+void ScaleDouble(double *d, double factor, size_t n)
+{
+    hipLaunchKernelGGL(scaleKernel, dim3(gridFor(n)), dim3(kLanes), 0, stream(), d, factor, n);
+    ACRO_HIP_CHECK(hipGetLastError());
+}
+
+}  // namespace hip
+
+void HipGPUOps::BatchMatrixInverse(Tensor &Ainv, Tensor &A)
+{
+    launchBatchMatrix<true, false>(A.GetDim(A.GetRank() - 1), A.GetDeviceData(), Ainv.GetDeviceData(), nullptr,
+                                   numMatrices(A));
+}
+
+void HipGPUOps::BatchMatrixDet(Tensor &Adet, Tensor &A)
+{
+    launchBatchMatrix<false, true>(A.GetDim(A.GetRank() - 1), A.GetDeviceData(), nullptr, Adet.GetDeviceData(),
+                                   numMatrices(A));
+}
+
+void HipGPUOps::BatchMatrixInvDet(Tensor &Ainv, Tensor &Adet, Tensor &A)
+{
+    launchBatchMatrix<true, true>(A.GetDim(A.GetRank() - 1), A.GetDeviceData(), Ainv.GetDeviceData(),
+                                  Adet.GetDeviceData(), numMatrices(A));
+}
+
+void HipGPUOps::FlatIndexedScatter(Tensor &Aout, Tensor &Ain, IndexMapping &M)
+{
+    const int n = M.GetRangeSize();
+    hipLaunchKernelGGL(scatterKernel, dim3(gridFor(n)), dim3(kLanes), 0, stream(), Aout.GetDeviceData(),
+                       Ain.GetDeviceData(), M.GetMap().GetDeviceData(), n);
+    ACRO_HIP_CHECK(hipGetLastError());
+}
+
+void HipGPUOps::FlatIndexedSumGather(Tensor &Aout, Tensor &Ain, IndexMapping &M)
+{
+    const int n = M.GetDomainSize();
+    hipLaunchKernelGGL(sumGatherKernel, dim3(gridFor(n)), dim3(kLanes), 0, stream(), Aout.GetDeviceData(),
+                       Ain.GetDeviceData(), M.GetInvMap().GetDeviceData(), M.GetInvMapOffsets().GetDeviceData(), n);
+    ACRO_HIP_CHECK(hipGetLastError());
+}
+
+}  // namespace acro

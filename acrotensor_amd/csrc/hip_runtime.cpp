@@ -1,0 +1,116 @@
+// Device memory and stream layer: the only place that owns a stream, allocates, copies and checks HIP errors.
+// Replaces the reference's util/CudaUtil.hpp:59-108 (error macros, context) and the cudaMalloc/cudaMemcpy/cudaFree
+// call sites of tensor/Tensor.cpp:370-428.
+#include <hip/hip_runtime.h>
+
+#include <iostream>
+#include <mutex>
+
+#include "HipRuntime.hpp"
+
+namespace acro
+{
+
+bool isHipReady()
+{
+    int n = 0;
+    hipError_t err = hipGetDeviceCount(&n);
+    if (err != hipSuccess)
+    {
+        (void)hipGetLastError();  // clear the sticky "no device" state
+        return false;
+    }
+    return n > 0;
+}
+
+namespace hip
+{
+
+void Check(int code, const char *file, int line)
+{
+    if (code == static_cast<int>(hipSuccess)) return;
+    std::string msg = std::string("HIP error: ") + hipGetErrorString(static_cast<hipError_t>(code));
+    std::cerr << file << ":" << line << "  " << msg << std::endl;
+    ::acro::detail::fail(file, line, msg);
+}
+
+namespace
+{
+std::mutex g_lock;
+hipStream_t g_own_stream = nullptr;
+hipStream_t g_adopted_stream = nullptr;
+bool g_have_info = false;
+DeviceInfo g_info;
+}  // namespace
+
+void *Stream()
+{
+    std::lock_guard<std::mutex> guard(g_lock);
+    if (g_adopted_stream != nullptr) return g_adopted_stream;
+    if (g_own_stream == nullptr)
+    {
+        ACRO_HIP_CHECK(hipStreamCreateWithFlags(&g_own_stream, hipStreamNonBlocking));
+    }
+    return g_own_stream;
+}
+
+void SetStream(void *hip_stream)
+{
+    std::lock_guard<std::mutex> guard(g_lock);
+    g_adopted_stream = static_cast<hipStream_t>(hip_stream);
+}
+
+void Synchronize()
+{
+    ACRO_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(Stream())));
+}
+
+void *Malloc(size_t bytes)
+{
+    void *p = nullptr;
+    ACRO_HIP_CHECK(hipMalloc(&p, bytes));
+    return p;
+}
+
+void Free(void *dptr)
+{
+    if (dptr == nullptr) return;
+    // Work that still uses the buffer may be queued on the stream.
+    ACRO_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(Stream())));
+    ACRO_HIP_CHECK(hipFree(dptr));
+}
+
+void CopyToDevice(void *dst, const void *src, size_t bytes)
+{
+    hipStream_t s = static_cast<hipStream_t>(Stream());
+    ACRO_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s));
+    ACRO_HIP_CHECK(hipStreamSynchronize(s));
+}
+
+void CopyToHost(void *dst, const void *src, size_t bytes)
+{
+    hipStream_t s = static_cast<hipStream_t>(Stream());
+    ACRO_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
+    ACRO_HIP_CHECK(hipStreamSynchronize(s));
+}
+
+const DeviceInfo &Info()
+{
+    std::lock_guard<std::mutex> guard(g_lock);
+    if (!g_have_info)
+    {
+        int dev = 0;
+        ACRO_HIP_CHECK(hipGetDevice(&dev));
+        hipDeviceProp_t prop;
+        ACRO_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+        g_info.num_cus = prop.multiProcessorCount;
+        g_info.lds_per_block = prop.sharedMemPerBlock;
+        g_info.wavefront = prop.warpSize;
+        g_info.arch = prop.gcnArchName;
+        g_have_info = true;
+    }
+    return g_info;
+}
+
+}  // namespace hip
+}  // namespace acro

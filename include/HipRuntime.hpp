@@ -1,0 +1,55 @@
+// Device memory and stream layer of the "HIP" policy (replaces the role of the reference's
+// util/CudaUtil.hpp:59-108,175-184: error checks, context handling, isCudaReady, and the cudaMalloc /
+// cudaMemcpy / cudaFree call sites in tensor/Tensor.cpp:370-428 and tensor/IndexVector.cpp:88-154).
+//
+// All device work of the library (copies, fills, generated kernels, batched ops) is issued on ONE stream that
+// this layer owns, so stream order alone makes producer/consumer sequences correct; only device-to-host
+// copies and explicit Synchronize() calls block the host.  Byte counts are size_t throughout.
+#ifndef ACRO_HIP_RUNTIME_HPP
+#define ACRO_HIP_RUNTIME_HPP
+
+#include <cstddef>
+#include <string>
+#include "Error.hpp"
+
+namespace acro
+{
+
+// True when a HIP device can be used by this process (hipGetDeviceCount > 0).  Never throws.
+bool isHipReady();
+
+namespace hip
+{
+// The stream every operation of the library is enqueued on (a hipStream_t passed as void* so that public
+// headers do not need the HIP headers).  Created lazily with default priority; never the null stream.
+void *Stream();
+// Adopt an externally created stream (the library then never destroys it).  nullptr restores the own stream.
+void SetStream(void *hip_stream);
+void Synchronize();
+
+void *Malloc(size_t bytes);
+void Free(void *dptr);
+void CopyToDevice(void *dst, const void *src, size_t bytes);    // returns after the host buffer may be reused
+void CopyToHost(void *dst, const void *src, size_t bytes);      // returns after the data has arrived
+void FillDouble(double *d, double value, size_t n);             // d[i] = value   (async on Stream())
+void ScaleDouble(double *d, double factor, size_t n);           // d[i] *= factor (async on Stream())
+
+// Multiprocessor count, LDS bytes per workgroup, wavefront size of the current device (cached).
+struct DeviceInfo
+{
+    int num_cus;
+    size_t lds_per_block;
+    int wavefront;
+    std::string arch;
+};
+const DeviceInfo &Info();
+
+// Throws std::runtime_error("<file>:  <line>  HIP error: ...") when code != hipSuccess.
+void Check(int hip_error_code, const char *file, int line);
+}  // namespace hip
+
+}  // namespace acro
+
+#define ACRO_HIP_CHECK(call) ::acro::hip::Check(static_cast<int>(call), __FILE__, __LINE__)
+
+#endif

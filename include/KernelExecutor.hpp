@@ -1,0 +1,53 @@
+// acro::KernelExecutor — the execution-policy plug-in boundary.  An executor is built for one
+// DimensionedMultiKernel and runs it on tensors supplied per call.  Interface as in the reference's
+// exec/KernelExecutor.hpp:16-45; the string-keyed factory (exec/KernelExecutor.cpp:106-121) is a registry here,
+// so a policy is added by registering a creator instead of editing a switch.
+#ifndef ACRO_HIP_KERNEL_EXECUTOR_HPP
+#define ACRO_HIP_KERNEL_EXECUTOR_HPP
+
+#include <string>
+#include <vector>
+#include "DimensionedMultiKernel.hpp"
+#include "Tensor.hpp"
+
+namespace acro
+{
+
+class KernelExecutor
+{
+  public:
+    explicit KernelExecutor(DimensionedMultiKernel *multi_kernel);
+    virtual ~KernelExecutor();
+
+    typedef KernelExecutor *(*Creator)(DimensionedMultiKernel *);
+    // Policy registry.  "HIP" is registered by the library itself.
+    static void Register(const std::string &exec_type, Creator creator);
+    static bool IsRegistered(const std::string &exec_type);
+    static KernelExecutor *Create(std::string exec_type, DimensionedMultiKernel *multi_kernel);
+
+    virtual std::string GetImplementation() = 0;
+    // Implementation that a launch on exactly these tensors would use (policies whose code depends on tensor
+    // properties override this; nothing is executed).
+    virtual std::string GetImplementation(std::vector<Tensor *> &, std::vector<std::vector<Tensor *>> &)
+    {
+        return GetImplementation();
+    }
+    virtual std::string GetExecType() = 0;
+    virtual void ExecuteSingle(Tensor *output, std::vector<Tensor *> &inputs) = 0;
+    // Default: one single-kernel executor per kernel, run in order
+    virtual void ExecuteMulti(std::vector<Tensor *> &output, std::vector<std::vector<Tensor *>> &inputs);
+
+  protected:
+    void MoveTensorsFromGPU(Tensor *output, std::vector<Tensor *> &inputs);
+    void MoveTensorsToGPU(Tensor *output, std::vector<Tensor *> &inputs);
+    void MoveTensorsToOutputLocation(Tensor *output, std::vector<Tensor *> &inputs);
+
+    DimensionedMultiKernel *MultiKernel;
+    DimensionedKernel *FirstKernel;
+    std::vector<DimensionedMultiKernel *> SubKernels;
+    std::vector<KernelExecutor *> SubExecutors;
+};
+
+}  // namespace acro
+
+#endif
