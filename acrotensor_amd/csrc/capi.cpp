@@ -495,7 +495,15 @@ int acro_describe_kernels(int num_kernels, const char *const *kernels, const int
                << ",\"contraction_indices\":" << jsonList(tk.ContractionIndexNames)
                << ",\"num_outer\":" << tk.GetNumOuterIndices() << ",\"loop_dims\":" << jsonList(dk.GetLoopDims())
                << ",\"flat_size\":" << dk.GetFlatIdxSize() << ",\"out_size\":" << dk.GetOutIdxSize()
-               << ",\"cont_size\":" << dk.GetContIdxSize() << ",\"vars\":[";
+               << ",\"cont_size\":" << dk.GetContIdxSize();
+            std::vector<int> out_req, in_req;
+            for (int nl = 0; nl <= dk.GetNumIndices(); ++nl)
+            {
+                out_req.push_back(dk.GetOutputStorageReqForInnerLoops(nl));
+                in_req.push_back(dk.GetInputStorageReqForInnerLoops(nl));
+            }
+            js << ",\"out_storage_inner\":" << jsonList(out_req) << ",\"in_storage_inner\":" << jsonList(in_req)
+               << ",\"vars\":[";
             for (int v = -1; v < tk.GetNumInputVars(); ++v)
             {
                 js << (v >= 0 ? "," : "") << "{\"name\":\"" << tk.GetVarName(v) << "\",\"indices\":"

@@ -1,0 +1,154 @@
+#!/usr/bin/env python3
+"""Headline benchmark: p=3 sum-factorised hex mass-operator apply, fp64, 2^18 elements, one MI355X.
+
+A step is one fused multi-kernel launch (7 contractions, X -> Y) over all elements with every tensor already
+resident in HBM.  Prints ONE JSON line:
+
+  value           GDOF/s over the timed steps, host-side TensorEngine overhead included (wall clock between two
+                  device synchronisations)
+  roofline        algorithmic bytes of one launch (X + D + Y = 2024 B per element) over the launch duration
+                  measured with HIP events on the library's stream, against the 8 TB/s HBM peak
+  cpu_baseline    the same chain on the host: the reference's own CPUInterpreted executor (oracle/_ref, kind
+                  "reference") or, if that library is absent, the plain-C restatement (kind "port"), one thread,
+                  on a bounded sample of elements
+  store_all       the same launch when the six intermediates are ordinary (non-transient) tensors, i.e. also
+                  written to HBM as the reference's generated kernel always does
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+METRIC = "GDOF/s + % HBM peak, p=3 sum-factorised hex mass apply fp64 (1 GPU)"
+
+# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a
+# copy kernel of known size); None until the profile summary under profiles/ has been taken for this kernel.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def time_steps(at, workloads, wl, engine, tensors, steps, warmup):
+    for _ in range(warmup):
+        workloads.launch(wl, engine, tensors)
+    at.synchronize()
+    t0 = time.perf_counter()
+    with at.hip_event_timer() as ev:
+        for _ in range(steps):
+            workloads.launch(wl, engine, tensors)
+    at.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, ev.ms * 1e-3
+
+
+def cpu_baseline(workloads, sample_elems):
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle  # tests/oracle.py - checker access, used here only for the reported CPU baseline
+
+    wl = workloads.config4(E=sample_elems)
+    if oracle.have_reference():
+        checker, kind = oracle.Reference(), "reference"
+    else:
+        checker, kind = oracle.Oracle(), "port"
+    t0 = time.perf_counter()
+    workloads.run_on_checker(wl, checker)
+    dt = time.perf_counter() - t0
+    return {
+        "value": wl.dof / dt * 1e-9,
+        "unit": "GDOF/s",
+        "cores": 1,
+        "kind": kind,
+        "sample": "%d of 262144 elements, whole 7-kernel chain, one pass, %.1f s" % (sample_elems, dt),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--elements", type=int, default=262144)
+    ap.add_argument("--cpu-sample-elems", type=int, default=131072)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-store-all", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the workload shards trivially over "
+                 "elements; see DESIGN.md).  Run with --gpus 1.")
+
+    import acrotensor_amd as at
+    from acrotensor_amd import workloads
+
+    if not at.is_hip_ready():
+        sys.exit("bench.py needs a HIP device; there is no host fallback.")
+
+    wl = workloads.config4(E=args.elements)
+    engine = at.TensorEngine("HIP")
+    tensors = workloads.bind_to_engine(wl, at, transient=True)
+    for t in tensors.values():
+        t.MoveToGPU()
+
+    wall, dev = time_steps(at, workloads, wl, engine, tensors, args.steps, args.warmup)
+    ms_per_step = wall / args.steps * 1e3
+    launch_s = dev / args.steps
+    achieved = wl.algorithmic_bytes / launch_s * 1e-9
+
+    result = {
+        "metric": METRIC,
+        "value": wl.dof * args.steps / wall * 1e-9,
+        "unit": "GDOF/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f64",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[3]: p=3 sum-factorised hex mass apply, E=%d, B[5,4] X[E,4,4,4] D[E,5,5,5], "
+                        "7-kernel multi-kernel launch, intermediates T1..V2 marked transient" % args.elements,
+            "elements": args.elements,
+            "dof": wl.dof,
+            "seed": wl.seed,
+        },
+        "pct_hbm_peak": 100.0 * achieved / HBM_PEAK_GBS,
+        "kernel_gdof_per_s": wl.dof / launch_s * 1e-9,
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": MEASURED_TRAFFIC_BYTES,
+            "algorithmic_bytes": wl.algorithmic_bytes,
+            "launch_us": launch_s * 1e6,
+        },
+    }
+
+    if not args.no_store_all:
+        for name in wl.transient:
+            tensors[name].SetTransient(False)
+        wall2, dev2 = time_steps(at, workloads, wl, engine, tensors, max(10, args.steps // 4), 5)
+        n2 = max(10, args.steps // 4)
+        stored_bytes = args.elements * (64 + 125 + 64 + 610) * 8
+        result["store_all"] = {
+            "value": wl.dof * n2 / wall2 * 1e-9,
+            "unit": "GDOF/s",
+            "launch_us": dev2 / n2 * 1e6,
+            "hbm_bytes_moved": stored_bytes,
+            "achieved_GBs_incl_intermediates": stored_bytes / (dev2 / n2) * 1e-9,
+        }
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(workloads, min(args.cpu_sample_elems, args.elements))
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,86 @@
+"""The code generator and the hipRTC compile step run without a device: generate, compile for gfx950 and inspect
+the source of kernels for the five baseline configurations and for the schedule's corner cases."""
+import numpy as np
+import pytest
+
+import acrotensor_amd as at
+from acrotensor_amd import workloads
+
+
+@pytest.fixture(scope="module")
+def TE():
+    return at.TensorEngine("HIP")
+
+
+def chain_source(TE, wl, transient):
+    tensors = workloads.bind_to_engine(wl, at, transient=transient)
+    TE.BeginMultiKernelLaunch()
+    for k, out, ins in wl.kernels:
+        TE(k, tensors[out], *[tensors[n] for n in ins])
+    return TE.EndMultiKernelLaunchGetImplementation()
+
+
+def test_single_contraction_source(TE):
+    A, C, B = at.Tensor(64, 9), at.Tensor(64, 9, 5), at.Tensor(5)
+    src = TE.GetImplementation("A_e_i = C_e_i_j B_j", A, C, B)
+    assert 'extern "C" __global__' in src and "__launch_bounds__" in src
+    assert "A_e_i = C_e_i_j B_j" in src                      # the kernel string is quoted in a comment
+    assert "batch index e extent 64" in src
+    assert "address_space(4)" in src and "B<-scalar" in src   # the small invariant operand is read with scalar loads
+
+
+def test_mass_apply_chain_keeps_intermediates_on_chip(TE):
+    src = chain_source(TE, workloads.config4(E=64), transient=True)
+    assert src.count("__syncthreads()") == 5                  # 7 kernels, one applied in registers: 6 phases
+    assert "in-register after previous" in src
+    assert "T1->lds" in src and "V2->lds" in src and "Y->global" in src
+    assert "T3<-registers" in src and "D<-global" in src
+    # no store of a transient intermediate to device memory: only Y (parameter of the last kernel) is written
+    stores = [l for l in src.splitlines() if l.strip().startswith("T") and "] = r" in l]
+    assert stores and all(l.strip().startswith("T9[") for l in stores)
+
+
+def test_mass_apply_chain_stores_everything_by_default(TE):
+    src = chain_source(TE, workloads.config4(E=64), transient=False)
+    for name in ("T1", "T2", "U", "V1", "V2"):
+        assert name + "->lds+global" in src
+    assert "T3->global" in src
+
+
+def test_mass_assembly_is_sum_factorised_inside_the_lane(TE):
+    wl = workloads.config3(E=16)
+    tensors = workloads.bind_to_engine(wl, at)
+    k, out, ins = wl.kernels[0]
+    src = TE.GetImplementation(k, tensors[out], *[tensors[n] for n in ins])
+    assert ")=9 contraction=64 unrolled" in src           # a 3x3 tile of outputs per lane
+    # as written the kernel has 729 * 64 * 6 multiplications per element; hoisting leaves a small fraction
+    assert src.count("*") < 81 * 400
+
+
+def test_long_contraction_uses_counted_loops(TE):
+    wl = workloads.config1(n=4096)
+    tensors = workloads.bind_to_engine(wl, at)
+    k, out, ins = wl.kernels[0]
+    src = TE.GetImplementation(k, tensors[out], *[tensors[n] for n in ins])
+    assert "looped" in src or "split" in src
+
+
+def test_diffusion_chain_with_aliased_slices_is_not_fused_blindly(TE):
+    src = chain_source(TE, workloads.config5(E=2, Q=5, P=4), transient=True)
+    assert "__global__" in src or "not fused" in src
+
+
+def test_rebinding_one_name_to_two_tensors_switches_to_positional_operands(TE):
+    A, B1, B2 = at.Tensor(5, 5), at.Tensor(5, 3), at.Tensor(5, 3)
+    src = TE.GetImplementation("A_i_j = B_i_k B_j_k", A, B1, B2)
+    assert src.count("const double *") >= 2
+
+
+def test_compile_errors_surface_as_exceptions_with_the_log():
+    import ctypes
+    from acrotensor_amd import _capi
+    # an engine created for an unknown policy is the only host-forcible failure of the boundary besides bad
+    # kernels; a bad kernel string must fail before any code is generated
+    TE = at.TensorEngine("HIP")
+    with pytest.raises(at.AcroError):
+        TE.GetImplementation("A_i = b_i", at.Tensor(3), at.Tensor(3))

@@ -1,0 +1,313 @@
+"""The reference's engine suite (unittest/kernel/test_TensorEngine.cpp) re-expressed for the "HIP" policy, driven
+through the C ABI.  Expected values come from the checker (the restated CPU interpreter) and, as in the reference's
+tests, from closed forms.  Integer-valued inputs make results exact in fp64 whatever the summation order, so those
+comparisons are bit-exact (index mapping); random inputs are held to 1e-12 relative to the largest entry."""
+import numpy as np
+import pytest
+
+from gpu_helpers import output_shape, rel_err, run_single, to_tensor
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-12
+
+
+def seq(shape, mod=None, scale=1.0):
+    a = np.arange(int(np.prod(shape)), dtype=np.float64)
+    if mod:
+        a = a % mod
+    return (a * scale).reshape(shape)
+
+
+def test_assert_compatible_dimensions(at, engine):
+    # unittest/kernel/test_TensorEngine.cpp:37-47
+    T1out_3, T1_3, T1_2, T2_3_3 = at.Tensor(3), at.Tensor(3), at.Tensor(2), at.Tensor(3, 3)
+    for t in (T1_3, T1_2, T2_3_3):
+        t.Set(1.0)
+    engine("A_i=B_iC_i", T1out_3, T1_3, T1_3)
+    with pytest.raises(at.AcroError):
+        engine("A_i=B_iC_i", T1out_3, T1_3, T1_2)
+    engine("A_i=B_i_jC_i", T1out_3, T2_3_3, T1_3)
+    with pytest.raises(at.AcroError):
+        engine("A_i=B_i_jC_i", T1out_3, T2_3_3, T1_2)
+    with pytest.raises(at.AcroError):
+        engine("A_i=B_i_jC_i", T1out_3, T2_3_3)                 # wrong number of inputs
+    with pytest.raises(at.AcroError):
+        engine("A_i_j=B_i_jC_i", T1out_3, T2_3_3, T1_3)         # wrong output rank
+    with pytest.raises(at.AcroError):
+        engine("Blah=Alah", T1out_3, T1_3)
+    with pytest.raises(at.AcroError):
+        engine.EndMultiKernelLaunch()                           # End without Begin
+    engine.BeginMultiKernelLaunch()
+    with pytest.raises(at.AcroError):
+        engine.BeginMultiKernelLaunch()                         # Begin twice
+    engine.EndMultiKernelLaunch()                               # empty capture is a no-op
+
+
+BASIC = [
+    ("A_i=B_i", [(3,)]),                       # simple copy
+    ("A_i=B_i_i", [(3, 3)]),                   # diagonal
+    ("A_i=B_j_j", [(3, 3)]),                   # contraction + broadcast
+    ("A_i = C_i_j B_j", [(3, 3), (3,)]),       # matvec
+    ("A_i_j=B_j_i", [(4, 4)]),                 # transpose
+    ("A_m_n=B_m_j B_n_j", [(3, 3), (3, 3)]),   # B B^T (same tensor under one name, see below)
+    ("A_i=B_j_k_l_m_n", [(1, 2, 1, 3, 2)]),    # singleton dimensions, everything contracted
+    ("A_i_j_k = B_k_j_i", [(5, 1, 7)]),
+    ("A_e_i = B_e_i_j_k C_j D_k", [(17, 4, 5, 2), (5,), (2,)]),
+    ("A_i_j = B_i_k C_k_j", [(33, 65), (65, 17)]),
+    ("A_i_i = B_i", [(4,)]),                   # repeated output index: only the diagonal is written
+]
+
+
+@pytest.mark.parametrize("kernel,shapes", BASIC)
+def test_basic_computations_exact_on_integer_data(at, engine, checker, kernel, shapes):
+    ins = [seq(s, mod=11) - 3.0 for s in shapes]
+    if kernel.startswith("A_m_n"):
+        ins[1] = ins[0]
+    init = np.full(output_shape(kernel, shapes), 7.0)
+    got, expected = run_single(at, engine, checker, kernel, init, *ins)
+    assert np.array_equal(got, expected)
+
+
+def test_same_name_bound_to_one_tensor(at, engine):
+    B = to_tensor(at, seq((3, 3)))
+    A = at.Tensor(3, 3)
+    engine("A_m_n=B_m_j B_n_j", A, B, B)
+    A.MoveFromGPU()
+    assert np.array_equal(A.data, B.data @ B.data.T)
+
+
+@pytest.mark.parametrize("kernel,shapes", BASIC[:6] + [("A_i += B_i_j C_j", [(300, 7), (7,)]),
+                                                       ("A_e_i += B_e_i_j_k C_j D_k", [(17, 4, 5, 2), (5,), (2,)])])
+def test_basic_computations_random_data(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(abs(hash(kernel)) % 2 ** 31)
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    init = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, init, *ins)
+    assert rel_err(got, expected) <= TOL
+
+
+def test_minus_equal_subtracts(at, engine, checker):
+    # The reference's device generator honours "-=" (exec/CudaExecutor.cpp:534-536) while its host interpreter adds
+    # (exec/CPUInterpretedExecutor.cpp:106); the HIP policy subtracts, i.e. init - (what "+=" would add).
+    rng = np.random.default_rng(11)
+    B, C, init = rng.uniform(-1, 1, (40, 6)), rng.uniform(-1, 1, 6), rng.uniform(-1, 1, 40)
+    got, added = run_single(at, engine, checker, "A_i -= B_i_j C_j", init, B, C)
+    assert rel_err(got, init - (added - init)) <= TOL
+
+
+def test_multi_kernel_launch_second_kernel_overwrites_first(at, engine):
+    # unittest/kernel/test_TensorEngine.cpp:211-228
+    A, B1, B2, C = at.Tensor(3), at.Tensor(3), at.Tensor(3), at.Tensor(3, 3)
+    B1.data[...] = [1.0, 2.0, 3.0]
+    B2.Set(1.0)
+    C.Set(1.0)
+    engine.BeginMultiKernelLaunch()
+    engine("A_i = B1_i", A, B1)
+    engine("A_i = C_i_j B2_j", A, C, B2)
+    engine.EndMultiKernelLaunch()
+    A.MoveFromGPU()
+    assert np.array_equal(A.data, [3.0, 3.0, 3.0])
+
+
+def test_multi_kernel_launch_without_common_outer_index_runs_kernel_by_kernel(at, engine):
+    A, B, C, D = at.Tensor(4), to_tensor(at, seq((4,))), at.Tensor(6), to_tensor(at, seq((6,)))
+    engine.BeginMultiKernelLaunch()
+    engine("A_i = B_i", A, B)
+    engine("C_j = D_j", C, D)
+    engine.EndMultiKernelLaunch()
+    assert "not fused" in engine.GetLastImplementation()
+    A.MoveFromGPU()
+    C.MoveFromGPU()
+    assert np.array_equal(A.data, B.data) and np.array_equal(C.data, D.data)
+
+
+def test_2d_mass_matrix(at, engine, checker):
+    # unittest/kernel/test_TensorEngine.cpp:232-309
+    rng = np.random.default_rng(2)
+    B, W, T = seq((3, 2)), seq((3, 3)) + 1.0, rng.uniform(0.5, 1.5, (5, 3, 3))
+    D, expD = run_single(at, engine, checker, "D_e_k1_k2 = W_k1_k2 T_e_k1_k2", np.zeros((5, 3, 3)), W, T)
+    assert rel_err(D, W[None] * T) <= TOL
+    M, expM = run_single(at, engine, checker, "M_e_i1_i2_j1_j2=B_k1_i1 B_k1_j1 B_k2_i2 B_k2_j2 D_e_k1_k2",
+                         np.zeros((5, 2, 2, 2, 2)), B, B, B, B, D)
+    assert rel_err(M, expM) <= TOL
+    assert rel_err(M, np.einsum("ai,aj,bk,bl,eab->eikjl", B, B, B, B, D)) <= TOL
+
+
+def test_2d_stiffness_partial_assembly_with_slices(at, engine, checker):
+    # unittest/kernel/test_TensorEngine.cpp:311-435: integer-valued data, slices as outputs and inputs
+    B, G, X, D = seq((4, 4)), seq((4, 4), scale=0.5), seq((5, 4, 4)), seq((5, 2, 2, 4, 4))
+    tB, tG, tX, tD = (to_tensor(at, a) for a in (B, G, X, D))
+    T, U, Z, Y = at.Tensor(5, 4, 4), at.Tensor(2, 5, 4, 4), at.Tensor(2, 5, 4, 4), at.Tensor(5, 4, 4)
+    U1, U2 = at.SliceTensor(U, 0), at.SliceTensor(U, 1)
+    Z1, Z2 = at.SliceTensor(Z, 0), at.SliceTensor(Z, 1)
+
+    engine("BX_e_i1_k2 = B_k2_i2 X_e_i1_i2", T, tB, tX)
+    engine("U1_e_k1_k2 = G_k1_i1 BX_e_i1_k2", U1, tG, T)
+    engine("GX_e_i1_k2 = G_k2_i2 X_e_i1_i2", T, tG, tX)
+    engine("U2_e_k1_k2 = B_k1_i1 GX_e_i1_k2", U2, tB, T)
+    engine("Z_m_e_k1_k2 = D_e_m_n_k1_k2 U_n_e_k1_k2", Z, tD, U)
+    U.MoveFromGPU()
+    expU = np.stack([np.einsum("ai,bj,eij->eab", G, B, X), np.einsum("ai,bj,eij->eab", B, G, X)])
+    assert np.array_equal(U.data, expU)
+    expZ = np.einsum("emnab,neab->meab", D, expU)
+    Z.MoveFromGPU()
+    assert np.array_equal(Z.data, expZ)
+
+    engine("BZ1_e_i2_k1 = B_k2_i2 Z1_e_k1_k2", T, tB, Z1)
+    engine("Y_e_i1_i2 = G_k1_i1 BZ1_e_i2_k1", Y, tG, T)
+    Y.MoveFromGPU()
+    assert np.array_equal(Y.data, np.einsum("ai,bj,eab->eij", G, B, expZ[0]))
+    engine("GZ2_e_i2_k1 = G_k2_i2 Z2_e_k1_k2", T, tG, Z2)
+    engine("Y_e_i1_i2 = B_k1_i1 GZ2_e_i2_k1", Y, tB, T)
+    Y.MoveFromGPU()
+    assert np.array_equal(Y.data, np.einsum("ai,bj,eab->eij", B, G, expZ[1]))
+
+
+def test_2d_stiffness_as_one_multi_kernel_launch_with_aliased_slices(at, engine):
+    # Same computation captured as ONE multi-kernel launch: U1/U2 are written under their own names and read
+    # back through U, so the variables overlap in memory and the launch must not be fused blindly.
+    B, G, X, D = seq((4, 4)), seq((4, 4), scale=0.5), seq((5, 4, 4)), seq((5, 2, 2, 4, 4))
+    tB, tG, tX, tD = (to_tensor(at, a) for a in (B, G, X, D))
+    T1, T2, U, Z = at.Tensor(5, 4, 4), at.Tensor(5, 4, 4), at.Tensor(2, 5, 4, 4), at.Tensor(2, 5, 4, 4)
+    U1, U2 = at.SliceTensor(U, 0), at.SliceTensor(U, 1)
+    engine.BeginMultiKernelLaunch()
+    engine("BX_e_i1_k2 = B_k2_i2 X_e_i1_i2", T1, tB, tX)
+    engine("U1_e_k1_k2 = G_k1_i1 BX_e_i1_k2", U1, tG, T1)
+    engine("GX_e_i1_k2 = G_k2_i2 X_e_i1_i2", T2, tG, tX)
+    engine("U2_e_k1_k2 = B_k1_i1 GX_e_i1_k2", U2, tB, T2)
+    engine("Z_m_e_k1_k2 = D_e_m_n_k1_k2 U_n_e_k1_k2", Z, tD, U)
+    engine.EndMultiKernelLaunch()
+    Z.MoveFromGPU()
+    expU = np.stack([np.einsum("ai,bj,eij->eab", G, B, X), np.einsum("ai,bj,eij->eab", B, G, X)])
+    assert np.array_equal(Z.data, np.einsum("emnab,neab->meab", D, expU))
+
+
+def test_3d_stiffness_twelve_loops(at, engine, checker):
+    # unittest/kernel/test_TensorEngine.cpp:437-496 (contraction of 1125 terms: counted-loop path), E reduced to 4
+    k = "S_e_i1_i2_i3_j1_j2_j3 = B1_i1_j1_k1_m_n B2_i2_j2_k2_m_n B3_i3_j3_k3_m_n D_e_k1_k2_k3_m_n"
+    B1 = seq((5, 5, 5, 3, 3), mod=11)
+    B2 = seq((5, 5, 5, 3, 3), mod=7, scale=2.0)
+    B3 = seq((5, 5, 5, 3, 3), mod=13, scale=3.0)
+    D = seq((4, 5, 5, 5, 3, 3), mod=5, scale=3.5)
+    got, expected = run_single(at, engine, checker, k, np.zeros((4, 5, 5, 5, 5, 5, 5)), B1, B2, B3, D)
+    assert np.array_equal(got, expected)          # all terms are multiples of 0.5 below 2^53: exact
+
+
+@pytest.mark.parametrize("order", [1, 4])
+def test_d_tensor_construction(at, engine, checker, order):
+    # unittest/kernel/test_TensorEngine.cpp:498-590
+    rng = np.random.default_rng(order)
+    n, E = order + 1, 6
+    W, C = rng.uniform(0.5, 1, (E, n, n)), rng.uniform(0.5, 1, (E, n, n))
+    J = np.eye(2) + 0.1 * rng.uniform(-1, 1, (E, n, n, 2, 2))
+    tJ, Jinv, Jdet = to_tensor(at, J), at.Tensor(E, n, n, 2, 2), at.Tensor(E, n, n)
+    engine.BatchMatrixInvDet(Jinv, Jdet, tJ)
+    Jinv.MoveFromGPU()
+    Jdet.MoveFromGPU()
+    ji, jd = Jinv.data.copy(), Jdet.data.copy()
+    got, expected = run_single(at, engine, checker,
+                               "D_e_m_n_k1_k2 = W_e_k1_k2 C_e_k1_k2 Jdet_e_k1_k2 Jinv_e_k1_k2_m_j Jinv_e_k1_k2_n_j",
+                               np.zeros((E, 2, 2, n, n)), W, C, jd, ji, ji)
+    assert rel_err(got, expected) <= TOL
+    assert rel_err(got, np.einsum("eab,eab,eab,eabmj,eabnj->emnab", W, C, jd, ji, ji)) <= TOL
+
+
+@pytest.mark.parametrize("m", [1, 2, 3])
+def test_batch_matrix_inverse_and_determinant(at, engine, checker, m):
+    # unittest/kernel/test_TensorEngine.cpp:594-706; non-symmetric matrices on purpose
+    rng = np.random.default_rng(m)
+    A = np.eye(m) + 0.2 * rng.uniform(-1, 1, (37, 5, m, m))
+    tA, Ainv, Adet, Ainv2, Adet2 = to_tensor(at, A), at.Tensor(37, 5, m, m), at.Tensor(37, 5), at.Tensor(37, 5, m, m), at.Tensor(37, 5)
+    engine.BatchMatrixInverse(Ainv, tA)
+    engine.BatchMatrixDet(Adet, tA)
+    engine.BatchMatrixInvDet(Ainv2, Adet2, tA)
+    for t in (Ainv, Adet, Ainv2, Adet2):
+        t.MoveFromGPU()
+    ri, rd = checker.batch_matrix_inv_det(A)
+    assert np.array_equal(Ainv.data, ri) and np.array_equal(Ainv2.data, ri)      # bit for bit
+    assert np.array_equal(Adet.data, rd) and np.array_equal(Adet2.data, rd)
+    # invariants: A * Ainv^T = I for 3x3 (the reference's layout), A * Ainv = I otherwise; det(A) det(Ainv) = 1
+    prod = np.einsum("...ij,...kj->...ik", A, Ainv.data) if m == 3 else np.einsum("...ij,...jk->...ik", A, Ainv.data)
+    assert np.abs(prod - np.eye(m)).max() < 1e-13
+    # I_b_i_k = TI_b_i_j T_b_j_k through the engine, as the reference's test does
+    I = at.Tensor(37 * 5, m, m)
+    Ainv.Reshape(37 * 5, m, m)
+    tA.Reshape(37 * 5, m, m)
+    if m == 3:
+        engine("I_b_i_k = TI_b_j_i T_b_j_k", I, Ainv, tA)
+    else:
+        engine("I_b_i_k = TI_b_i_j T_b_j_k", I, Ainv, tA)
+    I.MoveFromGPU()
+    assert np.abs(I.data - np.eye(m)).max() < 1e-13
+
+
+def test_batch_matrix_shape_asserts(at, engine):
+    # unittest/kernel/test_TensorEngine.cpp:600-612
+    A4, A3, B3, d = at.Tensor(5, 4, 4), at.Tensor(5, 3, 3), at.Tensor(6, 3, 3), at.Tensor(5)
+    for t in (A4, A3, B3):
+        t.Set(1.0)
+    with pytest.raises(at.AcroError):
+        engine.BatchMatrixInverse(at.Tensor(5, 4, 4), A4)        # larger than 3x3
+    with pytest.raises(at.AcroError):
+        engine.BatchMatrixInverse(B3, A3)                        # batch mismatch
+    with pytest.raises(at.AcroError):
+        engine.BatchMatrixDet(at.Tensor(6), A3)
+    with pytest.raises(at.AcroError):
+        engine.BatchMatrixDet(d, at.Tensor(5, 3, 2))             # not square
+    with pytest.raises(at.AcroError):
+        engine.BatchMatrixInvDet(at.Tensor(5, 3, 3), at.Tensor(5, 1), A3)
+
+
+def test_batch_matrix_ragged_batch_sizes(at, engine, checker):
+    for n in (1, 255, 256, 257, 1000):
+        rng = np.random.default_rng(n)
+        A = np.eye(3) + 0.1 * rng.uniform(-1, 1, (n, 3, 3))
+        tA, Ainv, Adet = to_tensor(at, A), at.Tensor(n, 3, 3), at.Tensor(n)
+        engine.BatchMatrixInvDet(Ainv, Adet, tA)
+        Ainv.MoveFromGPU()
+        Adet.MoveFromGPU()
+        ri, rd = checker.batch_matrix_inv_det(A)
+        assert np.array_equal(Ainv.data, ri) and np.array_equal(Adet.data, rd)
+
+
+def test_scatter_and_sum_gather(at, engine, checker):
+    # unittest/kernel/test_TensorEngine.cpp:708-745: the 8 -> 6 map
+    M = at.IndexMapping(6, 8)
+    M.map[:] = [0, 1, 2, 3, 4, 5, 1, 3]
+    src = to_tensor(at, np.arange(6, dtype=np.float64) * 10)
+    out = at.Tensor(8)
+    engine.FlatIndexedScatter(out, src, M)
+    out.MoveFromGPU()
+    assert np.array_equal(out.data, [0, 10, 20, 30, 40, 50, 10, 30])
+    vals = to_tensor(at, np.arange(1, 9, dtype=np.float64))
+    acc = at.Tensor(6)
+    engine.FlatIndexedSumGather(acc, vals, M)
+    acc.MoveFromGPU()
+    assert np.array_equal(acc.data, [1, 9, 3, 12, 5, 6])
+    with pytest.raises(at.AcroError):
+        engine.FlatIndexedScatter(at.Tensor(7), src, M)
+    with pytest.raises(at.AcroError):
+        engine.FlatIndexedSumGather(at.Tensor(5), vals, M)
+
+
+def test_sum_gather_large_random_map_bit_exact(at, engine, checker):
+    rng = np.random.default_rng(8)
+    domain, rsize = 5000, 40000
+    M = at.IndexMapping(domain, rsize)
+    M.map[:] = rng.integers(0, domain - 7, rsize)              # the last domain entries have no preimage
+    vals = rng.uniform(-1, 1, rsize)
+    acc = at.Tensor(domain)
+    engine.FlatIndexedSumGather(acc, to_tensor(at, vals), M)
+    acc.MoveFromGPU()
+    assert np.array_equal(acc.data, checker.sum_gather(vals, M.map, domain))
+    src = rng.uniform(-1, 1, domain)
+    out = at.Tensor(rsize)
+    engine.FlatIndexedScatter(out, to_tensor(at, src), M)
+    out.MoveFromGPU()
+    assert np.array_equal(out.data, checker.scatter(src, M.map))
+
+
+def test_get_implementation_returns_hip_source(at, engine):
+    A, B = at.Tensor(8, 3), at.Tensor(8, 3)
+    src = engine.GetImplementation("A_e_i = B_e_i", A, B)
+    assert "__global__" in src and "A_e_i = B_e_i" in src

@@ -1,0 +1,84 @@
+"""Tensor / SliceTensor / IndexMapping residency semantics on the device, as the reference tests them in
+unittest/tensor/test_Tensor.cpp:155-184 and unittest/tensor/test_SliceTensor.cpp:105-168."""
+import numpy as np
+import pytest
+
+from gpu_helpers import to_tensor
+
+pytestmark = pytest.mark.gpu
+
+
+def test_map_switch_set_move(at):
+    T = at.Tensor(10, 10)
+    T.Set(3.0)
+    assert not T.IsMappedToGPU() and not T.IsOnGPU() and T.GetDeviceData() is None
+    T.MapToGPU()
+    assert T.IsMappedToGPU() and not T.IsOnGPU() and T.GetDeviceData()
+    with pytest.raises(at.AcroError):
+        T.MapToGPU()                                     # mapping twice
+    T.SwitchToGPU()
+    assert T.IsOnGPU()
+    T.Set(9.0)                                           # on the device only
+    assert np.all(T.data == 3.0)
+    T.MoveFromGPU()
+    assert not T.IsOnGPU() and np.all(T.data == 9.0)
+    T.Set(2.0)
+    T.MoveToGPU()
+    T.Mult(2.5)
+    assert np.all(T.data == 2.0)
+    T.SwitchFromGPU()                                    # drop the device result
+    assert np.all(T.data == 2.0)
+    T.SwitchToGPU()
+    T.MoveFromGPU()
+    assert np.all(T.data == 5.0)
+    T.UnmapFromGPU()
+    assert not T.IsMappedToGPU() and not T.IsOnGPU()
+    with pytest.raises(at.AcroError):
+        T.UnmapFromGPU()
+
+
+def test_move_to_gpu_maps_on_demand_and_is_idempotent(at):
+    T = to_tensor(at, np.arange(12.0).reshape(3, 4))
+    T.MoveToGPU()
+    T.data[...] = -1.0                                   # host copy is stale now
+    T.MoveToGPU()                                        # no copy: the device copy is current
+    T.MoveFromGPU()
+    assert np.array_equal(T.data, np.arange(12.0).reshape(3, 4))
+
+
+def test_slices_share_storage_and_residency(at):
+    T = to_tensor(at, np.zeros((3, 4, 5)))
+    S1, S12 = at.SliceTensor(T, 1), at.SliceTensor(T, 1, 2)
+    assert S1.dims == (4, 5) and S12.dims == (5,)
+    S1.MoveToGPU()
+    assert T.IsOnGPU() and S12.IsOnGPU() and T.IsMappedToGPU()
+    S1.Set(4.0)
+    S12.Set(7.0)
+    T.MoveFromGPU()
+    assert not S1.IsOnGPU()
+    expected = np.zeros((3, 4, 5))
+    expected[1] = 4.0
+    expected[1, 2] = 7.0
+    assert np.array_equal(T.data, expected)
+    assert np.array_equal(S12.data, expected[1, 2])
+    with pytest.raises(at.AcroError):
+        at.SliceTensor(T, 3)
+    with pytest.raises(at.AcroError):
+        at.SliceTensor(T, 0, 0, 0)
+
+
+def test_engine_moves_host_tensors_and_leaves_output_on_device(at, engine):
+    A, B = at.Tensor(6), to_tensor(at, np.arange(6.0))
+    engine("A_i = B_i", A, B)
+    assert A.IsOnGPU() and B.IsOnGPU()
+    A.MoveFromGPU()
+    assert np.array_equal(A.data, np.arange(6.0))
+
+
+def test_large_fill_and_scale(at):
+    T = at.Tensor(1031, 257)
+    T.SwitchToGPU()
+    T.Set(1.5)
+    T.Mult(-2.0)
+    T.MoveFromGPU()
+    assert np.all(T.data == -3.0)
