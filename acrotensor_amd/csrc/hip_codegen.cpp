@@ -65,7 +65,8 @@ struct UVarInfo
     int tileSize = 0;             // doubles per batch entry
     std::vector<int> ldsStride;   // per dimension (0 for batch dimensions)
     int ldsOffset = 0;            // in doubles, start of the NB tiles
-    int liveFrom = 0, liveTo = 0;
+    int liveFrom = 0, liveTo = 0; // first producing and last consuming kernel
+    int phaseFrom = 0, phaseTo = 0;  // the same in barrier-separated phases (fused kernels share a phase)
     bool elide = false;           // no store to device memory
 };
 
@@ -252,6 +253,14 @@ class Generator
     bool CheckFusable(std::string &why)
     {
         if (mk.GetNumKernels() == 1) return true;  // a single kernel always has a private batch index
+        for (const auto &s : subs)
+        {
+            if (s.out.repeated && s.op == '=')
+            {
+                why = "an assigned output repeats an index and needs a zero fill between kernels";
+                return false;
+            }
+        }
         if (batch < 0)
         {
             why = "the kernels share no outer index";
@@ -306,7 +315,8 @@ class Generator
         return loads;
     }
 
-    static constexpr long kUnrollBudget = 8192;   // multiply-adds emitted per work item
+    static constexpr long kUnrollBudget = 8192;   // multiply-adds emitted per work item (before hoisting)
+    static constexpr long kMaxUnrolledContraction = 512;  // terms of one unrolled sum
     static constexpr long kMaxTile = 32;
     static constexpr long kMaxLiveValues = 160;   // loaded operands + accumulators held by one lane
 
@@ -320,7 +330,7 @@ class Generator
                 if (id != batch) mid.push_back(id);
             }
             const long nin = static_cast<long>(s.in.size());
-            if (s.contrCount * nin > kUnrollBudget)
+            if (s.contrCount > kMaxUnrolledContraction || s.contrCount * nin > kUnrollBudget)
             {
                 s.loopMode = true;
                 s.tile.clear();
@@ -453,6 +463,18 @@ class Generator
             u.wantLds = true;
             u.liveFrom = u.firstWrite;
             u.liveTo = lastReader;
+            // Kernels fused into one item loop run without a barrier between them, so LDS lifetimes are counted in
+            // phases: a tile read in a phase and a tile written in the same phase must not share storage.
+            auto phaseOf = [&](int k) {
+                int p = 0;
+                for (int j = 1; j <= k; ++j)
+                {
+                    if (!subs[j].fusedWithPrev) ++p;
+                }
+                return p;
+            };
+            u.phaseFrom = phaseOf(u.liveFrom);
+            u.phaseTo = phaseOf(u.liveTo);
             u.tileSize = u.size / u.dims[u.batchDims[0]];
             u.ldsStride.assign(u.dims.size(), 0);
             int st = 1;
@@ -474,7 +496,7 @@ class Generator
             if (uvars[ui].wantLds && uvars[ui].inLds) order.push_back(static_cast<int>(ui));
         }
         std::sort(order.begin(), order.end(), [&](int a, int b) {
-            if (uvars[a].liveFrom != uvars[b].liveFrom) return uvars[a].liveFrom < uvars[b].liveFrom;
+            if (uvars[a].phaseFrom != uvars[b].phaseFrom) return uvars[a].phaseFrom < uvars[b].phaseFrom;
             return a < b;
         });
         int total = 0;
@@ -491,7 +513,7 @@ class Generator
                 for (int pj : placed)
                 {
                     const UVarInfo &p = uvars[pj];
-                    const bool timeOverlap = !(p.liveTo < u.liveFrom || u.liveTo < p.liveFrom);
+                    const bool timeOverlap = !(p.phaseTo < u.phaseFrom || u.phaseTo < p.phaseFrom);
                     const int pneed = p.tileSize * nb;
                     const bool spaceOverlap = !(p.ldsOffset + pneed <= offset || offset + need <= p.ldsOffset);
                     if (timeOverlap && spaceOverlap)
@@ -1028,6 +1050,10 @@ class Generator
         {
             plan.param_occurrence[u] = FirstOccurrence(u);
             plan.stored[u] = uvars[u].written && !uvars[u].elide;
+        }
+        for (const auto &s : subs)
+        {
+            if (s.out.repeated && s.op == '=') plan.zero_fill_params.push_back(s.out.uvar);
         }
     }
 };

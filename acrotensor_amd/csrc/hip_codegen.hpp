@@ -52,6 +52,10 @@ struct HipKernelPlan
     // occurrence; variable number -1 is that kernel's output.
     std::vector<std::pair<int, int>> param_occurrence;
     std::vector<bool> stored;      // per parameter: the kernel writes it to device memory
+    // Parameters that must be set to zero before the launch: an output assigned with "=" whose index list repeats
+    // an index ("A_i_i = B_i") is only written on its diagonal by the kernel, while assignment means zero-fill
+    // followed by accumulation (reference exec/CPUInterpretedExecutor.cpp:63-67).
+    std::vector<int> zero_fill_params;
     int lds_bytes = 0;
     int nb = 0;
     std::string schedule;          // human readable schedule summary (also a comment in the source)

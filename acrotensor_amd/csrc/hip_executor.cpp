@@ -180,6 +180,12 @@ class HipExecutor : public KernelExecutor
             ACROBATIC_ASSERT(ptr[i] != nullptr, "Tensor has no device memory.");
             args[i] = &ptr[i];
         }
+        for (int i : v.plan.zero_fill_params)
+        {
+            const auto &occ = v.plan.param_occurrence[i];
+            Tensor *t = occ.second < 0 ? outputs[occ.first] : inputs[occ.first][occ.second];
+            hip::FillDouble(ptr[i], 0.0, static_cast<size_t>(t->GetSize()));
+        }
         v.kernel->Launch(v.plan.grid, v.plan.block, args.data());
     }
 

@@ -124,6 +124,15 @@ def test_config4_full_size_properties(at, engine, checker):
     sub.arrays["D"][...] = D[sample]
     expected = workloads.run_on_checker(sub, checker)["Y"]
     assert rel_err(Y[sample], expected) <= TOL
+    # (1b) every element against the chain evaluated with numpy (different summation order: 1e-12, not bit-exact)
+    T = np.einsum("qi,eijk->eqjk", B, X)
+    T = np.einsum("rj,eqjk->eqrk", B, T)
+    T = np.einsum("sk,eqrk->eqrs", B, T) * D
+    T = np.einsum("qi,eqrs->eirs", B, T)
+    T = np.einsum("rj,eirs->eijs", B, T)
+    T = np.einsum("sk,eijs->eijk", B, T)
+    per_element = np.abs(Y - T).reshape(E, -1).max(axis=1)
+    assert per_element.max() <= TOL * np.abs(T).max(), "first bad element %d" % int(per_element.argmax())
     # (2) linearity: apply(2 X) = 2 apply(X) exactly (scaling by 2 is exact in binary floating point)
     tensors["X"].data[...] = 2.0 * X
     tensors["X"].SwitchFromGPU()
