@@ -28,7 +28,17 @@ METRIC = "GDOF/s + % HBM peak, p=3 sum-factorised hex mass apply fp64 (1 GPU)"
 
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a
 # copy kernel of known size); None until the profile summary under profiles/ has been taken for this kernel.
-MEASURED_TRAFFIC_BYTES = None
+MEASURED_TRAFFIC_BYTES = 536845452  # profiles/cfg4_mass_apply_hbm_traffic.md
+
+
+def settle_clocks(at, workloads, wl, engine, tensors, seconds):
+    """Untimed launches before the warm-up: the first ~20 ms of sustained load run through a power-management
+    transient (boost clocks, then a clamp, then the sustainable state); measurements start after it."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(100):
+            workloads.launch(wl, engine, tensors)
+        at.synchronize()
 
 
 def time_steps(at, workloads, wl, engine, tensors, steps, warmup):
@@ -68,12 +78,17 @@ def cpu_baseline(workloads, sample_elems):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--settle-seconds", type=float, default=0.25,
+                    help="untimed launches before the warm-up, until clocks have settled under sustained load")
     ap.add_argument("--elements", type=int, default=262144)
-    ap.add_argument("--cpu-sample-elems", type=int, default=131072)
+    ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store-all", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one scale-by-1.0 kernel over X (reads and writes E*512 bytes): the known-size "
+                         "kernel that hardware-counter runs are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the workload shards trivially over "
@@ -91,6 +106,11 @@ def main():
     for t in tensors.values():
         t.MoveToGPU()
 
+    if args.calibration_copy:
+        tensors["X"].Mult(1.0)
+        at.synchronize()
+
+    settle_clocks(at, workloads, wl, engine, tensors, args.settle_seconds)
     wall, dev = time_steps(at, workloads, wl, engine, tensors, args.steps, args.warmup)
     ms_per_step = wall / args.steps * 1e3
     launch_s = dev / args.steps
@@ -133,8 +153,8 @@ def main():
     if not args.no_store_all:
         for name in wl.transient:
             tensors[name].SetTransient(False)
-        wall2, dev2 = time_steps(at, workloads, wl, engine, tensors, max(10, args.steps // 4), 5)
         n2 = max(10, args.steps // 4)
+        wall2, dev2 = time_steps(at, workloads, wl, engine, tensors, n2, max(5, args.warmup // 4))
         stored_bytes = args.elements * (64 + 125 + 64 + 610) * 8
         result["store_all"] = {
             "value": wl.dof * n2 / wall2 * 1e-9,
