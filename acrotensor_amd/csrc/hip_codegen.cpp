@@ -47,6 +47,7 @@ struct Sub
     long laneCount = 1, tileCount = 1, contrCount = 1;
 };
 
+// An operand of the group: a unique variable (by name) or, in positional mode, one occurrence.
 struct UVarInfo
 {
     std::string name;
@@ -59,14 +60,33 @@ struct UVarInfo
     bool consistent = true;       // same shape and batch positions in every occurrence
     std::vector<int> batchDims;   // dimensions carrying the batch index
     bool anyRepeated = false;
+    // the storage this operand is a view of
+    int storage = -1;
+    long viewOffset = 0;          // first element inside the storage
+    std::vector<int> fixed;       // leading indices of the storage that the view fixes
+    bool plainView = true;        // the view is "leading indices fixed, all trailing dimensions kept"
+};
+
+// A tensor's memory: what kernel parameters point to, what LDS tiles mirror and what stores are elided for.
+struct Storage
+{
+    std::vector<int> dims;        // extents of the root tensor
+    std::vector<long> stride;     // its row-major strides
+    std::vector<int> members;     // operands that are views of it
+    bool written = false;
+    bool transient = true;        // every member is marked transient
+    int batchDim = -1;            // root dimension carrying the batch index
+    bool elementLocal = true;     // every member carries the batch index exactly once, at batchDim
+    bool anyRepeated = false;
+    int firstWrite = -1;          // kernel numbers
     // LDS residency of the per-batch-entry tile
     bool wantLds = false;
     bool inLds = false;
     int tileSize = 0;             // doubles per batch entry
-    std::vector<int> ldsStride;   // per dimension (0 for batch dimensions)
+    std::vector<int> ldsStride;   // per root dimension (0 for the batch dimension)
     int ldsOffset = 0;            // in doubles, start of the NB tiles
-    int liveFrom = 0, liveTo = 0; // first producing and last consuming kernel
-    int phaseFrom = 0, phaseTo = 0;  // the same in barrier-separated phases (fused kernels share a phase)
+    int liveTo = -1;              // last kernel that reads the tile from LDS
+    int phaseFrom = 0, phaseTo = 0;  // lifetime in barrier-separated phases (fused kernels share a phase)
     bool elide = false;           // no store to device memory
 };
 
@@ -120,11 +140,16 @@ class Generator
             plan.why_not = why;
             return plan;
         }
+        plan.fusable = true;
+        if (UseReductionSchedule())
+        {
+            EmitReduction(plan);
+            return plan;
+        }
         ChooseTiles();
         PlanFusion();
         ChooseBatching();
         Emit(plan);
-        plan.fusable = true;
         return plan;
     }
 
@@ -137,6 +162,11 @@ class Generator
     std::vector<int> extent;
     std::vector<Sub> subs;
     std::vector<UVarInfo> uvars;
+    std::vector<Storage> stores;
+    // Per kernel and input occurrence: every entry it reads has been written to the storage's tile by an earlier
+    // kernel of the group (so it can be served from LDS); per kernel: the same for the old value of a += output.
+    std::vector<std::vector<bool>> readCovered;
+    std::vector<bool> oldCovered;
     int batch = -1;
     long E = 1;
     int NB = 1, NT = 128;
@@ -248,6 +278,143 @@ class Generator
             auto first = FirstOccurrence(u);
             uvars[u].name = mk.Kernels[first.first]->GetVarName(first.second);
         }
+        BuildStorages();
+        AnalyseCoverage();
+    }
+
+    void BuildStorages()
+    {
+        const int U = NumOperands();
+        int nstore = 0;
+        for (int u = 0; u < U; ++u)
+        {
+            UVarInfo &op = uvars[u];
+            if (static_cast<size_t>(u) < opt.views.size() && opt.views[u].storage >= 0)
+            {
+                op.storage = opt.views[u].storage;
+                op.viewOffset = opt.views[u].offset;
+            }
+            else
+            {
+                op.storage = -1 - u;  // renumbered below
+            }
+        }
+        // Dense storage numbers in order of first appearance.
+        std::map<int, int> renumber;
+        for (int u = 0; u < U; ++u)
+        {
+            auto it = renumber.find(uvars[u].storage);
+            if (it == renumber.end()) it = renumber.emplace(uvars[u].storage, nstore++).first;
+            uvars[u].storage = it->second;
+        }
+        stores.assign(nstore, Storage());
+        for (int u = 0; u < U; ++u)
+        {
+            UVarInfo &op = uvars[u];
+            Storage &st = stores[op.storage];
+            const bool hasView = static_cast<size_t>(u) < opt.views.size() && !opt.views[u].root_dims.empty();
+            if (st.dims.empty())
+            {
+                st.dims = hasView ? opt.views[u].root_dims : op.dims;
+                st.stride.assign(st.dims.size(), 1);
+                for (int d = static_cast<int>(st.dims.size()) - 2; d >= 0; --d)
+                    st.stride[d] = st.stride[d + 1] * st.dims[d + 1];
+            }
+            st.members.push_back(u);
+            st.written = st.written || op.written;
+            st.anyRepeated = st.anyRepeated || op.anyRepeated;
+            const bool tr = static_cast<size_t>(u) < opt.transient.size() && opt.transient[u];
+            st.transient = st.transient && tr;
+            if (op.written && (st.firstWrite < 0 || op.firstWrite < st.firstWrite)) st.firstWrite = op.firstWrite;
+
+            // The view must be "leading indices fixed, trailing dimensions kept" to be resolved exactly.
+            const int nfixed = static_cast<int>(st.dims.size()) - static_cast<int>(op.dims.size());
+            op.plainView = nfixed >= 0;
+            if (op.plainView)
+            {
+                for (size_t d = 0; d < op.dims.size(); ++d) op.plainView = op.plainView && st.dims[d + nfixed] == op.dims[d];
+                long rest = op.viewOffset;
+                op.fixed.assign(nfixed, 0);
+                for (int d = 0; d < nfixed; ++d)
+                {
+                    op.fixed[d] = static_cast<int>(rest / st.stride[d]);
+                    rest -= op.fixed[d] * st.stride[d];
+                    op.plainView = op.plainView && op.fixed[d] < st.dims[d];
+                }
+                op.plainView = op.plainView && rest == 0;
+            }
+            if (!op.plainView || !op.consistent || op.batchDims.size() != 1)
+            {
+                st.elementLocal = false;
+            }
+            else
+            {
+                const int bd = op.batchDims[0] + nfixed;
+                if (st.batchDim < 0) st.batchDim = bd;
+                if (st.batchDim != bd) st.elementLocal = false;
+            }
+        }
+        for (auto &st : stores)
+        {
+            if (batch < 0 || st.batchDim < 0) st.elementLocal = false;
+            if (!st.elementLocal) continue;
+            st.tileSize = 1;
+            st.ldsStride.assign(st.dims.size(), 0);
+            for (int d = static_cast<int>(st.dims.size()) - 1; d >= 0; --d)
+            {
+                if (d == st.batchDim) continue;
+                st.ldsStride[d] = st.tileSize;
+                st.tileSize *= st.dims[d];
+            }
+        }
+    }
+
+    // Is the region "storage at fixed leading indices `fixed`" contained in the union of the written regions?
+    bool Covered(const Storage &st, const std::vector<int> &fixed, const std::vector<std::vector<int>> &written) const
+    {
+        for (const auto &w : written)
+        {
+            if (w.size() <= fixed.size() && std::equal(w.begin(), w.end(), fixed.begin())) return true;
+        }
+        const int next = static_cast<int>(fixed.size());
+        if (next >= static_cast<int>(st.dims.size()) || next == st.batchDim) return false;
+        bool finer = false;
+        for (const auto &w : written)
+        {
+            if (w.size() > fixed.size() && std::equal(fixed.begin(), fixed.end(), w.begin())) finer = true;
+        }
+        if (!finer) return false;
+        std::vector<int> sub = fixed;
+        sub.push_back(0);
+        for (int v = 0; v < st.dims[next]; ++v)
+        {
+            sub.back() = v;
+            if (!Covered(st, sub, written)) return false;
+        }
+        return true;
+    }
+
+    void AnalyseCoverage()
+    {
+        const int K = static_cast<int>(subs.size());
+        std::vector<std::vector<std::vector<int>>> written(stores.size());
+        readCovered.assign(K, std::vector<bool>());
+        oldCovered.assign(K, false);
+        for (int k = 0; k < K; ++k)
+        {
+            const Sub &s = subs[k];
+            readCovered[k].assign(s.in.size(), false);
+            for (size_t v = 0; v < s.in.size(); ++v)
+            {
+                const UVarInfo &op = uvars[s.in[v].uvar];
+                const Storage &st = stores[op.storage];
+                readCovered[k][v] = st.elementLocal && op.plainView && Covered(st, op.fixed, written[op.storage]);
+            }
+            const UVarInfo &oo = uvars[s.out.uvar];
+            const Storage &so = stores[oo.storage];
+            oldCovered[k] = so.elementLocal && oo.plainView && Covered(so, oo.fixed, written[oo.storage]);
+            if (so.elementLocal && oo.plainView && !s.out.repeated) written[oo.storage].push_back(oo.fixed);
+        }
     }
 
     bool CheckFusable(std::string &why)
@@ -271,11 +438,14 @@ class Generator
             why = "an index name has different extents in different kernels";
             return false;
         }
-        for (const auto &u : uvars)
+        for (const auto &st : stores)
         {
-            if (u.written && !u.consistent)
+            // Everything that touches a written tensor must address it through the batch index in one fixed
+            // position, or one workgroup would depend on another's results.
+            if (st.written && !st.elementLocal)
             {
-                why = "variable " + u.name + " is written and used with different shapes or element positions";
+                why = "variable " + uvars[st.members[0]].name +
+                      " is written and used with different shapes, element positions or an unresolvable view";
                 return false;
             }
         }
@@ -283,7 +453,7 @@ class Generator
     }
 
     // --------------------------------------------------------------------------------------- schedule
-    bool IsPureInput(int uvar) const { return !uvars[uvar].written; }
+    bool IsPureInput(int uvar) const { return !stores[uvars[uvar].storage].written; }
 
     // Operand can be read with scalar loads: never written here, no aliasing, small, and its address does not
     // depend on the lane (only on tile / contraction indices, which are literals or uniform loop counters).
@@ -372,8 +542,7 @@ class Generator
         // when it is stored to device memory, otherwise the largest operand read from device memory.
         const VarRef *order = &s.out;
         const UVarInfo &uo = uvars[s.out.uvar];
-        const bool out_stays_on_chip = opt.transient.size() > static_cast<size_t>(s.out.uvar) &&
-                                       opt.transient[s.out.uvar] && uo.lastUse > uo.firstWrite;
+        const bool out_stays_on_chip = stores[uo.storage].transient && uo.lastUse > uo.firstWrite;
         if (out_stays_on_chip)
         {
             const VarRef *big = nullptr;
@@ -433,57 +602,50 @@ class Generator
         }
     }
 
+    bool FromRegisters(int k, int v) const { return subs[k].fusedWithPrev && subs[k].forwardedInput == v; }
+
+    int PhaseOf(int k) const
+    {
+        int p = 0;
+        for (int j = 1; j <= k; ++j)
+        {
+            if (!subs[j].fusedWithPrev) ++p;
+        }
+        return p;
+    }
+
     void ComputeLdsWishes()
     {
         const int K = static_cast<int>(subs.size());
-        for (auto &u : uvars)
+        for (auto &st : stores)
         {
-            u.wantLds = false;
-            u.inLds = false;
+            st.wantLds = false;
+            st.inLds = false;
+            st.liveTo = -1;
         }
         if (batch < 0) return;
-        for (size_t ui = 0; ui < uvars.size(); ++ui)
+        for (size_t si = 0; si < stores.size(); ++si)
         {
-            UVarInfo &u = uvars[ui];
-            if (!u.written || !u.consistent || u.anyRepeated || u.batchDims.size() != 1) continue;
-            // Readers after the first write that are not served from registers.
-            int lastReader = -1;
-            for (int k = u.firstWrite + 1; k < K; ++k)
+            Storage &st = stores[si];
+            if (!st.written || !st.elementLocal || st.anyRepeated) continue;
+            // Last kernel that could take entries of this storage from an LDS tile.
+            for (int k = st.firstWrite + 1; k < K; ++k)
             {
                 const Sub &s = subs[k];
                 for (size_t v = 0; v < s.in.size(); ++v)
                 {
-                    if (s.in[v].uvar != static_cast<int>(ui)) continue;
-                    if (s.fusedWithPrev && s.forwardedInput == static_cast<int>(v)) continue;
-                    lastReader = k;
+                    if (uvars[s.in[v].uvar].storage != static_cast<int>(si)) continue;
+                    if (FromRegisters(k, static_cast<int>(v)) || !readCovered[k][v]) continue;
+                    st.liveTo = k;
                 }
-                if (s.out.uvar == static_cast<int>(ui) && s.op != '=') lastReader = k;
+                if (uvars[s.out.uvar].storage == static_cast<int>(si) && s.op != '=' && oldCovered[k]) st.liveTo = k;
             }
-            if (lastReader < 0) continue;
-            u.wantLds = true;
-            u.liveFrom = u.firstWrite;
-            u.liveTo = lastReader;
+            if (st.liveTo < 0) continue;
+            st.wantLds = true;
             // Kernels fused into one item loop run without a barrier between them, so LDS lifetimes are counted in
             // phases: a tile read in a phase and a tile written in the same phase must not share storage.
-            auto phaseOf = [&](int k) {
-                int p = 0;
-                for (int j = 1; j <= k; ++j)
-                {
-                    if (!subs[j].fusedWithPrev) ++p;
-                }
-                return p;
-            };
-            u.phaseFrom = phaseOf(u.liveFrom);
-            u.phaseTo = phaseOf(u.liveTo);
-            u.tileSize = u.size / u.dims[u.batchDims[0]];
-            u.ldsStride.assign(u.dims.size(), 0);
-            int st = 1;
-            for (int d = static_cast<int>(u.dims.size()) - 1; d >= 0; --d)
-            {
-                if (d == u.batchDims[0]) continue;
-                u.ldsStride[d] = st;
-                st *= u.dims[d];
-            }
+            st.phaseFrom = PhaseOf(st.firstWrite);
+            st.phaseTo = PhaseOf(st.liveTo);
         }
     }
 
@@ -491,19 +653,19 @@ class Generator
     int PlaceLds(int nb)
     {
         std::vector<int> order;
-        for (size_t ui = 0; ui < uvars.size(); ++ui)
+        for (size_t si = 0; si < stores.size(); ++si)
         {
-            if (uvars[ui].wantLds && uvars[ui].inLds) order.push_back(static_cast<int>(ui));
+            if (stores[si].wantLds && stores[si].inLds) order.push_back(static_cast<int>(si));
         }
         std::sort(order.begin(), order.end(), [&](int a, int b) {
-            if (uvars[a].phaseFrom != uvars[b].phaseFrom) return uvars[a].phaseFrom < uvars[b].phaseFrom;
+            if (stores[a].phaseFrom != stores[b].phaseFrom) return stores[a].phaseFrom < stores[b].phaseFrom;
             return a < b;
         });
         int total = 0;
         std::vector<int> placed;
-        for (int ui : order)
+        for (int si : order)
         {
-            UVarInfo &u = uvars[ui];
+            Storage &u = stores[si];
             const int need = u.tileSize * nb;
             int offset = 0;
             bool moved = true;
@@ -512,7 +674,7 @@ class Generator
                 moved = false;
                 for (int pj : placed)
                 {
-                    const UVarInfo &p = uvars[pj];
+                    const Storage &p = stores[pj];
                     const bool timeOverlap = !(p.phaseTo < u.phaseFrom || u.phaseTo < p.phaseFrom);
                     const int pneed = p.tileSize * nb;
                     const bool spaceOverlap = !(p.ldsOffset + pneed <= offset || offset + need <= p.ldsOffset);
@@ -524,7 +686,7 @@ class Generator
                 }
             }
             u.ldsOffset = offset;
-            placed.push_back(ui);
+            placed.push_back(si);
             total = std::max(total, offset + need);
         }
         return total;
@@ -549,10 +711,10 @@ class Generator
         if (batch < 0) NB = 1;
         NB = static_cast<int>(std::min<long>(NB, E));
 
-        // Everything that wants LDS gets it while the workgroup stays within the budget; otherwise shrink the
-        // batch, and finally leave the largest tiles in device memory.
-        const int budgetDoubles = 48 * 1024 / 8;
-        for (auto &u : uvars) u.inLds = u.wantLds;
+        // Everything that wants LDS gets it while the workgroup stays within the 64 KB a workgroup may declare
+        // statically; otherwise shrink the batch, and finally leave the largest tiles in device memory.
+        const int budgetDoubles = 64 * 1024 / 8;
+        for (auto &st : stores) st.inLds = st.wantLds;
         while (true)
         {
             ldsDoubles = PlaceLds(NB);
@@ -563,46 +725,63 @@ class Generator
                 continue;
             }
             int biggest = -1;
-            for (size_t ui = 0; ui < uvars.size(); ++ui)
+            for (size_t si = 0; si < stores.size(); ++si)
             {
-                if (uvars[ui].inLds && (biggest < 0 || uvars[ui].tileSize > uvars[biggest].tileSize))
-                    biggest = static_cast<int>(ui);
+                if (stores[si].inLds && (biggest < 0 || stores[si].tileSize > stores[biggest].tileSize))
+                    biggest = static_cast<int>(si);
             }
             if (biggest < 0) break;
-            uvars[biggest].inLds = false;
+            stores[biggest].inLds = false;
         }
 
-        // Stores to device memory that may be dropped: transient, produced by a plain assignment before any
-        // read, and every later read is served on chip.
-        for (size_t ui = 0; ui < uvars.size(); ++ui)
+        // Stores to device memory that may be dropped: every view of the tensor is transient, and every read of it
+        // inside the group (operands and old values of += / -=) is served from registers or from the LDS tile.
+        const int K = static_cast<int>(subs.size());
+        for (size_t si = 0; si < stores.size(); ++si)
         {
-            UVarInfo &u = uvars[ui];
-            u.elide = false;
-            if (ui >= opt.transient.size() || !opt.transient[ui] || !u.written) continue;
-            bool ok = subs[u.firstWrite].op == '=';
-            bool laterRead = false;
-            for (int k = 0; k < static_cast<int>(subs.size()); ++k)
+            Storage &st = stores[si];
+            st.elide = false;
+            if (!st.transient || !st.written) continue;
+            bool ok = true, anyRead = false;
+            for (int k = 0; k < K; ++k)
             {
                 const Sub &s = subs[k];
                 for (size_t v = 0; v < s.in.size(); ++v)
                 {
-                    if (s.in[v].uvar != static_cast<int>(ui)) continue;
-                    if (k <= u.firstWrite) ok = false;  // read before (or while) first produced
-                    laterRead = true;
-                    const bool fromRegs = s.fusedWithPrev && s.forwardedInput == static_cast<int>(v);
-                    if (!fromRegs && !u.inLds) ok = false;
+                    if (uvars[s.in[v].uvar].storage != static_cast<int>(si)) continue;
+                    anyRead = true;
+                    if (FromRegisters(k, static_cast<int>(v))) continue;
+                    if (!(st.inLds && readCovered[k][v])) ok = false;
                 }
-                if (s.out.uvar == static_cast<int>(ui) && s.op != '=' && !u.inLds) ok = false;
+                if (uvars[s.out.uvar].storage == static_cast<int>(si) && s.op != '=')
+                {
+                    if (!(st.inLds && oldCovered[k])) ok = false;
+                }
             }
-            u.elide = ok && laterRead;
+            st.elide = ok && anyRead;
         }
     }
 
     // --------------------------------------------------------------------------------------- emission
     std::ostringstream out;
 
-    std::string PtrName(int uvar) const { return "T" + str(uvar); }
-    std::string ConstPtrName(int uvar) const { return "C" + str(uvar); }
+    // Kernel parameters are storages; an operand addresses its storage at viewOffset.
+    std::string PtrName(int uvar) const { return "T" + str(uvars[uvar].storage); }
+    std::string ConstPtrName(int uvar) const { return "C" + str(uvars[uvar].storage); }
+    const Storage &StoreOf(int uvar) const { return stores[uvars[uvar].storage]; }
+    // LDS stride of a view dimension, and the constant LDS offset of the view inside the storage's tile
+    int LdsStride(int uvar, size_t d) const
+    {
+        const UVarInfo &op = uvars[uvar];
+        return StoreOf(uvar).ldsStride[d + op.fixed.size()];
+    }
+    long LdsViewOffset(int uvar) const
+    {
+        const UVarInfo &op = uvars[uvar];
+        long off = 0;
+        for (size_t d = 0; d < op.fixed.size(); ++d) off += static_cast<long>(op.fixed[d]) * StoreOf(uvar).ldsStride[d];
+        return off;
+    }
     std::string IdxVar(int id) const { return "i_" + idxName[id]; }
 
     // Offset of an occurrence split into a run-time part (batch entry + lane indices) and, for a given
@@ -610,20 +789,24 @@ class Generator
     std::string RuntimeOffset(const VarRef &r, const Sub &s, bool lds) const
     {
         const UVarInfo &u = uvars[r.uvar];
+        const Storage &st = StoreOf(r.uvar);
         std::string expr;
         auto add = [&](const std::string &term) { expr += (expr.empty() ? "" : " + ") + term; };
-        if (lds) add(str(u.ldsOffset) + " + b * " + str(u.tileSize));
+        if (lds)
+            add(str(st.ldsOffset + LdsViewOffset(r.uvar)) + " + b * " + str(st.tileSize));
+        else if (u.viewOffset != 0)
+            add(str(u.viewOffset));
         for (size_t d = 0; d < r.idx.size(); ++d)
         {
             const int id = r.idx[d];
-            const long st = lds ? u.ldsStride[d] : r.stride[d];
+            const long stride = lds ? LdsStride(r.uvar, d) : r.stride[d];
             if (id == batch)
             {
-                if (!lds) add("e * " + str(st));
+                if (!lds) add("e * " + str(stride));
             }
             else if (has(s.lane, id))
             {
-                add(IdxVar(id) + " * " + str(st));
+                add(IdxVar(id) + " * " + str(stride));
             }
         }
         return expr.empty() ? "0" : expr;
@@ -631,13 +814,12 @@ class Generator
 
     long LiteralOffset(const VarRef &r, const Sub &s, bool lds, const std::vector<int> &value) const
     {
-        const UVarInfo &u = uvars[r.uvar];
         long off = 0;
         for (size_t d = 0; d < r.idx.size(); ++d)
         {
             const int id = r.idx[d];
             if (id == batch || has(s.lane, id)) continue;
-            off += static_cast<long>(value[id]) * (lds ? u.ldsStride[d] : r.stride[d]);
+            off += static_cast<long>(value[id]) * (lds ? LdsStride(r.uvar, d) : r.stride[d]);
         }
         return off;
     }
@@ -654,9 +836,8 @@ class Generator
     {
         const Sub &s = subs[k];
         const VarRef &r = s.in[v];
-        if (s.fusedWithPrev && s.forwardedInput == v) return kFromRegisters;
-        const UVarInfo &u = uvars[r.uvar];
-        if (u.inLds && u.written && u.firstWrite < k) return kFromLds;
+        if (FromRegisters(k, v)) return kFromRegisters;
+        if (StoreOf(r.uvar).inLds && readCovered[k][v]) return kFromLds;
         if (IsUniform(s, r, s.tile)) return kFromConstant;
         return kFromGlobal;
     }
@@ -686,7 +867,7 @@ class Generator
         }
         if (src == kFromConstant)
         {
-            return ConstPtrName(r.uvar) + "[" + str(LiteralOffset(r, s, false, value)) + "]";
+            return ConstPtrName(r.uvar) + "[" + str(uvars[r.uvar].viewOffset + LiteralOffset(r, s, false, value)) + "]";
         }
         const bool lds = (src == kFromLds);
         const long off = LiteralOffset(r, s, lds, value);
@@ -777,21 +958,42 @@ class Generator
                                  RuntimeOffset(s.in[v], s, src == kFromLds) + ";");
         }
         body.bases.push_back("const int o_k" + str(k) + "g = " + RuntimeOffset(s.out, s, false) + ";");
-        if (uvars[s.out.uvar].inLds)
+        if (StoreOf(s.out.uvar).inLds)
             body.bases.push_back("const int o_k" + str(k) + "l = " + RuntimeOffset(s.out, s, true) + ";");
     }
 
     // Is the output variable's tile already on chip before kernel k (needed by += and -=)?
-    bool OldValueInLds(int k) const
+    bool OldValueInLds(int k) const { return StoreOf(subs[k].out.uvar).inLds && oldCovered[k]; }
+
+    // The store of kernel k's output to device memory is dead when a later kernel of the group rewrites the same
+    // view completely, takes the old value from the LDS tile (or does not need it), and every read in between is
+    // served from the tile as well.
+    bool StoreIsDead(int k) const
     {
-        const UVarInfo &u = uvars[subs[k].out.uvar];
-        return u.inLds && u.firstWrite < k;
+        const int out = subs[k].out.uvar;
+        const Storage &st = StoreOf(out);
+        if (!st.inLds || subs[k].out.repeated) return false;
+        const int si = uvars[out].storage;
+        for (int j = k + 1; j < static_cast<int>(subs.size()); ++j)
+        {
+            const Sub &s = subs[j];
+            for (size_t v = 0; v < s.in.size(); ++v)
+            {
+                if (uvars[s.in[v].uvar].storage != si) continue;
+                if (!FromRegisters(j, static_cast<int>(v)) && !readCovered[j][v]) return false;
+            }
+            if (uvars[s.out.uvar].storage == si && s.out.uvar != out) return false;  // keep it simple: same view only
+            if (s.out.uvar == out) return s.op == '=' ? true : oldCovered[j];
+        }
+        return false;
     }
+
+    bool StoresToGlobal(int k) const { return !StoreOf(subs[k].out.uvar).elide && !StoreIsDead(k); }
 
     bool NeedsLdsCopy(int k) const
     {
-        const UVarInfo &u = uvars[subs[k].out.uvar];
-        return u.inLds && u.liveTo > k;
+        const Storage &st = StoreOf(subs[k].out.uvar);
+        return st.inLds && st.liveTo > k;
     }
 
     // Unrolled body of kernel k for one work item.  `forwarded` maps the literal output offsets of the previous
@@ -842,7 +1044,7 @@ class Generator
                 rhs = prod + " * " + rest;
 
             const long goff = LiteralOffset(s.out, s, false, value);
-            const long loff = uvars[s.out.uvar].inLds ? LiteralOffset(s.out, s, true, value) : 0;
+            const long loff = StoreOf(s.out.uvar).inLds ? LiteralOffset(s.out, s, true, value) : 0;
             const std::string gaddr = PtrName(s.out.uvar) + "[o_k" + str(k) + "g + " + str(goff) + "]";
             const std::string laddr = "lds[o_k" + str(k) + "l + " + str(loff) + "]";
             const std::string name = "r" + str(k) + "_" + str(t);
@@ -856,7 +1058,7 @@ class Generator
                 body.compute.push_back("const double " + name + " = " + old + (s.op == '+' ? " + " : " - ") + rhs + ";");
             }
             if (NeedsLdsCopy(k)) body.stores.push_back(laddr + " = " + name + ";");
-            if (!uvars[s.out.uvar].elide) body.stores.push_back(gaddr + " = " + name + ";");
+            if (StoresToGlobal(k)) body.stores.push_back(gaddr + " = " + name + ";");
             produced[goff] = name;
         }
 
@@ -897,13 +1099,13 @@ class Generator
             {
                 const int id = r.idx[d];
                 if (!has(s.contr, id)) continue;
-                const long st = lds ? uvars[r.uvar].ldsStride[d] : r.stride[d];
+                const long st = lds ? LdsStride(r.uvar, d) : r.stride[d];
                 off += (off.empty() ? "" : " + ") + IdxVar(id) + " * " + str(st);
             }
             if (off.empty()) off = "0";
             std::string opnd;
             if (src == kFromConstant)
-                opnd = ConstPtrName(r.uvar) + "[" + off + "]";
+                opnd = ConstPtrName(r.uvar) + "[" + str(uvars[r.uvar].viewOffset) + " + " + off + "]";
             else if (lds)
                 opnd = "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
             else
@@ -924,7 +1126,188 @@ class Generator
             lines.push_back(std::string("const double r = ") + (OldValueInLds(k) ? laddr : gaddr) +
                             (s.op == '+' ? " + sum;" : " - sum;"));
         if (NeedsLdsCopy(k)) lines.push_back(laddr + " = r;");
-        if (!uvars[s.out.uvar].elide) lines.push_back(gaddr + " = r;");
+        if (StoresToGlobal(k)) lines.push_back(gaddr + " = r;");
+    }
+
+    // ------------------------------------------------------------------------------ reduction schedule
+    // A single kernel with few output entries and a very long contraction ("S_i_j = A_n_i_j B_n" with n = 2^20):
+    // mapping lanes to outputs would leave the device idle, so the flattened contraction range is split over
+    // workgroups and over the lanes of a workgroup.  Lane (slice, output entry) accumulates a private partial sum
+    // over its share, the workgroup adds its slices in LDS and writes one partial per output entry to a scratch
+    // buffer, and a second, single-workgroup kernel adds the per-workgroup partials in a fixed order (no atomics:
+    // results are reproducible from run to run).
+    static constexpr long kReductionMinContraction = 2048;
+    static constexpr long kReductionMaxOutputs = 128;
+    static constexpr int kReductionLanes = 256;
+
+    bool UseReductionSchedule() const
+    {
+        if (subs.size() != 1) return false;
+        const Sub &s = subs[0];
+        if (s.out.repeated) return false;
+        return s.contrCount >= kReductionMinContraction && product(s.outIdx, extent) <= kReductionMaxOutputs;
+    }
+
+    // Expression for the element offset of an occurrence given variables named i_<index> for every loop index.
+    std::string FullOffset(const VarRef &r) const
+    {
+        std::string expr = uvars[r.uvar].viewOffset != 0 ? str(uvars[r.uvar].viewOffset) : std::string();
+        for (size_t d = 0; d < r.idx.size(); ++d)
+            expr += (expr.empty() ? "" : " + ") + IdxVar(r.idx[d]) + " * " + str(r.stride[d]);
+        return expr.empty() ? "0" : expr;
+    }
+
+    // Kernel parameters: one pointer per storage, taken from a representative member occurrence.
+    void FillParams(HipKernelPlan &plan, bool honour_elision) const
+    {
+        const int S = static_cast<int>(stores.size());
+        plan.param_occurrence.resize(S);
+        plan.param_offset.assign(S, 0);
+        plan.stored.assign(S, false);
+        for (int si = 0; si < S; ++si)
+        {
+            const int rep = stores[si].members[0];
+            plan.param_occurrence[si] = FirstOccurrence(rep);
+            plan.param_offset[si] = uvars[rep].viewOffset;
+            plan.stored[si] = stores[si].written && !(honour_elision && stores[si].elide);
+        }
+    }
+
+    std::string ParamList() const
+    {
+        std::string p;
+        for (size_t si = 0; si < stores.size(); ++si)
+        {
+            p += std::string(si ? ", " : "") + (stores[si].written ? "double *" : "const double *") +
+                 (opt.noalias ? "__restrict__ " : "") + "T" + str(static_cast<long>(si));
+        }
+        return p;
+    }
+
+    void EmitReduction(HipKernelPlan &plan)
+    {
+        const Sub &s = subs[0];
+        const long O = product(s.outIdx, extent);
+        const long Nc = s.contrCount;
+        const int NTr = kReductionLanes;
+        const long Sn = NTr / O;  // contraction slices per workgroup
+        // Lanes follow the memory order of the largest operand: output entries fastest when its innermost
+        // dimension is an output index, contraction slices fastest otherwise.
+        const VarRef *big = &s.in[0];
+        for (const auto &r : s.in)
+        {
+            if (r.size > big->size) big = &r;
+        }
+        const bool outputsFastest = has(s.outIdx, big->idx.back());
+        long G = std::min<long>(2048, std::max<long>(1, Nc / (Sn * 16)));
+        const long chunk = ((Nc + G - 1) / G + Sn - 1) / Sn * Sn;  // contraction entries per workgroup
+        G = (Nc + chunk - 1) / chunk;
+        const long S2 = NTr / O;
+
+        const std::string dimName = mk.GetDimensionedNameString();
+        char hex[32];
+        std::snprintf(hex, sizeof(hex), "%016llx",
+                      static_cast<unsigned long long>(hashString(dimName + "/reduction/" + (opt.noalias ? "n" : "a") +
+                                                                 (Positional() ? "p" : "u"))));
+        plan.module_name = std::string("acro_red_") + hex;
+        const std::string fPartial = plan.module_name + "_partial", fFinal = plan.module_name + "_final";
+
+        std::ostringstream sched;
+        sched << "reduction schedule: " << O << " output entries, contraction of " << Nc << " terms split over " << G
+              << " workgroups x " << Sn << " slices (" << (outputsFastest ? "output entries" : "slices")
+              << " on adjacent lanes), deterministic two-stage finish\n  [0] " << s.text << "\n";
+        plan.schedule = sched.str();
+
+        out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
+        {
+            std::istringstream lines(plan.schedule);
+            std::string l;
+            while (std::getline(lines, l)) out << "// " << l << "\n";
+        }
+        auto decompose = [&](const std::vector<int> &ids, const std::string &flat, const std::string &indent) {
+            long st = product(ids, extent);
+            for (size_t j = 0; j < ids.size(); ++j)
+            {
+                st /= extent[ids[j]];
+                out << indent << "const int " << IdxVar(ids[j]) << " = (int)(";
+                if (j == 0)
+                    out << flat << " / " << st;
+                else
+                    out << "(" << flat << " / " << st << ") % " << extent[ids[j]];
+                out << ");\n";
+            }
+        };
+
+        // ---- stage 1: per-workgroup partial sums
+        out << "\nextern \"C\" __global__ __launch_bounds__(" << NTr << ") void " << fPartial << "(" << ParamList()
+            << ", double *__restrict__ scratch)\n{\n";
+        out << "    __shared__ double red[" << NTr << "];\n";
+        out << "    const int lane = threadIdx.x;\n";
+        if (outputsFastest)
+            out << "    const int sl = lane / " << O << ", o = lane % " << O << ";\n";
+        else
+            out << "    const int o = lane / " << Sn << ", sl = lane % " << Sn << ";\n";
+        out << "    double sum = 0.0;\n";
+        out << "    if (lane < " << Sn * O << ")\n    {\n";
+        decompose(s.outIdx, "o", "        ");
+        out << "        const long first = (long)blockIdx.x * " << chunk << ";\n";
+        out << "        const long last = first + " << chunk << " < " << Nc << " ? first + " << chunk << " : " << Nc << ";\n";
+        out << "#pragma unroll 4\n";
+        out << "        for (long c = first + sl; c < last; c += " << Sn << ")\n        {\n";
+        decompose(s.contr, "c", "            ");
+        std::string prod;
+        for (const auto &r : s.in)
+        {
+            const std::string opnd = PtrName(r.uvar) + "[" + FullOffset(r) + "]";
+            prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
+        }
+        out << "            sum += " << prod << ";\n        }\n    }\n";
+        out << "    red[lane] = sum;\n    __syncthreads();\n";
+        out << "    if (lane < " << O << ")\n    {\n        double t = 0.0;\n";
+        out << "        for (int k = 0; k < " << Sn << "; ++k) t += red["
+            << (outputsFastest ? "k * " + str(O) + " + lane" : "lane * " + str(Sn) + " + k") << "];\n";
+        out << "        scratch[(long)blockIdx.x * " << O << " + lane] = t;\n    }\n}\n";
+
+        // ---- stage 2: add the per-workgroup partials in a fixed order and apply the assignment operator
+        out << "\nextern \"C\" __global__ __launch_bounds__(" << NTr << ") void " << fFinal << "(double *"
+            << (opt.noalias ? "__restrict__ " : "") << "result, const double *__restrict__ scratch)\n{\n";
+        out << "    __shared__ double red[" << NTr << "];\n";
+        out << "    const int lane = threadIdx.x;\n";
+        out << "    const int g2 = lane / " << O << ", o = lane % " << O << ";\n";
+        out << "    double sum = 0.0;\n";
+        out << "    if (lane < " << S2 * O << ")\n    {\n";
+        out << "        for (long g = g2; g < " << G << "; g += " << S2 << ") sum += scratch[g * " << O << " + o];\n    }\n";
+        out << "    red[lane] = sum;\n    __syncthreads();\n";
+        out << "    if (lane < " << O << ")\n    {\n        double t = 0.0;\n";
+        out << "        for (int k = 0; k < " << S2 << "; ++k) t += red[k * " << O << " + lane];\n";
+        decompose(s.outIdx, "lane", "        ");
+        const std::string dst = "result[" + FullOffset(s.out) + "]";
+        if (s.op == '=')
+            out << "        " << dst << " = t;\n";
+        else
+            out << "        " << dst << " = " << dst << (s.op == '+' ? " + t;\n" : " - t;\n");
+        out << "    }\n}\n";
+
+        plan.source = out.str();
+        plan.scratch_doubles = static_cast<size_t>(G * O);
+        plan.nb = 1;
+        plan.lds_bytes = NTr * 8;
+        FillParams(plan, false);
+        const int S = static_cast<int>(stores.size());
+        HipLaunch partial;
+        partial.function_name = fPartial;
+        partial.grid = static_cast<unsigned>(G);
+        partial.block = NTr;
+        for (int si = 0; si < S; ++si) partial.params.push_back(si);
+        partial.params.push_back(-1);
+        HipLaunch fin;
+        fin.function_name = fFinal;
+        fin.grid = 1;
+        fin.block = NTr;
+        fin.params.push_back(uvars[s.out.uvar].storage);
+        fin.params.push_back(-1);
+        plan.launches.push_back(partial);
+        plan.launches.push_back(fin);
     }
 
     void Emit(HipKernelPlan &plan)
@@ -933,10 +1316,12 @@ class Generator
         const int U = static_cast<int>(uvars.size());
         const std::string dimName = mk.GetDimensionedNameString();
         std::string variant = str(NB) + "/" + str(NT) + "/" + (opt.noalias ? "n" : "a") + (Positional() ? "p" : "u");
-        for (int u = 0; u < U; ++u) variant += uvars[u].elide ? "e" : (uvars[u].inLds ? "l" : "g");
+        for (const auto &st : stores) variant += st.elide ? "e" : (st.inLds ? "l" : "g");
+        for (int u = 0; u < U; ++u) variant += "s" + str(uvars[u].storage) + "@" + str(uvars[u].viewOffset);
         char hex[32];
         std::snprintf(hex, sizeof(hex), "%016llx", static_cast<unsigned long long>(hashString(dimName + variant)));
-        plan.function_name = std::string("acro_mk_") + hex;
+        plan.module_name = std::string("acro_mk_") + hex;
+        const std::string function_name = plan.module_name;
 
         std::ostringstream sched;
         sched << "batch index " << (batch >= 0 ? idxName[batch] : std::string("(none)")) << " extent " << E << ", " << NB
@@ -956,8 +1341,9 @@ class Generator
                 sched << " " << uvars[s.in[v].uvar].name << "<-" << names[SourceOf(k, static_cast<int>(v))];
             }
             const UVarInfo &uo = uvars[s.out.uvar];
-            sched << "; " << uo.name << "->" << (NeedsLdsCopy(k) ? "lds" : "") << (uo.elide ? "" : (NeedsLdsCopy(k) ? "+global" : "global"))
-                  << "\n";
+            const bool elided = !StoresToGlobal(k);
+            sched << "; " << uo.name << "->" << (NeedsLdsCopy(k) ? "lds" : "")
+                  << (elided ? "" : (NeedsLdsCopy(k) ? "+global" : "global")) << "\n";
         }
         plan.schedule = sched.str();
 
@@ -968,25 +1354,21 @@ class Generator
             while (std::getline(lines, l)) out << "// " << l << "\n";
         }
         out << "typedef const __attribute__((address_space(4))) double *acro_scalar_ptr;\n\n";
-        out << "extern \"C\" __global__ __launch_bounds__(" << NT << ") void " << plan.function_name << "(";
-        for (int u = 0; u < U; ++u)
-        {
-            const bool constant = !uvars[u].written;
-            out << (u ? ", " : "") << (constant ? "const double *" : "double *") << (opt.noalias ? "__restrict__ " : "")
-                << PtrName(u);
-        }
+        out << "extern \"C\" __global__ __launch_bounds__(" << NT << ") void " << function_name << "(";
+        out << ParamList();
         out << ")\n{\n";
         if (ldsDoubles > 0) out << "    __shared__ double lds[" << ldsDoubles << "];\n";
-        std::set<int> scalarVars;
+        std::set<int> scalarStores;
         for (int k = 0; k < K; ++k)
         {
             for (size_t v = 0; v < subs[k].in.size(); ++v)
             {
-                if (SourceOf(k, static_cast<int>(v)) == kFromConstant) scalarVars.insert(subs[k].in[v].uvar);
+                if (SourceOf(k, static_cast<int>(v)) == kFromConstant)
+                    scalarStores.insert(uvars[subs[k].in[v].uvar].storage);
             }
         }
-        for (int u : scalarVars)
-            out << "    const acro_scalar_ptr " << ConstPtrName(u) << " = (acro_scalar_ptr)" << PtrName(u) << ";\n";
+        for (int si : scalarStores)
+            out << "    const acro_scalar_ptr C" << si << " = (acro_scalar_ptr)T" << si << ";\n";
         out << "    const int tid = threadIdx.x;\n";
         out << "    const int e0 = blockIdx.x * " << NB << ";\n";
 
@@ -1040,20 +1422,19 @@ class Generator
         out << "}\n";
 
         plan.source = out.str();
-        plan.grid = static_cast<unsigned>((E + NB - 1) / NB);
-        plan.block = static_cast<unsigned>(NT);
+        HipLaunch launch;
+        launch.function_name = function_name;
+        launch.grid = static_cast<unsigned>((E + NB - 1) / NB);
+        launch.block = static_cast<unsigned>(NT);
+        for (size_t si = 0; si < stores.size(); ++si) launch.params.push_back(static_cast<int>(si));
+        plan.launches.push_back(launch);
         plan.nb = NB;
         plan.lds_bytes = ldsDoubles * 8;
-        plan.param_occurrence.resize(U);
-        plan.stored.assign(U, false);
-        for (int u = 0; u < U; ++u)
-        {
-            plan.param_occurrence[u] = FirstOccurrence(u);
-            plan.stored[u] = uvars[u].written && !uvars[u].elide;
-        }
+        FillParams(plan, true);
         for (const auto &s : subs)
         {
-            if (s.out.repeated && s.op == '=') plan.zero_fill_params.push_back(s.out.uvar);
+            if (s.out.repeated && s.op == '=')
+                plan.zero_fills.push_back({uvars[s.out.uvar].storage, uvars[s.out.uvar].viewOffset, s.out.size});
         }
     }
 };

@@ -25,10 +25,22 @@
 namespace acro
 {
 
+// Where an operand lives: operands that are views (leading-index slices) of one tensor share a storage number;
+// offset is the view's first element inside that tensor and root_dims the tensor's own extents.
+struct HipOperandView
+{
+    int storage = -1;
+    long offset = 0;
+    std::vector<int> root_dims;
+};
+
 struct HipCodegenOptions
 {
-    // Per unique variable: the executor allows the store to device memory to be dropped (transient tensor).
+    // Per operand: the executor allows the store to device memory to be dropped (transient tensor).
     std::vector<bool> transient;
+    // Per operand (empty: every operand is a tensor of its own).  Views of one storage may be written under one
+    // name and read under another inside a fused launch; the generator resolves them exactly.
+    std::vector<HipOperandView> views;
     // False when two unique variables overlap in device memory and one of them is written: pointers are then
     // not declared restrict and nothing is read through the constant address space.
     bool noalias = true;
@@ -40,22 +52,40 @@ struct HipCodegenOptions
     int force_nt = 0;  // 0 = choose
 };
 
+// One kernel launch of a plan.  params: >= 0 is an index into HipKernelPlan::param_occurrence (a storage's device
+// pointer), -1 is the plan's scratch buffer.
+struct HipLaunch
+{
+    std::string function_name;
+    unsigned grid = 0;
+    unsigned block = 0;
+    std::vector<int> params;
+};
+
 struct HipKernelPlan
 {
     bool fusable = false;        // false: the group must be run as one launch per kernel
     std::string why_not;         // reason when !fusable
-    std::string function_name;
-    std::string source;
-    unsigned grid = 0;
-    unsigned block = 0;
-    // Kernel parameter i is the device pointer of the tensor bound to this (kernel number, variable number)
-    // occurrence; variable number -1 is that kernel's output.
+    std::string module_name;
+    std::string source;            // one translation unit defining every function of `launches`
+    std::vector<HipLaunch> launches;  // executed in order on the library's stream
+    size_t scratch_doubles = 0;    // device scratch the launches share (partial sums of split contractions)
+    // Kernel parameter i is the device pointer of a storage: the device pointer of the tensor bound to this
+    // (kernel number, variable number) occurrence (variable number -1 is that kernel's output) minus param_offset[i]
+    // elements (the occurrence may be a view into the storage).
     std::vector<std::pair<int, int>> param_occurrence;
+    std::vector<long> param_offset;
     std::vector<bool> stored;      // per parameter: the kernel writes it to device memory
     // Parameters that must be set to zero before the launch: an output assigned with "=" whose index list repeats
     // an index ("A_i_i = B_i") is only written on its diagonal by the kernel, while assignment means zero-fill
     // followed by accumulation (reference exec/CPUInterpretedExecutor.cpp:63-67).
-    std::vector<int> zero_fill_params;
+    struct ZeroFill
+    {
+        int param;    // storage parameter
+        long offset;  // first element
+        long count;   // number of elements
+    };
+    std::vector<ZeroFill> zero_fills;
     int lds_bytes = 0;
     int nb = 0;
     std::string schedule;          // human readable schedule summary (also a comment in the source)

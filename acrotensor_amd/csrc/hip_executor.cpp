@@ -13,6 +13,7 @@
 
 #include "HipRuntime.hpp"
 #include "KernelExecutor.hpp"
+#include "SliceTensor.hpp"
 #include "hip_codegen.hpp"
 #include "hip_kernel.hpp"
 
@@ -61,6 +62,17 @@ class HipExecutor : public KernelExecutor
     {
         HipKernelPlan plan;
         std::unique_ptr<HipKernel> kernel;  // null when the group is not fusable
+        double *scratch = nullptr;          // device buffer shared by the plan's launches
+        ~Variant()
+        {
+            try
+            {
+                hip::Free(scratch);
+            }
+            catch (...)
+            {
+            }
+        }
     };
 
     std::string Describe(const Variant &v)
@@ -73,12 +85,17 @@ class HipExecutor : public KernelExecutor
     {
         std::string key = std::string(options.noalias ? "n" : "a") + (options.positional ? "p" : "u");
         for (bool t : options.transient) key += t ? '1' : '0';
+        for (const auto &v : options.views)
+        {
+            key += "|" + std::to_string(v.storage) + "@" + std::to_string(v.offset);
+            for (int d : v.root_dims) key += "," + std::to_string(d);
+        }
         auto it = Variants.find(key);
         if (it == Variants.end())
         {
             std::unique_ptr<Variant> v(new Variant);
             v->plan = GenerateHipKernel(*MultiKernel, options);
-            if (v->plan.fusable) v->kernel.reset(new HipKernel(v->plan.function_name, v->plan.source));
+            if (v->plan.fusable) v->kernel.reset(new HipKernel(v->plan.module_name, v->plan.source));
             it = Variants.emplace(key, std::move(v)).first;
         }
         LastVariant = it->second.get();
@@ -132,15 +149,45 @@ class HipExecutor : public KernelExecutor
                 written.push_back(MultiKernel->IsOutputUVar(u));
             }
         }
-        options.transient.assign(operand.size(), false);
-        bool hazard = false;
-        for (size_t a = 0; a < operand.size(); ++a)
+        // Storage of every operand: slices are followed up to the tensor they are a view of, so that views of one
+        // tensor are recognised as such (the generator resolves them exactly).
+        const size_t n = operand.size();
+        std::vector<const Tensor *> root(n);
+        std::vector<size_t> root_offset(n, 0);
+        options.views.assign(n, HipOperandView());
+        options.transient.assign(n, false);
+        for (size_t a = 0; a < n; ++a)
         {
-            options.transient[a] = operand[a]->IsTransient();
-            for (size_t b = a + 1; b < operand.size(); ++b)
+            const Tensor *t = operand[a];
+            while (const SliceTensor *sl = dynamic_cast<const SliceTensor *>(t))
             {
-                const double *pa = operand[a]->GetData(), *pb = operand[b]->GetData();
-                const bool overlap = pa < pb + operand[b]->GetSize() && pb < pa + operand[a]->GetSize();
+                root_offset[a] += sl->GetOffset();
+                t = sl->GetParent();
+            }
+            root[a] = t;
+            options.transient[a] = operand[a]->IsTransient();
+            size_t first = a;
+            for (size_t b = 0; b < a; ++b)
+            {
+                if (root[b] == root[a])
+                {
+                    first = b;
+                    break;
+                }
+            }
+            options.views[a].storage = static_cast<int>(first);
+            options.views[a].offset = static_cast<long>(root_offset[a]);
+            options.views[a].root_dims = root[a]->GetDims();
+        }
+        // Two different storages that overlap in memory (external buffers) are a hazard when one is written.
+        bool hazard = false;
+        for (size_t a = 0; a < n; ++a)
+        {
+            for (size_t b = a + 1; b < n; ++b)
+            {
+                if (root[a] == root[b]) continue;
+                const double *pa = root[a]->GetData(), *pb = root[b]->GetData();
+                const bool overlap = pa < pb + root[b]->GetSize() && pb < pa + root[a]->GetSize();
                 if (overlap && (written[a] || written[b])) hazard = true;
             }
         }
@@ -172,21 +219,30 @@ class HipExecutor : public KernelExecutor
         }
         const size_t nparam = v.plan.param_occurrence.size();
         std::vector<double *> ptr(nparam);
-        std::vector<void *> args(nparam);
         for (size_t i = 0; i < nparam; ++i)
         {
             const auto &occ = v.plan.param_occurrence[i];
             ptr[i] = (occ.second < 0 ? outputs[occ.first] : inputs[occ.first][occ.second])->GetDeviceData();
             ACROBATIC_ASSERT(ptr[i] != nullptr, "Tensor has no device memory.");
-            args[i] = &ptr[i];
+            ptr[i] -= v.plan.param_offset[i];
         }
-        for (int i : v.plan.zero_fill_params)
+        if (v.plan.scratch_doubles > 0 && v.scratch == nullptr)
         {
-            const auto &occ = v.plan.param_occurrence[i];
-            Tensor *t = occ.second < 0 ? outputs[occ.first] : inputs[occ.first][occ.second];
-            hip::FillDouble(ptr[i], 0.0, static_cast<size_t>(t->GetSize()));
+            v.scratch = static_cast<double *>(hip::Malloc(v.plan.scratch_doubles * sizeof(double)));
         }
-        v.kernel->Launch(v.plan.grid, v.plan.block, args.data());
+        for (const auto &z : v.plan.zero_fills)
+        {
+            hip::FillDouble(ptr[z.param] + z.offset, 0.0, static_cast<size_t>(z.count));
+        }
+        for (const HipLaunch &launch : v.plan.launches)
+        {
+            std::vector<void *> args(launch.params.size());
+            for (size_t i = 0; i < args.size(); ++i)
+            {
+                args[i] = launch.params[i] < 0 ? static_cast<void *>(&v.scratch) : static_cast<void *>(&ptr[launch.params[i]]);
+            }
+            v.kernel->Launch(launch.function_name, launch.grid, launch.block, args.data());
+        }
     }
 
     std::map<std::string, std::unique_ptr<Variant>> Variants;

@@ -88,8 +88,8 @@ void rtcCheck(hiprtcResult r, const char *what)
 
 }  // namespace
 
-HipKernel::HipKernel(const std::string &function_name, const std::string &source)
-    : FunctionName(function_name), Source(source), CacheHit(false), Module(nullptr), Function(nullptr)
+HipKernel::HipKernel(const std::string &module_name, const std::string &source)
+    : FunctionName(module_name), Source(source), CacheHit(false), Module(nullptr)
 {
     Compile();
 }
@@ -156,19 +156,23 @@ void HipKernel::Compile()
 
 void HipKernel::EnsureLoaded()
 {
-    if (Function != nullptr) return;
+    if (Module != nullptr) return;
     hipModule_t module;
     ACRO_HIP_CHECK(hipModuleLoadData(&module, CodeObject.data()));
     Module = module;
-    hipFunction_t function;
-    ACRO_HIP_CHECK(hipModuleGetFunction(&function, module, FunctionName.c_str()));
-    Function = function;
 }
 
-void HipKernel::Launch(unsigned grid, unsigned block, void **args)
+void HipKernel::Launch(const std::string &function_name, unsigned grid, unsigned block, void **args)
 {
     EnsureLoaded();
-    ACRO_HIP_CHECK(hipModuleLaunchKernel(static_cast<hipFunction_t>(Function), grid, 1, 1, block, 1, 1, 0,
+    auto it = Functions.find(function_name);
+    if (it == Functions.end())
+    {
+        hipFunction_t function;
+        ACRO_HIP_CHECK(hipModuleGetFunction(&function, static_cast<hipModule_t>(Module), function_name.c_str()));
+        it = Functions.emplace(function_name, function).first;
+    }
+    ACRO_HIP_CHECK(hipModuleLaunchKernel(static_cast<hipFunction_t>(it->second), grid, 1, 1, block, 1, 1, 0,
                                          static_cast<hipStream_t>(hip::Stream()), args, nullptr));
 }
 

@@ -9,6 +9,7 @@
 #ifndef ACRO_HIP_KERNEL_HPP
 #define ACRO_HIP_KERNEL_HPP
 
+#include <map>
 #include <string>
 #include <vector>
 
@@ -18,17 +19,18 @@ namespace acro
 class HipKernel
 {
   public:
-    // Compiles immediately; throws std::runtime_error carrying the compiler log on failure.
-    HipKernel(const std::string &function_name, const std::string &source);
+    // Compiles immediately; throws std::runtime_error carrying the compiler log on failure.  module_name labels
+    // the translation unit; the source may define several extern "C" __global__ functions.
+    HipKernel(const std::string &module_name, const std::string &source);
     ~HipKernel();
     HipKernel(const HipKernel &) = delete;
     HipKernel &operator=(const HipKernel &) = delete;
 
     // args: one pointer per kernel parameter (as for hipModuleLaunchKernel)
-    void Launch(unsigned grid, unsigned block, void **args);
+    void Launch(const std::string &function_name, unsigned grid, unsigned block, void **args);
 
     const std::string &GetSource() const { return Source; }
-    const std::string &GetFunctionName() const { return FunctionName; }
+    const std::string &GetModuleName() const { return FunctionName; }
     void WriteCodeToFile(const std::string &path) const;
     size_t GetCodeObjectSize() const { return CodeObject.size(); }
     bool WasCacheHit() const { return CacheHit; }
@@ -41,8 +43,8 @@ class HipKernel
     std::string Source;
     std::vector<char> CodeObject;
     bool CacheHit;
-    void *Module;    // hipModule_t
-    void *Function;  // hipFunction_t
+    void *Module;                            // hipModule_t
+    std::map<std::string, void *> Functions;  // hipFunction_t by name
 };
 
 }  // namespace acro

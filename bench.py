@@ -75,6 +75,60 @@ def cpu_baseline(workloads, sample_elems):
     }
 
 
+FP64_PEAK_GFLOPS = 78600.0
+
+
+def other_workload(at, workloads, args):
+    """Same measurement for cfg1 / cfg2 / cfg3 / cfg5 at the sizes of the baseline configurations."""
+    engine = at.TensorEngine("HIP")
+    name = args.workload
+    if name == "cfg2":
+        J = workloads.config2_inputs()
+        E, Q = J.shape[:2]
+        tJ, Jinv, Jdet = at.Tensor(*J.shape), at.Tensor(*J.shape), at.Tensor(E, Q)
+        tJ.data[...] = J
+        for t in (tJ, Jinv, Jdet):
+            t.MoveToGPU()
+        step = lambda: engine.BatchMatrixInvDet(Jinv, Jdet, tJ)
+        label = "configs[1]: BatchMatrixInvDet, J[65536,64,3,3]"
+        units, unit_name, abytes, flops = E * Q, "Gmatrices/s", E * Q * 152, E * Q * 54
+    else:
+        wl = {"cfg1": workloads.config1, "cfg3": workloads.config3, "cfg5": workloads.config5}[name]()
+        tensors = workloads.bind_to_engine(wl, at, transient=True)
+        for t in tensors.values():
+            t.MoveToGPU()
+        step = lambda: workloads.launch(wl, engine, tensors)
+        label = {"cfg1": "configs[0]: S_i_j = A_n_i_j B_n, n=2^20", "cfg3": "configs[2]: p=2 hex mass assembly, E=32768",
+                 "cfg5": "configs[4]: p=7 hex diffusion apply, E=65536"}[name]
+        abytes, flops = wl.algorithmic_bytes, wl.flops
+        units, unit_name = (wl.dof, "GDOF/s") if wl.dof else (abytes, "GB/s")
+    steps, warmup = min(args.steps, 200), min(args.warmup, 20)
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < args.settle_seconds:
+        step()
+        at.synchronize()
+    for _ in range(warmup):
+        step()
+    at.synchronize()
+    t0 = time.perf_counter()
+    with at.hip_event_timer() as ev:
+        for _ in range(steps):
+            step()
+    at.synchronize()
+    wall = time.perf_counter() - t0
+    launch_s = ev.ms * 1e-3 / steps
+    achieved = abytes / launch_s * 1e-9
+    return {
+        "metric": "%s throughput (1 GPU)" % name, "value": units * steps / wall * 1e-9, "unit": unit_name, "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": wall / steps * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic", "config": {"workload": label},
+        "gflops": flops / launch_s * 1e-9, "pct_fp64_peak": 100.0 * flops / launch_s * 1e-9 / FP64_PEAK_GFLOPS,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": abytes,
+                     "launch_us": launch_s * 1e6},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -86,6 +140,9 @@ def main():
     ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store-all", action="store_true")
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"],
+                    help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
+                         "remaining baseline configurations at their full sizes")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one scale-by-1.0 kernel over X (reads and writes E*512 bytes): the known-size "
                          "kernel that hardware-counter runs are scaled by")
@@ -99,6 +156,10 @@ def main():
 
     if not at.is_hip_ready():
         sys.exit("bench.py needs a HIP device; there is no host fallback.")
+
+    if args.workload != "cfg4":
+        print(json.dumps(other_workload(at, workloads, args)))
+        return
 
     wl = workloads.config4(E=args.elements)
     engine = at.TensorEngine("HIP")

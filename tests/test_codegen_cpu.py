@@ -65,9 +65,26 @@ def test_long_contraction_uses_counted_loops(TE):
     assert "looped" in src or "split" in src
 
 
-def test_diffusion_chain_with_aliased_slices_is_not_fused_blindly(TE):
+def test_diffusion_chain_resolves_slices_of_one_tensor_and_fuses(TE):
+    # U0, U1, U2 are written under their own names and read back through U (and Z the other way round): the
+    # generator resolves the views of one tensor exactly and keeps all of it on chip
     src = chain_source(TE, workloads.config5(E=2, Q=5, P=4), transient=True)
-    assert "__global__" in src or "not fused" in src
+    assert src.count("__global__") == 1 and "not fused" not in src
+    assert "U<-lds" in src and "Z0<-lds" in src and "Z2<-lds" in src
+    assert "U0->lds\n" in src and "Z->lds\n" in src            # transient: no store to device memory
+    # Y is accumulated by three kernels; only the last one stores it
+    assert src.count("Y->lds\n") == 2 and "Y->global" in src
+
+
+def test_views_that_cannot_be_resolved_fall_back(TE):
+    # the same parent viewed with the element index in two different positions cannot be fused
+    T = at.Tensor(4, 4)
+    A, B = at.Tensor(4, 4), at.Tensor(4, 4)
+    TE.BeginMultiKernelLaunch()
+    TE("T_e_i = A_e_i", T, A)
+    TE("B_e_i = T_i_e", B, T)
+    src = TE.EndMultiKernelLaunchGetImplementation()
+    assert "not fused" in src
 
 
 def test_rebinding_one_name_to_two_tensors_switches_to_positional_operands(TE):
