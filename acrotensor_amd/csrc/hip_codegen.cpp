@@ -149,6 +149,35 @@ class Generator
         ChooseTiles();
         PlanFusion();
         ChooseBatching();
+        if (NB == 1 && batch >= 0 && opt.noalias)
+        {
+            // One batch entry per workgroup makes the batch index uniform across the workgroup: operands that
+            // depend on it but on no lane index can then be read with scalar loads too.  Plan again under that
+            // assumption and keep the result if it still puts one entry in a workgroup.
+            batchUniform = true;
+            for (auto &s : subs)
+            {
+                s.fusedWithPrev = false;
+                s.forwardedInput = -1;
+                s.loopMode = false;
+            }
+            ChooseTiles();
+            PlanFusion();
+            ChooseBatching();
+            if (NB != 1)
+            {
+                batchUniform = false;
+                for (auto &s : subs)
+                {
+                    s.fusedWithPrev = false;
+                    s.forwardedInput = -1;
+                    s.loopMode = false;
+                }
+                ChooseTiles();
+                PlanFusion();
+                ChooseBatching();
+            }
+        }
         Emit(plan);
         return plan;
     }
@@ -172,6 +201,7 @@ class Generator
     int NB = 1, NT = 128;
     int ldsDoubles = 0;
     bool extentsConsistent = true;
+    bool batchUniform = false;  // one batch entry per workgroup: the batch index is a scalar
 
     // ------------------------------------------------------------------------------------------ model
     // Operand numbering: unique variables by name, or one operand per occurrence in positional mode.
@@ -459,13 +489,21 @@ class Generator
     // depend on the lane (only on tile / contraction indices, which are literals or uniform loop counters).
     bool IsUniform(const Sub &s, const VarRef &r, const std::vector<int> &tile) const
     {
-        if (!opt.noalias || !IsPureInput(r.uvar) || r.size > 4096) return false;
+        if (!opt.noalias || !IsPureInput(r.uvar)) return false;
+        bool carriesBatch = false;
         for (int id : r.idx)
         {
-            if (id == batch) return false;
+            if (id == batch)
+            {
+                if (!batchUniform) return false;
+                carriesBatch = true;
+                continue;
+            }
             if (!has(tile, id) && !has(s.contr, id)) return false;
         }
-        return true;
+        // What one workgroup reads must be small enough to live in the scalar cache.
+        const long perEntry = carriesBatch ? r.size / extent[batch] : r.size;
+        return perEntry <= 4096;
     }
 
     long LoadsPerItem(const Sub &s, const std::vector<int> &tile) const
@@ -489,6 +527,7 @@ class Generator
     static constexpr long kMaxUnrolledContraction = 512;  // terms of one unrolled sum
     static constexpr long kMaxTile = 32;
     static constexpr long kMaxLiveValues = 160;   // loaded operands + accumulators held by one lane
+    static constexpr long kPrefetchDoubles = 48;  // per lane, held in registers from kernel entry to their phase
 
     void ChooseTiles()
     {
@@ -711,6 +750,48 @@ class Generator
         if (batch < 0) NB = 1;
         NB = static_cast<int>(std::min<long>(NB, E));
 
+        // Lane utilisation at wavefront granularity (a wavefront with a single busy lane costs as much issue time as
+        // a full one).  When the default leaves many lanes idle, look for a batch size / workgroup size that packs
+        // wavefronts better; only switch for a clear gain, small workgroups overlap memory latency better.
+        if (opt.force_nb <= 0 && opt.force_nt <= 0 && envInt("ACRO_HIP_NB") <= 0 && envInt("ACRO_HIP_NT") <= 0 && batch >= 0)
+        {
+            auto utilisation = [&](int nb, int nt) {
+                double busy = 0.0, issued = 0.0;
+                for (const auto &s : subs)
+                {
+                    if (s.fusedWithPrev) continue;
+                    const long items = static_cast<long>(nb) * s.laneCount;
+                    const long passes = (items + nt - 1) / nt;
+                    const long tail = items - (passes - 1) * nt;
+                    const double weight = static_cast<double>(std::max<long>(1, s.tileCount * s.contrCount));
+                    busy += weight * items;
+                    issued += weight * 64.0 * ((passes - 1) * (nt / 64) + (tail + 63) / 64);
+                }
+                return busy / issued;
+            };
+            const double base = utilisation(NB, NT);
+            double best = base;
+            int bestNB = NB, bestNT = NT;
+            for (int nt : {128, 256})
+            {
+                for (int nb = 1; nb <= 16 && nb <= E && nb * maxLane <= nt; ++nb)
+                {
+                    const double u = utilisation(nb, nt);
+                    if (u > best * 1.02)
+                    {
+                        best = u;
+                        bestNB = nb;
+                        bestNT = nt;
+                    }
+                }
+            }
+            if (envInt("ACRO_HIP_PACK") > 0 && best >= 1.25 * base)
+            {
+                NB = bestNB;
+                NT = bestNT;
+            }
+        }
+
         // Everything that wants LDS gets it while the workgroup stays within the 64 KB a workgroup may declare
         // statically; otherwise shrink the batch, and finally leave the largest tiles in device memory.
         const int budgetDoubles = 64 * 1024 / 8;
@@ -842,6 +923,17 @@ class Generator
         return kFromGlobal;
     }
 
+    // Batch part of a scalar operand's address ("e0 * stride + ", e0 being uniform) or nothing.
+    std::string ScalarBase(const VarRef &r) const
+    {
+        std::string base;
+        for (size_t d = 0; d < r.idx.size(); ++d)
+        {
+            if (r.idx[d] == batch) base += "e0 * " + str(r.stride[d]) + " + ";
+        }
+        return base;
+    }
+
     struct Body
     {
         std::vector<std::string> bases;    // run-time base offsets
@@ -851,7 +943,18 @@ class Generator
         std::map<std::string, std::string> loadMemo;
         std::map<std::string, std::string> sumMemo;
         int counter = 0;
+        // Loads of per-entry pure inputs from device memory, in order of first use: (memo key, right-hand side).
+        // They are what a prefetch at kernel entry would issue.
+        std::vector<std::pair<std::string, std::string>> globalLoads;
     };
+
+    // Device-memory operand that a phase may load long before it is used: never written by the group and
+    // addressed through the batch index (the streaming inputs, not small tables).
+    bool Prefetchable(int k, int v) const
+    {
+        const VarRef &r = subs[k].in[v];
+        return SourceOf(k, v) == kFromGlobal && IsPureInput(r.uvar) && has(r.idx, batch);
+    }
 
     std::string OperandExpr(int k, int v, const std::vector<int> &value, Body &body,
                             const std::map<long, std::string> &forwarded)
@@ -867,7 +970,7 @@ class Generator
         }
         if (src == kFromConstant)
         {
-            return ConstPtrName(r.uvar) + "[" + str(uvars[r.uvar].viewOffset + LiteralOffset(r, s, false, value)) + "]";
+            return ConstPtrName(r.uvar) + "[" + ScalarBase(r) + str(uvars[r.uvar].viewOffset + LiteralOffset(r, s, false, value)) + "]";
         }
         const bool lds = (src == kFromLds);
         const long off = LiteralOffset(r, s, lds, value);
@@ -877,9 +980,15 @@ class Generator
         const std::string name = "x" + str(k) + "_" + str(body.counter++);
         const std::string base = "o_" + tag;
         if (lds)
+        {
             body.loads.push_back("const double " + name + " = lds[" + base + " + " + str(off) + "];");
+        }
         else
-            body.loads.push_back("const double " + name + " = " + PtrName(r.uvar) + "[" + base + " + " + str(off) + "];");
+        {
+            const std::string rhs = PtrName(r.uvar) + "[" + base + " + " + str(off) + "]";
+            body.loads.push_back("const double " + name + " = " + rhs + ";");
+            if (Prefetchable(k, v)) body.globalLoads.push_back(std::make_pair(key, rhs));
+        }
         body.loadMemo[key] = name;
         return name;
     }
@@ -998,10 +1107,13 @@ class Generator
 
     // Unrolled body of kernel k for one work item.  `forwarded` maps the literal output offsets of the previous
     // kernel to the registers holding them; on return it describes this kernel's outputs.
-    void EmitUnrolledBody(int k, std::map<long, std::string> &forwarded, std::vector<std::string> &lines)
+    void EmitUnrolledBody(int k, std::map<long, std::string> &forwarded, std::vector<std::string> &lines,
+                          const std::map<std::string, std::string> *preloaded = nullptr,
+                          std::vector<std::pair<std::string, std::string>> *globalLoads = nullptr)
     {
         const Sub &s = subs[k];
         Body body;
+        if (preloaded != nullptr) body.loadMemo = *preloaded;
         EmitBases(k, body);
 
         const int n = static_cast<int>(s.contr.size());
@@ -1068,6 +1180,7 @@ class Generator
         for (const auto &l : body.compute) lines.push_back(l);
         for (const auto &l : body.stores) lines.push_back(l);
         forwarded.swap(produced);
+        if (globalLoads != nullptr) *globalLoads = body.globalLoads;
     }
 
     // Counted-loop body (long contractions): one output per work item, no tile.
@@ -1105,7 +1218,7 @@ class Generator
             if (off.empty()) off = "0";
             std::string opnd;
             if (src == kFromConstant)
-                opnd = ConstPtrName(r.uvar) + "[" + str(uvars[r.uvar].viewOffset) + " + " + off + "]";
+                opnd = ConstPtrName(r.uvar) + "[" + ScalarBase(r) + str(uvars[r.uvar].viewOffset) + " + " + off + "]";
             else if (lds)
                 opnd = "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
             else
@@ -1373,51 +1486,162 @@ class Generator
         out << "    const int e0 = blockIdx.x * " << NB << ";\n";
 
         const bool guardBatch = (E % NB) != 0;
-        int k = 0;
-        bool first = true;
-        while (k < K)
-        {
-            int last = k;
-            while (last + 1 < K && subs[last + 1].fusedWithPrev) ++last;
-            const Sub &s = subs[k];
-            if (!first) out << "    __syncthreads();\n";
-            first = false;
-            const long W = static_cast<long>(NB) * s.laneCount;
-            out << "    for (int w = tid; w < " << W << "; w += " << NT << ")\n    {\n";
-            out << "        const int b = w / " << s.laneCount << ";\n";
-            out << "        const int e = e0 + b;\n";
-            if (guardBatch) out << "        if (e >= " << E << ") break;\n";
+
+        // Work-item header: batch entry and lane indices of item `w` of the phase that kernel `ks` opens.
+        auto emitHeader = [&](const Sub &s, const std::string &indent) {
+            out << indent << "const int b = w / " << s.laneCount << ";\n";
+            out << indent << "const int e = e0 + b;\n";
             if (!s.lane.empty())
             {
-                out << "        const int r_ = w - b * " << s.laneCount << ";\n";
+                out << indent << "const int r_ = w - b * " << s.laneCount << ";\n";
                 long st = s.laneCount;
                 for (size_t j = 0; j < s.lane.size(); ++j)
                 {
                     const int id = s.lane[j];
                     st /= extent[id];
-                    out << "        const int " << IdxVar(id) << " = ";
+                    out << indent << "const int " << IdxVar(id) << " = ";
                     if (j == 0)
                         out << "r_ / " << st << ";\n";
                     else
                         out << "(r_ / " << st << ") % " << extent[id] << ";\n";
                 }
             }
+        };
+
+        // Phases (groups of fused kernels) and what each may prefetch at kernel entry: the loads of streaming
+        // inputs of every phase after the first are issued before the first phase starts, so that their latency
+        // overlaps with the earlier phases instead of stalling a workgroup that few others can cover for.
+        struct Phase
+        {
+            int first, last;
+            long W, passes;
+            // per kernel of the phase and pass: memo key -> register name
+            std::vector<std::vector<std::map<std::string, std::string>>> names;
+            bool prefetched = false;
+        };
+        std::vector<Phase> phases;
+        for (int k = 0; k < K;)
+        {
+            Phase ph;
+            ph.first = k;
+            ph.last = k;
+            while (ph.last + 1 < K && subs[ph.last + 1].fusedWithPrev) ++ph.last;
+            ph.W = static_cast<long>(NB) * subs[k].laneCount;
+            ph.passes = (ph.W + NT - 1) / NT;
+            phases.push_back(ph);
+            k = ph.last + 1;
+        }
+        long prefetchBudget = envInt("ACRO_HIP_PREFETCH") < 0 ? 0 : kPrefetchDoubles;
+        for (size_t pi = 1; pi < phases.size() && phases.size() > 1; ++pi)
+        {
+            Phase &ph = phases[pi];
+            std::vector<std::vector<std::pair<std::string, std::string>>> loads(ph.last - ph.first + 1);
+            long perPass = 0;
+            bool ok = true;
             std::map<long, std::string> forwarded;
-            for (int kk = k; kk <= last; ++kk)
+            for (int kk = ph.first; kk <= ph.last; ++kk)
             {
-                std::vector<std::string> lines;
                 if (subs[kk].loopMode)
-                    EmitLoopBody(kk, lines);
-                else
-                    EmitUnrolledBody(kk, forwarded, lines);
-                // Scopes nest (closed after the group) so that a kernel applied in registers sees the values
-                // of its producer.
-                out << "        {\n";
-                for (const auto &l : lines) out << "            " << l << "\n";
+                {
+                    ok = false;
+                    break;
+                }
+                std::vector<std::string> scratchLines;
+                EmitUnrolledBody(kk, forwarded, scratchLines, nullptr, &loads[kk - ph.first]);
+                perPass += static_cast<long>(loads[kk - ph.first].size());
             }
-            for (int kk = k; kk <= last; ++kk) out << "        }\n";
-            out << "    }\n";
-            k = last + 1;
+            if (!ok || perPass == 0 || perPass * ph.passes > prefetchBudget) continue;
+            prefetchBudget -= perPass * ph.passes;
+            ph.prefetched = true;
+            ph.names.assign(ph.last - ph.first + 1, std::vector<std::map<std::string, std::string>>(ph.passes));
+            out << "    // streaming inputs of kernel " << ph.first << (ph.last > ph.first ? " (and fused followers)" : "")
+                << ", requested before the first phase\n";
+            for (long j = 0; j < ph.passes; ++j)
+            {
+                for (int kk = ph.first; kk <= ph.last; ++kk)
+                {
+                    int n = 0;
+                    for (const auto &ld : loads[kk - ph.first])
+                    {
+                        const std::string name = "pf" + str(kk) + "_" + str(j) + "_" + str(n++);
+                        ph.names[kk - ph.first][j][ld.first] = name;
+                        out << "    double " << name << " = 0.0;\n";
+                    }
+                }
+                out << "    {\n        const int w = tid + " << j * NT << ";\n        if (w < " << ph.W << ")\n        {\n";
+                emitHeader(subs[ph.first], "            ");
+                std::string indent = "            ";
+                if (guardBatch)
+                {
+                    out << indent << "if (e < " << E << ")\n" << indent << "{\n";
+                    indent += "    ";
+                }
+                for (int kk = ph.first; kk <= ph.last; ++kk)
+                {
+                    if (loads[kk - ph.first].empty()) continue;
+                    Body bases;
+                    EmitBases(kk, bases);
+                    for (const auto &l : bases.bases) out << indent << l << "\n";
+                    for (const auto &ld : loads[kk - ph.first])
+                        out << indent << ph.names[kk - ph.first][j][ld.first] << " = " << ld.second << ";\n";
+                }
+                if (guardBatch) out << "            }\n";
+                out << "        }\n    }\n";
+            }
+        }
+
+        bool first = true;
+        for (const Phase &ph : phases)
+        {
+            const Sub &s = subs[ph.first];
+            if (!first) out << "    __syncthreads();\n";
+            first = false;
+            const long npass = ph.prefetched ? ph.passes : 1;
+            for (long j = 0; j < npass; ++j)
+            {
+                std::string indent;
+                if (ph.prefetched)
+                {
+                    out << "    {\n        const int w = tid + " << j * NT << ";\n        if (w < " << ph.W << ")\n        {\n";
+                    indent = "            ";
+                    emitHeader(s, indent);
+                    if (guardBatch)
+                    {
+                        out << indent << "if (e < " << E << ")\n" << indent << "{\n";
+                        indent += "    ";
+                    }
+                }
+                else
+                {
+                    out << "    for (int w = tid; w < " << ph.W << "; w += " << NT << ")\n    {\n";
+                    indent = "        ";
+                    emitHeader(s, indent);
+                    if (guardBatch) out << indent << "if (e >= " << E << ") break;\n";
+                }
+                std::map<long, std::string> forwarded;
+                for (int kk = ph.first; kk <= ph.last; ++kk)
+                {
+                    std::vector<std::string> lines;
+                    if (subs[kk].loopMode)
+                        EmitLoopBody(kk, lines);
+                    else
+                        EmitUnrolledBody(kk, forwarded, lines, ph.prefetched ? &ph.names[kk - ph.first][j] : nullptr);
+                    // Scopes nest (closed after the group) so that a kernel applied in registers sees the values
+                    // of its producer.
+                    out << indent << "{\n";
+                    for (const auto &l : lines) out << indent << "    " << l << "\n";
+                }
+                for (int kk = ph.first; kk <= ph.last; ++kk) out << indent << "}\n";
+                if (ph.prefetched)
+                {
+                    if (guardBatch) out << "            }\n";
+                    out << "        }\n    }\n";
+                }
+                else
+                {
+                    out << "    }\n";
+                }
+            }
         }
         out << "}\n";
 
