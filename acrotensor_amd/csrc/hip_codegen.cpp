@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <cstdint>
 #include <cstdlib>
+#include <functional>
 #include <map>
 #include <set>
 #include <sstream>
@@ -44,6 +45,8 @@ struct Sub
     bool loopMode = false;    // contraction as counted loops instead of unrolled code
     bool fusedWithPrev = false;
     int forwardedInput = -1;  // input occurrence served from the previous kernel's registers
+    bool forwardedOld = false;  // the old value of a += / -= output is the previous kernel's result, in registers
+    int phase = 0;              // barrier-separated phase the kernel runs in
     long laneCount = 1, tileCount = 1, contrCount = 1;
 };
 
@@ -159,6 +162,7 @@ class Generator
             {
                 s.fusedWithPrev = false;
                 s.forwardedInput = -1;
+                s.forwardedOld = false;
                 s.loopMode = false;
             }
             ChooseTiles();
@@ -171,6 +175,7 @@ class Generator
                 {
                     s.fusedWithPrev = false;
                     s.forwardedInput = -1;
+                    s.forwardedOld = false;
                     s.loopMode = false;
                 }
                 ChooseTiles();
@@ -639,19 +644,88 @@ class Generator
             s.tileCount = p.tileCount;
             s.loopMode = false;
         }
+        // Accumulation chains ("Y = ...", "Y += ...", "Y += ..."): a kernel that adds into exactly what the previous
+        // kernel produced, with the same pencil decomposition, takes the old value from that kernel's registers.
+        for (int k = 1; k < K; ++k)
+        {
+            Sub &s = subs[k];
+            const Sub &p = subs[k - 1];
+            if (s.fusedWithPrev || s.op == '=' || s.loopMode || p.loopMode || s.out.repeated) continue;
+            if (s.out.uvar != p.out.uvar || s.out.idx != p.out.idx || s.tile != p.tile || s.lane != p.lane) continue;
+            bool reads_it = false;
+            for (const auto &r : s.in) reads_it = reads_it || uvars[r.uvar].storage == uvars[p.out.uvar].storage;
+            if (reads_it) continue;
+            s.fusedWithPrev = true;
+            s.forwardedInput = -1;
+            s.forwardedOld = true;
+        }
+        AssignPhases();
+    }
+
+    // Two operands address overlapping memory: same storage and neither view's fixed leading indices exclude the
+    // other's.
+    bool ViewsOverlap(int ua, int ub) const
+    {
+        const UVarInfo &a = uvars[ua], &b = uvars[ub];
+        if (a.storage != b.storage) return false;
+        if (!a.plainView || !b.plainView) return true;
+        const size_t n = std::min(a.fixed.size(), b.fixed.size());
+        for (size_t d = 0; d < n; ++d)
+        {
+            if (a.fixed[d] != b.fixed[d]) return false;
+        }
+        return true;
+    }
+
+    bool KernelsIndependent(int ka, int kb) const
+    {
+        const Sub &a = subs[ka], &b = subs[kb];
+        if (ViewsOverlap(a.out.uvar, b.out.uvar)) return false;
+        for (const auto &r : b.in)
+        {
+            if (ViewsOverlap(a.out.uvar, r.uvar)) return false;
+        }
+        for (const auto &r : a.in)
+        {
+            if (ViewsOverlap(b.out.uvar, r.uvar)) return false;
+        }
+        return true;
+    }
+
+    // Chains (a kernel with the kernels applied in its registers) that do not depend on each other share a phase:
+    // their work items are laid side by side across the workgroup's wavefronts, which shortens the sequence of
+    // barrier-separated steps one workgroup walks through.
+    void AssignPhases()
+    {
+        const int K = static_cast<int>(subs.size());
+        int phase = 0;
+        int phaseStart = 0;  // first kernel of the current phase
+        for (int k = 0; k < K; ++k)
+        {
+            if (k > 0 && !subs[k].fusedWithPrev)
+            {
+                // k opens a new chain: may the whole chain join the current phase?
+                int last = k;
+                while (last + 1 < K && subs[last + 1].fusedWithPrev) ++last;
+                bool join = envInt("ACRO_HIP_MERGE") >= 0 && !subs[k].loopMode;
+                for (int a = phaseStart; a < k && join; ++a)
+                {
+                    if (subs[a].loopMode) join = false;
+                    for (int b = k; b <= last && join; ++b) join = KernelsIndependent(a, b);
+                }
+                if (!join)
+                {
+                    ++phase;
+                    phaseStart = k;
+                }
+            }
+            subs[k].phase = phase;
+        }
     }
 
     bool FromRegisters(int k, int v) const { return subs[k].fusedWithPrev && subs[k].forwardedInput == v; }
 
-    int PhaseOf(int k) const
-    {
-        int p = 0;
-        for (int j = 1; j <= k; ++j)
-        {
-            if (!subs[j].fusedWithPrev) ++p;
-        }
-        return p;
-    }
+    int PhaseOf(int k) const { return subs[k].phase; }
 
     void ComputeLdsWishes()
     {
@@ -677,7 +751,8 @@ class Generator
                     if (FromRegisters(k, static_cast<int>(v)) || !readCovered[k][v]) continue;
                     st.liveTo = k;
                 }
-                if (uvars[s.out.uvar].storage == static_cast<int>(si) && s.op != '=' && oldCovered[k]) st.liveTo = k;
+                if (uvars[s.out.uvar].storage == static_cast<int>(si) && s.op != '=' && !s.forwardedOld && oldCovered[k])
+                    st.liveTo = k;
             }
             if (st.liveTo < 0) continue;
             st.wantLds = true;
@@ -834,7 +909,7 @@ class Generator
                     if (FromRegisters(k, static_cast<int>(v))) continue;
                     if (!(st.inLds && readCovered[k][v])) ok = false;
                 }
-                if (uvars[s.out.uvar].storage == static_cast<int>(si) && s.op != '=')
+                if (uvars[s.out.uvar].storage == static_cast<int>(si) && s.op != '=' && !s.forwardedOld)
                 {
                     if (!(st.inLds && oldCovered[k])) ok = false;
                 }
@@ -1081,7 +1156,9 @@ class Generator
     {
         const int out = subs[k].out.uvar;
         const Storage &st = StoreOf(out);
-        if (!st.inLds || subs[k].out.repeated) return false;
+        if (subs[k].out.repeated) return false;
+        const bool nextTakesRegisters = k + 1 < static_cast<int>(subs.size()) && subs[k + 1].forwardedOld;
+        if (!st.inLds && !nextTakesRegisters) return false;
         const int si = uvars[out].storage;
         for (int j = k + 1; j < static_cast<int>(subs.size()); ++j)
         {
@@ -1089,10 +1166,10 @@ class Generator
             for (size_t v = 0; v < s.in.size(); ++v)
             {
                 if (uvars[s.in[v].uvar].storage != si) continue;
-                if (!FromRegisters(j, static_cast<int>(v)) && !readCovered[j][v]) return false;
+                if (!FromRegisters(j, static_cast<int>(v)) && !(st.inLds && readCovered[j][v])) return false;
             }
             if (uvars[s.out.uvar].storage == si && s.out.uvar != out) return false;  // keep it simple: same view only
-            if (s.out.uvar == out) return s.op == '=' ? true : oldCovered[j];
+            if (s.out.uvar == out) return s.op == '=' || s.forwardedOld || (st.inLds && oldCovered[j]);
         }
         return false;
     }
@@ -1166,7 +1243,7 @@ class Generator
             }
             else
             {
-                const std::string old = OldValueInLds(k) ? laddr : gaddr;
+                const std::string old = s.forwardedOld ? forwarded.at(goff) : (OldValueInLds(k) ? laddr : gaddr);
                 body.compute.push_back("const double " + name + " = " + old + (s.op == '+' ? " + " : " - ") + rhs + ";");
             }
             if (NeedsLdsCopy(k)) body.stores.push_back(laddr + " = " + name + ";");
@@ -1447,7 +1524,7 @@ class Generator
             sched << ")=" << s.laneCount << " tile(";
             for (size_t j = 0; j < s.tile.size(); ++j) sched << (j ? "," : "") << idxName[s.tile[j]];
             sched << ")=" << s.tileCount << " contraction=" << s.contrCount << (s.loopMode ? " looped" : " unrolled")
-                  << (s.fusedWithPrev ? " in-register after previous" : "") << "; operands:";
+                  << (s.fusedWithPrev ? " in-register after previous" : "") << " phase " << s.phase << "; operands:";
             for (size_t v = 0; v < s.in.size(); ++v)
             {
                 static const char *const names[] = {"registers", "scalar", "lds", "global"};
@@ -1508,139 +1585,173 @@ class Generator
             }
         };
 
-        // Phases (groups of fused kernels) and what each may prefetch at kernel entry: the loads of streaming
-        // inputs of every phase after the first are issued before the first phase starts, so that their latency
-        // overlaps with the earlier phases instead of stalling a workgroup that few others can cover for.
-        struct Phase
+        // Phases, the chains (a kernel plus the kernels applied in its registers) each of them runs side by side, and
+        // what each may prefetch at kernel entry: the loads of streaming inputs of every phase after the first are
+        // issued before the first phase starts, so that their latency overlaps with the earlier phases instead of
+        // stalling a workgroup that few others can cover for.
+        struct Chain
         {
             int first, last;
-            long W, passes;
-            // per kernel of the phase and pass: memo key -> register name
+            long W;       // work items
+            long offset;  // first item slot in the phase (multiple of the wavefront size)
+            std::vector<std::vector<std::pair<std::string, std::string>>> loads;  // per kernel: prefetchable loads
+            // per kernel and pass: memo key -> register name
             std::vector<std::vector<std::map<std::string, std::string>>> names;
+        };
+        struct Phase
+        {
+            std::vector<Chain> chains;
+            long slots = 0, passes = 1;
             bool prefetched = false;
         };
         std::vector<Phase> phases;
         for (int k = 0; k < K;)
         {
-            Phase ph;
-            ph.first = k;
-            ph.last = k;
-            while (ph.last + 1 < K && subs[ph.last + 1].fusedWithPrev) ++ph.last;
-            ph.W = static_cast<long>(NB) * subs[k].laneCount;
-            ph.passes = (ph.W + NT - 1) / NT;
-            phases.push_back(ph);
-            k = ph.last + 1;
+            Chain c;
+            c.first = k;
+            c.last = k;
+            while (c.last + 1 < K && subs[c.last + 1].fusedWithPrev) ++c.last;
+            c.W = static_cast<long>(NB) * subs[k].laneCount;
+            if (phases.empty() || subs[k].phase != subs[phases.back().chains.back().first].phase) phases.push_back(Phase());
+            Phase &ph = phases.back();
+            c.offset = ph.slots;
+            ph.slots += (c.W + 63) / 64 * 64;
+            ph.chains.push_back(c);
+            k = c.last + 1;
         }
+        for (auto &ph : phases)
+        {
+            if (ph.chains.size() == 1) ph.slots = ph.chains[0].W;
+            ph.passes = (ph.slots + NT - 1) / NT;
+        }
+
         long prefetchBudget = envInt("ACRO_HIP_PREFETCH") < 0 ? 0 : kPrefetchDoubles;
-        for (size_t pi = 1; pi < phases.size() && phases.size() > 1; ++pi)
+        for (size_t pi = 1; pi < phases.size(); ++pi)
         {
             Phase &ph = phases[pi];
-            std::vector<std::vector<std::pair<std::string, std::string>>> loads(ph.last - ph.first + 1);
-            long perPass = 0;
+            long perLane = 0;  // registers one lane needs: a lane serves at most one chain per pass
             bool ok = true;
-            std::map<long, std::string> forwarded;
-            for (int kk = ph.first; kk <= ph.last; ++kk)
+            for (auto &c : ph.chains)
             {
-                if (subs[kk].loopMode)
+                c.loads.assign(c.last - c.first + 1, {});
+                std::map<long, std::string> forwarded;
+                long perPass = 0;
+                for (int kk = c.first; kk <= c.last; ++kk)
                 {
-                    ok = false;
-                    break;
-                }
-                std::vector<std::string> scratchLines;
-                EmitUnrolledBody(kk, forwarded, scratchLines, nullptr, &loads[kk - ph.first]);
-                perPass += static_cast<long>(loads[kk - ph.first].size());
-            }
-            if (!ok || perPass == 0 || perPass * ph.passes > prefetchBudget) continue;
-            prefetchBudget -= perPass * ph.passes;
-            ph.prefetched = true;
-            ph.names.assign(ph.last - ph.first + 1, std::vector<std::map<std::string, std::string>>(ph.passes));
-            out << "    // streaming inputs of kernel " << ph.first << (ph.last > ph.first ? " (and fused followers)" : "")
-                << ", requested before the first phase\n";
-            for (long j = 0; j < ph.passes; ++j)
-            {
-                for (int kk = ph.first; kk <= ph.last; ++kk)
-                {
-                    int n = 0;
-                    for (const auto &ld : loads[kk - ph.first])
+                    if (subs[kk].loopMode)
                     {
-                        const std::string name = "pf" + str(kk) + "_" + str(j) + "_" + str(n++);
-                        ph.names[kk - ph.first][j][ld.first] = name;
-                        out << "    double " << name << " = 0.0;\n";
+                        ok = false;
+                        break;
                     }
+                    std::vector<std::string> scratchLines;
+                    EmitUnrolledBody(kk, forwarded, scratchLines, nullptr, &c.loads[kk - c.first]);
+                    perPass += static_cast<long>(c.loads[kk - c.first].size());
                 }
-                out << "    {\n        const int w = tid + " << j * NT << ";\n        if (w < " << ph.W << ")\n        {\n";
-                emitHeader(subs[ph.first], "            ");
-                std::string indent = "            ";
-                if (guardBatch)
+                perLane = std::max(perLane, perPass);
+            }
+            if (!ok || perLane == 0 || perLane * ph.passes > prefetchBudget) continue;
+            prefetchBudget -= perLane * ph.passes;
+            ph.prefetched = true;
+        }
+
+        // Emits, for pass j of a phase (or for the item loop when j < 0), the selection of the chain a lane works
+        // for and calls `body` inside the guarded scope of one work item.
+        auto emitItems = [&](const Phase &ph, long j, const std::function<void(const Chain &, const std::string &)> &body) {
+            std::string indent = "        ";
+            if (j < 0)
+                out << "    for (int w0 = tid; w0 < " << ph.slots << "; w0 += " << NT << ")\n    {\n";
+            else
+                out << "    {\n        const int w0 = tid + " << j * NT << ";\n";
+            for (size_t ci = 0; ci < ph.chains.size(); ++ci)
+            {
+                const Chain &c = ph.chains[ci];
+                const long end = c.offset + (ph.chains.size() == 1 ? c.W : (c.W + 63) / 64 * 64);
+                if (ph.chains.size() > 1)
                 {
-                    out << indent << "if (e < " << E << ")\n" << indent << "{\n";
+                    out << indent << (ci ? "else if" : "if") << " (w0 < " << end << ")\n" << indent << "{\n";
                     indent += "    ";
                 }
-                for (int kk = ph.first; kk <= ph.last; ++kk)
+                out << indent << "const int w = w0 - " << c.offset << ";\n";
+                out << indent << "if (w < " << c.W << ")\n" << indent << "{\n";
+                emitHeader(subs[c.first], indent + "    ");
+                std::string inner = indent + "    ";
+                if (guardBatch)
                 {
-                    if (loads[kk - ph.first].empty()) continue;
-                    Body bases;
-                    EmitBases(kk, bases);
-                    for (const auto &l : bases.bases) out << indent << l << "\n";
-                    for (const auto &ld : loads[kk - ph.first])
-                        out << indent << ph.names[kk - ph.first][j][ld.first] << " = " << ld.second << ";\n";
+                    out << inner << "if (e < " << E << ")\n" << inner << "{\n";
+                    inner += "    ";
                 }
-                if (guardBatch) out << "            }\n";
-                out << "        }\n    }\n";
+                body(c, inner);
+                if (guardBatch) out << indent << "    }\n";
+                out << indent << "}\n";
+                if (ph.chains.size() > 1)
+                {
+                    indent.resize(indent.size() - 4);
+                    out << indent << "}\n";
+                }
+            }
+            out << "    }\n";
+        };
+
+        for (auto &ph : phases)
+        {
+            if (!ph.prefetched) continue;
+            out << "    // streaming inputs of phase " << subs[ph.chains[0].first].phase << ", requested before the first phase\n";
+            for (auto &c : ph.chains)
+                c.names.assign(c.last - c.first + 1, std::vector<std::map<std::string, std::string>>(ph.passes));
+            for (long j = 0; j < ph.passes; ++j)
+            {
+                // One register set per pass, shared by the chains (a lane serves one chain in a pass).
+                long widest = 0;
+                for (auto &c : ph.chains)
+                {
+                    long n = 0;
+                    for (int kk = c.first; kk <= c.last; ++kk)
+                    {
+                        for (const auto &ld : c.loads[kk - c.first])
+                            c.names[kk - c.first][j][ld.first] = "pf" + str(subs[c.first].phase) + "_" + str(j) + "_" + str(n++);
+                    }
+                    widest = std::max(widest, n);
+                }
+                for (long n = 0; n < widest; ++n)
+                    out << "    double pf" << subs[ph.chains[0].first].phase << "_" << j << "_" << n << " = 0.0;\n";
+                emitItems(ph, j, [&](const Chain &c, const std::string &indent) {
+                    for (int kk = c.first; kk <= c.last; ++kk)
+                    {
+                        if (c.loads[kk - c.first].empty()) continue;
+                        Body bases;
+                        EmitBases(kk, bases);
+                        for (const auto &l : bases.bases) out << indent << l << "\n";
+                        for (const auto &ld : c.loads[kk - c.first])
+                            out << indent << c.names[kk - c.first][j].at(ld.first) << " = " << ld.second << ";\n";
+                    }
+                });
             }
         }
 
         bool first = true;
         for (const Phase &ph : phases)
         {
-            const Sub &s = subs[ph.first];
             if (!first) out << "    __syncthreads();\n";
             first = false;
             const long npass = ph.prefetched ? ph.passes : 1;
             for (long j = 0; j < npass; ++j)
             {
-                std::string indent;
-                if (ph.prefetched)
-                {
-                    out << "    {\n        const int w = tid + " << j * NT << ";\n        if (w < " << ph.W << ")\n        {\n";
-                    indent = "            ";
-                    emitHeader(s, indent);
-                    if (guardBatch)
+                emitItems(ph, ph.prefetched ? j : -1, [&](const Chain &c, const std::string &indent) {
+                    std::map<long, std::string> forwarded;
+                    for (int kk = c.first; kk <= c.last; ++kk)
                     {
-                        out << indent << "if (e < " << E << ")\n" << indent << "{\n";
-                        indent += "    ";
+                        std::vector<std::string> lines;
+                        if (subs[kk].loopMode)
+                            EmitLoopBody(kk, lines);
+                        else
+                            EmitUnrolledBody(kk, forwarded, lines, ph.prefetched ? &c.names[kk - c.first][j] : nullptr);
+                        // Scopes nest (closed after the chain) so that a kernel applied in registers sees the
+                        // values of its producer.
+                        out << indent << "{\n";
+                        for (const auto &l : lines) out << indent << "    " << l << "\n";
                     }
-                }
-                else
-                {
-                    out << "    for (int w = tid; w < " << ph.W << "; w += " << NT << ")\n    {\n";
-                    indent = "        ";
-                    emitHeader(s, indent);
-                    if (guardBatch) out << indent << "if (e >= " << E << ") break;\n";
-                }
-                std::map<long, std::string> forwarded;
-                for (int kk = ph.first; kk <= ph.last; ++kk)
-                {
-                    std::vector<std::string> lines;
-                    if (subs[kk].loopMode)
-                        EmitLoopBody(kk, lines);
-                    else
-                        EmitUnrolledBody(kk, forwarded, lines, ph.prefetched ? &ph.names[kk - ph.first][j] : nullptr);
-                    // Scopes nest (closed after the group) so that a kernel applied in registers sees the values
-                    // of its producer.
-                    out << indent << "{\n";
-                    for (const auto &l : lines) out << indent << "    " << l << "\n";
-                }
-                for (int kk = ph.first; kk <= ph.last; ++kk) out << indent << "}\n";
-                if (ph.prefetched)
-                {
-                    if (guardBatch) out << "            }\n";
-                    out << "        }\n    }\n";
-                }
-                else
-                {
-                    out << "    }\n";
-                }
+                    for (int kk = c.first; kk <= c.last; ++kk) out << indent << "}\n";
+                });
             }
         }
         out << "}\n";
