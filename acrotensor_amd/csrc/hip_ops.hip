@@ -87,6 +87,9 @@ struct SmallMatrix<3>
 };
 
 // One workgroup = kLanes consecutive matrices.  WANT_INV / WANT_DET select the outputs.
+// The matrices of a workgroup are contiguous in memory, so the workgroup copies them to and from LDS as one
+// stream of 16-byte pieces (full-rate HBM access), and lane t works on matrix t out of LDS.  For 2x2 the lane
+// stride in LDS is padded from 4 to 5 doubles so that lanes fall into distinct banks; 9 and 1 are odd already.
 template <int M, bool WANT_INV, bool WANT_DET>
 __global__ __launch_bounds__(kLanes) void batchMatrixKernel(const double *__restrict__ A, double *__restrict__ Ainv,
                                                             double *__restrict__ Adet, size_t num_mat)
@@ -100,7 +103,23 @@ __global__ __launch_bounds__(kLanes) void batchMatrixKernel(const double *__rest
     const int ndbl = static_cast<int>(count) * MM;
     const double *src = A + first * MM;
 
-    for (int i = threadIdx.x; i < ndbl; i += kLanes) tile[(i / MM) * LS + (i % MM)] = src[i];
+    // first * MM * 8 bytes is a multiple of 16 (kLanes is even), so pairs of doubles are aligned
+    const double2 *src2 = reinterpret_cast<const double2 *>(src);
+    for (int i = threadIdx.x; i < ndbl / 2; i += kLanes)
+    {
+        const double2 v = src2[i];
+        if (LS == MM)
+        {
+            tile[2 * i] = v.x;
+            tile[2 * i + 1] = v.y;
+        }
+        else
+        {
+            tile[((2 * i) / MM) * LS + ((2 * i) % MM)] = v.x;
+            tile[((2 * i + 1) / MM) * LS + ((2 * i + 1) % MM)] = v.y;
+        }
+    }
+    if ((ndbl & 1) && threadIdx.x == 0) tile[((ndbl - 1) / MM) * LS + ((ndbl - 1) % MM)] = src[ndbl - 1];
     __syncthreads();
 
     double a[MM], r[MM];
@@ -123,7 +142,23 @@ __global__ __launch_bounds__(kLanes) void batchMatrixKernel(const double *__rest
         }
         __syncthreads();
         double *dst = Ainv + first * MM;
-        for (int i = threadIdx.x; i < ndbl; i += kLanes) dst[i] = tile[(i / MM) * LS + (i % MM)];
+        double2 *dst2 = reinterpret_cast<double2 *>(dst);
+        for (int i = threadIdx.x; i < ndbl / 2; i += kLanes)
+        {
+            double2 v;
+            if (LS == MM)
+            {
+                v.x = tile[2 * i];
+                v.y = tile[2 * i + 1];
+            }
+            else
+            {
+                v.x = tile[((2 * i) / MM) * LS + ((2 * i) % MM)];
+                v.y = tile[((2 * i + 1) / MM) * LS + ((2 * i + 1) % MM)];
+            }
+            dst2[i] = v;
+        }
+        if ((ndbl & 1) && threadIdx.x == 0) dst[ndbl - 1] = tile[((ndbl - 1) / MM) * LS + ((ndbl - 1) % MM)];
     }
 }
 
