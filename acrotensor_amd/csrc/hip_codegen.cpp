@@ -1389,7 +1389,7 @@ class Generator
             if (r.size > big->size) big = &r;
         }
         const bool outputsFastest = has(s.outIdx, big->idx.back());
-        long G = std::min<long>(2048, std::max<long>(1, Nc / (Sn * 16)));
+        long G = std::min<long>(512, std::max<long>(1, Nc / (Sn * 16)));
         const long chunk = ((Nc + G - 1) / G + Sn - 1) / Sn * Sn;  // contraction entries per workgroup
         G = (Nc + chunk - 1) / chunk;
         const long S2 = NTr / O;
@@ -1466,6 +1466,7 @@ class Generator
         out << "    const int g2 = lane / " << O << ", o = lane % " << O << ";\n";
         out << "    double sum = 0.0;\n";
         out << "    if (lane < " << S2 * O << ")\n    {\n";
+        out << "#pragma unroll 8\n";
         out << "        for (long g = g2; g < " << G << "; g += " << S2 << ") sum += scratch[g * " << O << " + o];\n    }\n";
         out << "    red[lane] = sum;\n    __syncthreads();\n";
         out << "    if (lane < " << O << ")\n    {\n        double t = 0.0;\n";
@@ -1505,7 +1506,8 @@ class Generator
         const int K = static_cast<int>(subs.size());
         const int U = static_cast<int>(uvars.size());
         const std::string dimName = mk.GetDimensionedNameString();
-        std::string variant = str(NB) + "/" + str(NT) + "/" + (opt.noalias ? "n" : "a") + (Positional() ? "p" : "u");
+        std::string variant = str(NB) + "/" + str(NT) + "/" + (opt.noalias ? "n" : "a") + (Positional() ? "p" : "u") +
+                              "/" + str(envInt("ACRO_HIP_PERSIST"));
         for (const auto &st : stores) variant += st.elide ? "e" : (st.inLds ? "l" : "g");
         for (int u = 0; u < U; ++u) variant += "s" + str(uvars[u].storage) + "@" + str(uvars[u].viewOffset);
         char hex[32];
@@ -1560,7 +1562,15 @@ class Generator
         for (int si : scalarStores)
             out << "    const acro_scalar_ptr C" << si << " = (acro_scalar_ptr)T" << si << ";\n";
         out << "    const int tid = threadIdx.x;\n";
-        out << "    const int e0 = blockIdx.x * " << NB << ";\n";
+        // Persistent form (ACRO_HIP_PERSIST=<workgroups per CU>): a fixed grid walks over the batch in a loop.
+        const long totalGroups = (E + NB - 1) / NB;
+        const long persist = envInt("ACRO_HIP_PERSIST");
+        const long gridGroups = persist > 0 ? std::min<long>(totalGroups, persist * 256) : totalGroups;
+        const bool looped = gridGroups < totalGroups;
+        if (looped)
+            out << "    for (int e0 = blockIdx.x * " << NB << "; e0 < " << E << "; e0 += " << gridGroups * NB << ")\n    {\n";
+        else
+            out << "    const int e0 = blockIdx.x * " << NB << ";\n    {\n";
 
         const bool guardBatch = (E % NB) != 0;
 
@@ -1754,12 +1764,13 @@ class Generator
                 });
             }
         }
-        out << "}\n";
+        if (looped && ldsDoubles > 0) out << "    __syncthreads();\n";
+        out << "    }\n}\n";
 
         plan.source = out.str();
         HipLaunch launch;
         launch.function_name = function_name;
-        launch.grid = static_cast<unsigned>((E + NB - 1) / NB);
+        launch.grid = static_cast<unsigned>(gridGroups);
         launch.block = static_cast<unsigned>(NT);
         for (size_t si = 0; si < stores.size(); ++si) launch.params.push_back(static_cast<int>(si));
         plan.launches.push_back(launch);

@@ -150,6 +150,48 @@ def test_config4_full_size_properties(at, engine, checker):
     assert np.array_equal(Y1, np.broadcast_to(Y1[0], Y1.shape))
 
 
+def numpy_diffusion(wl):
+    B, G, X, D = (wl.arrays[n] for n in "BGXD")
+    combos = ((G, B, B), (B, G, B), (B, B, G))
+    U = np.stack([np.einsum("qi,rj,sk,eijk->eqrs", a, b, c, X, optimize=True) for a, b, c in combos])
+    Z = np.einsum("eqrsmn,neqrs->meqrs", D, U)
+    return sum(np.einsum("qi,rj,sk,eqrs->eijk", a, b, c, Z[m], optimize=True) for m, (a, b, c) in enumerate(combos))
+
+
+def test_config5_every_element_against_numpy(at, engine):
+    """p=7 diffusion apply on 4096 elements: every element against the operator evaluated with numpy."""
+    wl = workloads.config5(E=4096)
+    tensors = run_workload(at, engine, wl, True)
+    Y = fetch(tensors, "Y")
+    expected = numpy_diffusion(wl)
+    per_element = np.abs(Y - expected).reshape(4096, -1).max(axis=1)
+    assert per_element.max() <= TOL * np.abs(expected).max(), "first bad element %d" % int(per_element.argmax())
+    # run to run reproducibility (no atomics, fixed summation order)
+    workloads.launch(wl, engine, tensors)
+    assert np.array_equal(fetch(tensors, "Y"), Y)
+
+
+def test_config5_full_size_properties(at, engine, checker):
+    """E = 65536 (D alone is 4.7 GB, more bytes than an int can count): sampled elements against the checker and
+    exact linearity in X."""
+    E = 65536
+    wl = workloads.config5(E=E)
+    tensors = run_workload(at, engine, wl, True)
+    Y = fetch(tensors, "Y")
+    sample = np.array([0, 1, E // 2, E - 1, 12345])
+    sub = workloads.config5(E=len(sample))
+    for name in ("B", "G"):
+        sub.arrays[name][...] = wl.arrays[name]
+    for name in ("X", "D"):
+        sub.arrays[name][...] = wl.arrays[name][sample]
+    expected = workloads.run_on_checker(sub, checker)["Y"]
+    assert rel_err(Y[sample], expected) <= TOL
+    tensors["X"].data[...] = 2.0 * wl.arrays["X"]
+    tensors["X"].SwitchFromGPU()
+    workloads.launch(wl, engine, tensors)
+    assert np.array_equal(fetch(tensors, "Y"), 2.0 * Y)
+
+
 def test_config2_full_size_properties(at, engine):
     """4 194 304 matrices: J (Jinv)^T = I and det(J) det(Jinv) = 1 everywhere."""
     J = workloads.config2_inputs()
