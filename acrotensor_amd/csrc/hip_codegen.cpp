@@ -916,6 +916,145 @@ class Generator
             }
             st.elide = ok && anyRead;
         }
+        if (envInt("ACRO_HIP_LDS_PAD") > 0) PadLdsTiles(budgetDoubles);  // opt-in: see PadLdsTiles
+    }
+
+    // ----------------------------------------------------------------------------- LDS bank conflicts
+    // LDS has 64 banks of 4 bytes; a wavefront's 8-byte accesses are served 32 lanes at a time, and lanes of such a
+    // group that hit the same bank at different addresses serialise.  All addresses are known here (lane index
+    // decomposition, tile strides), so the cost of every LDS access instruction can be counted and the tile strides
+    // padded until the count stops improving.  The count models 8-byte accesses only; the compiler merges adjacent
+    // ones into 16-byte accesses that padding can break apart, and on the p=7 diffusion chain the padded layout
+    // measured 20 % slower, so padding is opt-in (ACRO_HIP_LDS_PAD=1) until the model covers merged accesses.
+
+    // Serialisation cycles of one access instruction whose lane l of the chain's item w reads `base(w)` doubles.
+    static long ConflictCycles(const std::vector<long> &addr)
+    {
+        long cycles = 0;
+        for (size_t g = 0; g < addr.size(); g += 32)
+        {
+            // distinct addresses per bank (a double covers two consecutive 4-byte banks: bank pair = addr mod 32)
+            std::map<long, std::set<long>> perBank;
+            for (size_t l = g; l < std::min(addr.size(), g + 32); ++l) perBank[((addr[l] % 32) + 32) % 32].insert(addr[l]);
+            size_t worst = 1;
+            for (const auto &b : perBank) worst = std::max(worst, b.second.size());
+            cycles += static_cast<long>(worst);
+        }
+        return cycles;
+    }
+
+    // Lane part of the LDS address of an occurrence for every work item of its kernel.
+    std::vector<long> LaneAddresses(const Sub &s, const VarRef &r, int nb) const
+    {
+        const Storage &st = StoreOf(r.uvar);
+        const long items = static_cast<long>(nb) * s.laneCount;
+        std::vector<long> addr(items);
+        for (long w = 0; w < items; ++w)
+        {
+            const long b = w / s.laneCount;
+            long rest = w % s.laneCount;
+            std::vector<int> value(nidx, 0);
+            for (int j = static_cast<int>(s.lane.size()) - 1; j >= 0; --j)
+            {
+                value[s.lane[j]] = static_cast<int>(rest % extent[s.lane[j]]);
+                rest /= extent[s.lane[j]];
+            }
+            long a = b * st.tileSize;
+            for (size_t d = 0; d < r.idx.size(); ++d)
+            {
+                if (r.idx[d] != batch && has(s.lane, r.idx[d])) a += static_cast<long>(value[r.idx[d]]) * LdsStride(r.uvar, d);
+            }
+            addr[w] = a;
+        }
+        return addr;
+    }
+
+    long LdsCostOfStorage(int si, int nb) const
+    {
+        long cost = 0;
+        for (int k = 0; k < static_cast<int>(subs.size()); ++k)
+        {
+            const Sub &s = subs[k];
+            if (s.loopMode) continue;
+            for (size_t v = 0; v < s.in.size(); ++v)
+            {
+                if (uvars[s.in[v].uvar].storage != si || SourceOf(k, static_cast<int>(v)) != kFromLds) continue;
+                std::set<int> seen;
+                long ninstr = 1;
+                for (int id : s.in[v].idx)
+                {
+                    if ((has(s.tile, id) || has(s.contr, id)) && seen.insert(id).second) ninstr *= extent[id];
+                }
+                cost += ninstr * ConflictCycles(LaneAddresses(s, s.in[v], nb));
+            }
+            if (uvars[s.out.uvar].storage == si && (NeedsLdsCopy(k) || (s.op != '=' && !s.forwardedOld && OldValueInLds(k))))
+                cost += s.tileCount * ConflictCycles(LaneAddresses(s, s.out, nb));
+        }
+        return cost;
+    }
+
+    void SetLdsStrides(Storage &st, const std::vector<int> &pad, int padEntry) const
+    {
+        long run = 1;
+        st.ldsStride.assign(st.dims.size(), 0);
+        int p = 0;
+        for (int d = static_cast<int>(st.dims.size()) - 1; d >= 0; --d)
+        {
+            if (d == st.batchDim) continue;
+            st.ldsStride[d] = static_cast<int>(run);
+            run = run * st.dims[d] + pad[p++];
+        }
+        st.tileSize = static_cast<int>(run + padEntry);
+    }
+
+    void PadLdsTiles(int budgetDoubles)
+    {
+        // Padding must not cost a resident workgroup: a CU has 160 KB of LDS.
+        const long cuDoubles = 160 * 1024 / 8;
+        const long residentBefore = cuDoubles / std::max(1, PlaceLds(NB));
+        for (size_t si = 0; si < stores.size(); ++si)
+        {
+            Storage &st = stores[si];
+            if (!st.inLds) continue;
+            const int ndim = static_cast<int>(st.dims.size()) - 1;
+            std::vector<int> pad(ndim, 0), bestPad(ndim, 0);
+            int bestEntry = 0;
+            SetLdsStrides(st, pad, 0);
+            long best = LdsCostOfStorage(static_cast<int>(si), NB);
+            const long unpadded = best;
+            // coordinate descent: one stride at a time, innermost first, two sweeps
+            for (int sweep = 0; sweep < 2 && best > 0; ++sweep)
+            {
+                for (int p = 0; p <= ndim; ++p)
+                {
+                    const int limit = p == ndim ? 16 : 8;
+                    for (int cand = 0; cand <= limit; ++cand)
+                    {
+                        std::vector<int> trial = bestPad;
+                        int trialEntry = bestEntry;
+                        if (p == ndim)
+                            trialEntry = cand;
+                        else
+                            trial[p] = cand;
+                        SetLdsStrides(st, trial, trialEntry);
+                        const long c = LdsCostOfStorage(static_cast<int>(si), NB);
+                        if (c < best)
+                        {
+                            best = c;
+                            bestPad = trial;
+                            bestEntry = trialEntry;
+                        }
+                    }
+                }
+            }
+            SetLdsStrides(st, bestPad, bestEntry);
+            const int total = PlaceLds(NB);
+            if (total > budgetDoubles || best >= unpadded || (envInt("ACRO_HIP_LDS_PAD") < 2 && cuDoubles / std::max(1, total) < residentBefore))
+            {
+                SetLdsStrides(st, std::vector<int>(ndim, 0), 0);  // no room or no gain: natural layout
+            }
+        }
+        ldsDoubles = PlaceLds(NB);
     }
 
     // --------------------------------------------------------------------------------------- emission

@@ -148,8 +148,8 @@ def main():
                          "kernel that hardware-counter runs are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the workload shards trivially over "
-                 "elements; see DESIGN.md).  Run with --gpus 1.")
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the workload shards over elements "
+                 "without any exchange, so N GPUs would each run this same kernel on 1/N of them).  Run with --gpus 1.")
 
     import acrotensor_amd as at
     from acrotensor_amd import workloads
