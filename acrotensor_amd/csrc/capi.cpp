@@ -8,6 +8,7 @@
 
 #include "AcroTensor.hpp"
 #include "acrotensor_hip.h"
+#include "hip_kernel.hpp"
 
 using namespace acro;
 
@@ -449,6 +450,15 @@ int acro_engine_flat_indexed_sum_gather(acro_engine *e, acro_tensor *Aout, acro_
     return guarded([&] {
         require(e && Aout && Ain && M, "null handle");
         e->te.FlatIndexedSumGather(*Aout->t, *Ain->t, *M->m);
+    });
+}
+
+int acro_hip_compile(const char *module_name, const char *source, size_t *code_size)
+{
+    return guarded([&] {
+        require(module_name != nullptr && source != nullptr, "null argument");
+        HipKernel kernel(module_name, source);
+        if (code_size != nullptr) *code_size = kernel.GetCodeObjectSize();
     });
 }
 

@@ -109,6 +109,11 @@ int acro_engine_flat_indexed_scatter(acro_engine *e, acro_tensor *Aout, acro_ten
 int acro_engine_flat_indexed_sum_gather(acro_engine *e, acro_tensor *Aout, acro_tensor *Ain,
                                         acro_index_mapping *M);
 
+/* ---- runtime compiler, host only (stands for CudaKernel::GenerateFunction, util/CudaUtil.cpp:43-84) ---- */
+/* Compiles HIP C++ source for gfx950 with the options the library uses for generated kernels; needs no device.
+ * Returns 0 and the code-object size in *code_size, or non-zero with the compiler log in acro_last_error(). */
+int acro_hip_compile(const char *module_name, const char *source, size_t *code_size);
+
 /* ---- kernel IR introspection, host only (kernel/TensorKernel.hpp, DimensionedKernel.hpp,
  *      DimensionedMultiKernel.hpp) ---- */
 /* Parses num_kernels kernel strings and binds them to shapes.  For kernel k its tensors are listed output first,

@@ -95,11 +95,20 @@ def test_rebinding_one_name_to_two_tensors_switches_to_positional_operands(TE):
     assert src.count("const double *") >= 2
 
 
-def test_compile_errors_surface_as_exceptions_with_the_log():
+def test_runtime_compiler_reports_errors_with_the_log():
     import ctypes
     from acrotensor_amd import _capi
-    # an engine created for an unknown policy is the only host-forcible failure of the boundary besides bad
-    # kernels; a bad kernel string must fail before any code is generated
+    lib = _capi.load()
+    size = ctypes.c_size_t(0)
+    good = b'extern "C" __global__ void k(double *p) { p[threadIdx.x] = 1.0; }'
+    assert lib.acro_hip_compile(b"unit_good", good, ctypes.byref(size)) == 0 and size.value > 0
+    bad = b'extern "C" __global__ void k(double *p) { p[threadIdx.x] = undeclared_symbol; }'
+    assert lib.acro_hip_compile(b"unit_bad", bad, ctypes.byref(size)) != 0
+    message = lib.acro_last_error().decode()
+    assert "undeclared_symbol" in message and "unit_bad" in message
+
+
+def test_bad_kernel_strings_fail_before_code_generation():
     TE = at.TensorEngine("HIP")
     with pytest.raises(at.AcroError):
         TE.GetImplementation("A_i = b_i", at.Tensor(3), at.Tensor(3))
