@@ -23,7 +23,8 @@ namespace acro
 namespace
 {
 
-constexpr int kLanes = 256;
+constexpr int kLanes = 256;    // fill, scale, scatter, gather: one lane per entry
+constexpr int kMatLanes = 64;  // batched matrices: one wavefront per workgroup, so its barriers are free
 
 __global__ __launch_bounds__(kLanes) void fillKernel(double *__restrict__ d, double value, size_t n)
 {
@@ -86,26 +87,26 @@ struct SmallMatrix<3>
     }
 };
 
-// One workgroup = kLanes consecutive matrices.  WANT_INV / WANT_DET select the outputs.
+// One workgroup = kMatLanes consecutive matrices.  WANT_INV / WANT_DET select the outputs.
 // The matrices of a workgroup are contiguous in memory, so the workgroup copies them to and from LDS as one
 // stream of 16-byte pieces (full-rate HBM access), and lane t works on matrix t out of LDS.  For 2x2 the lane
 // stride in LDS is padded from 4 to 5 doubles so that lanes fall into distinct banks; 9 and 1 are odd already.
 template <int M, bool WANT_INV, bool WANT_DET>
-__global__ __launch_bounds__(kLanes) void batchMatrixKernel(const double *__restrict__ A, double *__restrict__ Ainv,
+__global__ __launch_bounds__(kMatLanes) void batchMatrixKernel(const double *__restrict__ A, double *__restrict__ Ainv,
                                                             double *__restrict__ Adet, size_t num_mat)
 {
     constexpr int MM = M * M;
     constexpr int LS = (MM % 2 == 0) ? MM + 1 : MM;  // odd lane stride in doubles: no LDS bank conflicts
-    __shared__ double tile[kLanes * LS];
+    __shared__ double tile[kMatLanes * LS];
 
-    const size_t first = static_cast<size_t>(blockIdx.x) * kLanes;
-    const size_t count = (num_mat - first < static_cast<size_t>(kLanes)) ? num_mat - first : kLanes;
+    const size_t first = static_cast<size_t>(blockIdx.x) * kMatLanes;
+    const size_t count = (num_mat - first < static_cast<size_t>(kMatLanes)) ? num_mat - first : kMatLanes;
     const int ndbl = static_cast<int>(count) * MM;
     const double *src = A + first * MM;
 
-    // first * MM * 8 bytes is a multiple of 16 (kLanes is even), so pairs of doubles are aligned
+    // first * MM * 8 bytes is a multiple of 16 (kMatLanes is even), so pairs of doubles are aligned
     const double2 *src2 = reinterpret_cast<const double2 *>(src);
-    for (int i = threadIdx.x; i < ndbl / 2; i += kLanes)
+    for (int i = threadIdx.x; i < ndbl / 2; i += kMatLanes)
     {
         const double2 v = src2[i];
         if (LS == MM)
@@ -143,7 +144,7 @@ __global__ __launch_bounds__(kLanes) void batchMatrixKernel(const double *__rest
         __syncthreads();
         double *dst = Ainv + first * MM;
         double2 *dst2 = reinterpret_cast<double2 *>(dst);
-        for (int i = threadIdx.x; i < ndbl / 2; i += kLanes)
+        for (int i = threadIdx.x; i < ndbl / 2; i += kMatLanes)
         {
             double2 v;
             if (LS == MM)
@@ -198,19 +199,21 @@ hipStream_t stream()
 template <bool WANT_INV, bool WANT_DET>
 void launchBatchMatrix(int mdim, const double *A, double *Ainv, double *Adet, size_t num_mat)
 {
-    const unsigned grid = gridFor(num_mat);
+    const size_t groups = (num_mat + kMatLanes - 1) / kMatLanes;
+    ACROBATIC_ASSERT(groups <= 0x7fffffffu, "Operand too large for a one-dimensional grid.");
+    const unsigned grid = static_cast<unsigned>(groups == 0 ? 1 : groups);
     switch (mdim)
     {
         case 1:
-            hipLaunchKernelGGL((batchMatrixKernel<1, WANT_INV, WANT_DET>), dim3(grid), dim3(kLanes), 0, stream(), A,
+            hipLaunchKernelGGL((batchMatrixKernel<1, WANT_INV, WANT_DET>), dim3(grid), dim3(kMatLanes), 0, stream(), A,
                                Ainv, Adet, num_mat);
             break;
         case 2:
-            hipLaunchKernelGGL((batchMatrixKernel<2, WANT_INV, WANT_DET>), dim3(grid), dim3(kLanes), 0, stream(), A,
+            hipLaunchKernelGGL((batchMatrixKernel<2, WANT_INV, WANT_DET>), dim3(grid), dim3(kMatLanes), 0, stream(), A,
                                Ainv, Adet, num_mat);
             break;
         case 3:
-            hipLaunchKernelGGL((batchMatrixKernel<3, WANT_INV, WANT_DET>), dim3(grid), dim3(kLanes), 0, stream(), A,
+            hipLaunchKernelGGL((batchMatrixKernel<3, WANT_INV, WANT_DET>), dim3(grid), dim3(kMatLanes), 0, stream(), A,
                                Ainv, Adet, num_mat);
             break;
         default:

@@ -259,7 +259,7 @@ def test_batch_matrix_shape_asserts(at, engine):
 
 
 def test_batch_matrix_ragged_batch_sizes(at, engine, checker):
-    for n in (1, 255, 256, 257, 1000):
+    for n in (1, 63, 64, 65, 255, 256, 257, 1000):
         rng = np.random.default_rng(n)
         A = np.eye(3) + 0.1 * rng.uniform(-1, 1, (n, 3, 3))
         tA, Ainv, Adet = to_tensor(at, A), at.Tensor(n, 3, 3), at.Tensor(n)
