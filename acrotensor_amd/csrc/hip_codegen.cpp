@@ -57,7 +57,6 @@ struct UVarInfo
     std::vector<int> dims;
     int size = 0;
     bool written = false;
-    bool read = false;
     int firstWrite = -1;
     int lastUse = -1;
     bool consistent = true;       // same shape and batch positions in every occurrence
@@ -299,10 +298,7 @@ class Generator
                     if (!u.written) u.firstWrite = ki;
                     u.written = true;
                 }
-                else
-                {
-                    u.read = true;
-                }
+
             };
             for (const auto &r : s.in) note(r, false);
             if (s.op != '=') note(s.out, false);

@@ -14,6 +14,15 @@
 //    device memory is skipped when the tensor is marked transient.  A kernel without contraction whose operand
 //    was just produced with the same index set is applied in registers (no LDS round trip).
 //  * Contractions too long to unroll fall back to counted loops with the same lane mapping.
+//
+// Experiment switches (environment, read when a kernel is generated; defaults are what measured best on MI355X):
+//   ACRO_HIP_NB / ACRO_HIP_NT   batch entries per workgroup / lanes per workgroup (default: chosen per kernel)
+//   ACRO_HIP_MERGE=-1           one phase per chain instead of sharing phases between independent kernels
+//   ACRO_HIP_PREFETCH=-1        no prefetch of later phases' streaming inputs at kernel entry
+//   ACRO_HIP_NT_STORE=-1        ordinary instead of non-temporal stores for results that stream out
+//   ACRO_HIP_LDS_PAD=1|2        pad LDS tile strides against bank conflicts (2: even if a resident workgroup is lost)
+//   ACRO_HIP_PACK=1             pick batch / workgroup size for wavefront utilisation
+//   ACRO_HIP_PERSIST=<n>        persistent grid of n workgroups per CU looping over the batch
 #ifndef ACRO_HIP_CODEGEN_HPP
 #define ACRO_HIP_CODEGEN_HPP
 
