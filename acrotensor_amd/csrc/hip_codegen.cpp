@@ -1317,10 +1317,14 @@ class Generator
     // Such stores complete later, which delays the retirement of the workgroup: where LDS allows only a few resident
     // workgroups per CU that costs more than it gains (p=7 diffusion apply, 3 workgroups per CU: -14 %), so they are
     // only used while at least 8 workgroups fit.
+    // They also get less write combining, so they are only used when one store instruction of a wavefront fills at
+    // least about half of every 128-byte line it touches (scattered 8-byte pieces written this way measured 1.7x
+    // slower than ordinary stores).
     bool StreamsOut(int k) const
     {
         if (envInt("ACRO_HIP_NT_STORE") < 0) return false;
         if (static_cast<long>(ldsDoubles) * 8 > 20 * 1024) return false;
+        if (WaveStoreLineCoverage(k) < 0.45) return false;
         const int si = uvars[subs[k].out.uvar].storage;
         for (int j = k + 1; j < static_cast<int>(subs.size()); ++j)
         {
@@ -1332,6 +1336,65 @@ class Generator
             if (uvars[s.out.uvar].storage == si && s.op != '=' && !s.forwardedOld && !OldValueInLds(j)) return false;
         }
         return true;
+    }
+
+    // How much of the 128-byte lines that one store instruction of kernel k touches does it fill, on average over
+    // the instructions of the first wavefront?  A lane's stores to consecutive addresses are counted as one
+    // instruction per pair of doubles (the compiler merges them into 16-byte stores).
+    double WaveStoreLineCoverage(int k) const
+    {
+        const Sub &s = subs[k];
+        const long items = std::min<long>(64, static_cast<long>(NB) * s.laneCount);
+        std::vector<std::vector<long>> perLane(items);
+        for (long w = 0; w < items; ++w)
+        {
+            std::vector<int> value(nidx, 0);
+            long rest = w % s.laneCount;
+            for (int j = static_cast<int>(s.lane.size()) - 1; j >= 0; --j)
+            {
+                value[s.lane[j]] = static_cast<int>(rest % extent[s.lane[j]]);
+                rest /= extent[s.lane[j]];
+            }
+            if (batch >= 0) value[batch] = static_cast<int>(w / s.laneCount);
+            const long tiles = s.loopMode ? 1 : s.tileCount;
+            for (long t = 0; t < tiles; ++t)
+            {
+                long rem = t;
+                for (int j = static_cast<int>(s.tile.size()) - 1; j >= 0; --j)
+                {
+                    value[s.tile[j]] = static_cast<int>(rem % extent[s.tile[j]]);
+                    rem /= extent[s.tile[j]];
+                }
+                long a = uvars[s.out.uvar].viewOffset;
+                for (size_t d = 0; d < s.out.idx.size(); ++d) a += static_cast<long>(value[s.out.idx[d]]) * s.out.stride[d];
+                perLane[w].push_back(a);
+            }
+            std::sort(perLane[w].begin(), perLane[w].end());
+        }
+        // instruction g of a lane = its g-th group of (up to two) consecutive addresses
+        std::vector<std::map<long, int>> doublesPerLine;
+        for (long w = 0; w < items; ++w)
+        {
+            size_t g = 0;
+            for (size_t i = 0; i < perLane[w].size(); ++g)
+            {
+                const size_t n = (i + 1 < perLane[w].size() && perLane[w][i + 1] == perLane[w][i] + 1) ? 2 : 1;
+                if (doublesPerLine.size() <= g) doublesPerLine.resize(g + 1);
+                for (size_t j = 0; j < n; ++j) doublesPerLine[g][perLane[w][i + j] / 16] += 1;
+                i += n;
+            }
+        }
+        double sum = 0.0;
+        long lines = 0;
+        for (const auto &instr : doublesPerLine)
+        {
+            for (const auto &l : instr)
+            {
+                sum += std::min(16, l.second) / 16.0;
+                ++lines;
+            }
+        }
+        return lines == 0 ? 0.0 : sum / static_cast<double>(lines);
     }
 
     std::string GlobalStore(int k, const std::string &gaddr, const std::string &value) const
