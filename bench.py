@@ -28,7 +28,7 @@ METRIC = "GDOF/s + % HBM peak, p=3 sum-factorised hex mass apply fp64 (1 GPU)"
 
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a
 # copy kernel of known size); None until the profile summary under profiles/ has been taken for this kernel.
-MEASURED_TRAFFIC_BYTES = 536846085  # profiles/cfg4_mass_apply_hbm_traffic.md
+MEASURED_TRAFFIC_BYTES = 541836805  # profiles/cfg4_mass_apply_hbm_traffic.md
 
 
 def settle_clocks(at, workloads, wl, engine, tensors, seconds):
