@@ -311,3 +311,44 @@ def test_get_implementation_returns_hip_source(at, engine):
     A, B = at.Tensor(8, 3), at.Tensor(8, 3)
     src = engine.GetImplementation("A_e_i = B_e_i", A, B)
     assert "__global__" in src and "A_e_i = B_e_i" in src
+
+
+def test_partially_written_parent_is_read_back_from_device_memory(at, engine):
+    # U0 is produced inside the launch, U1 keeps what it held before; the whole-U read must see both
+    rng = np.random.default_rng(77)
+    E = 13
+    X, G, D = rng.uniform(-1, 1, (E, 4)), rng.uniform(-1, 1, (5, 4)), rng.uniform(-1, 1, (E, 5, 2, 2))
+    U_init = rng.uniform(-1, 1, (2, E, 5))
+    for transient in (False, True):
+        tX, tG, tD, U, Z = to_tensor(at, X), to_tensor(at, G), to_tensor(at, D), to_tensor(at, U_init), at.Tensor(2, E, 5)
+        U.SetTransient(transient)
+        U0 = at.SliceTensor(U, 0)
+        engine.BeginMultiKernelLaunch()
+        engine("U0_e_q = G_q_i X_e_i", U0, tG, tX)
+        engine("Z_m_e_q = D_e_q_m_n U_n_e_q", Z, tD, U)
+        engine.EndMultiKernelLaunch()
+        Z.MoveFromGPU()
+        expU = U_init.copy()
+        expU[0] = X @ G.T
+        assert rel_err(Z.data, np.einsum("eqmn,neq->meq", D, expU)) <= TOL
+
+
+def test_slice_of_a_slice_inside_a_fused_launch(at, engine):
+    rng = np.random.default_rng(78)
+    E = 9
+    P = at.Tensor(2, 3, E, 4)
+    P.data[...] = rng.uniform(-1, 1, (2, 3, E, 4))
+    before = P.data.copy()
+    S1 = at.SliceTensor(P, 1)            # [3, E, 4]
+    S12 = at.SliceTensor(S1, 2)          # [E, 4]  = P[1, 2]
+    A, R = to_tensor(at, rng.uniform(-1, 1, (E, 4))), at.Tensor(3, E)
+    engine.BeginMultiKernelLaunch()
+    engine("V_e_i = A_e_i", S12, A)
+    engine("R_a_e = W_a_e_i", R, S1)
+    engine.EndMultiKernelLaunch()
+    R.MoveFromGPU()
+    P.MoveFromGPU()
+    expected = before.copy()
+    expected[1, 2] = A.data
+    assert np.array_equal(P.data, expected)
+    assert rel_err(R.data, expected[1].sum(axis=2)) <= TOL
