@@ -6,6 +6,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <cstdio>
 #include <cstdlib>
 #include <functional>
 #include <map>
@@ -67,6 +68,7 @@ struct UVarInfo
     long viewOffset = 0;          // first element inside the storage
     std::vector<int> fixed;       // leading indices of the storage that the view fixes
     bool plainView = true;        // the view is "leading indices fixed, all trailing dimensions kept"
+    bool isVirtual = false;       // intermediate of a factorised kernel: lives in LDS only, no kernel parameter
 };
 
 // A tensor's memory: what kernel parameters point to, what LDS tiles mirror and what stores are elided for.
@@ -129,7 +131,16 @@ int envInt(const char *name)
 class Generator
 {
   public:
-    Generator(const DimensionedMultiKernel &mk_, const HipCodegenOptions &opt_) : mk(mk_), opt(opt_) {}
+    // max_virtual_tile: largest partial result (doubles per batch entry) a reordered single kernel may keep in LDS;
+    // 0 = evaluate single kernels as written.
+    Generator(const DimensionedMultiKernel &mk_, const HipCodegenOptions &opt_, long max_virtual_tile)
+        : mk(mk_), opt(opt_), factorise(max_virtual_tile > 0), maxVirtualTile(max_virtual_tile)
+    {
+    }
+
+    // The factorised form of a kernel was planned but its intermediates did not all stay on chip: the caller
+    // generates the kernel again as written.
+    bool factorisationAbandoned = false;
 
     HipKernelPlan Run()
     {
@@ -182,6 +193,20 @@ class Generator
                 ChooseBatching();
             }
         }
+        if (factorised)
+        {
+            for (const auto &st : stores)
+            {
+                // every read of a partial result must be served from registers or from its LDS tile
+                if (uvars[st.members[0]].isVirtual && !st.elide) factorisationAbandoned = true;
+            }
+            if (factorisationAbandoned)
+            {
+                plan.fusable = false;
+                plan.why_not = "intermediates of the factorised kernel do not fit on chip";
+                return plan;
+            }
+        }
         Emit(plan);
         return plan;
     }
@@ -189,6 +214,9 @@ class Generator
   private:
     const DimensionedMultiKernel &mk;
     const HipCodegenOptions &opt;
+    const bool factorise;
+    const long maxVirtualTile;
+    bool factorised = false;
 
     int nidx = 0;
     std::vector<std::string> idxName;
@@ -270,8 +298,10 @@ class Generator
             E = extent[batch];
         }
 
+        if (factorise && K == 1 && envInt("ACRO_HIP_FACTORISE") >= 0) FactoriseSingleKernel();
+
         // Unique-variable facts, in program order (a kernel reads its inputs before it writes its output).
-        for (int ki = 0; ki < K; ++ki)
+        for (int ki = 0; ki < static_cast<int>(subs.size()); ++ki)
         {
             const Sub &s = subs[ki];
             auto note = [&](const VarRef &r, bool is_write) {
@@ -313,9 +343,208 @@ class Generator
         AnalyseCoverage();
     }
 
+    // --------------------------------------------------------------------------- contraction ordering
+    // A single kernel with three or more operands, written as one big sum
+    // ("M_e_i_j_k_l_m_n = B_q_i B_q_l B_r_j B_r_m B_s_k B_s_n W_e_q_r_s": 64 terms of 7 factors for each of 729
+    // outputs), is evaluated as a chain of smaller contractions when that takes far fewer multiply-adds: a
+    // contraction index is summed as soon as every operand carrying it has been multiplied in, and the partial
+    // result becomes the operand of the next step.  The partial results are tensors of the generator's own: one
+    // tile per batch entry in LDS, never a kernel parameter.  The steps then run through the same machinery as a
+    // user-written multi-kernel group.  The order of the steps is the cheapest (in multiply-adds) among those whose
+    // every intermediate carries the batch index and fits in LDS; nothing changes unless the gain is large, because
+    // one lane already shares partial sums between the outputs of its pencil.
+    static constexpr double kFactoriseMinWork = 8192.0;   // multiply-adds per batch entry as written
+    static constexpr double kFactoriseMinGain = 4.0;
+
+    struct FactorStep
+    {
+        std::vector<int> group;   // operand ids multiplied in this step (inputs: 0..n-1, result of step t: n + t)
+        std::vector<int> summed;  // loop ids summed in this step
+        std::vector<int> result;  // loop ids of the result, in storage order
+    };
+
+    double NonBatchVolume(const std::set<int> &ids) const
+    {
+        double v = 1.0;
+        for (int id : ids)
+        {
+            if (id != batch) v *= extent[id];
+        }
+        return v;
+    }
+
+    void FactoriseSearch(const Sub &orig, std::vector<int> &live, std::vector<std::vector<int>> &idxOf,
+                         std::vector<int> &remaining, double cost, std::vector<FactorStep> &steps, double &best,
+                         long &bestSlowest, std::vector<FactorStep> &bestSteps, long &visits) const
+    {
+        if (++visits > 20000) return;
+        // Finish here: one kernel over everything that is left.
+        {
+            std::set<int> all(orig.outIdx.begin(), orig.outIdx.end());
+            for (int o : live) all.insert(idxOf[o].begin(), idxOf[o].end());
+            const double total = cost + NonBatchVolume(all) * static_cast<double>(live.size());
+            // Among equally cheap orders prefer the one whose last kernel introduces the slowest-varying output
+            // indices: they become its register tile, and the lanes then follow the fast output dimensions, which
+            // keeps the stores of a wavefront contiguous.
+            long slowest = 0;
+            const int nin = static_cast<int>(orig.in.size());
+            for (size_t d = 0; d < orig.out.idx.size(); ++d)
+            {
+                const int id = orig.out.idx[d];
+                bool inIntermediate = false, inInput = false;
+                for (int o : live) (o >= nin ? inIntermediate : inInput) |= has(idxOf[o], id);
+                if (id != batch && inInput && !inIntermediate) slowest = slowest == 0 ? orig.out.stride[d] : std::min<long>(slowest, orig.out.stride[d]);
+            }
+            if (total < best * (1.0 - 1e-9) || (total <= best * (1.0 + 1e-9) && slowest > bestSlowest))
+            {
+                best = total;
+                bestSlowest = slowest;
+                bestSteps = steps;
+            }
+        }
+        for (size_t ci = 0; ci < remaining.size(); ++ci)
+        {
+            const int c = remaining[ci];
+            std::vector<int> group, rest;
+            for (int o : live) (has(idxOf[o], c) ? group : rest).push_back(o);
+            if (rest.empty() || group.empty()) continue;  // that is the final kernel
+            std::set<int> all;
+            for (int o : group) all.insert(idxOf[o].begin(), idxOf[o].end());
+            FactorStep st;
+            st.group = group;
+            for (int id : remaining)
+            {
+                if (all.count(id) == 0) continue;
+                bool outside = false;
+                for (int o : rest) outside = outside || has(idxOf[o], id);
+                if (!outside) st.summed.push_back(id);
+            }
+            std::set<int> kept = all;
+            for (int id : st.summed) kept.erase(id);
+            if (kept.count(batch) == 0 || NonBatchVolume(kept) > static_cast<double>(maxVirtualTile)) continue;
+            const double stepCost = cost + NonBatchVolume(all) * static_cast<double>(group.size());
+            if (stepCost > best) continue;
+            // Storage order of the result: batch index, the output's indices in the output's order, then the
+            // contraction indices still open (read by the next step as literal offsets, unit stride innermost).
+            st.result.push_back(batch);
+            for (int id : orig.outIdx)
+            {
+                if (id != batch && kept.count(id)) st.result.push_back(id);
+            }
+            for (int id : orig.contr)
+            {
+                if (kept.count(id)) st.result.push_back(id);
+            }
+            std::vector<int> nextLive = rest, nextRemaining;
+            nextLive.push_back(static_cast<int>(idxOf.size()));
+            for (int id : remaining)
+            {
+                if (!has(st.summed, id)) nextRemaining.push_back(id);
+            }
+            idxOf.push_back(st.result);
+            steps.push_back(st);
+            FactoriseSearch(orig, nextLive, idxOf, nextRemaining, stepCost, steps, best, bestSlowest, bestSteps, visits);
+            steps.pop_back();
+            idxOf.pop_back();
+        }
+    }
+
+    void FactoriseSingleKernel()
+    {
+        const Sub orig = subs[0];
+        const int nin = static_cast<int>(orig.in.size());
+        if (batch < 0 || nin < 3 || orig.contr.empty() || !opt.noalias || orig.out.repeated) return;
+        if (orig.contrCount >= kReductionMinContraction && product(orig.outIdx, extent) <= kReductionMaxOutputs) return;
+        for (const auto &r : orig.in)
+        {
+            if (r.repeated || r.uvar == orig.out.uvar) return;
+        }
+        std::vector<int> live;
+        std::vector<std::vector<int>> idxOf;
+        for (int v = 0; v < nin; ++v)
+        {
+            live.push_back(v);
+            idxOf.push_back(orig.in[v].idx);
+        }
+        std::vector<int> remaining = orig.contr;
+        std::vector<FactorStep> steps, bestSteps;
+        double best = 1e300;
+        long visits = 0, bestSlowest = -1;
+        std::set<int> all(orig.outIdx.begin(), orig.outIdx.end());
+        all.insert(orig.contr.begin(), orig.contr.end());
+        const double asWritten = NonBatchVolume(all) * static_cast<double>(nin);
+        FactoriseSearch(orig, live, idxOf, remaining, 0.0, steps, best, bestSlowest, bestSteps, visits);
+        if (bestSteps.empty() || asWritten < kFactoriseMinWork || best * kFactoriseMinGain > asWritten) return;
+
+        DimensionedKernel *kernel = mk.Kernels[0];
+        auto refText = [&](const std::string &name, const std::vector<int> &ids) {
+            std::string t = name;
+            for (int id : ids) t += "_" + idxName[id];
+            return t;
+        };
+        std::vector<VarRef> refOf(orig.in.begin(), orig.in.end());
+        std::vector<std::string> textOf;
+        for (int v = 0; v < nin; ++v) textOf.push_back(refText(kernel->GetVarName(v), orig.in[v].idx));
+        std::vector<bool> used(nin, false);
+        subs.clear();
+        for (size_t t = 0; t < bestSteps.size(); ++t)
+        {
+            const FactorStep &st = bestSteps[t];
+            UVarInfo info;
+            info.isVirtual = true;
+            info.name = "_F" + str(static_cast<long>(t + 1));
+            VarRef out;
+            out.uvar = static_cast<int>(uvars.size());
+            out.idx = st.result;
+            for (int id : st.result) out.ext.push_back(extent[id]);
+            out.stride.assign(out.idx.size(), 1);
+            for (int d = static_cast<int>(out.idx.size()) - 2; d >= 0; --d) out.stride[d] = out.stride[d + 1] * out.ext[d + 1];
+            for (int x : out.ext) out.size *= x;
+            uvars.push_back(info);
+
+            Sub s;
+            s.op = '=';
+            s.out = out;
+            s.outIdx = st.result;
+            s.contr = st.summed;
+            s.contrCount = product(s.contr, extent);
+            s.text = refText(info.name, st.result) + " =";
+            for (int o : st.group)
+            {
+                s.in.push_back(refOf[o]);
+                s.text += " " + textOf[o];
+                used[o] = true;
+            }
+            subs.push_back(s);
+            refOf.push_back(out);
+            textOf.push_back(refText(info.name, st.result));
+            used.push_back(false);
+        }
+        Sub fin = orig;
+        fin.in.clear();
+        fin.contr.clear();
+        fin.text = refText(kernel->GetVarName(-1), orig.out.idx) + " " + (orig.op == '=' ? "=" : std::string(1, orig.op) + "=");
+        for (size_t o = 0; o < refOf.size(); ++o)
+        {
+            if (used[o]) continue;
+            fin.in.push_back(refOf[o]);
+            fin.text += " " + textOf[o];
+        }
+        for (int id : orig.contr)
+        {
+            bool summedEarlier = false;
+            for (const auto &st : bestSteps) summedEarlier = summedEarlier || has(st.summed, id);
+            if (!summedEarlier) fin.contr.push_back(id);
+        }
+        fin.contrCount = product(fin.contr, extent);
+        fin.text += "   (steps of: " + orig.text + ")";
+        subs.push_back(fin);
+        factorised = true;
+    }
+
     void BuildStorages()
     {
-        const int U = NumOperands();
+        const int U = static_cast<int>(uvars.size());
         int nstore = 0;
         for (int u = 0; u < U; ++u)
         {
@@ -354,7 +583,7 @@ class Generator
             st.members.push_back(u);
             st.written = st.written || op.written;
             st.anyRepeated = st.anyRepeated || op.anyRepeated;
-            const bool tr = static_cast<size_t>(u) < opt.transient.size() && opt.transient[u];
+            const bool tr = op.isVirtual || (static_cast<size_t>(u) < opt.transient.size() && opt.transient[u]);
             st.transient = st.transient && tr;
             if (op.written && (st.firstWrite < 0 || op.firstWrite < st.firstWrite)) st.firstWrite = op.firstWrite;
 
@@ -1575,9 +1804,21 @@ class Generator
     }
 
     // Kernel parameters: one pointer per storage, taken from a representative member occurrence.
+    // Storages that are kernel parameters: all but the intermediates of a factorised kernel, which are numbered last.
+    int NumParamStores() const
+    {
+        int n = 0;
+        for (const auto &st : stores)
+        {
+            if (!uvars[st.members[0]].isVirtual) ++n;
+        }
+        for (int si = 0; si < n; ++si) ACROBATIC_ASSERT(!uvars[stores[si].members[0]].isVirtual, "HIP generator: storage order");
+        return n;
+    }
+
     void FillParams(HipKernelPlan &plan, bool honour_elision) const
     {
-        const int S = static_cast<int>(stores.size());
+        const int S = NumParamStores();
         plan.param_occurrence.resize(S);
         plan.param_offset.assign(S, 0);
         plan.stored.assign(S, false);
@@ -1593,7 +1834,7 @@ class Generator
     std::string ParamList() const
     {
         std::string p;
-        for (size_t si = 0; si < stores.size(); ++si)
+        for (size_t si = 0; si < static_cast<size_t>(NumParamStores()); ++si)
         {
             p += std::string(si ? ", " : "") + (stores[si].written ? "double *" : "const double *") +
                  (opt.noalias ? "__restrict__ " : "") + "T" + str(static_cast<long>(si));
@@ -1999,7 +2240,7 @@ class Generator
         launch.function_name = function_name;
         launch.grid = static_cast<unsigned>(gridGroups);
         launch.block = static_cast<unsigned>(NT);
-        for (size_t si = 0; si < stores.size(); ++si) launch.params.push_back(static_cast<int>(si));
+        for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
         plan.launches.push_back(launch);
         plan.nb = NB;
         plan.lds_bytes = ldsDoubles * 8;
@@ -2016,7 +2257,16 @@ class Generator
 
 HipKernelPlan GenerateHipKernel(const DimensionedMultiKernel &mk, const HipCodegenOptions &options)
 {
-    Generator g(mk, options);
+    // Partial results of a reordered kernel may take up to 48 KB of LDS per batch entry; when the tiles that are
+    // live together do not fit in a workgroup's 64 KB, plan again with tiles of half that size (any two fit), and
+    // finally evaluate the kernel as written.
+    for (long maxTile : {6144L, 3072L})
+    {
+        Generator g(mk, options, maxTile);
+        HipKernelPlan plan = g.Run();
+        if (!g.factorisationAbandoned) return plan;
+    }
+    Generator g(mk, options, 0);
     return g.Run();
 }
 

@@ -48,14 +48,51 @@ def test_mass_apply_chain_stores_everything_by_default(TE):
     assert "T3->global" in src
 
 
-def test_mass_assembly_is_sum_factorised_inside_the_lane(TE):
+def test_mass_assembly_is_evaluated_as_a_chain_of_small_contractions(TE):
     wl = workloads.config3(E=16)
+    tensors = workloads.bind_to_engine(wl, at)
+    k, out, ins = wl.kernels[0]
+    src = TE.GetImplementation(k, tensors[out], *[tensors[n] for n in ins])
+    # one index is summed per step; the two partial results are tensors of the generator's own that live in LDS
+    assert src.count("contraction=4 unrolled") == 3 and "contraction=64" not in src
+    assert "_F1->lds\n" in src and "_F2->lds\n" in src and "_F2<-lds" in src and "M->global" in src
+    assert src.count("__syncthreads()") == 2
+    # kernel parameters are the user's tensors only: M, B, W
+    signature = [l for l in src.splitlines() if "__global__" in l][0]
+    assert signature.count("double *") == 3
+    # the last step keeps the slowest output indices in the lane's tile, so lanes follow the fast dimensions
+    assert "lanes(j,k,m,n)=81 tile(i,l)=9" in src
+    # as written: 729 * 64 * 6 multiplications per element; the chain needs about 4 800 multiply-adds
+    assert src.count("*") < 1500
+
+
+def test_mass_assembly_without_reordering_shares_partial_sums_inside_the_lane(TE, monkeypatch):
+    monkeypatch.setenv("ACRO_HIP_FACTORISE", "-1")
+    wl = workloads.config3(E=17)
     tensors = workloads.bind_to_engine(wl, at)
     k, out, ins = wl.kernels[0]
     src = TE.GetImplementation(k, tensors[out], *[tensors[n] for n in ins])
     assert ")=9 contraction=64 unrolled" in src           # a 3x3 tile of outputs per lane
     # as written the kernel has 729 * 64 * 6 multiplications per element; hoisting leaves a small fraction
     assert src.count("*") < 81 * 400
+
+
+def test_small_or_barely_cheaper_kernels_are_not_reordered(TE):
+    # geometric-factor setup (reference unittest/kernel/test_TensorEngine.cpp:543-590): summing j first would save
+    # a third of the multiplications, which one lane's shared partial sums already do
+    D, W, C, Jdet, Jinv = at.Tensor(10, 3, 3, 5, 5, 5), at.Tensor(5, 5, 5), at.Tensor(10, 5, 5, 5), at.Tensor(10, 5, 5, 5), at.Tensor(10, 5, 5, 5, 3, 3)
+    src = TE.GetImplementation("D_e_m_n_k1_k2_k3 = W_k1_k2_k3 C_e_k1_k2_k3 Jdet_e_k1_k2_k3 Jinv_e_k1_k2_k3_n_j Jinv_e_k1_k2_k3_m_j",
+                               D, W, C, Jdet, Jinv, Jinv)
+    assert "_F1" not in src and src.count("__syncthreads()") == 0
+
+
+def test_stiffness_assembly_sums_one_direction_early(TE):
+    # 3D stiffness assembly (reference unittest/kernel/test_TensorEngine.cpp:437-496): 1 125 terms of 4 factors per
+    # output as written; the k3 sum is taken first, the remaining directions would not fit in LDS
+    S, B1, B2, B3, D = at.Tensor(10, 5, 5, 5, 5, 5, 5), at.Tensor(5, 5, 5, 3, 3), at.Tensor(5, 5, 5, 3, 3), at.Tensor(5, 5, 5, 3, 3), at.Tensor(10, 5, 5, 5, 3, 3)
+    src = TE.GetImplementation("S_e_i1_i2_i3_j1_j2_j3 = B1_i1_j1_k1_m_n B2_i2_j2_k2_m_n B3_i3_j3_k3_m_n D_e_k1_k2_k3_m_n",
+                               S, B1, B2, B3, D)
+    assert "_F1->lds\n" in src and "_F1<-lds" in src and "S->global" in src
 
 
 def test_long_contraction_uses_counted_loops(TE):

@@ -1,0 +1,106 @@
+"""Single kernels that the HIP policy evaluates as a chain of smaller contractions (partial results in LDS) must give
+what the reference's interpreter gives for the kernel as written (exec/CPUInterpretedExecutor.cpp:59-121), for every
+assignment operator, binding mode and index layout.  Through the C ABI, against the oracle."""
+import numpy as np
+import pytest
+
+from gpu_helpers import output_shape, rel_err, run_single, to_tensor
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-12
+
+
+def is_reordered(engine):
+    return "_F1" in engine.GetLastImplementation()
+
+
+# kernel, input shapes; every one of them is large enough and gains enough for the generator to reorder it
+REORDERED = [
+    # p=2 mass assembly, config 3 of the baseline at a ragged element count
+    ("M_e_i_j_k_l_m_n = B_q_i B_q_l B_r_j B_r_m B_s_k B_s_n W_e_q_r_s", [(4, 3)] * 6 + [(37, 4, 4, 4)]),
+    # the element index is not the first dimension of the output or of the streamed input
+    ("M_i_j_e_k_l = B_q_i B_q_k B_r_j B_r_l W_q_e_r", [(6, 5)] * 4 + [(6, 50, 6)]),
+    # three different tables, an input that has no contraction index at all (pointwise factor C_e)
+    ("Y_e_a_b_c = P_a_i Q_b_j R_c_k X_e_i_j_k C_e", [(7, 6), (5, 6), (4, 6), (21, 6, 6, 6), (21,)]),
+    # two contraction indices leave together (n and m only meet in F and G)
+    ("Z_e_i_j = F_i_n_m G_n_m_p H_p_j_q X_e_q", [(9, 4, 3), (4, 3, 8), (8, 9, 7), (19, 7)]),
+    # a contraction index that a single operand carries alone (T_e_i_j = sum_k A_e_i_j_k, then the rest)
+    ("Y_e_i = A_e_i_j_k B_j_l C_l_m D_m_i", [(11, 12, 9, 8), (9, 10), (10, 9), (9, 12)]),
+]
+
+
+@pytest.mark.parametrize("op", ["=", "+=", "-="])
+@pytest.mark.parametrize("kernel,shapes", REORDERED)
+def test_reordered_kernel_matches_the_kernel_as_written(at, engine, checker, kernel, shapes, op):
+    kernel = kernel.replace(" = ", " %s " % op)
+    rng = np.random.default_rng(len(kernel) * 7 + len(op))
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    init = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, init, *ins)
+    assert is_reordered(engine), engine.GetLastImplementation().splitlines()[1:6]
+    if op == "-=":
+        expected = init - (expected - init)  # the interpreter adds for "-=" (exec/CPUInterpretedExecutor.cpp:106)
+    assert rel_err(got, expected) <= TOL
+
+
+def test_reordered_kernel_is_exact_on_integer_data(at, engine, checker):
+    kernel, shapes = REORDERED[0]
+    ins = [np.arange(np.prod(s), dtype=np.float64).reshape(s) % 5 - 2.0 for s in shapes]
+    got, expected = run_single(at, engine, checker, kernel, np.zeros(output_shape(kernel, shapes)), *ins)
+    assert is_reordered(engine)
+    assert np.array_equal(got, expected)
+
+
+def test_reordered_kernel_with_one_name_bound_to_two_tensors(at, engine, checker):
+    # "B" names two different tensors: operands are taken by position (reference kernel/TensorEngine.cpp:290-336
+    # passes the tensors of a call in order, whatever their names say)
+    kernel = "M_e_i_j_k_l = B_q_i B_q_k B_r_j B_r_l W_e_q_r"
+    rng = np.random.default_rng(5)
+    tables = [rng.uniform(-1, 1, (6, 5)) for _ in range(4)]
+    W = rng.uniform(0.5, 1.5, (40, 6, 6))
+    got, expected = run_single(at, engine, checker, kernel, np.zeros((40, 5, 5, 5, 5)), *tables, W)
+    assert is_reordered(engine)
+    assert rel_err(got, expected) <= TOL
+    assert rel_err(got, np.einsum("qi,qk,rj,rl,eqr->eijkl", *tables, W)) <= TOL
+
+
+def test_reordered_kernel_writes_into_a_slice_and_reads_a_slice(at, engine, checker):
+    rng = np.random.default_rng(6)
+    B, W = rng.uniform(-1, 1, (6, 5)), rng.uniform(0.5, 1.5, (2, 30, 6, 6))
+    tB, tW, M = to_tensor(at, B), to_tensor(at, W), at.Tensor(2, 30, 5, 5, 5, 5)
+    M.Set(-1.0)
+    M1, W1 = at.SliceTensor(M, 1), at.SliceTensor(tW, 1)
+    engine("M_e_i_j_k_l = B_q_i B_q_k B_r_j B_r_l W_e_q_r", M1, tB, tB, tB, tB, W1)
+    assert is_reordered(engine)
+    M.MoveFromGPU()
+    assert rel_err(M.data[1], np.einsum("qi,qk,rj,rl,eqr->eijkl", B, B, B, B, W[1])) <= TOL
+    assert np.all(M.data[0] == -1.0)
+
+
+def test_kernel_runs_as_written_when_no_partial_result_fits_in_lds(at, engine, checker):
+    # both candidate partial results (8 x 800 doubles per batch entry) exceed 48 KB
+    kernel = "Y_e_a_b = P_a_i Q_b_j X_e_i_j"
+    shapes = [(8, 800), (8, 800), (10, 800, 800)]
+    rng = np.random.default_rng(8)
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    got, expected = run_single(at, engine, checker, kernel, np.zeros((10, 8, 8)), *ins)
+    assert not is_reordered(engine)
+    assert rel_err(got, expected) <= TOL
+
+
+def test_partial_results_that_do_not_fit_together_fall_back(at, engine, checker):
+    # the cheapest order keeps two partial results of 17^3 doubles alive at once (79 KB) and no order with smaller
+    # ones exists, so the kernel runs as written
+    kernel = "Y_e_a_b_c = P_a_i Q_b_j R_c_k X_e_i_j_k"
+    shapes = [(17, 17)] * 3 + [(18, 17, 17, 17)]
+    rng = np.random.default_rng(9)
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    got, expected = run_single(at, engine, checker, kernel, np.zeros((18, 17, 17, 17)), *ins)
+    assert not is_reordered(engine)
+    assert rel_err(got, expected) <= TOL
+    # one size down both fit (16^3 doubles each, 64 KB together) and the chain is used
+    shapes = [(16, 16)] * 3 + [(17, 16, 16, 16)]
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    got, expected = run_single(at, engine, checker, kernel, np.zeros((17, 16, 16, 16)), *ins)
+    assert is_reordered(engine)
+    assert rel_err(got, expected) <= TOL
