@@ -1780,8 +1780,8 @@ class Generator
     // mapping lanes to outputs would leave the device idle, so the flattened contraction range is split over
     // workgroups and over the lanes of a workgroup.  Lane (slice, output entry) accumulates a private partial sum
     // over its share, the workgroup adds its slices in LDS and writes one partial per output entry to a scratch
-    // buffer, and a second, single-workgroup kernel adds the per-workgroup partials in a fixed order (no atomics:
-    // results are reproducible from run to run).
+    // buffer, and a second, single-workgroup kernel adds the per-workgroup partials in a fixed order (no
+    // floating-point atomics: results are reproducible from run to run).
     static constexpr long kReductionMinContraction = 2048;
     static constexpr long kReductionMaxOutputs = 128;
     static constexpr int kReductionLanes = 256;
@@ -1860,20 +1860,31 @@ class Generator
         long G = std::min<long>(512, std::max<long>(1, Nc / (Sn * 16)));
         const long chunk = ((Nc + G - 1) / G + Sn - 1) / Sn * Sn;  // contraction entries per workgroup
         G = (Nc + chunk - 1) / chunk;
-        const long S2 = NTr / O;
+        // Lanes of the finishing kernel: enough for every lane to have all its loads of partials in flight at once
+        // (the kernel is a chain of memory latencies: launch, one round of loads, LDS; 1024 lanes instead of 256
+        // measured 16.8 instead of 17.2 us for the pair of launches at n = 2^20), at most 1024.  The one-pass
+        // variant finishes with the lanes of the partial kernel.
+        int NTf = NTr;
+        if (envInt("ACRO_HIP_ONE_PASS") <= 0)
+        {
+            while (NTf < 1024 && G * O > NTf * 4) NTf *= 2;
+        }
+        const long S2 = NTf / O;
 
         const std::string dimName = mk.GetDimensionedNameString();
         char hex[32];
         std::snprintf(hex, sizeof(hex), "%016llx",
                       static_cast<unsigned long long>(hashString(dimName + "/reduction/" + (opt.noalias ? "n" : "a") +
-                                                                 (Positional() ? "p" : "u"))));
+                                                                 (Positional() ? "p" : "u") +
+                                                                 (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "2" : "1"))));
         plan.module_name = std::string("acro_red_") + hex;
         const std::string fPartial = plan.module_name + "_partial", fFinal = plan.module_name + "_final";
 
         std::ostringstream sched;
         sched << "reduction schedule: " << O << " output entries, contraction of " << Nc << " terms split over " << G
               << " workgroups x " << Sn << " slices (" << (outputsFastest ? "output entries" : "slices")
-              << " on adjacent lanes), deterministic two-stage finish\n  [0] " << s.text << "\n";
+              << " on adjacent lanes), partials added in a fixed order by "
+              << (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "a second kernel" : "the workgroup that finishes last") << "\n  [0] " << s.text << "\n";
         plan.schedule = sched.str();
 
         out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
@@ -1896,10 +1907,14 @@ class Generator
             }
         };
 
+        const bool twoKernels = envInt("ACRO_HIP_ONE_PASS") <= 0;
+        const std::string counter = "(unsigned int *)(scratch + " + str(G * O) + ")";
+
         // ---- stage 1: per-workgroup partial sums
         out << "\nextern \"C\" __global__ __launch_bounds__(" << NTr << ") void " << fPartial << "(" << ParamList()
             << ", double *__restrict__ scratch)\n{\n";
         out << "    __shared__ double red[" << NTr << "];\n";
+        if (!twoKernels) out << "    __shared__ int isLast;\n";
         out << "    const int lane = threadIdx.x;\n";
         if (outputsFastest)
             out << "    const int sl = lane / " << O << ", o = lane % " << O << ";\n";
@@ -1924,31 +1939,62 @@ class Generator
         out << "    if (lane < " << O << ")\n    {\n        double t = 0.0;\n";
         out << "        for (int k = 0; k < " << Sn << "; ++k) t += red["
             << (outputsFastest ? "k * " + str(O) + " + lane" : "lane * " + str(Sn) + " + k") << "];\n";
-        out << "        scratch[(long)blockIdx.x * " << O << " + lane] = t;\n    }\n}\n";
-
-        // ---- stage 2: add the per-workgroup partials in a fixed order and apply the assignment operator
-        out << "\nextern \"C\" __global__ __launch_bounds__(" << NTr << ") void " << fFinal << "(double *"
-            << (opt.noalias ? "__restrict__ " : "") << "result, const double *__restrict__ scratch)\n{\n";
-        out << "    __shared__ double red[" << NTr << "];\n";
-        out << "    const int lane = threadIdx.x;\n";
-        out << "    const int g2 = lane / " << O << ", o = lane % " << O << ";\n";
-        out << "    double sum = 0.0;\n";
-        out << "    if (lane < " << S2 * O << ")\n    {\n";
-        out << "#pragma unroll 8\n";
-        out << "        for (long g = g2; g < " << G << "; g += " << S2 << ") sum += scratch[g * " << O << " + o];\n    }\n";
-        out << "    red[lane] = sum;\n    __syncthreads();\n";
-        out << "    if (lane < " << O << ")\n    {\n        double t = 0.0;\n";
-        out << "        for (int k = 0; k < " << S2 << "; ++k) t += red[k * " << O << " + lane];\n";
-        decompose(s.outIdx, "lane", "        ");
-        const std::string dst = "result[" + FullOffset(s.out) + "]";
-        if (s.op == '=')
-            out << "        " << dst << " = t;\n";
+        if (twoKernels)
+            out << "        scratch[(long)blockIdx.x * " << O << " + lane] = t;\n    }\n}\n";
         else
-            out << "        " << dst << " = " << dst << (s.op == '+' ? " + t;\n" : " - t;\n");
-        out << "    }\n}\n";
+            out << "        __hip_atomic_store(&scratch[(long)blockIdx.x * " << O
+                << " + lane], t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n    }\n";
+
+        // ---- stage 2: add the per-workgroup partials in a fixed order and apply the assignment operator.
+        // Default: a second, single-workgroup kernel.
+        // ACRO_HIP_ONE_PASS=1: the workgroup that arrives last at a device-wide counter does it instead (partials and
+        // counter exchanged with device-scope atomics and fences; the counter lives behind the partials in the scratch
+        // buffer, which the executor zeroes when it allocates it, and the last workgroup sets it back to zero).  The
+        // device-scope fences write back and invalidate the L2 of the workgroup's XCD every time; with 507 workgroups
+        // the single launch measured 55.9 us against 17.3 us for the two launches, so it is not the default.
+        auto emitFinish = [&](const std::string &load) {
+            out << "    const int g2 = lane / " << O << ", o2 = lane % " << O << ";\n";
+            out << "    double sum2 = 0.0;\n";
+            out << "    if (lane < " << S2 * O << ")\n    {\n";
+            out << "#pragma unroll 8\n";
+            out << "        for (long g = g2; g < " << G << "; g += " << S2 << ") sum2 += " << load << ";\n    }\n";
+            out << "    red[lane] = sum2;\n    __syncthreads();\n";
+            out << "    if (lane < " << O << ")\n    {\n        double t = 0.0;\n";
+            out << "        for (int k = 0; k < " << S2 << "; ++k) t += red[k * " << O << " + lane];\n";
+            decompose(s.outIdx, "lane", "        ");
+            const std::string dst = (twoKernels ? std::string("result") : PtrName(s.out.uvar)) + "[" + FullOffset(s.out) + "]";
+            if (s.op == '=')
+                out << "        " << dst << " = t;\n";
+            else
+                out << "        " << dst << " = " << dst << (s.op == '+' ? " + t;\n" : " - t;\n");
+            out << "    }\n";
+        };
+        if (twoKernels)
+        {
+            out << "\nextern \"C\" __global__ __launch_bounds__(" << NTf << ") void " << fFinal << "(double *"
+                << (opt.noalias ? "__restrict__ " : "") << "result, const double *__restrict__ scratch)\n{\n";
+            out << "    __shared__ double red[" << NTf << "];\n";
+            out << "    const int lane = threadIdx.x;\n";
+            emitFinish("scratch[g * " + str(O) + " + o2]");
+            out << "}\n";
+        }
+        else
+        {
+            out << "    __threadfence();\n    __syncthreads();\n";
+            out << "    if (lane == 0)\n    {\n";
+            out << "        const unsigned int arrived = __hip_atomic_fetch_add(" << counter
+                << ", 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);\n";
+            out << "        isLast = (arrived == " << G - 1 << "u);\n    }\n";
+            out << "    __syncthreads();\n";
+            out << "    if (!isLast) return;\n";
+            out << "    __threadfence();\n";
+            emitFinish("__hip_atomic_load(&scratch[g * " + str(O) + " + o2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)");
+            out << "    if (lane == 0) __hip_atomic_store(" << counter << ", 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+            out << "}\n";
+        }
 
         plan.source = out.str();
-        plan.scratch_doubles = static_cast<size_t>(G * O);
+        plan.scratch_doubles = static_cast<size_t>(G * O) + (twoKernels ? 0 : 1);
         plan.nb = 1;
         plan.lds_bytes = NTr * 8;
         FillParams(plan, false);
@@ -1959,14 +2005,17 @@ class Generator
         partial.block = NTr;
         for (int si = 0; si < S; ++si) partial.params.push_back(si);
         partial.params.push_back(-1);
-        HipLaunch fin;
-        fin.function_name = fFinal;
-        fin.grid = 1;
-        fin.block = NTr;
-        fin.params.push_back(uvars[s.out.uvar].storage);
-        fin.params.push_back(-1);
         plan.launches.push_back(partial);
-        plan.launches.push_back(fin);
+        if (twoKernels)
+        {
+            HipLaunch fin;
+            fin.function_name = fFinal;
+            fin.grid = 1;
+            fin.block = NTf;
+            fin.params.push_back(uvars[s.out.uvar].storage);
+            fin.params.push_back(-1);
+            plan.launches.push_back(fin);
+        }
     }
 
     void Emit(HipKernelPlan &plan)

@@ -23,6 +23,9 @@
 //   ACRO_HIP_LDS_PAD=1|2        pad LDS tile strides against bank conflicts (2: even if a resident workgroup is lost)
 //   ACRO_HIP_PACK=1             pick batch / workgroup size for wavefront utilisation
 //   ACRO_HIP_PERSIST=<n>        persistent grid of n workgroups per CU looping over the batch
+//   ACRO_HIP_FACTORISE=-1       evaluate multi-operand single kernels as written instead of as a chain of steps
+//   ACRO_HIP_ONE_PASS=1         split contractions: the workgroup that finishes last adds the per-workgroup partials
+//                               instead of a second kernel (measured 3x slower: device-scope fences flush the L2)
 #ifndef ACRO_HIP_CODEGEN_HPP
 #define ACRO_HIP_CODEGEN_HPP
 
@@ -78,7 +81,9 @@ struct HipKernelPlan
     std::string module_name;
     std::string source;            // one translation unit defining every function of `launches`
     std::vector<HipLaunch> launches;  // executed in order on the library's stream
-    size_t scratch_doubles = 0;    // device scratch the launches share (partial sums of split contractions)
+    // Device scratch the launches share (partial sums of split contractions and their arrival counter).  The
+    // executor zeroes it once, when it allocates it; the kernels leave the counter at zero when they finish.
+    size_t scratch_doubles = 0;
     // Kernel parameter i is the device pointer of a storage: the device pointer of the tensor bound to this
     // (kernel number, variable number) occurrence (variable number -1 is that kernel's output) minus param_offset[i]
     // elements (the occurrence may be a view into the storage).

@@ -229,6 +229,7 @@ class HipExecutor : public KernelExecutor
         if (v.plan.scratch_doubles > 0 && v.scratch == nullptr)
         {
             v.scratch = static_cast<double *>(hip::Malloc(v.plan.scratch_doubles * sizeof(double)));
+            hip::FillDouble(v.scratch, 0.0, v.plan.scratch_doubles);  // on the stream, ahead of the first launch
         }
         for (const auto &z : v.plan.zero_fills)
         {

@@ -214,6 +214,36 @@ def test_config1_full_size_closed_form(at, engine):
     assert rel_err(S, expected) <= TOL
 
 
+@pytest.mark.parametrize("one_pass", [False, True])
+def test_config1_repeated_launches_are_bit_identical_and_accumulate(at, engine, monkeypatch, one_pass):
+    # the partial sums of the split contraction are added in a fixed order, by a second kernel or (experiment
+    # switch) by whichever workgroup finishes last; neither the result nor the state left behind for the next launch
+    # may depend on timing
+    if one_pass:
+        monkeypatch.setenv("ACRO_HIP_ONE_PASS", "1")
+    wl = workloads.config1(n=1048576 - 8 * one_pass)
+    tensors = run_workload(at, engine, wl, False)
+    first = fetch(tensors, "S")
+    k, out, ins = wl.kernels[0]
+    for _ in range(50):
+        engine(k, tensors[out], *[tensors[n] for n in ins])
+    assert np.array_equal(fetch(tensors, "S"), first)
+    tensors["S"].MoveToGPU()
+    for _ in range(3):
+        engine(k.replace(" = ", " += "), tensors[out], *[tensors[n] for n in ins])
+    got = fetch(tensors, "S")
+    assert rel_err(got, 4.0 * first) <= TOL
+    # and a second shape on the same engine (its own scratch buffer and counter)
+    n = 300007 + one_pass
+    A = (np.arange(n * 9) % 13).astype(np.float64).reshape(n, 3, 3)
+    S = at.Tensor(3, 3)
+    tA, tB = to_tensor(at, A), to_tensor(at, np.ones(n))
+    for _ in range(5):
+        engine("S_i_j = A_n_i_j B_n", S, tA, tB)
+    S.MoveFromGPU()
+    assert np.array_equal(S.data, A.sum(axis=0))
+
+
 def test_config3_full_size_symmetry_and_sample(at, engine, checker):
     E = 32768
     wl = workloads.config3(E=E)
