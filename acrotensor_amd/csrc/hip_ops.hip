@@ -12,6 +12,8 @@
 // without multiply-add contraction, so results are bit-identical to the host formulas.
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
+
 #include "HipRuntime.hpp"
 #include "NonContractionOps.hpp"
 
@@ -163,6 +165,17 @@ __global__ __launch_bounds__(kMatLanes) void batchMatrixKernel(const double *__r
     }
 }
 
+// Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with an L2 of its own.  The index kernels
+// gather through a map with spatial locality (neighbouring range entries touch neighbouring domain entries), so
+// each XCD is given one contiguous eighth of the work instead of every eighth workgroup: lines that neighbouring
+// workgroups share are then fetched from HBM once, not once per XCD.
+__device__ inline unsigned xcdContiguousBlock()
+{
+    const unsigned per = gridDim.x / 8;
+    const unsigned b = blockIdx.x;
+    return b < per * 8 ? (b % 8) * per + b / 8 : b;
+}
+
 __global__ __launch_bounds__(kLanes) void scatterKernel(double *__restrict__ Aout, const double *__restrict__ Ain,
                                                         const int *__restrict__ M, int range_size)
 {
@@ -170,18 +183,87 @@ __global__ __launch_bounds__(kLanes) void scatterKernel(double *__restrict__ Aou
     if (i < range_size) Aout[i] = Ain[M[i]];
 }
 
+// Four consecutive range entries per lane: one 16-byte load of map entries, four gathers in flight, two 16-byte
+// stores.  Needs Aout and M aligned to 16 bytes; the entries past the last multiple of four go to the last lane.
+__global__ __launch_bounds__(kLanes) void scatterKernel4(double *__restrict__ Aout, const double *__restrict__ Ain,
+                                                         const int *__restrict__ M, int range_size)
+{
+    const int quads = range_size / 4;
+    const int q = xcdContiguousBlock() * kLanes + threadIdx.x;
+    if (q < quads)
+    {
+        const int4 m = reinterpret_cast<const int4 *>(M)[q];
+        const double a0 = Ain[m.x], a1 = Ain[m.y], a2 = Ain[m.z], a3 = Ain[m.w];
+        double2 *dst = reinterpret_cast<double2 *>(Aout) + 2 * static_cast<size_t>(q);
+        dst[0] = make_double2(a0, a1);
+        dst[1] = make_double2(a2, a3);
+    }
+    if (q == quads - 1)
+    {
+        for (int i = quads * 4; i < range_size; ++i) Aout[i] = Ain[M[i]];
+    }
+}
+
 // Row d of the inverse map lists, in increasing range order, the entries that are added into Aout[d]; summing
 // them front to back reproduces the sequential host scatter-add bit for bit and needs no atomics.
+// A workgroup owns kGatherRows * kLanes consecutive rows.  Their entries are consecutive in the inverse map, so the workgroup
+// walks that range in chunks: all lanes gather a chunk into LDS (unit-stride reads of the map, eight gathers in
+// flight per lane whatever the row lengths are), then the lane of each row adds the part of its row that lies in
+// the chunk, in row order.  Rows are short on average (2.3 entries for a hexahedral mesh) and uneven (1 to 8), so
+// one lane walking its own row leaves most of a wavefront's gather slots empty.
+constexpr int kGatherChunk = 8 * kLanes;
+constexpr int kGatherRows = 4;  // rows per lane: a workgroup's range of entries should fill a chunk
+
 __global__ __launch_bounds__(kLanes) void sumGatherKernel(double *__restrict__ Aout, const double *__restrict__ Ain,
                                                           const int *__restrict__ InvM,
                                                           const int *__restrict__ InvMOff, int domain_size)
 {
-    int d = blockIdx.x * kLanes + threadIdx.x;
-    if (d >= domain_size) return;
-    double sum = 0.0;
-    const int end = InvMOff[d + 1];
-    for (int k = InvMOff[d]; k < end; ++k) sum += Ain[InvM[k]];
-    Aout[d] = sum;
+    __shared__ double vals[kGatherChunk];
+    const int d0 = xcdContiguousBlock() * (kLanes * kGatherRows);  // first row of this workgroup
+    if (d0 >= domain_size) return;
+    const int dEnd = d0 + kLanes * kGatherRows < domain_size ? d0 + kLanes * kGatherRows : domain_size;
+    const int first = InvMOff[d0], last = InvMOff[dEnd];
+    int rowBegin[kGatherRows], rowEnd[kGatherRows];
+    double sum[kGatherRows];
+#pragma unroll
+    for (int r = 0; r < kGatherRows; ++r)
+    {
+        const int d = d0 + r * kLanes + threadIdx.x;
+        rowBegin[r] = d < domain_size ? InvMOff[d] : 0;
+        rowEnd[r] = d < domain_size ? InvMOff[d + 1] : 0;
+        sum[r] = 0.0;
+    }
+    for (int c = first; c < last; c += kGatherChunk)
+    {
+        const int n = last - c < kGatherChunk ? last - c : kGatherChunk;
+        int idx[8];
+        double a[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+        {
+            const int j = threadIdx.x + u * kLanes;
+            idx[u] = j < n ? InvM[c + j] : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a[u] = idx[u] >= 0 ? Ain[idx[u]] : 0.0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) vals[threadIdx.x + u * kLanes] = a[u];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < kGatherRows; ++r)
+        {
+            const int lo = rowBegin[r] > c ? rowBegin[r] : c;
+            const int hi = rowEnd[r] < c + n ? rowEnd[r] : c + n;
+            for (int k = lo; k < hi; ++k) sum[r] += vals[k - c];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int r = 0; r < kGatherRows; ++r)
+    {
+        const int d = d0 + r * kLanes + threadIdx.x;
+        if (d < domain_size) Aout[d] = sum[r];
+    }
 }
 
 unsigned gridFor(size_t n)
@@ -268,15 +350,21 @@ void HipGPUOps::BatchMatrixInvDet(Tensor &Ainv, Tensor &Adet, Tensor &A)
 void HipGPUOps::FlatIndexedScatter(Tensor &Aout, Tensor &Ain, IndexMapping &M)
 {
     const int n = M.GetRangeSize();
-    hipLaunchKernelGGL(scatterKernel, dim3(gridFor(n)), dim3(kLanes), 0, stream(), Aout.GetDeviceData(),
-                       Ain.GetDeviceData(), M.GetMap().GetDeviceData(), n);
+    const bool aligned = reinterpret_cast<uintptr_t>(Aout.GetDeviceData()) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(M.GetMap().GetDeviceData()) % 16 == 0;
+    if (aligned && n >= 4)
+        hipLaunchKernelGGL(scatterKernel4, dim3(gridFor(n / 4)), dim3(kLanes), 0, stream(), Aout.GetDeviceData(),
+                           Ain.GetDeviceData(), M.GetMap().GetDeviceData(), n);
+    else
+        hipLaunchKernelGGL(scatterKernel, dim3(gridFor(n)), dim3(kLanes), 0, stream(), Aout.GetDeviceData(),
+                           Ain.GetDeviceData(), M.GetMap().GetDeviceData(), n);
     ACRO_HIP_CHECK(hipGetLastError());
 }
 
 void HipGPUOps::FlatIndexedSumGather(Tensor &Aout, Tensor &Ain, IndexMapping &M)
 {
     const int n = M.GetDomainSize();
-    hipLaunchKernelGGL(sumGatherKernel, dim3(gridFor(n)), dim3(kLanes), 0, stream(), Aout.GetDeviceData(),
+    hipLaunchKernelGGL(sumGatherKernel, dim3(gridFor((static_cast<size_t>(n) + kGatherRows - 1) / kGatherRows)), dim3(kLanes), 0, stream(), Aout.GetDeviceData(),
                        Ain.GetDeviceData(), M.GetInvMap().GetDeviceData(), M.GetInvMapOffsets().GetDeviceData(), n);
     ACRO_HIP_CHECK(hipGetLastError());
 }

@@ -188,3 +188,18 @@ def config5(E=65536, seed=0xAC25, Q=10, P=8):
     return Workload("cfg5_diffusion_apply_p7", arrays, kernels, transient=transient, slices=slices, outputs=("Y",),
                     dof=E * P ** 3, algorithmic_bytes=E * (P ** 3 + 9 * Q ** 3 + P ** 3) * 8,
                     flops=E * flops_per_elem, seed=seed)
+
+
+def hex_mesh_dof_map(nx, ny, nz, p):
+    """Element-to-node numbering of a structured nx x ny x nz hexahedral mesh of continuous degree-p elements:
+    int32 array [E, p+1, p+1, p+1] of node numbers in [0, (nx p + 1)(ny p + 1)(nz p + 1)).  This is the IndexMapping an
+    FE code uses with FlatIndexedScatter (node vector -> element vector) before an operator apply and with
+    FlatIndexedSumGather (element vector -> node vector) after it (reference ops/NonContractionOps.hpp:27-31)."""
+    n1 = p + 1
+    gx, gy, gz = nx * p + 1, ny * p + 1, nz * p + 1
+    ex, ey, ez = np.meshgrid(np.arange(nx), np.arange(ny), np.arange(nz), indexing="ij")
+    base = ((ex * p) * gy + ey * p) * gz + ez * p                      # node of local (0, 0, 0), shape [nx, ny, nz]
+    li, lj, lk = np.meshgrid(np.arange(n1), np.arange(n1), np.arange(n1), indexing="ij")
+    local = (li * gy + lj) * gz + lk                                  # offsets of the local nodes
+    dofs = base.reshape(-1, 1, 1, 1) + local[None]
+    return dofs.astype(np.int32), gx * gy * gz

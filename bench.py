@@ -79,7 +79,8 @@ FP64_PEAK_GFLOPS = 78600.0
 
 
 def other_workload(at, workloads, args):
-    """Same measurement for cfg1 / cfg2 / cfg3 / cfg5 at the sizes of the baseline configurations."""
+    """Same measurement for cfg1 / cfg2 / cfg3 / cfg5 at the sizes of the baseline configurations, and for
+    FlatIndexedScatter / FlatIndexedSumGather on the headline mesh."""
     engine = at.TensorEngine("HIP")
     name = args.workload
     if name == "cfg2":
@@ -92,6 +93,26 @@ def other_workload(at, workloads, args):
         step = lambda: engine.BatchMatrixInvDet(Jinv, Jdet, tJ)
         label = "configs[1]: BatchMatrixInvDet, J[65536,64,3,3]"
         units, unit_name, abytes, flops = E * Q, "Gmatrices/s", E * Q * 152, E * Q * 54
+    elif name in ("scatter", "sumgather"):
+        # node vector <-> element vector of the headline mesh size: 64^3 hex elements of degree 3
+        import numpy as np
+        dofs, nodes = workloads.hex_mesh_dof_map(64, 64, 64, 3)
+        M = at.IndexMapping(nodes, dofs.size)
+        M.map[:] = dofs.ravel()
+        L, Ev = at.Tensor(nodes), at.Tensor(dofs.size)
+        L.data[...] = workloads.counter_uniform(0xAC26, 0, (nodes,), -1.0, 1.0)
+        Ev.data[...] = workloads.counter_uniform(0xAC26, 1, (dofs.size,), -1.0, 1.0)
+        for t in (L, Ev):
+            t.MoveToGPU()
+        if name == "scatter":
+            step = lambda: engine.FlatIndexedScatter(Ev, L, M)
+            label = "E-vector[262144*64] = L-vector[7189057] through the element-to-node map"
+            abytes = dofs.size * (4 + 8) + nodes * 8          # map + E-vector written + every node read once
+        else:
+            step = lambda: engine.FlatIndexedSumGather(L, Ev, M)
+            label = "L-vector[7189057] = sum of E-vector[262144*64] entries through the element-to-node map"
+            abytes = dofs.size * (4 + 8) + nodes * (4 + 8)    # inverse map + E-vector read + row offsets + L written
+        units, unit_name, flops = dofs.size, "GDOF/s", dofs.size
     else:
         wl = {"cfg1": workloads.config1, "cfg3": workloads.config3, "cfg5": workloads.config5}[name]()
         tensors = workloads.bind_to_engine(wl, at, transient=True)
@@ -140,9 +161,10 @@ def main():
     ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store-all", action="store_true")
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"],
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather"],
                     help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
-                         "remaining baseline configurations at their full sizes")
+                         "remaining baseline configurations at their full sizes and for the node-vector <-> "
+                         "element-vector steps either side of the operator apply")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one scale-by-1.0 kernel over X (reads and writes E*512 bytes): the known-size "
                          "kernel that hardware-counter runs are scaled by")

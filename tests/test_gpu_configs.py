@@ -257,3 +257,21 @@ def test_config3_full_size_symmetry_and_sample(at, engine, checker):
     sub.arrays["B"][...] = wl.arrays["B"]
     sub.arrays["W"][...] = wl.arrays["W"][sample]
     assert rel_err(M[sample], workloads.run_on_checker(sub, checker)["M"]) <= TOL
+
+
+def test_node_vector_to_element_vector_and_back_full_size(at, engine):
+    # FlatIndexedScatter / FlatIndexedSumGather on the mesh of the headline configuration (64^3 hexahedra of degree
+    # 3: 16.8 M element entries, 7.2 M nodes); integer-valued data make every sum exact whatever the row length
+    dofs, nodes = workloads.hex_mesh_dof_map(64, 64, 64, 3)
+    M = at.IndexMapping(nodes, dofs.size)
+    M.map[:] = dofs.ravel()
+    Lv = (np.arange(nodes) % 97 - 48).astype(np.float64)
+    L, Ev, back = to_tensor(at, Lv), at.Tensor(dofs.size), at.Tensor(nodes)
+    engine.FlatIndexedScatter(Ev, L, M)
+    Ev.MoveFromGPU()
+    assert np.array_equal(Ev.data, Lv[dofs.ravel()])
+    engine.FlatIndexedSumGather(back, Ev, M)
+    back.MoveFromGPU()
+    multiplicity = np.bincount(dofs.ravel(), minlength=nodes)
+    assert multiplicity.min() == 1 and multiplicity.max() == 8
+    assert np.array_equal(back.data, multiplicity * Lv)

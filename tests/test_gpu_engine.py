@@ -307,6 +307,45 @@ def test_sum_gather_large_random_map_bit_exact(at, engine, checker):
     assert np.array_equal(out.data, checker.scatter(src, M.map))
 
 
+@pytest.mark.parametrize("domain,rsize,skew", [(1, 9001, 0), (1030, 3, 0), (2500, 70001, 3), (4099, 4099, 0)])
+def test_scatter_and_sum_gather_ragged_maps_bit_exact(at, engine, checker, domain, rsize, skew):
+    # rows of the inverse map from empty to tens of thousands of entries (longer than one staging chunk), domain and
+    # range sizes that are not multiples of the workgroup or vector width
+    rng = np.random.default_rng(domain + rsize)
+    M = at.IndexMapping(domain, rsize)
+    m = rng.integers(0, domain, rsize)
+    if skew:
+        m[rng.uniform(size=rsize) < 0.6] = domain // skew          # one very long row
+    M.map[:] = m
+    vals = rng.uniform(-1, 1, rsize)
+    acc = at.Tensor(domain)
+    acc.Set(99.0)                                                  # must be overwritten, also where no entry maps
+    engine.FlatIndexedSumGather(acc, to_tensor(at, vals), M)
+    acc.MoveFromGPU()
+    assert np.array_equal(acc.data, checker.sum_gather(vals, M.map, domain))
+    src = rng.uniform(-1, 1, domain)
+    out = at.Tensor(rsize)
+    engine.FlatIndexedScatter(out, to_tensor(at, src), M)
+    out.MoveFromGPU()
+    assert np.array_equal(out.data, checker.scatter(src, M.map))
+
+
+def test_scatter_into_a_slice_that_is_not_vector_aligned(at, engine, checker):
+    rng = np.random.default_rng(77)
+    domain, rsize = 300, 1001                                       # slices start at odd multiples of 8 bytes
+    M = at.IndexMapping(domain, rsize)
+    M.map[:] = rng.integers(0, domain, rsize)
+    src = rng.uniform(-1, 1, domain)
+    parent = at.Tensor(3, rsize)
+    parent.Set(-5.0)
+    parent.MoveToGPU()      # an output that is still on the host is switched, not copied (kernel/TensorEngine.cpp:692-699)
+    out = at.SliceTensor(parent, 1)
+    engine.FlatIndexedScatter(out, to_tensor(at, src), M)
+    parent.MoveFromGPU()
+    assert np.array_equal(parent.data[1], checker.scatter(src, M.map))
+    assert np.all(parent.data[0] == -5.0) and np.all(parent.data[2] == -5.0)
+
+
 def test_get_implementation_returns_hip_source(at, engine):
     A, B = at.Tensor(8, 3), at.Tensor(8, 3)
     src = engine.GetImplementation("A_e_i = B_e_i", A, B)
