@@ -93,6 +93,25 @@ def other_workload(at, workloads, args):
         step = lambda: engine.BatchMatrixInvDet(Jinv, Jdet, tJ)
         label = "configs[1]: BatchMatrixInvDet, J[65536,64,3,3]"
         units, unit_name, abytes, flops = E * Q, "Gmatrices/s", E * Q * 152, E * Q * 54
+    elif name == "dsetup":
+        # geometric factors of the diffusion operator from the inverse Jacobians (reference
+        # unittest/kernel/test_TensorEngine.cpp:543-590), at the quadrature size of configs[4], E = 16384
+        import numpy as np
+        E, Q = 16384, 10
+        W, C, Jdet = at.Tensor(Q, Q, Q), at.Tensor(E, Q, Q, Q), at.Tensor(E, Q, Q, Q)
+        Jinv, D = at.Tensor(E, Q, Q, Q, 3, 3), at.Tensor(E, 3, 3, Q, Q, Q)
+        W.data[...] = workloads.counter_uniform(0xAC27, 0, (Q, Q, Q), 0.1, 1.0)
+        C.data[...] = workloads.counter_uniform(0xAC27, 1, (E, Q, Q, Q), 0.5, 1.5)
+        Jdet.data[...] = workloads.counter_uniform(0xAC27, 2, (E, Q, Q, Q), 0.5, 1.5)
+        Jinv.data[...] = workloads.counter_uniform(0xAC27, 3, (E, Q, Q, Q, 3, 3), -1.0, 1.0)
+        for t in (W, C, Jdet, Jinv, D):
+            t.MoveToGPU()
+        k = "D_e_m_n_k1_k2_k3 = W_k1_k2_k3 C_e_k1_k2_k3 Jdet_e_k1_k2_k3 Jinv_e_k1_k2_k3_n_j Jinv_e_k1_k2_k3_m_j"
+        step = lambda: engine(k, D, W, C, Jdet, Jinv, Jinv)
+        label = "geometric factor setup D[16384,3,3,10,10,10] from Jinv, Jdet, C, W"
+        points = E * Q * Q * Q
+        abytes, flops = points * (9 + 1 + 1 + 9) * 8, points * 9 * 3 * 5
+        units, unit_name = points, "Gpoints/s"
     elif name in ("scatter", "sumgather"):
         # node vector <-> element vector of the headline mesh size: 64^3 hex elements of degree 3
         import numpy as np
@@ -161,7 +180,7 @@ def main():
     ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store-all", action="store_true")
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather"],
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup"],
                     help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
                          "remaining baseline configurations at their full sizes and for the node-vector <-> "
                          "element-vector steps either side of the operator apply")
