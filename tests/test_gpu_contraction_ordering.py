@@ -104,3 +104,44 @@ def test_partial_results_that_do_not_fit_together_fall_back(at, engine, checker)
     got, expected = run_single(at, engine, checker, kernel, np.zeros((17, 16, 16, 16)), *ins)
     assert is_reordered(engine)
     assert rel_err(got, expected) <= TOL
+
+
+def random_multi_operand_kernel(rng):
+    letters = list("abcdfghijklmnopqrstuvwxyz")
+    n_out, n_con = int(rng.integers(1, 4)), int(rng.integers(1, 5))
+    names = list(rng.choice(letters, size=n_out + n_con, replace=False))
+    out_idx, con_idx = names[:n_out], names[n_out:]
+    extent = {n: int(rng.integers(1, 6)) for n in names}
+    extent[out_idx[0]] = int(rng.integers(6, 40))              # the batch index
+    n_in = int(rng.integers(3, 6))
+    ins = []
+    for v in range(n_in):
+        k = int(rng.integers(1, min(4, len(names)) + 1))
+        ins.append(list(rng.choice(names, size=k, replace=False)))
+    for c in con_idx:
+        if not any(c in i for i in ins):
+            ins[int(rng.integers(0, n_in))].append(c)
+    op = str(rng.choice(["=", "=", "+=", "-="]))
+    kernel = "O_" + "_".join(out_idx) + " " + op + " " + " ".join("I%d_%s" % (v, "_".join(i)) for v, i in enumerate(ins))
+    return kernel, tuple(extent[n] for n in out_idx), [tuple(extent[n] for n in i) for i in ins], op
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_kernels_reordered_whenever_possible(at, engine, checker, monkeypatch, seed):
+    # the size and gain thresholds are switched off, so every kernel with a cheaper chain of steps takes that path:
+    # odd index patterns (inputs without the batch index, indices shared by all operands, broadcast output indices,
+    # several indices leaving in one step) go through the ordering search and the LDS-only partial results
+    monkeypatch.setenv("ACRO_HIP_FACTORISE", "2")
+    rng = np.random.default_rng(9000 + seed)
+    kernel, out_shape, shapes, op = random_multi_operand_kernel(rng)
+    print(kernel, out_shape, shapes, flush=True)
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    init = rng.uniform(-1, 1, out_shape)
+    out = to_tensor(at, init)
+    engine(kernel, out, *[to_tensor(at, a) for a in ins])
+    out.MoveFromGPU()
+    expected = init.copy()
+    checker.contract(kernel.replace("-=", "+="), expected, *ins)
+    if op == "-=":
+        expected = init - (expected - init)
+    assert rel_err(out.data, expected) <= TOL
