@@ -25,19 +25,43 @@ namespace acro
 namespace
 {
 
-constexpr int kLanes = 256;    // fill, scale, scatter, gather: one lane per entry
+typedef double Double2 __attribute__((ext_vector_type(2)));  // a 16-byte access the compiler keeps whole
+
+constexpr int kLanes = 256;    // fill, scale, scatter, gather
 constexpr int kMatLanes = 64;  // batched matrices: one wavefront per workgroup, so its barriers are free
 
+// Fill and scale move 16 bytes per lane and write with non-temporal stores (the result is not read again by the
+// kernel).  When the buffer starts on an odd multiple of 8 bytes its first entry is handled alone, so that the body
+// is 16-byte aligned; that entry and an odd last one go to the lane after the last pair.
 __global__ __launch_bounds__(kLanes) void fillKernel(double *__restrict__ d, double value, size_t n)
 {
-    size_t i = static_cast<size_t>(blockIdx.x) * kLanes + threadIdx.x;
-    if (i < n) d[i] = value;
+    const size_t head = ((reinterpret_cast<uintptr_t>(d) & 8) != 0 && n > 0) ? 1 : 0;
+    const size_t pairs = (n - head) / 2;
+    const size_t p = static_cast<size_t>(blockIdx.x) * kLanes + threadIdx.x;
+    if (p < pairs) __builtin_nontemporal_store(Double2{value, value}, reinterpret_cast<Double2 *>(d + head) + p);
+    if (p == pairs)
+    {
+        if (head) d[0] = value;
+        if ((n - head) & 1) d[n - 1] = value;
+    }
 }
 
 __global__ __launch_bounds__(kLanes) void scaleKernel(double *__restrict__ d, double factor, size_t n)
 {
-    size_t i = static_cast<size_t>(blockIdx.x) * kLanes + threadIdx.x;
-    if (i < n) d[i] *= factor;
+    const size_t head = ((reinterpret_cast<uintptr_t>(d) & 8) != 0 && n > 0) ? 1 : 0;
+    const size_t pairs = (n - head) / 2;
+    const size_t p = static_cast<size_t>(blockIdx.x) * kLanes + threadIdx.x;
+    if (p < pairs)
+    {
+        Double2 *q = reinterpret_cast<Double2 *>(d + head) + p;
+        const Double2 v = *q;
+        __builtin_nontemporal_store(Double2{v.x * factor, v.y * factor}, q);
+    }
+    if (p == pairs)
+    {
+        if (head) d[0] *= factor;
+        if ((n - head) & 1) d[n - 1] *= factor;
+    }
 }
 
 template <int M>
@@ -132,7 +156,7 @@ __global__ __launch_bounds__(kMatLanes) void batchMatrixKernel(const double *__r
 #pragma unroll
         for (int j = 0; j < MM; ++j) a[j] = tile[threadIdx.x * LS + j];
         const double det = SmallMatrix<M>::det(a);
-        if (WANT_DET) Adet[first + threadIdx.x] = det;
+        if (WANT_DET) __builtin_nontemporal_store(det, &Adet[first + threadIdx.x]);
         if (WANT_INV) SmallMatrix<M>::inv(r, a, det);
     }
     if (WANT_INV)
@@ -145,7 +169,6 @@ __global__ __launch_bounds__(kMatLanes) void batchMatrixKernel(const double *__r
         }
         __syncthreads();
         double *dst = Ainv + first * MM;
-        double2 *dst2 = reinterpret_cast<double2 *>(dst);
         for (int i = threadIdx.x; i < ndbl / 2; i += kMatLanes)
         {
             double2 v;
@@ -159,7 +182,9 @@ __global__ __launch_bounds__(kMatLanes) void batchMatrixKernel(const double *__r
                 v.x = tile[((2 * i) / MM) * LS + ((2 * i) % MM)];
                 v.y = tile[((2 * i + 1) / MM) * LS + ((2 * i + 1) % MM)];
             }
-            dst2[i] = v;
+            // results stream out and are not read again here: non-temporal, like the generated kernels' outputs
+            __builtin_nontemporal_store(v.x, &dst[2 * i]);
+            __builtin_nontemporal_store(v.y, &dst[2 * i + 1]);
         }
         if ((ndbl & 1) && threadIdx.x == 0) dst[ndbl - 1] = tile[((ndbl - 1) / MM) * LS + ((ndbl - 1) % MM)];
     }
@@ -183,24 +208,39 @@ __global__ __launch_bounds__(kLanes) void scatterKernel(double *__restrict__ Aou
     if (i < range_size) Aout[i] = Ain[M[i]];
 }
 
-// Four consecutive range entries per lane: one 16-byte load of map entries, four gathers in flight, two 16-byte
-// stores.  Needs Aout and M aligned to 16 bytes; the entries past the last multiple of four go to the last lane.
-__global__ __launch_bounds__(kLanes) void scatterKernel4(double *__restrict__ Aout, const double *__restrict__ Ain,
+// Two consecutive range entries per access and kScatterPairs accesses per lane, adjacent lanes on adjacent pairs:
+// every load of map entries (8 bytes per lane) and every store (16 bytes per lane) of a wavefront covers whole
+// lines, and a lane has 2 * kScatterPairs gathers in flight.  The result streams out with non-temporal stores
+// (they only pay off when one store instruction fills its lines: with four consecutive entries per lane, i.e. two
+// half-covering instructions per line, they were 1.5x slower than ordinary stores).  Needs Aout aligned to 16 and
+// M to 8 bytes; an odd last entry goes to the lane after the last pair.
+constexpr int kScatterPairs = 2;
+
+__global__ __launch_bounds__(kLanes) void scatterKernel2(double *__restrict__ Aout, const double *__restrict__ Ain,
                                                          const int *__restrict__ M, int range_size)
 {
-    const int quads = range_size / 4;
-    const int q = xcdContiguousBlock() * kLanes + threadIdx.x;
-    if (q < quads)
+    const int pairs = range_size / 2;
+    const int base = xcdContiguousBlock() * (kLanes * kScatterPairs) + threadIdx.x;
+    int2 m[kScatterPairs];
+#pragma unroll
+    for (int u = 0; u < kScatterPairs; ++u)
     {
-        const int4 m = reinterpret_cast<const int4 *>(M)[q];
-        const double a0 = Ain[m.x], a1 = Ain[m.y], a2 = Ain[m.z], a3 = Ain[m.w];
-        double2 *dst = reinterpret_cast<double2 *>(Aout) + 2 * static_cast<size_t>(q);
-        dst[0] = make_double2(a0, a1);
-        dst[1] = make_double2(a2, a3);
+        const int p = base + u * kLanes;
+        m[u] = p < pairs ? reinterpret_cast<const int2 *>(M)[p] : make_int2(0, 0);
     }
-    if (q == quads - 1)
+    double a[kScatterPairs][2];
+#pragma unroll
+    for (int u = 0; u < kScatterPairs; ++u)
     {
-        for (int i = quads * 4; i < range_size; ++i) Aout[i] = Ain[M[i]];
+        a[u][0] = Ain[m[u].x];
+        a[u][1] = Ain[m[u].y];
+    }
+#pragma unroll
+    for (int u = 0; u < kScatterPairs; ++u)
+    {
+        const int p = base + u * kLanes;
+        if (p < pairs) __builtin_nontemporal_store(Double2{a[u][0], a[u][1]}, reinterpret_cast<Double2 *>(Aout) + p);
+        if (p == pairs && (range_size & 1)) Aout[range_size - 1] = Ain[M[range_size - 1]];
     }
 }
 
@@ -262,7 +302,7 @@ __global__ __launch_bounds__(kLanes) void sumGatherKernel(double *__restrict__ A
     for (int r = 0; r < kGatherRows; ++r)
     {
         const int d = d0 + r * kLanes + threadIdx.x;
-        if (d < domain_size) Aout[d] = sum[r];
+        if (d < domain_size) __builtin_nontemporal_store(sum[r], &Aout[d]);
     }
 }
 
@@ -317,13 +357,13 @@ namespace hip
 
 void FillDouble(double *d, double value, size_t n)
 {
-    hipLaunchKernelGGL(fillKernel, dim3(gridFor(n)), dim3(kLanes), 0, stream(), d, value, n);
+    hipLaunchKernelGGL(fillKernel, dim3(gridFor(n / 2 + 1)), dim3(kLanes), 0, stream(), d, value, n);
     ACRO_HIP_CHECK(hipGetLastError());
 }
 
 void ScaleDouble(double *d, double factor, size_t n)
 {
-    hipLaunchKernelGGL(scaleKernel, dim3(gridFor(n)), dim3(kLanes), 0, stream(), d, factor, n);
+    hipLaunchKernelGGL(scaleKernel, dim3(gridFor(n / 2 + 1)), dim3(kLanes), 0, stream(), d, factor, n);
     ACRO_HIP_CHECK(hipGetLastError());
 }
 
@@ -351,10 +391,11 @@ void HipGPUOps::FlatIndexedScatter(Tensor &Aout, Tensor &Ain, IndexMapping &M)
 {
     const int n = M.GetRangeSize();
     const bool aligned = reinterpret_cast<uintptr_t>(Aout.GetDeviceData()) % 16 == 0 &&
-                         reinterpret_cast<uintptr_t>(M.GetMap().GetDeviceData()) % 16 == 0;
-    if (aligned && n >= 4)
-        hipLaunchKernelGGL(scatterKernel4, dim3(gridFor(n / 4)), dim3(kLanes), 0, stream(), Aout.GetDeviceData(),
-                           Ain.GetDeviceData(), M.GetMap().GetDeviceData(), n);
+                         reinterpret_cast<uintptr_t>(M.GetMap().GetDeviceData()) % 8 == 0;
+    if (aligned)
+        hipLaunchKernelGGL(scatterKernel2, dim3(gridFor((static_cast<size_t>(n) / 2 + 1 + kScatterPairs - 1) / kScatterPairs)),
+                           dim3(kLanes), 0, stream(), Aout.GetDeviceData(), Ain.GetDeviceData(),
+                           M.GetMap().GetDeviceData(), n);
     else
         hipLaunchKernelGGL(scatterKernel, dim3(gridFor(n)), dim3(kLanes), 0, stream(), Aout.GetDeviceData(),
                            Ain.GetDeviceData(), M.GetMap().GetDeviceData(), n);

@@ -82,3 +82,22 @@ def test_large_fill_and_scale(at):
     T.Mult(-2.0)
     T.MoveFromGPU()
     assert np.all(T.data == -3.0)
+
+
+@pytest.mark.parametrize("rows,cols", [(4, 1), (3, 7), (5, 8), (3, 1025)])
+def test_fill_and_scale_of_slices_touch_exactly_their_entries(at, rows, cols):
+    # slices start at any multiple of 8 bytes and have odd or even lengths; device fill and scale move 16 bytes per
+    # lane and must neither miss the unaligned first / odd last entry nor touch a neighbour
+    T = to_tensor(at, np.arange(rows * cols, dtype=np.float64).reshape(rows, cols))
+    T.MoveToGPU()
+    expected = T.data.copy()
+    for r in range(rows):
+        S = at.SliceTensor(T, r)
+        if r % 2 == 0:
+            S.Mult(-3.0)
+            expected[r] *= -3.0
+        else:
+            S.Set(0.25 + r)
+            expected[r] = 0.25 + r
+    T.MoveFromGPU()
+    assert np.array_equal(T.data, expected)
