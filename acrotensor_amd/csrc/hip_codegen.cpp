@@ -496,18 +496,18 @@ class Generator
             UVarInfo info;
             info.isVirtual = true;
             info.name = "_F" + str(static_cast<long>(t + 1));
-            VarRef out;
-            out.uvar = static_cast<int>(uvars.size());
-            out.idx = st.result;
-            for (int id : st.result) out.ext.push_back(extent[id]);
-            out.stride.assign(out.idx.size(), 1);
-            for (int d = static_cast<int>(out.idx.size()) - 2; d >= 0; --d) out.stride[d] = out.stride[d + 1] * out.ext[d + 1];
-            for (int x : out.ext) out.size *= x;
+            VarRef res;
+            res.uvar = static_cast<int>(uvars.size());
+            res.idx = st.result;
+            for (int id : st.result) res.ext.push_back(extent[id]);
+            res.stride.assign(res.idx.size(), 1);
+            for (int d = static_cast<int>(res.idx.size()) - 2; d >= 0; --d) res.stride[d] = res.stride[d + 1] * res.ext[d + 1];
+            for (int x : res.ext) res.size *= x;
             uvars.push_back(info);
 
             Sub s;
             s.op = '=';
-            s.out = out;
+            s.out = res;
             s.outIdx = st.result;
             s.contr = st.summed;
             s.contrCount = product(s.contr, extent);
@@ -519,7 +519,7 @@ class Generator
                 used[o] = true;
             }
             subs.push_back(s);
-            refOf.push_back(out);
+            refOf.push_back(res);
             textOf.push_back(refText(info.name, st.result));
             used.push_back(false);
         }
@@ -1521,12 +1521,12 @@ class Generator
     // served from the tile as well.
     bool StoreIsDead(int k) const
     {
-        const int out = subs[k].out.uvar;
-        const Storage &st = StoreOf(out);
+        const int outVar = subs[k].out.uvar;
+        const Storage &st = StoreOf(outVar);
         if (subs[k].out.repeated) return false;
         const bool nextTakesRegisters = k + 1 < static_cast<int>(subs.size()) && subs[k + 1].forwardedOld;
         if (!st.inLds && !nextTakesRegisters) return false;
-        const int si = uvars[out].storage;
+        const int si = uvars[outVar].storage;
         for (int j = k + 1; j < static_cast<int>(subs.size()); ++j)
         {
             const Sub &s = subs[j];
@@ -1535,8 +1535,8 @@ class Generator
                 if (uvars[s.in[v].uvar].storage != si) continue;
                 if (!FromRegisters(j, static_cast<int>(v)) && !(st.inLds && readCovered[j][v])) return false;
             }
-            if (uvars[s.out.uvar].storage == si && s.out.uvar != out) return false;  // keep it simple: same view only
-            if (s.out.uvar == out) return s.op == '=' || s.forwardedOld || (st.inLds && oldCovered[j]);
+            if (uvars[s.out.uvar].storage == si && s.out.uvar != outVar) return false;  // keep it simple: same view only
+            if (s.out.uvar == outVar) return s.op == '=' || s.forwardedOld || (st.inLds && oldCovered[j]);
         }
         return false;
     }
