@@ -298,7 +298,7 @@ class Generator
             E = extent[batch];
         }
 
-        if (factorise && K == 1 && envInt("ACRO_HIP_FACTORISE") >= 0) FactoriseSingleKernel();
+        if (factorise && envInt("ACRO_HIP_FACTORISE") >= 0) FactoriseKernels();
 
         // Unique-variable facts, in program order (a kernel reads its inputs before it writes its output).
         for (int ki = 0; ki < static_cast<int>(subs.size()); ++ki)
@@ -344,7 +344,7 @@ class Generator
     }
 
     // --------------------------------------------------------------------------- contraction ordering
-    // A single kernel with three or more operands, written as one big sum
+    // A kernel with three or more operands, written as one big sum
     // ("M_e_i_j_k_l_m_n = B_q_i B_q_l B_r_j B_r_m B_s_k B_s_n W_e_q_r_s": 64 terms of 7 factors for each of 729
     // outputs), is evaluated as a chain of smaller contractions when that takes far fewer multiply-adds: a
     // contraction index is summed as soon as every operand carrying it has been multiplied in, and the partial
@@ -449,15 +449,29 @@ class Generator
         }
     }
 
-    void FactoriseSingleKernel()
+    // Every kernel of the group that qualifies is replaced by its steps (a kernel of a multi-kernel launch just as
+    // a kernel launched alone).
+    void FactoriseKernels()
     {
-        const Sub orig = subs[0];
+        std::vector<Sub> expanded;
+        int counter = 0;
+        for (size_t ki = 0; ki < subs.size(); ++ki)
+        {
+            if (!FactoriseKernel(static_cast<int>(ki), subs[ki], subs.size() == 1, expanded, counter)) expanded.push_back(subs[ki]);
+        }
+        subs.swap(expanded);
+    }
+
+    // Appends the steps of kernel ki to `result` and returns true, or returns false when the kernel stays as written.
+    bool FactoriseKernel(int ki, const Sub &orig, bool alone, std::vector<Sub> &result, int &counter)
+    {
         const int nin = static_cast<int>(orig.in.size());
-        if (batch < 0 || nin < 3 || orig.contr.empty() || !opt.noalias || orig.out.repeated) return;
-        if (orig.contrCount >= kReductionMinContraction && product(orig.outIdx, extent) <= kReductionMaxOutputs) return;
+        if (batch < 0 || nin < 3 || orig.contr.empty() || !opt.noalias || orig.out.repeated) return false;
+        if (alone && orig.contrCount >= kReductionMinContraction && product(orig.outIdx, extent) <= kReductionMaxOutputs)
+            return false;  // the reduction schedule serves it
         for (const auto &r : orig.in)
         {
-            if (r.repeated || r.uvar == orig.out.uvar) return;
+            if (r.repeated || r.uvar == orig.out.uvar) return false;
         }
         std::vector<int> live;
         std::vector<std::vector<int>> idxOf;
@@ -476,10 +490,10 @@ class Generator
         FactoriseSearch(orig, live, idxOf, remaining, 0.0, steps, best, bestSlowest, bestSteps, visits);
         // ACRO_HIP_FACTORISE=2 (tests): reorder whenever any chain is cheaper at all, however small the kernel.
         const bool eager = envInt("ACRO_HIP_FACTORISE") >= 2;
-        if (bestSteps.empty()) return;
-        if (!eager && (asWritten < kFactoriseMinWork || best * kFactoriseMinGain > asWritten)) return;
+        if (bestSteps.empty()) return false;
+        if (!eager && (asWritten < kFactoriseMinWork || best * kFactoriseMinGain > asWritten)) return false;
 
-        DimensionedKernel *kernel = mk.Kernels[0];
+        DimensionedKernel *kernel = mk.Kernels[ki];
         auto refText = [&](const std::string &name, const std::vector<int> &ids) {
             std::string t = name;
             for (int id : ids) t += "_" + idxName[id];
@@ -489,13 +503,12 @@ class Generator
         std::vector<std::string> textOf;
         for (int v = 0; v < nin; ++v) textOf.push_back(refText(kernel->GetVarName(v), orig.in[v].idx));
         std::vector<bool> used(nin, false);
-        subs.clear();
         for (size_t t = 0; t < bestSteps.size(); ++t)
         {
             const FactorStep &st = bestSteps[t];
             UVarInfo info;
             info.isVirtual = true;
-            info.name = "_F" + str(static_cast<long>(t + 1));
+            info.name = "_F" + str(static_cast<long>(++counter));
             VarRef res;
             res.uvar = static_cast<int>(uvars.size());
             res.idx = st.result;
@@ -518,7 +531,7 @@ class Generator
                 s.text += " " + textOf[o];
                 used[o] = true;
             }
-            subs.push_back(s);
+            result.push_back(s);
             refOf.push_back(res);
             textOf.push_back(refText(info.name, st.result));
             used.push_back(false);
@@ -541,8 +554,9 @@ class Generator
         }
         fin.contrCount = product(fin.contr, extent);
         fin.text += "   (steps of: " + orig.text + ")";
-        subs.push_back(fin);
+        result.push_back(fin);
         factorised = true;
+        return true;
     }
 
     void BuildStorages()

@@ -23,7 +23,7 @@
 //   ACRO_HIP_LDS_PAD=1|2        pad LDS tile strides against bank conflicts (2: even if a resident workgroup is lost)
 //   ACRO_HIP_PACK=1             pick batch / workgroup size for wavefront utilisation
 //   ACRO_HIP_PERSIST=<n>        persistent grid of n workgroups per CU looping over the batch
-//   ACRO_HIP_FACTORISE=-1|2     -1: evaluate multi-operand single kernels as written instead of as a chain of steps;
+//   ACRO_HIP_FACTORISE=-1|2     -1: evaluate multi-operand kernels as written instead of as a chain of steps;
 //                               2: reorder whenever a chain is cheaper at all (default: only large kernels, 4x gain)
 //   ACRO_HIP_ONE_PASS=1         split contractions: the workgroup that finishes last adds the per-workgroup partials
 //                               instead of a second kernel (measured 3x slower: device-scope fences flush the L2)

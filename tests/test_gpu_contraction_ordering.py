@@ -145,3 +145,31 @@ def test_random_kernels_reordered_whenever_possible(at, engine, checker, monkeyp
     if op == "-=":
         expected = init - (expected - init)
     assert rel_err(out.data, expected) <= TOL
+
+
+@pytest.mark.parametrize("transient", [False, True])
+def test_kernel_inside_a_multi_kernel_launch_is_reordered_too(at, engine, checker, transient):
+    # assemble the element matrices and apply them in one launch: the 7-operand assembly kernel runs as three steps,
+    # its result M feeds the next kernel from LDS (and is not stored at all when marked transient)
+    rng = np.random.default_rng(12)
+    E = 29
+    B, W, X = rng.uniform(-1, 1, (4, 3)), rng.uniform(0.5, 1.5, (E, 4, 4, 4)), rng.uniform(-1, 1, (E, 3, 3, 3))
+    tB, tW, tX = to_tensor(at, B), to_tensor(at, W), to_tensor(at, X)
+    M, Y = at.Tensor(E, 3, 3, 3, 3, 3, 3), at.Tensor(E, 3, 3, 3)
+    M.SetTransient(transient)
+    engine.BeginMultiKernelLaunch()
+    engine("M_e_i_j_k_l_m_n = B_q_i B_q_l B_r_j B_r_m B_s_k B_s_n W_e_q_r_s", M, tB, tB, tB, tB, tB, tB, tW)
+    engine("Y_e_i_j_k = M_e_i_j_k_l_m_n X_e_l_m_n", Y, M, tX)
+    engine.EndMultiKernelLaunch()
+    src = engine.GetLastImplementation()
+    assert "_F1" in src and "_F2" in src and src.count("__global__") == 1
+    assert ("M->lds\n" in src) == transient
+    expM = np.zeros((E, 3, 3, 3, 3, 3, 3))
+    checker.contract("M_e_i_j_k_l_m_n = B_q_i B_q_l B_r_j B_r_m B_s_k B_s_n W_e_q_r_s", expM, B, B, B, B, B, B, W)
+    expY = np.zeros((E, 3, 3, 3))
+    checker.contract("Y_e_i_j_k = M_e_i_j_k_l_m_n X_e_l_m_n", expY, expM, X)
+    Y.MoveFromGPU()
+    assert rel_err(Y.data, expY) <= TOL
+    if not transient:
+        M.MoveFromGPU()
+        assert rel_err(M.data, expM) <= TOL

@@ -110,7 +110,19 @@ def random_chain(rng):
 
 @pytest.mark.parametrize("seed", range(40))
 def test_random_chains(at, engine, checker, seed):
-    rng = np.random.default_rng(5000 + seed)
+    run_random_chain(at, engine, checker, 5000 + seed)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_chains_with_every_possible_kernel_reordered(at, engine, checker, monkeypatch, seed):
+    # kernels of the chain with three or more operands are split into steps whenever that is cheaper at all
+    # (thresholds off): generator-owned partial results next to the user's intermediates in one fused launch
+    monkeypatch.setenv("ACRO_HIP_FACTORISE", "2")
+    run_random_chain(at, engine, checker, 7000 + seed)
+
+
+def run_random_chain(at, engine, checker, seed):
+    rng = np.random.default_rng(seed)
     strings, shapes, produced = random_chain(rng)
     for s, _, _ in strings:
         print(s, flush=True)
