@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <iostream>
 #include <numeric>
+#include <vector>
 
 #include "HipRuntime.hpp"
 #include "IndexMapping.hpp"
@@ -404,12 +405,10 @@ void IndexMapping::ComputeInverse()
     int *off = InvMOff.GetData();
     const int *map = M.GetData();
 
-    // Range entries ordered by the domain entry they map to; ties keep range order (stable), which makes the
-    // compressed-row sum visit contributions in the same order as a sequential scatter-add over the range.
-    std::iota(inv, inv + RangeSize, 0);
-    std::stable_sort(inv, inv + RangeSize, [map](int a, int b) { return map[a] < map[b]; });
-
-    // Row d of the inverse holds the range entries whose image is d: count, then prefix-sum.
+    // Row d of the inverse holds the range entries whose image is d, in increasing range order, which makes the
+    // compressed-row sum visit contributions in the same order as a sequential scatter-add over the range.  The
+    // reference sorts the range stably by image (tensor/IndexMapping.cpp:31-33); counting rows, prefix-summing and
+    // filling in range order gives the same rows in linear time (16.8 M entries: seconds -> tens of milliseconds).
     std::fill(off, off + DomainSize + 1, 0);
     for (int i = 0; i < RangeSize; ++i)
     {
@@ -417,6 +416,8 @@ void IndexMapping::ComputeInverse()
         ++off[map[i] + 1];
     }
     for (int d = 0; d < DomainSize; ++d) off[d + 1] += off[d];
+    std::vector<int> next(off, off + DomainSize);
+    for (int i = 0; i < RangeSize; ++i) inv[next[map[i]]++] = i;
 
     InverseComputed = true;
     if (OnGPU)
