@@ -30,9 +30,9 @@ SIGNATURES = {
     "acro_tensor_create_slice": (ctypes.c_int, [handle, ctypes.c_int, c_int_p, handle_p]),
     "acro_tensor_destroy": (ctypes.c_int, [handle]),
     "acro_tensor_rank": (ctypes.c_int, [handle]),
-    "acro_tensor_size": (ctypes.c_int, [handle]),
+    "acro_tensor_size": (ctypes.c_longlong, [handle]),
     "acro_tensor_dim": (ctypes.c_int, [handle, ctypes.c_int]),
-    "acro_tensor_stride": (ctypes.c_int, [handle, ctypes.c_int]),
+    "acro_tensor_stride": (ctypes.c_longlong, [handle, ctypes.c_int]),
     "acro_tensor_data": (ctypes.c_void_p, [handle]),
     "acro_tensor_device_data": (ctypes.c_void_p, [handle]),
     "acro_tensor_reshape": (ctypes.c_int, [handle, ctypes.c_int, c_int_p]),

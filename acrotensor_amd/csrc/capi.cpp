@@ -207,9 +207,9 @@ int acro_tensor_destroy(acro_tensor *t)
 }
 
 int acro_tensor_rank(const acro_tensor *t) { return t ? t->t->GetRank() : -1; }
-int acro_tensor_size(const acro_tensor *t) { return t ? t->t->GetSize() : -1; }
+long long acro_tensor_size(const acro_tensor *t) { return t ? static_cast<long long>(t->t->GetSize()) : -1; }
 int acro_tensor_dim(const acro_tensor *t, int d) { return (t && d >= 0 && d < t->t->GetRank()) ? t->t->GetDim(d) : -1; }
-int acro_tensor_stride(const acro_tensor *t, int d)
+long long acro_tensor_stride(const acro_tensor *t, int d)
 {
     return (t && d >= 0 && d < t->t->GetRank()) ? t->t->GetStride(d) : -1;
 }

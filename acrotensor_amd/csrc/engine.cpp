@@ -301,8 +301,8 @@ void TensorEngine::BatchMatrixInvDet(Tensor &Ainv, Tensor &Adet, Tensor &A)
 void TensorEngine::FlatIndexedScatter(Tensor &Aout, Tensor &Ain, IndexMapping &M)
 {
     ACROBATIC_ASSERT(Ops != nullptr, "The executor type of this engine provides no non-contraction ops.");
-    ACROBATIC_ASSERT(Aout.GetSize() == M.GetRangeSize(), "IndexMapping RangeSize does not match the output Tensor size.");
-    ACROBATIC_ASSERT(Ain.GetSize() == M.GetDomainSize(), "IndexMapping DomainSize does not match the input Tensor size.");
+    ACROBATIC_ASSERT(Aout.GetSize() == static_cast<size_t>(M.GetRangeSize()), "IndexMapping RangeSize does not match the output Tensor size.");
+    ACROBATIC_ASSERT(Ain.GetSize() == static_cast<size_t>(M.GetDomainSize()), "IndexMapping DomainSize does not match the input Tensor size.");
     SwitchToComputeLocation(Aout);
     MoveToComputeLocation(Ain);
     MoveToComputeLocation(M);
@@ -312,8 +312,8 @@ void TensorEngine::FlatIndexedScatter(Tensor &Aout, Tensor &Ain, IndexMapping &M
 void TensorEngine::FlatIndexedSumGather(Tensor &Aout, Tensor &Ain, IndexMapping &M)
 {
     ACROBATIC_ASSERT(Ops != nullptr, "The executor type of this engine provides no non-contraction ops.");
-    ACROBATIC_ASSERT(Aout.GetSize() == M.GetDomainSize(), "IndexMapping DomainSize does not match the output Tensor size.");
-    ACROBATIC_ASSERT(Ain.GetSize() == M.GetRangeSize(), "IndexMapping RangeSize does not match the input Tensor size.");
+    ACROBATIC_ASSERT(Aout.GetSize() == static_cast<size_t>(M.GetDomainSize()), "IndexMapping DomainSize does not match the output Tensor size.");
+    ACROBATIC_ASSERT(Ain.GetSize() == static_cast<size_t>(M.GetRangeSize()), "IndexMapping RangeSize does not match the input Tensor size.");
     if (!M.IsInverseComputed()) M.ComputeInverse();
     SwitchToComputeLocation(Aout);
     MoveToComputeLocation(Ain);

@@ -27,8 +27,8 @@ struct VarRef
     int uvar = -1;
     std::vector<int> idx;     // loop id of every dimension
     std::vector<int> ext;     // extent of every dimension
-    std::vector<int> stride;  // row-major element stride of every dimension
-    int size = 1;
+    std::vector<long> stride;  // row-major element stride of every dimension
+    long size = 1;
     bool repeated = false;    // some index occurs in two dimensions
 };
 
@@ -56,7 +56,7 @@ struct UVarInfo
 {
     std::string name;
     std::vector<int> dims;
-    int size = 0;
+    long size = 0;
     bool written = false;
     int firstWrite = -1;
     int lastUse = -1;
@@ -234,6 +234,11 @@ class Generator
     int ldsDoubles = 0;
     bool extentsConsistent = true;
     bool batchUniform = false;  // one batch entry per workgroup: the batch index is a scalar
+    bool wide = false;          // 64-bit device-memory offsets
+
+    // Literal of a device-memory stride or offset, and the type such offsets are computed in.
+    std::string Lit(long v) const { return std::to_string(v) + (wide ? "L" : ""); }
+    const char *OffsetType() const { return wide ? "long" : "int"; }
 
     // ------------------------------------------------------------------------------------------ model
     // Operand numbering: unique variables by name, or one operand per occurrence in positional mode.
@@ -341,6 +346,14 @@ class Generator
         }
         BuildStorages();
         AnalyseCoverage();
+        // Element offsets into device memory are 32-bit unless some tensor of the group reaches 2^31 entries
+        // (16 GiB of doubles; the device holds 288 GB): then every device-memory offset is computed in 64 bits.
+        for (const auto &st : stores)
+        {
+            long entries = 1;
+            for (int d : st.dims) entries *= d;
+            if (entries >= (1L << 31) - 1) wide = true;
+        }
     }
 
     // --------------------------------------------------------------------------- contraction ordering
@@ -1332,18 +1345,18 @@ class Generator
         if (lds)
             add(str(st.ldsOffset + LdsViewOffset(r.uvar)) + " + b * " + str(st.tileSize));
         else if (u.viewOffset != 0)
-            add(str(u.viewOffset));
+            add(Lit(u.viewOffset));
         for (size_t d = 0; d < r.idx.size(); ++d)
         {
             const int id = r.idx[d];
             const long stride = lds ? LdsStride(r.uvar, d) : r.stride[d];
             if (id == batch)
             {
-                if (!lds) add("e * " + str(stride));
+                if (!lds) add("e * " + Lit(stride));
             }
             else if (has(s.lane, id))
             {
-                add(IdxVar(id) + " * " + str(stride));
+                add(IdxVar(id) + " * " + (lds ? str(stride) : Lit(stride)));
             }
         }
         return expr.empty() ? "0" : expr;
@@ -1385,7 +1398,7 @@ class Generator
         std::string base;
         for (size_t d = 0; d < r.idx.size(); ++d)
         {
-            if (r.idx[d] == batch) base += "e0 * " + str(r.stride[d]) + " + ";
+            if (r.idx[d] == batch) base += "e0 * " + Lit(r.stride[d]) + " + ";
         }
         return base;
     }
@@ -1426,7 +1439,7 @@ class Generator
         }
         if (src == kFromConstant)
         {
-            return ConstPtrName(r.uvar) + "[" + ScalarBase(r) + str(uvars[r.uvar].viewOffset + LiteralOffset(r, s, false, value)) + "]";
+            return ConstPtrName(r.uvar) + "[" + ScalarBase(r) + Lit(uvars[r.uvar].viewOffset + LiteralOffset(r, s, false, value)) + "]";
         }
         const bool lds = (src == kFromLds);
         const long off = LiteralOffset(r, s, lds, value);
@@ -1441,7 +1454,7 @@ class Generator
         }
         else
         {
-            const std::string rhs = PtrName(r.uvar) + "[" + base + " + " + str(off) + "]";
+            const std::string rhs = PtrName(r.uvar) + "[" + base + " + " + Lit(off) + "]";
             body.loads.push_back("const double " + name + " = " + rhs + ";");
             if (Prefetchable(k, v)) body.globalLoads.push_back(std::make_pair(key, rhs));
         }
@@ -1519,10 +1532,10 @@ class Generator
         {
             const Source src = SourceOf(k, static_cast<int>(v));
             if (src == kFromRegisters || src == kFromConstant) continue;
-            body.bases.push_back("const int o_k" + str(k) + "v" + str(v) + " = " +
-                                 RuntimeOffset(s.in[v], s, src == kFromLds) + ";");
+            body.bases.push_back(std::string("const ") + (src == kFromLds ? "int" : OffsetType()) + " o_k" + str(k) + "v" +
+                                 str(v) + " = " + RuntimeOffset(s.in[v], s, src == kFromLds) + ";");
         }
-        body.bases.push_back("const int o_k" + str(k) + "g = " + RuntimeOffset(s.out, s, false) + ";");
+        body.bases.push_back(std::string("const ") + OffsetType() + " o_k" + str(k) + "g = " + RuntimeOffset(s.out, s, false) + ";");
         if (StoreOf(s.out.uvar).inLds)
             body.bases.push_back("const int o_k" + str(k) + "l = " + RuntimeOffset(s.out, s, true) + ";");
     }
@@ -1707,7 +1720,7 @@ class Generator
 
             const long goff = LiteralOffset(s.out, s, false, value);
             const long loff = StoreOf(s.out.uvar).inLds ? LiteralOffset(s.out, s, true, value) : 0;
-            const std::string gaddr = PtrName(s.out.uvar) + "[o_k" + str(k) + "g + " + str(goff) + "]";
+            const std::string gaddr = PtrName(s.out.uvar) + "[o_k" + str(k) + "g + " + Lit(goff) + "]";
             const std::string laddr = "lds[o_k" + str(k) + "l + " + str(loff) + "]";
             const std::string name = "r" + str(k) + "_" + str(t);
             if (s.op == '=')
@@ -1763,12 +1776,12 @@ class Generator
                 const int id = r.idx[d];
                 if (!has(s.contr, id)) continue;
                 const long st = lds ? LdsStride(r.uvar, d) : r.stride[d];
-                off += (off.empty() ? "" : " + ") + IdxVar(id) + " * " + str(st);
+                off += (off.empty() ? "" : " + ") + IdxVar(id) + " * " + (lds ? str(st) : Lit(st));
             }
             if (off.empty()) off = "0";
             std::string opnd;
             if (src == kFromConstant)
-                opnd = ConstPtrName(r.uvar) + "[" + ScalarBase(r) + str(uvars[r.uvar].viewOffset) + " + " + off + "]";
+                opnd = ConstPtrName(r.uvar) + "[" + ScalarBase(r) + Lit(uvars[r.uvar].viewOffset) + " + " + off + "]";
             else if (lds)
                 opnd = "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
             else
@@ -1814,9 +1827,9 @@ class Generator
     // Expression for the element offset of an occurrence given variables named i_<index> for every loop index.
     std::string FullOffset(const VarRef &r) const
     {
-        std::string expr = uvars[r.uvar].viewOffset != 0 ? str(uvars[r.uvar].viewOffset) : std::string();
+        std::string expr = uvars[r.uvar].viewOffset != 0 ? Lit(uvars[r.uvar].viewOffset) : std::string();
         for (size_t d = 0; d < r.idx.size(); ++d)
-            expr += (expr.empty() ? "" : " + ") + IdxVar(r.idx[d]) + " * " + str(r.stride[d]);
+            expr += (expr.empty() ? "" : " + ") + IdxVar(r.idx[d]) + " * " + Lit(r.stride[d]);
         return expr.empty() ? "0" : expr;
     }
 

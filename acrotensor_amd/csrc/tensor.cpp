@@ -45,7 +45,6 @@ void Tensor::Init(const std::vector<int> &dims, double *hdata, double *ddata, bo
     Dims = dims;
     UpdateStrides();
     ComputeSize();
-    ACROBATIC_ASSERT(Size <= static_cast<size_t>(0x7fffffff), "Tensor has more entries than an int can index.");
 
     OwnsData = (hdata == nullptr);
     Data = OwnsData ? new double[Size] : hdata;
@@ -86,14 +85,14 @@ void Tensor::ComputeSize()
     for (int d : Dims) Size *= static_cast<size_t>(d);
 }
 
-int Tensor::RawIndexOf(const int *idx, int n) const
+size_t Tensor::RawIndexOf(const int *idx, int n) const
 {
-    int raw = 0;
-    for (int d = 0; d < n; ++d) raw += idx[d] * Strides[d];
+    size_t raw = 0;
+    for (int d = 0; d < n; ++d) raw += static_cast<size_t>(idx[d]) * static_cast<size_t>(Strides[d]);
     return raw;
 }
 
-int Tensor::GetRawIndex(const std::vector<int> &indices) const
+size_t Tensor::GetRawIndex(const std::vector<int> &indices) const
 {
     return RawIndexOf(indices.data(), static_cast<int>(indices.size()));
 }
@@ -191,7 +190,7 @@ void Tensor::Print()
     std::cout << "Dims:  ";
     for (int d : Dims) std::cout << d << "  ";
     std::cout << "\nStrides:  ";
-    for (int s : Strides) std::cout << s << "  ";
+    for (long s : Strides) std::cout << s << "  ";
     std::cout << "\n";
     const double *p = GetData();
     for (size_t i = 0; i < Size; ++i) std::cout << p[i] << "\n";
@@ -210,7 +209,7 @@ void SliceTensor::SliceInit(Tensor &T, const std::vector<int> &sind)
         ACROBATIC_ASSERT(sind[d] >= 0 && sind[d] < T.GetDim(static_cast<int>(d)), "Slice index out of range.");
     }
     FullT = &T;
-    Offset = static_cast<size_t>(T.GetRawIndex(sind));
+    Offset = T.GetRawIndex(sind);
 
     std::vector<int> dims(T.GetDims().begin() + sind.size(), T.GetDims().end());
     double *hdata = T.GetData();

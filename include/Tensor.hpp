@@ -76,13 +76,13 @@ class Tensor
     }
 
     // Flat access to the host buffer
-    double &operator[](int raw_index) { return Data[raw_index]; }
-    const double &operator[](int raw_index) const { return Data[raw_index]; }
+    double &operator[](size_t raw_index) { return Data[raw_index]; }
+    const double &operator[](size_t raw_index) const { return Data[raw_index]; }
 
     // Row-major flat index of a multi-index ("most significant index on the left")
-    int GetRawIndex(const std::vector<int> &indices) const;
+    size_t GetRawIndex(const std::vector<int> &indices) const;
     template <typename... I>
-    int GetRawIndex(int i0, I... rest) const
+    size_t GetRawIndex(int i0, I... rest) const
     {
         const int idx[] = {i0, static_cast<int>(rest)...};
         return RawIndexOf(idx, 1 + static_cast<int>(sizeof...(rest)));
@@ -104,10 +104,12 @@ class Tensor
     }
 
     int GetRank() const { return static_cast<int>(Dims.size()); }
-    int GetSize() const { return static_cast<int>(Size); }
+    // Number of entries.  The reference returns int (tensor/Tensor.hpp:60); a tensor here may hold more than 2^31
+    // entries (16 GiB of doubles), so the count is a size_t.
+    size_t GetSize() const { return Size; }
     size_t GetByteSize() const { return Size * sizeof(double); }
     int GetDim(int d) const { return Dims[d]; }
-    int GetStride(int d) const { return Strides[d]; }
+    long GetStride(int d) const { return Strides[d]; }   // entries; tensors may exceed 2^31 entries
     const std::vector<int> &GetDims() const { return Dims; }
     virtual double *GetData() const { return Data; }
     virtual double *GetDeviceData() const { return DeviceData; }
@@ -140,10 +142,10 @@ class Tensor
   protected:
     void UpdateStrides();
     void ComputeSize();
-    int RawIndexOf(const int *idx, int n) const;
+    size_t RawIndexOf(const int *idx, int n) const;
 
     std::vector<int> Dims;
-    std::vector<int> Strides;
+    std::vector<long> Strides;
     size_t Size;
 
     bool Initialized;

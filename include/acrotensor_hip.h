@@ -51,9 +51,9 @@ int acro_tensor_create(int rank, const int *dims, double *hdata, double *ddata, 
 int acro_tensor_create_slice(acro_tensor *parent, int num_indices, const int *indices, acro_tensor **out);
 int acro_tensor_destroy(acro_tensor *t);
 int acro_tensor_rank(const acro_tensor *t);
-int acro_tensor_size(const acro_tensor *t);
+long long acro_tensor_size(const acro_tensor *t);      /* entries; may exceed 2^31 */
 int acro_tensor_dim(const acro_tensor *t, int d);
-int acro_tensor_stride(const acro_tensor *t, int d);
+long long acro_tensor_stride(const acro_tensor *t, int d);
 double *acro_tensor_data(const acro_tensor *t);        /* host buffer   (Tensor::GetData) */
 double *acro_tensor_device_data(const acro_tensor *t); /* device mirror (Tensor::GetDeviceData), may be NULL */
 int acro_tensor_reshape(acro_tensor *t, int rank, const int *dims);

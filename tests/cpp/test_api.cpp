@@ -54,7 +54,7 @@ static void hostTests()
     CHECK_THROWS(Tensor(3, -1));
     Tensor T(2, 3, 4);
     CHECK(T.GetRank() == 3 && T.GetSize() == 24 && T.GetDim(1) == 3 && T.GetStride(0) == 12);
-    for (int i = 0; i < T.GetSize(); ++i) T[i] = i;
+    for (size_t i = 0; i < T.GetSize(); ++i) T[i] = i;
     CHECK(T(1, 2, 3) == 23.0 && T.GetRawIndex(1, 0, 2) == 14);
     T.Reshape(4, 6);
     CHECK(T.GetRank() == 2 && T(3, 5) == 23.0);
@@ -74,7 +74,7 @@ static void hostTests()
 
     std::printf("host: slices\n");
     Tensor P(3, 4, 5);
-    for (int i = 0; i < P.GetSize(); ++i) P[i] = i;
+    for (size_t i = 0; i < P.GetSize(); ++i) P[i] = i;
     SliceTensor S(P, 2), S2(P, 1, 3);
     CHECK(S.GetRank() == 2 && S.GetDim(0) == 4 && S(1, 2) == P(2, 1, 2));
     CHECK(S2.GetRank() == 1 && S2(4) == P(1, 3, 4));
@@ -143,7 +143,7 @@ static void gpuTests()
     {
         const int n = 1000;
         Tensor A(n, 3, 3), B(n), S(3, 3);
-        for (int i = 0; i < A.GetSize(); ++i) A[i] = i % 7;
+        for (size_t i = 0; i < A.GetSize(); ++i) A[i] = i % 7;
         B.Set(1.0);
         A.MapToGPU();
         A.MoveToGPU();
@@ -209,9 +209,9 @@ static void gpuTests()
         const int E = 37;
         Tensor Bm(5, 4), X(E, 4, 4, 4), D(E, 5, 5, 5), Y(E, 4, 4, 4);
         Tensor T1(E, 5, 4, 4), T2(E, 5, 5, 4), T3(E, 5, 5, 5), U(E, 5, 5, 5), V1(E, 4, 5, 5), V2(E, 4, 4, 5);
-        for (int i = 0; i < Bm.GetSize(); ++i) Bm[i] = std::sin(1.0 + i);
-        for (int i = 0; i < X.GetSize(); ++i) X[i] = std::cos(0.1 * i);
-        for (int i = 0; i < D.GetSize(); ++i) D[i] = 1.0 + 0.5 * std::sin(0.3 * i);
+        for (size_t i = 0; i < Bm.GetSize(); ++i) Bm[i] = std::sin(1.0 + i);
+        for (size_t i = 0; i < X.GetSize(); ++i) X[i] = std::cos(0.1 * i);
+        for (size_t i = 0; i < D.GetSize(); ++i) D[i] = 1.0 + 0.5 * std::sin(0.3 * i);
         for (Tensor *t : {&T1, &T2, &T3, &U, &V1, &V2}) t->SetTransient(true);
         TE.BeginMultiKernelLaunch();
         TE("T1_e_q_j_k = B_q_i X_e_i_j_k", T1, Bm, X);
