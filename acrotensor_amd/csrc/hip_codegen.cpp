@@ -1068,7 +1068,22 @@ class Generator
         for (const auto &s : subs) maxLane = std::max(maxLane, s.laneCount);
 
         NT = opt.force_nt > 0 ? opt.force_nt : envInt("ACRO_HIP_NT");
-        if (NT <= 0) NT = maxLane > 128 ? 256 : 128;
+        if (NT <= 0)
+        {
+            NT = maxLane > 128 ? 256 : 128;
+            // A streaming group (one phase, nothing kept in LDS) with more work items per batch entry than that runs
+            // them in one pass of a larger workgroup instead of a loop of passes (geometric-factor setup, 1 000 items:
+            // 475.7 -> 457.0 us with 1 024 lanes).  Groups with barriers measured slower that way (p=7 diffusion
+            // apply: 1 283 against 940 us), so they keep 256.
+            bool streaming = subs.back().phase == 0;
+            for (const auto &st : stores) streaming = streaming && !st.wantLds;
+            // Larger workgroups leave fewer registers per lane (128 at 1 024 lanes, 256 at 512): size them by the
+            // values a lane holds at once.
+            long live = 0;
+            for (const auto &s : subs) live = std::max(live, s.loopMode ? 8 : LoadsPerItem(s, s.tile) + s.tileCount);
+            const long cap = live <= 48 ? 1024 : (live <= 100 ? 512 : 256);
+            if (streaming && maxLane > 256) NT = static_cast<int>(std::min<long>(cap, (maxLane + 63) / 64 * 64));
+        }
         NB = opt.force_nb > 0 ? opt.force_nb : envInt("ACRO_HIP_NB");
         if (NB <= 0)
         {
