@@ -1683,6 +1683,27 @@ class Generator
         return st.inLds && st.liveTo > k;
     }
 
+    // A result that must reach device memory AND stays in LDS for a later kernel is written to device memory from
+    // the LDS tiles, by the whole workgroup, right after the barrier that ends its phase: the tiles of a workgroup's
+    // batch entries are one contiguous range of the tensor, so every store instruction of a wavefront writes 512
+    // contiguous bytes, where the lanes' own stores are pencils (a few doubles per lane at a stride).  Needs the
+    // tensor to carry the batch index first, the kernel to be the only writer of the whole tensor in the group, and
+    // the natural (unpadded) tile layout.
+    bool CopiesOutFromLds(int k) const
+    {
+        if (envInt("ACRO_HIP_LDS_COPY_OUT") < 0 || envInt("ACRO_HIP_PERSIST") > 0 || envInt("ACRO_HIP_LDS_PAD") > 0) return false;
+        const Sub &s = subs[k];
+        if (!NeedsLdsCopy(k) || !StoresToGlobal(k) || s.out.repeated) return false;
+        const UVarInfo &u = uvars[s.out.uvar];
+        const Storage &st = stores[u.storage];
+        if (st.members.size() != 1 || st.batchDim != 0 || !u.fixed.empty() || u.viewOffset != 0) return false;
+        for (size_t j = 0; j < subs.size(); ++j)
+        {
+            if (static_cast<int>(j) != k && uvars[subs[j].out.uvar].storage == u.storage) return false;
+        }
+        return true;
+    }
+
     // Unrolled body of kernel k for one work item.  `forwarded` maps the literal output offsets of the previous
     // kernel to the registers holding them; on return it describes this kernel's outputs.
     void EmitUnrolledBody(int k, std::map<long, std::string> &forwarded, std::vector<std::string> &lines,
@@ -1748,7 +1769,7 @@ class Generator
                 body.compute.push_back("const double " + name + " = " + old + (s.op == '+' ? " + " : " - ") + rhs + ";");
             }
             if (NeedsLdsCopy(k)) body.stores.push_back(laddr + " = " + name + ";");
-            if (StoresToGlobal(k)) body.stores.push_back(GlobalStore(k, gaddr, name));
+            if (StoresToGlobal(k) && !CopiesOutFromLds(k)) body.stores.push_back(GlobalStore(k, gaddr, name));
             produced[goff] = name;
         }
 
@@ -1817,7 +1838,7 @@ class Generator
             lines.push_back(std::string("const double r = ") + (OldValueInLds(k) ? laddr : gaddr) +
                             (s.op == '+' ? " + sum;" : " - sum;"));
         if (NeedsLdsCopy(k)) lines.push_back(laddr + " = r;");
-        if (StoresToGlobal(k)) lines.push_back(GlobalStore(k, gaddr, "r"));
+        if (StoresToGlobal(k) && !CopiesOutFromLds(k)) lines.push_back(GlobalStore(k, gaddr, "r"));
     }
 
     // ------------------------------------------------------------------------------ reduction schedule
@@ -2304,6 +2325,30 @@ class Generator
         for (const Phase &ph : phases)
         {
             if (!first) out << "    __syncthreads();\n";
+            if (!first)
+            {
+                // results of the previous phase that leave through their LDS tiles
+                const int previous = subs[ph.chains[0].first].phase - 1;
+                for (int k = 0; k < K; ++k)
+                {
+                    if (subs[k].phase != previous || !CopiesOutFromLds(k)) continue;
+                    const Storage &st = StoreOf(subs[k].out.uvar);
+                    const bool streams = envInt("ACRO_HIP_NT_STORE") >= 0 && static_cast<long>(ldsDoubles) * 8 <= 20 * 1024;
+                    out << "    {   // " << uvars[subs[k].out.uvar].name << ": LDS tiles -> device memory\n";
+                    if (guardBatch)
+                        out << "        const int count = (" << E << " - e0 < " << NB << " ? " << E << " - e0 : " << NB << ") * "
+                            << st.tileSize << ";\n";
+                    else
+                        out << "        const int count = " << static_cast<long>(NB) * st.tileSize << ";\n";
+                    out << "        double *dst = " << PtrName(subs[k].out.uvar) << " + e0 * " << Lit(st.tileSize) << ";\n";
+                    out << "        for (int i = tid; i < count; i += " << NT << ") ";
+                    if (streams)
+                        out << "__builtin_nontemporal_store(lds[" << st.ldsOffset << " + i], &dst[i]);\n";
+                    else
+                        out << "dst[i] = lds[" << st.ldsOffset << " + i];\n";
+                    out << "    }\n";
+                }
+            }
             first = false;
             const long npass = ph.prefetched ? ph.passes : 1;
             for (long j = 0; j < npass; ++j)

@@ -25,6 +25,8 @@
 //   ACRO_HIP_PERSIST=<n>        persistent grid of n workgroups per CU looping over the batch
 //   ACRO_HIP_FACTORISE=-1|2     -1: evaluate multi-operand kernels as written instead of as a chain of steps;
 //                               2: reorder whenever a chain is cheaper at all (default: only large kernels, 4x gain)
+//   ACRO_HIP_LDS_COPY_OUT=-1    stored results that also live in LDS are written by the lanes that computed them instead
+//                               of by the workgroup from the LDS tiles
 //   ACRO_HIP_ONE_PASS=1         split contractions: the workgroup that finishes last adds the per-workgroup partials
 //                               instead of a second kernel (measured 3x slower: device-scope fences flush the L2)
 #ifndef ACRO_HIP_CODEGEN_HPP

@@ -45,7 +45,9 @@ def test_mass_apply_chain_stores_everything_by_default(TE):
     src = chain_source(TE, workloads.config4(E=64), transient=False)
     for name in ("T1", "T2", "U", "V1", "V2"):
         assert name + "->lds+global" in src
-    assert "T3->global" in src
+        # ... and they reach device memory from their LDS tiles, whole lines at a time, after the phase's barrier
+        assert "// %s: LDS tiles -> device memory" % name in src
+    assert "T3->global" in src and "// T3: LDS tiles" not in src     # applied in registers: the lanes store it
 
 
 def test_mass_assembly_is_evaluated_as_a_chain_of_small_contractions(TE):
