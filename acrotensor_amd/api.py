@@ -284,3 +284,42 @@ class hip_event_timer:
         for ev in (getattr(self, "_a", None), getattr(self, "_b", None)):
             if ev:
                 self._lib.acro_hip_event_destroy(ev)
+
+
+class recorded_launches:
+    """Records everything the library would launch inside the ``with`` block (hipGraph) instead of executing it;
+    ``launch()`` then enqueues the whole sequence with one call::
+
+        apply()                                   # once, eagerly: loads kernels, allocates scratch
+        with at.recorded_launches() as seq:
+            apply()
+        for _ in range(100):
+            seq.launch()
+
+    Tensors must be resident on the device and nothing inside the block may need the host (copies, allocation,
+    synchronisation raise ``AcroError``; the recording is then discarded)."""
+
+    def __init__(self):
+        self._lib = _capi.load()
+        self._g = ctypes.c_void_p()
+
+    def __enter__(self):
+        _check(self._lib.acro_hip_graph_begin_capture())
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        if exc_type is not None:
+            self._lib.acro_hip_graph_abort_capture()
+            return False
+        _check(self._lib.acro_hip_graph_end_capture(ctypes.byref(self._g)))
+        return False
+
+    def launch(self):
+        if not self._g:
+            raise AcroError("nothing has been recorded")
+        _check(self._lib.acro_hip_graph_launch(self._g))
+
+    def __del__(self):
+        g, self._g = getattr(self, "_g", None), None
+        if g:
+            self._lib.acro_hip_graph_destroy(g)

@@ -137,6 +137,7 @@ int acro_hip_event_create(void **event)
 int acro_hip_event_record(void *event)
 {
     return guarded([&] {
+        require(!hip::Capturing(), "events cannot be recorded while a launch sequence is being recorded");
         ACRO_HIP_CHECK(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(hip::Stream())));
     });
 }
@@ -153,6 +154,34 @@ int acro_hip_event_elapsed_ms(void *start, void *stop, float *ms)
 int acro_hip_event_destroy(void *event)
 {
     return guarded([&] { ACRO_HIP_CHECK(hipEventDestroy(static_cast<hipEvent_t>(event))); });
+}
+
+int acro_hip_graph_begin_capture(void)
+{
+    return guarded([] { hip::BeginCapture(); });
+}
+
+int acro_hip_graph_end_capture(acro_hip_graph **out)
+{
+    return guarded([&] {
+        require(out != nullptr, "null graph pointer");
+        *out = reinterpret_cast<acro_hip_graph *>(hip::EndCapture());
+    });
+}
+
+int acro_hip_graph_abort_capture(void)
+{
+    return guarded([] { hip::AbortCapture(); });
+}
+
+int acro_hip_graph_launch(acro_hip_graph *g)
+{
+    return guarded([&] { hip::Launch(reinterpret_cast<hip::Graph *>(g)); });
+}
+
+int acro_hip_graph_destroy(acro_hip_graph *g)
+{
+    return guarded([&] { hip::Destroy(reinterpret_cast<hip::Graph *>(g)); });
 }
 
 // ------------------------------------------------------------------------------------------------ tensor

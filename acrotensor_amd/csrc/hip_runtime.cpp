@@ -41,7 +41,21 @@ hipStream_t g_own_stream = nullptr;
 hipStream_t g_adopted_stream = nullptr;
 bool g_have_info = false;
 DeviceInfo g_info;
+bool g_capturing = false;
+
+void notWhileCapturing(const char *what)
+{
+    ACROBATIC_ASSERT(!g_capturing, std::string(what) +
+                                       " is not possible while a launch sequence is being recorded: make the tensors "
+                                       "resident and run the sequence once before recording it.");
+}
 }  // namespace
+
+struct Graph
+{
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
 
 void *Stream()
 {
@@ -56,17 +70,20 @@ void *Stream()
 
 void SetStream(void *hip_stream)
 {
+    notWhileCapturing("Changing the stream");
     std::lock_guard<std::mutex> guard(g_lock);
     g_adopted_stream = static_cast<hipStream_t>(hip_stream);
 }
 
 void Synchronize()
 {
+    notWhileCapturing("Synchronising");
     ACRO_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(Stream())));
 }
 
 void *Malloc(size_t bytes)
 {
+    notWhileCapturing("Allocating device memory");
     void *p = nullptr;
     ACRO_HIP_CHECK(hipMalloc(&p, bytes));
     return p;
@@ -75,13 +92,15 @@ void *Malloc(size_t bytes)
 void Free(void *dptr)
 {
     if (dptr == nullptr) return;
-    // Work that still uses the buffer may be queued on the stream.
-    ACRO_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(Stream())));
+    // Work that still uses the buffer may be queued on the stream (no wait is possible while a sequence is being
+    // recorded; this is reached from destructors and must not throw then).
+    if (!g_capturing) ACRO_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(Stream())));
     ACRO_HIP_CHECK(hipFree(dptr));
 }
 
 void CopyToDevice(void *dst, const void *src, size_t bytes)
 {
+    notWhileCapturing("Copying to the device");
     hipStream_t s = static_cast<hipStream_t>(Stream());
     ACRO_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s));
     ACRO_HIP_CHECK(hipStreamSynchronize(s));
@@ -89,9 +108,70 @@ void CopyToDevice(void *dst, const void *src, size_t bytes)
 
 void CopyToHost(void *dst, const void *src, size_t bytes)
 {
+    notWhileCapturing("Copying to the host");
     hipStream_t s = static_cast<hipStream_t>(Stream());
     ACRO_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
     ACRO_HIP_CHECK(hipStreamSynchronize(s));
+}
+
+void BeginCapture()
+{
+    ACROBATIC_ASSERT(!g_capturing, "A launch sequence is already being recorded.");
+    hipStream_t s = static_cast<hipStream_t>(Stream());
+    // Relaxed mode: loading the code object of a kernel that is used for the first time inside the recording is
+    // not a stream operation and must not invalidate it.
+    ACRO_HIP_CHECK(hipStreamBeginCapture(s, hipStreamCaptureModeRelaxed));
+    g_capturing = true;
+}
+
+Graph *EndCapture()
+{
+    ACROBATIC_ASSERT(g_capturing, "No launch sequence is being recorded.");
+    g_capturing = false;
+    hipStream_t s = static_cast<hipStream_t>(Stream());
+    Graph *g = new Graph;
+    hipError_t err = hipStreamEndCapture(s, &g->graph);
+    if (err == hipSuccess) err = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    if (err != hipSuccess)
+    {
+        if (g->graph != nullptr) (void)hipGraphDestroy(g->graph);
+        delete g;
+        (void)hipGetLastError();
+        ACRO_HIP_CHECK(err);
+    }
+    return g;
+}
+
+void AbortCapture()
+{
+    if (!g_capturing) return;
+    g_capturing = false;
+    hipGraph_t discarded = nullptr;
+    (void)hipStreamEndCapture(static_cast<hipStream_t>(Stream()), &discarded);
+    if (discarded != nullptr) (void)hipGraphDestroy(discarded);
+    (void)hipGetLastError();
+}
+
+bool Capturing()
+{
+    return g_capturing;
+}
+
+void Launch(Graph *graph)
+{
+    ACROBATIC_ASSERT(graph != nullptr && graph->exec != nullptr, "Not a recorded launch sequence.");
+    notWhileCapturing("Launching a recorded sequence");
+    ACRO_HIP_CHECK(hipGraphLaunch(graph->exec, static_cast<hipStream_t>(Stream())));
+}
+
+void Destroy(Graph *graph)
+{
+    if (graph == nullptr) return;
+    // A launch of the sequence may still be queued.
+    if (!g_capturing) ACRO_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(Stream())));
+    if (graph->exec != nullptr) (void)hipGraphExecDestroy(graph->exec);
+    if (graph->graph != nullptr) (void)hipGraphDestroy(graph->graph);
+    delete graph;
 }
 
 const DeviceInfo &Info()

@@ -34,6 +34,20 @@ void CopyToHost(void *dst, const void *src, size_t bytes);      // returns after
 void FillDouble(double *d, double value, size_t n);             // d[i] = value   (async on Stream())
 void ScaleDouble(double *d, double factor, size_t n);           // d[i] *= factor (async on Stream())
 
+// Recorded launch sequences (hipGraph).  Between BeginCapture() and EndCapture() everything the library enqueues on
+// Stream() (generated kernels, batched operations, fills) is recorded instead of executed; Launch() then enqueues
+// the whole recorded sequence with one call.  The recorded work must not need the host: allocations, host <-> device
+// copies and Synchronize() throw while recording, so tensors have to be resident and every kernel of the sequence
+// has to have run once before (its code object is then loaded and its scratch buffer allocated).  The reference
+// has no counterpart: it launches kernel by kernel on the null stream (exec/CudaExecutor.cpp:70-101).
+struct Graph;
+void BeginCapture();
+Graph *EndCapture();           // ends the recording (also after an error in between) and instantiates it
+void AbortCapture();           // ends a recording and discards it; no-op when none is active
+bool Capturing();
+void Launch(Graph *graph);     // asynchronous, in stream order with everything else on Stream()
+void Destroy(Graph *graph);
+
 // Multiprocessor count, LDS bytes per workgroup, wavefront size of the current device (cached).
 struct DeviceInfo
 {

@@ -42,6 +42,18 @@ int acro_hip_event_record(void *event);
 int acro_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for stop */
 int acro_hip_event_destroy(void *event);
 
+/* Recorded launch sequences (hipGraph): between begin_capture and end_capture every kernel the library would launch
+ * on its stream is recorded instead of executed; acro_hip_graph_launch then enqueues the whole sequence with one
+ * call, in stream order with everything else.  While recording, anything that needs the host fails (allocation,
+ * host <-> device copies, synchronisation): tensors must be resident and the sequence must have run once before.
+ * No counterpart in the reference, which launches kernel by kernel on the null stream (exec/CudaExecutor.cpp:70-101). */
+typedef struct acro_hip_graph acro_hip_graph;
+int acro_hip_graph_begin_capture(void);
+int acro_hip_graph_end_capture(acro_hip_graph **out);  /* also ends a recording in which a call failed */
+int acro_hip_graph_abort_capture(void);
+int acro_hip_graph_launch(acro_hip_graph *g);
+int acro_hip_graph_destroy(acro_hip_graph *g);
+
 /* ---- acro::Tensor (tensor/Tensor.hpp:15-126) and acro::SliceTensor (tensor/SliceTensor.hpp:14-58) ---- */
 /* hdata / ddata may be NULL (library-owned host buffer / no device mirror yet); ongpu marks the device copy
  * as the current one (Tensor::Init rules, tensor/Tensor.cpp:166-202). */
