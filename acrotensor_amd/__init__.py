@@ -7,7 +7,7 @@ operations); every call goes through ``libacrotensor_hip.so``.  Errors that the 
 ``AcroError``.  There is no host compute path in this package.
 """
 from .api import (AcroError, IndexMapping, SliceTensor, Tensor, TensorEngine, describe_kernels, hip_event_timer,
-                  is_hip_ready, recorded_launches, synchronize)
+                  is_hip_ready, recorded_launches, set_pinned_host_allocation, synchronize)
 
 __all__ = ["AcroError", "IndexMapping", "SliceTensor", "Tensor", "TensorEngine", "describe_kernels",
-           "hip_event_timer", "is_hip_ready", "recorded_launches", "synchronize"]
+           "hip_event_timer", "is_hip_ready", "recorded_launches", "set_pinned_host_allocation", "synchronize"]

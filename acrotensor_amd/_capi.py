@@ -24,6 +24,7 @@ SIGNATURES = {
     "acro_hip_get_stream": (ctypes.c_void_p, []),
     "acro_hip_event_create": (ctypes.c_int, [handle_p]),
     "acro_hip_event_record": (ctypes.c_int, [handle]),
+    "acro_tensor_set_pinned_host_allocation": (ctypes.c_int, [ctypes.c_int]),
     "acro_hip_graph_begin_capture": (ctypes.c_int, []),
     "acro_hip_graph_end_capture": (ctypes.c_int, [ctypes.POINTER(handle)]),
     "acro_hip_graph_abort_capture": (ctypes.c_int, []),

@@ -29,6 +29,11 @@ def synchronize():
     _check(_capi.load().acro_hip_synchronize())
 
 
+def set_pinned_host_allocation(flag=True):
+    """Host buffers of tensors created from now on are page-locked (faster ``MoveToGPU`` / ``MoveFromGPU``)."""
+    _check(_capi.load().acro_tensor_set_pinned_host_allocation(1 if flag else 0))
+
+
 class Tensor:
     """Dense row-major fp64 tensor: ``Tensor(d0, d1, ...)``.  ``.data`` is a numpy view of the host buffer."""
 

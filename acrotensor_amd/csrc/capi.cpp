@@ -186,6 +186,11 @@ int acro_hip_graph_destroy(acro_hip_graph *g)
 
 // ------------------------------------------------------------------------------------------------ tensor
 
+int acro_tensor_set_pinned_host_allocation(int pinned)
+{
+    return guarded([&] { Tensor::SetPinnedHostAllocation(pinned != 0); });
+}
+
 int acro_tensor_create(int rank, const int *dims, double *hdata, double *ddata, int ongpu, acro_tensor **out)
 {
     return guarded([&] {

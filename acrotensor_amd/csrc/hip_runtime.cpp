@@ -98,6 +98,20 @@ void Free(void *dptr)
     ACRO_HIP_CHECK(hipFree(dptr));
 }
 
+void *HostMalloc(size_t bytes)
+{
+    void *p = nullptr;
+    ACRO_HIP_CHECK(hipHostMalloc(&p, bytes, hipHostMallocDefault));
+    return p;
+}
+
+void HostFree(void *hptr)
+{
+    if (hptr == nullptr) return;
+    if (!g_capturing) ACRO_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(Stream())));
+    ACRO_HIP_CHECK(hipHostFree(hptr));
+}
+
 void CopyToDevice(void *dst, const void *src, size_t bytes)
 {
     notWhileCapturing("Copying to the device");

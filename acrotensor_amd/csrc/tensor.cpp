@@ -17,6 +17,22 @@ namespace acro
 
 // ---------------------------------------------------------------------------------------------- Tensor
 
+namespace
+{
+bool g_pinned_host_allocation = false;
+}
+
+void Tensor::SetPinnedHostAllocation(bool pinned)
+{
+    ACROBATIC_ASSERT(!pinned || isHipReady(), "Page-locked host memory needs a HIP device.");
+    g_pinned_host_allocation = pinned;
+}
+
+bool Tensor::GetPinnedHostAllocation()
+{
+    return g_pinned_host_allocation;
+}
+
 Tensor::Tensor()
     : Size(0), Initialized(false), OwnsData(false), MappedToGPU(false), OnGPU(false), Transient(false),
       Data(nullptr), DeviceData(nullptr)
@@ -47,7 +63,11 @@ void Tensor::Init(const std::vector<int> &dims, double *hdata, double *ddata, bo
     ComputeSize();
 
     OwnsData = (hdata == nullptr);
-    Data = OwnsData ? new double[Size] : hdata;
+    PinnedData = OwnsData && g_pinned_host_allocation;
+    if (PinnedData)
+        Data = static_cast<double *>(hip::HostMalloc(Size * sizeof(double)));
+    else
+        Data = OwnsData ? new double[Size] : hdata;
     DeviceData = ddata;
     MappedToGPU = (ddata != nullptr);
     OnGPU = ongpu;
@@ -57,7 +77,20 @@ void Tensor::Init(const std::vector<int> &dims, double *hdata, double *ddata, bo
 Tensor::~Tensor()
 {
     if (!OwnsData) return;
-    delete[] Data;
+    if (PinnedData)
+    {
+        try
+        {
+            hip::HostFree(Data);
+        }
+        catch (...)
+        {
+        }
+    }
+    else
+    {
+        delete[] Data;
+    }
     if (MappedToGPU && DeviceData != nullptr)
     {
         try

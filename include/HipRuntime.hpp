@@ -29,6 +29,8 @@ void Synchronize();
 
 void *Malloc(size_t bytes);
 void Free(void *dptr);
+void *HostMalloc(size_t bytes);   // page-locked host memory
+void HostFree(void *hptr);
 void CopyToDevice(void *dst, const void *src, size_t bytes);    // returns after the host buffer may be reused
 void CopyToHost(void *dst, const void *src, size_t bytes);      // returns after the data has arrived
 void FillDouble(double *d, double value, size_t n);             // d[i] = value   (async on Stream())

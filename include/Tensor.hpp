@@ -139,6 +139,12 @@ class Tensor
     void SetTransient(bool transient) { Transient = transient; }
     virtual bool IsTransient() const { return Transient; }
 
+    // Extension (no counterpart in the reference, which allocates with new[], tensor/Tensor.cpp:196): host buffers
+    // that tensors allocate from now on are page-locked, so MoveToGPU / MoveFromGPU run as direct transfers at
+    // the rate of the host link instead of through the runtime's staging of pageable memory.  Needs a HIP device.
+    static void SetPinnedHostAllocation(bool pinned);
+    static bool GetPinnedHostAllocation();
+
   protected:
     void UpdateStrides();
     void ComputeSize();
@@ -150,6 +156,7 @@ class Tensor
 
     bool Initialized;
     bool OwnsData;
+    bool PinnedData = false;  // the owned host buffer is page-locked
     bool MappedToGPU;
     bool OnGPU;
     bool Transient;

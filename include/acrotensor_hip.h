@@ -83,6 +83,10 @@ int acro_tensor_mult(acro_tensor *t, double factor); /* Tensor::Mult, tensor/Ten
 /* Extension without reference counterpart: a transient tensor is scratch of a fused multi-kernel launch; its
  * contents in device memory are unspecified after the launch (the store may be skipped). */
 int acro_tensor_set_transient(acro_tensor *t, int transient);
+/* Extension without reference counterpart (the reference allocates host buffers with new[], tensor/Tensor.cpp:196):
+ * host buffers that the library allocates for tensors created from now on are page-locked, so that host <-> device
+ * moves run at the rate of the host link.  Needs a HIP device. */
+int acro_tensor_set_pinned_host_allocation(int pinned);
 
 /* ---- acro::IndexMapping (tensor/IndexMapping.hpp:13-45) ---- */
 int acro_index_mapping_create(int domain_size, int range_size, acro_index_mapping **out);

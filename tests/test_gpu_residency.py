@@ -101,3 +101,20 @@ def test_fill_and_scale_of_slices_touch_exactly_their_entries(at, rows, cols):
             expected[r] = 0.25 + r
     T.MoveFromGPU()
     assert np.array_equal(T.data, expected)
+
+
+def test_page_locked_host_buffers_move_like_ordinary_ones(at):
+    at.set_pinned_host_allocation(True)
+    try:
+        T = at.Tensor(257, 129)
+    finally:
+        at.set_pinned_host_allocation(False)
+    U = at.Tensor(257, 129)                                     # ordinary again
+    ref = np.arange(257 * 129, dtype=np.float64).reshape(257, 129)
+    for X in (T, U):
+        X.data[...] = ref
+        X.MoveToGPU()
+        X.Mult(2.0)
+        X.MoveFromGPU()
+        assert np.array_equal(X.data, 2.0 * ref)
+    del T, U
