@@ -1187,6 +1187,30 @@ class Generator
             st.elide = ok && anyRead;
         }
         if (envInt("ACRO_HIP_LDS_PAD") > 0) PadLdsTiles(budgetDoubles);  // opt-in: see PadLdsTiles
+
+        // A launch that writes several times what it reads streams better with fewer workgroups resident per CU
+        // (fewer write streams interleave at the memory controllers): workgroups of 128 lanes become 256 lanes with
+        // the upper half idle, which halves the residency.  Measured: p=2 mass assembly 37.2 -> 34.3 us, p=3 mass
+        // apply with all intermediates stored 355 -> 335 us; the same change costs the read-dominated p=3 mass
+        // apply with transient intermediates 8 % (86.4 -> 93.6 us), hence the condition.
+        if (NT == 128 && opt.force_nt <= 0 && envInt("ACRO_HIP_NT") <= 0 && batch >= 0)
+        {
+            double stored = 0.0, loaded = 0.0;
+            std::set<int> counted;
+            for (int k = 0; k < K; ++k)
+            {
+                const Sub &s = subs[k];
+                if (StoresToGlobal(k)) stored += static_cast<double>(s.out.size) / static_cast<double>(E);
+                for (size_t v = 0; v < s.in.size(); ++v)
+                {
+                    const Source src = SourceOf(k, static_cast<int>(v));
+                    if ((src == kFromGlobal || src == kFromConstant) && has(s.in[v].idx, batch) &&
+                        counted.insert(s.in[v].uvar).second)
+                        loaded += static_cast<double>(s.in[v].size) / static_cast<double>(E);
+                }
+            }
+            if (stored >= 3.0 * loaded && stored > 0.0) NT = 256;
+        }
     }
 
     // ----------------------------------------------------------------------------- LDS bank conflicts
