@@ -2273,9 +2273,17 @@ class Generator
 
         // Emits, for pass j of a phase (or for the item loop when j < 0), the selection of the chain a lane works
         // for and calls `body` inside the guarded scope of one work item.
+        // A streaming group (one phase, no LDS) over few batch entries would leave most of the device idle with one
+        // workgroup per entry: the passes of its item loop become workgroups of a second grid dimension instead.
+        const long splitY = (phases.size() == 1 && ldsDoubles == 0 && !looped && phases[0].passes > 1 && totalGroups < 2048)
+                                ? std::min<long>(phases[0].passes, 65535)
+                                : 1;
         auto emitItems = [&](const Phase &ph, long j, const std::function<void(const Chain &, const std::string &)> &body) {
             std::string indent = "        ";
-            if (j < 0)
+            if (j < 0 && splitY > 1)
+                out << "    for (int w0 = tid + blockIdx.y * " << NT << "; w0 < " << ph.slots << "; w0 += " << splitY * NT
+                    << ")\n    {\n";
+            else if (j < 0)
                 out << "    for (int w0 = tid; w0 < " << ph.slots << "; w0 += " << NT << ")\n    {\n";
             else
                 out << "    {\n        const int w0 = tid + " << j * NT << ";\n";
@@ -2402,6 +2410,7 @@ class Generator
         HipLaunch launch;
         launch.function_name = function_name;
         launch.grid = static_cast<unsigned>(gridGroups);
+        launch.grid_y = static_cast<unsigned>(splitY);
         launch.block = static_cast<unsigned>(NT);
         for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
         plan.launches.push_back(launch);

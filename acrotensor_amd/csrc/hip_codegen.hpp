@@ -73,6 +73,7 @@ struct HipLaunch
 {
     std::string function_name;
     unsigned grid = 0;
+    unsigned grid_y = 1;  // > 1: the work items of one batch entry are spread over this many workgroups
     unsigned block = 0;
     std::vector<int> params;
 };

@@ -242,7 +242,7 @@ class HipExecutor : public KernelExecutor
             {
                 args[i] = launch.params[i] < 0 ? static_cast<void *>(&v.scratch) : static_cast<void *>(&ptr[launch.params[i]]);
             }
-            v.kernel->Launch(launch.function_name, launch.grid, launch.block, args.data());
+            v.kernel->Launch(launch.function_name, launch.grid, launch.grid_y, launch.block, args.data());
         }
     }
 

@@ -162,7 +162,7 @@ void HipKernel::EnsureLoaded()
     Module = module;
 }
 
-void HipKernel::Launch(const std::string &function_name, unsigned grid, unsigned block, void **args)
+void HipKernel::Launch(const std::string &function_name, unsigned grid, unsigned grid_y, unsigned block, void **args)
 {
     EnsureLoaded();
     auto it = Functions.find(function_name);
@@ -172,7 +172,7 @@ void HipKernel::Launch(const std::string &function_name, unsigned grid, unsigned
         ACRO_HIP_CHECK(hipModuleGetFunction(&function, static_cast<hipModule_t>(Module), function_name.c_str()));
         it = Functions.emplace(function_name, function).first;
     }
-    ACRO_HIP_CHECK(hipModuleLaunchKernel(static_cast<hipFunction_t>(it->second), grid, 1, 1, block, 1, 1, 0,
+    ACRO_HIP_CHECK(hipModuleLaunchKernel(static_cast<hipFunction_t>(it->second), grid, grid_y, 1, block, 1, 1, 0,
                                          static_cast<hipStream_t>(hip::Stream()), args, nullptr));
 }
 

@@ -27,7 +27,7 @@ class HipKernel
     HipKernel &operator=(const HipKernel &) = delete;
 
     // args: one pointer per kernel parameter (as for hipModuleLaunchKernel)
-    void Launch(const std::string &function_name, unsigned grid, unsigned block, void **args);
+    void Launch(const std::string &function_name, unsigned grid, unsigned grid_y, unsigned block, void **args);
 
     const std::string &GetSource() const { return Source; }
     const std::string &GetModuleName() const { return FunctionName; }

@@ -346,6 +346,19 @@ def test_scatter_into_a_slice_that_is_not_vector_aligned(at, engine, checker):
     assert np.all(parent.data[0] == -5.0) and np.all(parent.data[2] == -5.0)
 
 
+def test_few_batch_entries_with_many_work_items_spread_over_workgroups(at, engine, checker):
+    # 12 batch entries (the largest output index) x 4 950 work items: one workgroup per entry would use 12 of 256
+    # CUs, so the passes of the item loop become a second grid dimension
+    rng = np.random.default_rng(21)
+    B, C = rng.uniform(-1, 1, (12, 11, 10, 9, 5, 6)), rng.uniform(-1, 1, 6)
+    k = "A_a_b_c_d_f = B_a_b_c_d_f_k C_k"
+    got, expected = run_single(at, engine, checker, k, np.zeros((12, 11, 10, 9, 5)), B, C)
+    assert "blockIdx.y" in engine.GetLastImplementation()
+    assert rel_err(got, expected) <= TOL
+    got, expected = run_single(at, engine, checker, k.replace(" = ", " += "), rng.uniform(-1, 1, (12, 11, 10, 9, 5)), B, C)
+    assert rel_err(got, expected) <= TOL
+
+
 def test_get_implementation_returns_hip_source(at, engine):
     A, B = at.Tensor(8, 3), at.Tensor(8, 3)
     src = engine.GetImplementation("A_e_i = B_e_i", A, B)
