@@ -10,6 +10,7 @@
 #include <cstdlib>
 #include <functional>
 #include <map>
+#include <numeric>
 #include <set>
 #include <sstream>
 
@@ -1937,8 +1938,6 @@ class Generator
         const Sub &s = subs[0];
         const long O = product(s.outIdx, extent);
         const long Nc = s.contrCount;
-        const int NTr = kReductionLanes;
-        const long Sn = NTr / O;  // contraction slices per workgroup
         // Lanes follow the memory order of the largest operand: output entries fastest when its innermost
         // dimension is an output index, contraction slices fastest otherwise.
         const VarRef *big = &s.in[0];
@@ -1947,9 +1946,21 @@ class Generator
             if (r.size > big->size) big = &r;
         }
         const bool outputsFastest = has(s.outIdx, big->idx.back());
-        long G = std::min<long>(512, std::max<long>(1, Nc / (Sn * 16)));
-        const long chunk = ((Nc + G - 1) / G + Sn - 1) / Sn * Sn;  // contraction entries per workgroup
-        G = (Nc + chunk - 1) / chunk;
+        // Few output entries that are the fastest dimension of the big operand ("S_i_j = A_n_i_j B_n"): a lane owns
+        // whole contraction slices and keeps one accumulator per output entry ("pencil").  It reads the O entries of
+        // its slice of A as 16-byte pieces and the slice's entry of B once, i.e. 6 load instructions per 80 bytes;
+        // with one lane per (slice, output entry) every lane loads B again and the same bytes take 18 load
+        // instructions (A alone streamed at 6.1 TB/s that way, A and B together at 5.0 - 5.5 TB/s).
+        const bool pencil = outputsFastest && O <= 16 && envInt("ACRO_HIP_RED_PENCIL") >= 0;
+        const int NTr = kReductionLanes;
+        const long Sn = pencil ? NTr : NTr / O;  // contraction slices per workgroup and step
+        // First-stage workgroups.  Pencil: one per CU (256 on this device) without unrolling, i.e. about 20 KB of
+        // loads in flight per CU and one 4.7 MB window moving through the operands; more workgroups or deeper
+        // unrolling measured slower at every n (n = 2^24: 206 us with 256 workgroups, 216 with 512, 252 with 2 048;
+        // 214 / 263 us with the loop unrolled 2 / 4 times).  One lane per (slice, output entry): 8 bytes per lane
+        // and load, so up to 512 workgroups and four loads in flight per lane (also swept: 256 - 8 192 workgroups,
+        // unroll 1 - 8).
+        const long G = std::min<long>(pencil ? 256 : 512, std::max<long>(1, Nc / (Sn * (pencil ? 4 : 16))));
         // Lanes of the finishing kernel: enough for every lane to have all its loads of partials in flight at once
         // (the kernel is a chain of memory latencies: launch, one round of loads, LDS; 1024 lanes instead of 256
         // measured 16.8 instead of 17.2 us for the pair of launches at n = 2^20), at most 1024.  The one-pass
@@ -1957,6 +1968,7 @@ class Generator
         int NTf = NTr;
         if (envInt("ACRO_HIP_ONE_PASS") <= 0)
         {
+            NTf = kReductionLanes;
             while (NTf < 1024 && G * O > NTf * 4) NTf *= 2;
         }
         const long S2 = NTf / O;
@@ -1966,14 +1978,15 @@ class Generator
         std::snprintf(hex, sizeof(hex), "%016llx",
                       static_cast<unsigned long long>(hashString(dimName + "/reduction/" + (opt.noalias ? "n" : "a") +
                                                                  (Positional() ? "p" : "u") +
-                                                                 (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "2" : "1"))));
+                                                                 (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "2" : "1") + "/" + str(envInt("ACRO_HIP_RED_PENCIL")))));
         plan.module_name = std::string("acro_red_") + hex;
         const std::string fPartial = plan.module_name + "_partial", fFinal = plan.module_name + "_final";
 
         std::ostringstream sched;
         sched << "reduction schedule: " << O << " output entries, contraction of " << Nc << " terms split over " << G
-              << " workgroups x " << Sn << " slices (" << (outputsFastest ? "output entries" : "slices")
-              << " on adjacent lanes), partials added in a fixed order by "
+              << " workgroups x " << Sn << " slices ("
+              << (pencil ? "a lane owns whole slices" : (outputsFastest ? "output entries on adjacent lanes" : "slices on adjacent lanes"))
+              << "), partials added in a fixed order by "
               << (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "a second kernel" : "the workgroup that finishes last") << "\n  [0] " << s.text << "\n";
         plan.schedule = sched.str();
 
@@ -2003,32 +2016,103 @@ class Generator
         // ---- stage 1: per-workgroup partial sums
         out << "\nextern \"C\" __global__ __launch_bounds__(" << NTr << ") void " << fPartial << "(" << ParamList()
             << ", double *__restrict__ scratch)\n{\n";
-        out << "    __shared__ double red[" << NTr << "];\n";
+        out << "    __shared__ double red[" << (pencil ? NTr * O : NTr) << "];\n";
         if (!twoKernels) out << "    __shared__ int isLast;\n";
         out << "    const int lane = threadIdx.x;\n";
-        if (outputsFastest)
-            out << "    const int sl = lane / " << O << ", o = lane % " << O << ";\n";
-        else
-            out << "    const int o = lane / " << Sn << ", sl = lane % " << Sn << ";\n";
-        out << "    double sum = 0.0;\n";
-        out << "    if (lane < " << Sn * O << ")\n    {\n";
-        decompose(s.outIdx, "o", "        ");
-        out << "        const long first = (long)blockIdx.x * " << chunk << ";\n";
-        out << "        const long last = first + " << chunk << " < " << Nc << " ? first + " << chunk << " : " << Nc << ";\n";
-        out << "#pragma unroll 4\n";
-        out << "        for (long c = first + sl; c < last; c += " << Sn << ")\n        {\n";
-        decompose(s.contr, "c", "            ");
-        std::string prod;
-        for (const auto &r : s.in)
+        // Workgroups interleave: in every step the G workgroups together read one contiguous window of the
+        // operands, so the device-wide access pattern is a single moving front.  Neighbouring workgroups share the
+        // cache lines at their border, so neighbours run on the same XCD (one L2): hardware deals consecutive
+        // workgroup ids round-robin to the 8 XCDs.
+        const std::string gExpr = (G % 8 == 0) ? "(long)(blockIdx.x % 8) * " + str(G / 8) + " + blockIdx.x / 8" : std::string("blockIdx.x");
+        if (pencil)
         {
-            const std::string opnd = PtrName(r.uvar) + "[" + FullOffset(r) + "]";
-            prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
+            for (long o = 0; o < O; ++o) out << "    double acc" << o << " = 0.0;\n";
+            out << "    {\n        const long g = " << gExpr << ";\n";
+            out << "#pragma unroll 1\n";
+            out << "        for (long c = g * " << Sn << " + lane; c < " << Nc << "; c += " << G * Sn << ")\n        {\n";
+            decompose(s.contr, "c", "            ");
+            // operand bases (contraction part of the address) and memoised loads (output part is a literal)
+            std::vector<std::string> loads, sums;
+            std::map<std::string, std::string> memo;
+            for (size_t v = 0; v < s.in.size(); ++v)
+            {
+                const VarRef &r = s.in[v];
+                std::string base = uvars[r.uvar].viewOffset != 0 ? Lit(uvars[r.uvar].viewOffset) : std::string();
+                for (size_t d = 0; d < r.idx.size(); ++d)
+                {
+                    if (has(s.contr, r.idx[d])) base += (base.empty() ? "" : " + ") + IdxVar(r.idx[d]) + " * " + Lit(r.stride[d]);
+                }
+                out << "            const " << OffsetType() << " ob" << v << " = " << (base.empty() ? "0" : base) << ";\n";
+            }
+            std::vector<int> value(nidx, 0);
+            for (long o = 0; o < O; ++o)
+            {
+                long rem = o;
+                for (int j = static_cast<int>(s.outIdx.size()) - 1; j >= 0; --j)
+                {
+                    value[s.outIdx[j]] = static_cast<int>(rem % extent[s.outIdx[j]]);
+                    rem /= extent[s.outIdx[j]];
+                }
+                std::string prod;
+                for (size_t v = 0; v < s.in.size(); ++v)
+                {
+                    const VarRef &r = s.in[v];
+                    long lit = 0;
+                    for (size_t d = 0; d < r.idx.size(); ++d)
+                    {
+                        if (!has(s.contr, r.idx[d])) lit += static_cast<long>(value[r.idx[d]]) * r.stride[d];
+                    }
+                    const std::string key = str(static_cast<long>(v)) + ":" + str(lit);
+                    auto it = memo.find(key);
+                    if (it == memo.end())
+                    {
+                        const std::string name = "x" + str(static_cast<long>(v)) + "_" + str(static_cast<long>(memo.size()));
+                        loads.push_back("const double " + name + " = " + PtrName(r.uvar) + "[ob" + str(static_cast<long>(v)) + " + " + Lit(lit) + "];");
+                        it = memo.emplace(key, name).first;
+                    }
+                    prod = prod.empty() ? it->second : "(" + prod + " * " + it->second + ")";
+                }
+                sums.push_back("acc" + str(o) + " += " + prod + ";");
+            }
+            for (const auto &l : loads) out << "            " << l << "\n";
+            for (const auto &l : sums) out << "            " << l << "\n";
+            out << "        }\n    }\n";
+            // lanes -> 64 lanes -> one: fixed order, whatever the timing
+            for (long o = 0; o < O; ++o) out << "    red[lane * " << O << " + " << o << "] = acc" << o << ";\n";
+            out << "    __syncthreads();\n";
+            out << "    if (lane < 64)\n    {\n";
+            out << "        for (int o = 0; o < " << O << "; ++o)\n        {\n            double t = 0.0;\n";
+            out << "            for (int j = 0; j < " << NTr / 64 << "; ++j) t += red[(lane + 64 * j) * " << O << " + o];\n";
+            out << "            red[lane * " << O << " + o] = t;\n        }\n    }\n";
+            out << "    __syncthreads();\n";
+            out << "    if (lane < " << O << ")\n    {\n        double t = 0.0;\n";
+            out << "        for (int k = 0; k < 64; ++k) t += red[k * " << O << " + lane];\n";
         }
-        out << "            sum += " << prod << ";\n        }\n    }\n";
-        out << "    red[lane] = sum;\n    __syncthreads();\n";
-        out << "    if (lane < " << O << ")\n    {\n        double t = 0.0;\n";
-        out << "        for (int k = 0; k < " << Sn << "; ++k) t += red["
-            << (outputsFastest ? "k * " + str(O) + " + lane" : "lane * " + str(Sn) + " + k") << "];\n";
+        else
+        {
+            if (outputsFastest)
+                out << "    const int sl = lane / " << O << ", o = lane % " << O << ";\n";
+            else
+                out << "    const int o = lane / " << Sn << ", sl = lane % " << Sn << ";\n";
+            out << "    double sum = 0.0;\n";
+            out << "    if (lane < " << Sn * O << ")\n    {\n";
+            decompose(s.outIdx, "o", "        ");
+            out << "        const long g = " << gExpr << ";\n";
+            out << "#pragma unroll 4\n";
+            out << "        for (long c = g * " << Sn << " + sl; c < " << Nc << "; c += " << G * Sn << ")\n        {\n";
+            decompose(s.contr, "c", "            ");
+            std::string prod;
+            for (const auto &r : s.in)
+            {
+                const std::string opnd = PtrName(r.uvar) + "[" + FullOffset(r) + "]";
+                prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
+            }
+            out << "            sum += " << prod << ";\n        }\n    }\n";
+            out << "    red[lane] = sum;\n    __syncthreads();\n";
+            out << "    if (lane < " << O << ")\n    {\n        double t = 0.0;\n";
+            out << "        for (int k = 0; k < " << Sn << "; ++k) t += red["
+                << (outputsFastest ? "k * " + str(O) + " + lane" : "lane * " + str(Sn) + " + k") << "];\n";
+        }
         if (twoKernels)
             out << "        scratch[(long)blockIdx.x * " << O << " + lane] = t;\n    }\n}\n";
         else
@@ -2086,7 +2170,7 @@ class Generator
         plan.source = out.str();
         plan.scratch_doubles = static_cast<size_t>(G * O) + (twoKernels ? 0 : 1);
         plan.nb = 1;
-        plan.lds_bytes = NTr * 8;
+        plan.lds_bytes = static_cast<int>((pencil ? NTr * O : NTr) * 8);
         FillParams(plan, false);
         const int S = static_cast<int>(stores.size());
         HipLaunch partial;
