@@ -97,6 +97,21 @@ def test_stiffness_assembly_sums_one_direction_early(TE):
     assert "_F1->lds\n" in src and "_F1<-lds" in src and "S->global" in src
 
 
+def test_split_contraction_with_few_outputs_gives_a_lane_whole_slices(TE, monkeypatch):
+    S, A, B = at.Tensor(3, 3), at.Tensor(1 << 18, 3, 3), at.Tensor(1 << 18)
+    src = TE.GetImplementation("S_i_j = A_n_i_j B_n", S, A, B)
+    assert "a lane owns whole slices" in src and "split over 256 workgroups" in src
+    assert src.count("double acc") == 9 and src.count("T2[ob1") == 1      # B is loaded once per slice, not per output
+    assert src.count("__global__") == 2 and "atomic" not in src            # second kernel adds the partials
+    # many outputs, or outputs that are not the fastest dimension of the big operand: one lane per (slice, output)
+    S2, A2 = at.Tensor(40), at.Tensor(40, 1 << 14)
+    src = TE.GetImplementation("S_i = A_i_n B_n", S2, A2, at.Tensor(1 << 14))
+    assert "slices on adjacent lanes" in src
+    monkeypatch.setenv("ACRO_HIP_ONE_PASS", "1")
+    src = TE.GetImplementation("S_i_j = A_n_i_j B_n", S, at.Tensor((1 << 18) + 1, 3, 3), at.Tensor((1 << 18) + 1))
+    assert src.count("__global__") == 1 and "__hip_atomic_fetch_add" in src
+
+
 def test_long_contraction_uses_counted_loops(TE):
     wl = workloads.config1(n=4096)
     tensors = workloads.bind_to_engine(wl, at)
