@@ -1304,9 +1304,13 @@ class Generator
 
     void PadLdsTiles(int budgetDoubles)
     {
-        // Padding must not cost a resident workgroup: a CU has 160 KB of LDS.
-        const long cuDoubles = 160 * 1024 / 8;
-        const long residentBefore = cuDoubles / std::max(1, PlaceLds(NB));
+        // Padding must not cost a resident workgroup: a CU has 160 KB of LDS, handed out in granules of 1 280 bytes
+        // (the p=7 diffusion chain at 53 440 bytes fits three times, at 54 080 bytes only twice).
+        auto resident = [](long doubles) {
+            const long bytes = (std::max<long>(1, doubles) * 8 + 1279) / 1280 * 1280;
+            return 160L * 1024 / bytes;
+        };
+        const long residentBefore = resident(PlaceLds(NB));
         for (size_t si = 0; si < stores.size(); ++si)
         {
             Storage &st = stores[si];
@@ -1344,7 +1348,7 @@ class Generator
             }
             SetLdsStrides(st, bestPad, bestEntry);
             const int total = PlaceLds(NB);
-            if (total > budgetDoubles || best >= unpadded || (envInt("ACRO_HIP_LDS_PAD") < 2 && cuDoubles / std::max(1, total) < residentBefore))
+            if (total > budgetDoubles || best >= unpadded || (envInt("ACRO_HIP_LDS_PAD") < 2 && resident(total) < residentBefore))
             {
                 SetLdsStrides(st, std::vector<int>(ndim, 0), 0);  // no room or no gain: natural layout
             }
