@@ -1218,9 +1218,10 @@ class Generator
     // LDS has 64 banks of 4 bytes; a wavefront's 8-byte accesses are served 32 lanes at a time, and lanes of such a
     // group that hit the same bank at different addresses serialise.  All addresses are known here (lane index
     // decomposition, tile strides), so the cost of every LDS access instruction can be counted and the tile strides
-    // padded until the count stops improving.  The count models 8-byte accesses only; the compiler merges adjacent
-    // ones into 16-byte accesses that padding can break apart, and on the p=7 diffusion chain the padded layout
-    // measured 20 % slower, so padding is opt-in (ACRO_HIP_LDS_PAD=1) until the model covers merged accesses.
+    // padded until the count stops improving.  The count models 8-byte accesses only (the compiler merges adjacent
+    // ones into 16-byte accesses).  Padding is opt-in (ACRO_HIP_LDS_PAD=1): it changed nothing measurable for the
+    // p=3 mass apply, and on the p=7 diffusion chain a few hundred bytes of padding cost a resident workgroup (LDS is
+    // handed out in granules) and 20 % of the speed until the acceptance test counted in granules.
 
     // Serialisation cycles of one access instruction whose lane l of the chain's item w reads `base(w)` doubles.
     static long ConflictCycles(const std::vector<long> &addr)
