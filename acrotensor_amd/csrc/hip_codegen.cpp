@@ -2126,11 +2126,12 @@ class Generator
 
         // ---- stage 2: add the per-workgroup partials in a fixed order and apply the assignment operator.
         // Default: a second, single-workgroup kernel.
-        // ACRO_HIP_ONE_PASS=1: the workgroup that arrives last at a device-wide counter does it instead (partials and
-        // counter exchanged with device-scope atomics and fences; the counter lives behind the partials in the scratch
-        // buffer, which the executor zeroes when it allocates it, and the last workgroup sets it back to zero).  The
-        // device-scope fences write back and invalidate the L2 of the workgroup's XCD every time; with 507 workgroups
-        // the single launch measured 55.9 us against 17.3 us for the two launches, so it is not the default.
+        // ACRO_HIP_ONE_PASS=1: the workgroup that arrives last at a device-wide counter does it instead (partials
+        // written with device-scope atomic stores, arrival counted with a release, the last workgroup acquires; the
+        // counter lives behind the partials in the scratch buffer, which the executor zeroes when it allocates it,
+        // and the last workgroup sets it back to zero).  A release at device scope writes back the L2 of the
+        // workgroup's XCD; with 256 workgroups the single launch measured 18.4 us against 16.3 us for the two
+        // launches (55.9 us when every lane also fenced), so it is not the default.
         auto emitFinish = [&](const std::string &load) {
             out << "    const int g2 = lane / " << O << ", o2 = lane % " << O << ";\n";
             out << "    double sum2 = 0.0;\n";
@@ -2159,10 +2160,12 @@ class Generator
         }
         else
         {
-            out << "    __threadfence();\n    __syncthreads();\n";
+            // The partials were stored by the wavefront of lane 0 with device-scope atomic stores; its release on the
+            // counter orders them before the arrival.  Only the last workgroup needs the acquire side.
+            out << "    __syncthreads();\n";
             out << "    if (lane == 0)\n    {\n";
             out << "        const unsigned int arrived = __hip_atomic_fetch_add(" << counter
-                << ", 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);\n";
+                << ", 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);\n";
             out << "        isLast = (arrived == " << G - 1 << "u);\n    }\n";
             out << "    __syncthreads();\n";
             out << "    if (!isLast) return;\n";
