@@ -163,6 +163,46 @@ def test_runtime_compiler_reports_errors_with_the_log():
     assert "undeclared_symbol" in message and "unit_bad" in message
 
 
+def generated_sources(TE):
+    """Sources of every schedule the generator has: fused chains with and without stored intermediates, reordered
+    kernels, split contractions (both finishes), counted loops, a second grid dimension, positional operands."""
+    yield "mass apply, transient", chain_source(TE, workloads.config4(E=66), True)
+    yield "mass apply, stored", chain_source(TE, workloads.config4(E=66), False)
+    yield "diffusion apply", chain_source(TE, workloads.config5(E=3), True)
+    yield "diffusion apply, stored", chain_source(TE, workloads.config5(E=3, Q=5, P=4), False)
+    wl = workloads.config3(E=5)
+    t = workloads.bind_to_engine(wl, at)
+    k, out, ins = wl.kernels[0]
+    yield "mass assembly", TE.GetImplementation(k, t[out], *[t[n] for n in ins])
+    S, A, B = at.Tensor(3, 3), at.Tensor(70000, 3, 3), at.Tensor(70000)
+    yield "split contraction", TE.GetImplementation("S_i_j = A_n_i_j B_n", S, A, B)
+    yield "split contraction, += and many outputs", TE.GetImplementation("S_i += A_i_n B_n", at.Tensor(40), at.Tensor(40, 9000), at.Tensor(9000))
+    yield "counted loops", TE.GetImplementation("C_e = B_e_j V_j", at.Tensor(300), at.Tensor(300, 700), at.Tensor(700))
+    yield "second grid dimension", TE.GetImplementation("A_a_b_c_d_f = B_a_b_c_d_f_k C_k", at.Tensor(12, 11, 10, 9, 5),
+                                                        at.Tensor(12, 11, 10, 9, 5, 6), at.Tensor(6))
+    yield "stiffness assembly", TE.GetImplementation(
+        "S_e_i1_i2_i3_j1_j2_j3 = B1_i1_j1_k1_m_n B2_i2_j2_k2_m_n B3_i3_j3_k3_m_n D_e_k1_k2_k3_m_n",
+        at.Tensor(4, 5, 5, 5, 5, 5, 5), at.Tensor(5, 5, 5, 3, 3), at.Tensor(5, 5, 5, 3, 3), at.Tensor(5, 5, 5, 3, 3),
+        at.Tensor(4, 5, 5, 5, 3, 3))
+    yield "one name, two tensors", TE.GetImplementation("A_m_n = B_m_j B_n_j", at.Tensor(3, 3), at.Tensor(3, 4), at.Tensor(3, 4))
+    yield "repeated output index", TE.GetImplementation("A_i_i = B_i", at.Tensor(6, 6), at.Tensor(6))
+
+
+def test_every_kind_of_generated_kernel_compiles_for_gfx950(TE, monkeypatch):
+    import ctypes
+    from acrotensor_amd import _capi
+    lib = _capi.load()
+    sources = list(generated_sources(TE))
+    monkeypatch.setenv("ACRO_HIP_ONE_PASS", "1")
+    sources.append(("split contraction, one launch",
+                    TE.GetImplementation("S_i_j = A_n_i_j B_n", at.Tensor(3, 3), at.Tensor(70001, 3, 3), at.Tensor(70001))))
+    for name, src in sources:
+        assert "__global__" in src, name
+        size = ctypes.c_size_t(0)
+        rc = lib.acro_hip_compile(("unit_" + name.split(",")[0].replace(" ", "_")).encode(), src.encode(), ctypes.byref(size))
+        assert rc == 0 and size.value > 0, (name, lib.acro_last_error().decode()[-2000:])
+
+
 def test_bad_kernel_strings_fail_before_code_generation():
     TE = at.TensorEngine("HIP")
     with pytest.raises(at.AcroError):
