@@ -158,7 +158,19 @@ void HipKernel::EnsureLoaded()
 {
     if (Module != nullptr) return;
     hipModule_t module;
-    ACRO_HIP_CHECK(hipModuleLoadData(&module, CodeObject.data()));
+    hipError_t err = hipModuleLoadData(&module, CodeObject.data());
+    if (err != hipSuccess && CacheHit)
+    {
+        // A code object from the disk cache that does not load (damaged file, different driver): compile afresh.
+        (void)hipGetLastError();
+        const std::string path = cachePath(FunctionName, Source);
+        if (!path.empty()) std::remove(path.c_str());
+        CacheHit = false;
+        CodeObject.clear();
+        Compile();
+        err = hipModuleLoadData(&module, CodeObject.data());
+    }
+    ACRO_HIP_CHECK(err);
     Module = module;
 }
 
