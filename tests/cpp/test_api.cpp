@@ -295,6 +295,41 @@ static void gpuTests()
         }
         CHECK(result[7] == 7.0 && owner.IsMappedToGPU());  // the wrapper did not free the caller's allocation
     }
+
+    std::printf("gpu: recorded launch sequence, page-locked host buffers\n");
+    {
+        Tensor::SetPinnedHostAllocation(true);
+        Tensor A(64, 3), B(64, 3), C(3);
+        Tensor::SetPinnedHostAllocation(false);
+        for (size_t i = 0; i < B.GetSize(); ++i) B[i] = 0.5 * static_cast<double>(i);
+        C(0) = 1.0, C(1) = 2.0, C(2) = 3.0;
+        auto step = [&]() {
+            TE("A_e_i = B_e_i C_i", A, B, C);
+            TE("B_e_i = A_e_i", B, A);
+        };
+        step();  // once eagerly: kernels loaded, tensors resident
+        hip::BeginCapture();
+        step();
+        hip::Graph *sequence = hip::EndCapture();
+        for (int rep = 0; rep < 3; ++rep) hip::Launch(sequence);
+        B.MoveFromGPU();
+        // four applications of B_e_i *= C_i in total: one eager, three replays (recording executes nothing)
+        CHECK(B(63, 0) == 0.5 * 189 && B(63, 1) == 0.5 * 190 * 16.0 && B(63, 2) == 0.5 * 191 * 81.0);
+        bool refused = false;
+        Tensor H(64, 3);  // still on the host: using it while recording would need a copy
+        hip::BeginCapture();
+        try
+        {
+            TE("A_e_i = B_e_i", A, H);
+        }
+        catch (const std::runtime_error &)
+        {
+            refused = true;
+        }
+        hip::AbortCapture();
+        CHECK(refused && !hip::Capturing());
+        hip::Destroy(sequence);
+    }
 }
 
 int main(int argc, char **argv)
