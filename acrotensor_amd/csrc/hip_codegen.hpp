@@ -21,7 +21,8 @@
 //   ACRO_HIP_PREFETCH=-1        no prefetch of later phases' streaming inputs at kernel entry
 //   ACRO_HIP_NT_STORE=-1        ordinary instead of non-temporal stores for results that stream out
 //   ACRO_HIP_LDS_PAD=1|2        pad LDS tile strides against bank conflicts (2: even if a resident workgroup is lost)
-//   ACRO_HIP_PACK=1             pick batch / workgroup size for wavefront utilisation
+//   ACRO_HIP_PACK=1|-1          1: pick batch / workgroup size for wavefront utilisation also when one batch entry per
+//                               workgroup would do; -1: never (default: only for groups that batch several entries)
 //   ACRO_HIP_PERSIST=<n>        persistent grid of n workgroups per CU looping over the batch
 //   ACRO_HIP_FACTORISE=-1|2     -1: evaluate multi-operand kernels as written instead of as a chain of steps;
 //                               2: reorder whenever a chain is cheaper at all (default: only large kernels, 4x gain)
