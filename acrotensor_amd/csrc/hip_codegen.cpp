@@ -5,6 +5,7 @@
 #include "hip_codegen.hpp"
 
 #include <algorithm>
+#include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -176,10 +177,14 @@ class Generator
                 s.forwardedOld = false;
                 s.loopMode = false;
             }
+            const double busyBefore = busyLanes;
             ChooseTiles();
             PlanFusion();
             ChooseBatching();
-            if (NB != 1)
+            // Scalar operands take their indices out of the lanes; a plan that leaves the wavefronts much emptier than
+            // before costs more in issue slots than the scalar loads save (T1_e_q_j_k = B_q_i X_e_i_j_k with X scalar
+            // has 6 busy lanes instead of 25: p=4 diffusion apply at 44.8 % of the HBM peak against 72.3 %).
+            if (NB != 1 || busyLanes < 0.8 * busyBefore)
             {
                 batchUniform = false;
                 for (auto &s : subs)
@@ -235,6 +240,7 @@ class Generator
     int ldsDoubles = 0;
     bool extentsConsistent = true;
     bool batchUniform = false;  // one batch entry per workgroup: the batch index is a scalar
+    double busyLanes = 1.0;     // share of busy lanes in the wavefronts that the chosen batching issues
     bool wide = false;          // 64-bit device-memory offsets
 
     // Literal of a device-memory stride or offset, and the type such offsets are computed in.
@@ -1115,14 +1121,54 @@ class Generator
                 }
                 return busy / issued;
             };
-            const double base = utilisation(NB, NT);
+            // Share of the arithmetic in kernels that need more than one pass of the workgroup over their items.
+            auto multiPassShare = [&](int nb, int nt) {
+                double all = 0.0, looped = 0.0;
+                for (const auto &s : subs)
+                {
+                    const double work = static_cast<double>(s.laneCount) * std::max<long>(1, s.tileCount * s.contrCount);
+                    all += work;
+                    if (static_cast<long>(nb) * s.laneCount > nt) looped += work;
+                }
+                return all > 0.0 ? looped / all : 0.0;
+            };
+            // Workgroups that declare much LDS leave few wavefronts resident on a compute unit (160 KB of LDS, handed
+            // out in 1280-byte granules, 32 wavefronts at most) and so fewer loads in flight to cover the memory
+            // latency; the square root follows the measured rates (p=3 diffusion apply in 256 lanes: 77.3 % of the
+            // HBM peak with 32 resident wavefronts, 69.8 % with 12 and fuller wavefronts).
+            auto occupancy = [&](int nb, int nt) {
+                long bytes = static_cast<long>(PlaceLds(nb)) * 8;
+                bytes = std::max<long>(1280, (bytes + 1279) / 1280 * 1280);
+                const long groups = std::min<long>(160 * 1024 / bytes, 32 / (nt / 64));
+                // wavefronts of a workgroup that have items at all, averaged over the arithmetic
+                double all = 0.0, busy = 0.0;
+                for (const auto &s : subs)
+                {
+                    const double work = static_cast<double>(s.laneCount) * std::max<long>(1, s.tileCount * s.contrCount);
+                    all += work;
+                    busy += work * std::min<long>(nt / 64, (static_cast<long>(nb) * s.laneCount + 63) / 64);
+                }
+                const double waves = groups * (all > 0.0 ? busy / all : nt / 64.0);
+                return std::sqrt(std::min(1.0, waves / 32.0));
+            };
+            for (auto &st : stores) st.inLds = st.wantLds;
+            const double idle = utilisation(NB, NT);
+            const double base = idle * occupancy(NB, NT);
             double best = base;
             int bestNB = NB, bestNT = NT;
+            // Candidates: up to 16 entries per workgroup.  Kernels that carry at most a quarter of the arithmetic may
+            // need several passes (a wide but cheap pointwise kernel should not dictate one entry per workgroup to
+            // the narrow, expensive contractions around it); looping the contractions themselves measured slower
+            // (p=3 mass apply with 12 entries in 128 lanes: 62.5 % against 76.7 %).  Never smaller workgroups than the
+            // default, and everything that wants LDS must still fit.
             for (int nt : {128, 256})
             {
-                for (int nb = 1; nb <= 16 && nb <= E && nb * maxLane <= nt; ++nb)
+                if (nt < NT) continue;
+                for (int nb = 1; nb <= 16 && nb <= E; ++nb)
                 {
-                    const double u = utilisation(nb, nt);
+                    if (nb * maxLane > 8L * nt || multiPassShare(nb, nt) > 0.25) break;
+                    if (PlaceLds(nb) > 64 * 1024 / 8) break;
+                    const double u = utilisation(nb, nt) * occupancy(nb, nt);
                     if (u > best * 1.02)
                     {
                         best = u;
@@ -1131,16 +1177,18 @@ class Generator
                     }
                 }
             }
-            // A workgroup with one batch entry keeps it: the batch index is then uniform and operands that depend
-            // on it alone are read with scalar loads, which measured better than fuller wavefronts (p=2 mass
-            // assembly).  Groups that batch anyway take the better packing (p=1 mass apply: 8 -> 14 entries per
-            // workgroup, 62.9 -> 74.9 % of the HBM peak; p=4: 2 -> 5 entries in 256 lanes, 67.5 -> 72.0 %).
-            const bool wanted = envInt("ACRO_HIP_PACK") > 0 || (envInt("ACRO_HIP_PACK") == 0 && NB > 1);
-            if (wanted && best >= 1.25 * base)
+            // A workgroup with one batch entry and at least half of its lanes busy keeps it: the batch index is then
+            // uniform, so its share of the address arithmetic is scalar, which measured no worse than fuller
+            // wavefronts (p=2 mass assembly).  Groups that batch anyway take the better packing (p=1 mass apply:
+            // 8 -> 14 entries per workgroup, 62.9 -> 74.9 % of the HBM peak; p=4: 2 -> 5 entries in 256 lanes,
+            // 67.5 -> 72.0 %), and so do groups whose wavefronts would be mostly idle.
+            const bool wanted = envInt("ACRO_HIP_PACK") > 0 || (envInt("ACRO_HIP_PACK") == 0 && (NB > 1 || idle < 0.5));
+            if (wanted && best >= 1.1 * base)
             {
                 NB = bestNB;
                 NT = bestNT;
             }
+            busyLanes = utilisation(NB, NT);
         }
 
         // Everything that wants LDS gets it while the workgroup stays within the 64 KB a workgroup may declare
