@@ -133,6 +133,20 @@ def test_diffusion_chain_resolves_slices_of_one_tensor_and_fuses(TE):
     assert src.count("__syncthreads()") == 6
 
 
+def test_diffusion_chain_batching_follows_the_contractions_not_the_pointwise_kernel(TE):
+    # Q=6, P=5: the pointwise kernel Z = D U has 216 lanes, the 17 contractions 25 - 36.  One element per workgroup
+    # must not turn X into a scalar operand (6 busy lanes for T1 instead of 25) ...
+    src = chain_source(TE, workloads.config5(E=64, Q=6, P=5), transient=True)
+    assert "T1g_e_q_j_k = G_q_i X_e_i_j_k : lanes(j,k)=25" in src and "G<-scalar X<-global" in src
+    # ... and with Q=5, P=4 (125 lanes against 16 - 25) several elements share a workgroup although the pointwise
+    # kernel then needs more than one pass over its items
+    src = chain_source(TE, workloads.config5(E=64, Q=5, P=4), transient=True)
+    header = src.splitlines()[1]
+    per_group = int(header.split(",")[1].split()[0])
+    assert per_group >= 2 and "256 lanes" in header
+    assert src.count("__syncthreads()") == 6
+
+
 def test_views_that_cannot_be_resolved_fall_back(TE):
     # the same parent viewed with the element index in two different positions cannot be fused
     T = at.Tensor(4, 4)

@@ -71,7 +71,7 @@ def test_config4_mass_apply(at, engine, checker, E, transient):
             assert rel_err(fetch(tensors, name), expected[name]) <= TOL, name
 
 
-@pytest.mark.parametrize("E,Q,P", [(1, 5, 4), (5, 5, 4), (3, 10, 8)])
+@pytest.mark.parametrize("E,Q,P", [(1, 5, 4), (5, 5, 4), (3, 10, 8), (23, 3, 2), (19, 4, 3), (7, 6, 5), (3, 7, 6)])
 @pytest.mark.parametrize("transient", [False, True])
 def test_config5_diffusion_apply(at, engine, checker, E, Q, P, transient):
     wl = workloads.config5(E=E, Q=Q, P=P)
