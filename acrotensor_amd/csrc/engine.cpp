@@ -1,6 +1,7 @@
 // TensorEngine (kernel caches, multi-kernel capture, non-contraction front-ends) and the KernelExecutor base
 // class with its policy registry.  Call order and asserts follow the reference's kernel/TensorEngine.cpp:70-95,
 // 290-336,538-767 and exec/KernelExecutor.cpp:12-131.
+#include <algorithm>
 #include <map>
 
 #include "TensorEngine.hpp"
@@ -140,6 +141,7 @@ void TensorEngine::ResetCapture()
     MKLKernels.clear();
     MKLOutputT.clear();
     MKLInputT.clear();
+    MKLMatrixOps.clear();
 }
 
 void TensorEngine::operator()(const std::string &kernel_str, Tensor *output, std::vector<Tensor *> &inputs)
@@ -175,9 +177,170 @@ void TensorEngine::EndMultiKernelLaunch()
 {
     ACROBATIC_ASSERT(IsMultiKernelLaunch, "Found and EndMultiKernelLaunch before a BeginMultiKernelLaunch!");
     IsMultiKernelLaunch = false;
-    if (MKLKernels.empty()) return;
-    LastExecutor = GetAddKernelExecutor();
-    LastExecutor->ExecuteMulti(MKLOutputT, MKLInputT);
+    FinishCapture(nullptr);
+}
+
+// Index and variable names for a recorded matrix operation, taken from the first later kernel that reads its
+// result, so that the operation becomes one or two kernels of the group ("Jinv_e_k_m_n = J_e_k_m_n" as an inverse,
+// "Jdet_e_k = J_e_k_m_n" as a determinant).  False when no later kernel reads a result, or a result is the operand
+// itself: the operation then runs on its own.
+bool TensorEngine::MatrixOpAsKernels(const RecordedMatrixOp &op, const std::vector<DimensionedKernel *> &kernels,
+                                     const std::vector<Tensor *> &outputs, const std::vector<std::vector<Tensor *>> &inputs,
+                                     std::vector<DimensionedKernel *> &op_kernels, std::vector<Tensor *> &op_outputs,
+                                     std::vector<std::vector<Tensor *>> &op_inputs)
+{
+    if (op.inverse == op.matrices || op.determinant == op.matrices) return false;
+    const int rank = op.matrices->GetRank();
+    std::vector<std::string> lead;
+    std::string row, col, inverse_name, determinant_name, matrices_name;
+    auto reader = [&](Tensor *t, const KernelVar *&found) {
+        found = nullptr;
+        for (size_t k = op.position; k < kernels.size() && found == nullptr; ++k)
+        {
+            for (size_t v = 0; v < inputs[k].size() && found == nullptr; ++v)
+            {
+                if (inputs[k][v] == t) found = &kernels[k]->GetVar(static_cast<int>(v));
+            }
+        }
+    };
+    const KernelVar *inv_reader = nullptr, *det_reader = nullptr;
+    if (op.inverse != nullptr) reader(op.inverse, inv_reader);
+    if (op.determinant != nullptr) reader(op.determinant, det_reader);
+    if (inv_reader != nullptr)
+    {
+        lead.assign(inv_reader->IndexNames.begin(), inv_reader->IndexNames.end() - 2);
+        row = inv_reader->IndexNames[rank - 2];
+        col = inv_reader->IndexNames[rank - 1];
+        inverse_name = inv_reader->Name;
+        if (det_reader != nullptr && det_reader->IndexNames == lead) determinant_name = det_reader->Name;
+    }
+    else if (det_reader != nullptr)
+    {
+        lead = det_reader->IndexNames;
+        determinant_name = det_reader->Name;
+    }
+    else
+    {
+        return false;
+    }
+
+    // Names in use anywhere in the capture; made-up names must differ from all of them.
+    std::vector<std::string> index_names, var_names;
+    for (size_t k = 0; k < kernels.size(); ++k)
+    {
+        for (int v = -1; v < kernels[k]->GetNumInputVars(); ++v)
+        {
+            const KernelVar &var = kernels[k]->GetVar(v);
+            var_names.push_back(var.Name);
+            index_names.insert(index_names.end(), var.IndexNames.begin(), var.IndexNames.end());
+            Tensor *t = v < 0 ? outputs[k] : inputs[k][v];
+            if (t == op.matrices && matrices_name.empty()) matrices_name = var.Name;
+        }
+    }
+    auto fresh = [](const std::string &stem, std::vector<std::string> &taken) {
+        std::string name = stem;
+        for (int n = 0; std::find(taken.begin(), taken.end(), name) != taken.end(); ++n) name = stem + std::to_string(n);
+        taken.push_back(name);
+        return name;
+    };
+    if (row.empty()) row = fresh("mr", index_names);
+    if (col.empty()) col = fresh("mc", index_names);
+    if (op.inverse != nullptr && inverse_name.empty()) inverse_name = fresh("MatrixInverse", var_names);
+    if (op.determinant != nullptr && determinant_name.empty()) determinant_name = fresh("MatrixDeterminant", var_names);
+    if (matrices_name.empty()) matrices_name = fresh("MatrixOperand", var_names);
+    std::vector<std::string> all = lead;
+    all.push_back(row);
+    all.push_back(col);
+    for (size_t a = 0; a < all.size(); ++a)
+    {
+        for (size_t b = a + 1; b < all.size(); ++b)
+        {
+            if (all[a] == all[b]) return false;  // the reader addresses a diagonal: not a plain copy of the result
+        }
+    }
+    if (inverse_name == matrices_name || determinant_name == matrices_name ||
+        (op.inverse != nullptr && op.determinant != nullptr && inverse_name == determinant_name))
+        return false;
+
+    auto spell = [](const std::string &name, const std::vector<std::string> &idx) {
+        std::string s = name;
+        for (const auto &i : idx) s += "_" + i;
+        return s;
+    };
+    std::vector<Tensor *> operand(1, op.matrices);
+    if (op.inverse != nullptr)
+    {
+        TensorKernel *kernel = GetAddTensorKernel(spell(inverse_name, all) + " = " + spell(matrices_name, all), "inv");
+        op_kernels.push_back(GetAddDimensionedKernel(kernel, op.inverse, operand));
+        op_outputs.push_back(op.inverse);
+        op_inputs.push_back(operand);
+    }
+    if (op.determinant != nullptr)
+    {
+        TensorKernel *kernel = GetAddTensorKernel(spell(determinant_name, lead) + " = " + spell(matrices_name, all), "det");
+        op_kernels.push_back(GetAddDimensionedKernel(kernel, op.determinant, operand));
+        op_outputs.push_back(op.determinant);
+        op_inputs.push_back(operand);
+    }
+    return true;
+}
+
+void TensorEngine::FinishCapture(std::string *implementation)
+{
+    std::vector<DimensionedKernel *> kernels;
+    std::vector<Tensor *> outputs;
+    std::vector<std::vector<Tensor *>> inputs;
+    kernels.swap(MKLKernels);
+    outputs.swap(MKLOutputT);
+    inputs.swap(MKLInputT);
+    std::vector<RecordedMatrixOp> ops;
+    ops.swap(MKLMatrixOps);
+
+    auto flush = [&]() {
+        if (MKLKernels.empty()) return;
+        KernelExecutor *executor = GetAddKernelExecutor();
+        if (implementation != nullptr)
+        {
+            *implementation += executor->GetImplementation(MKLOutputT, MKLInputT);
+        }
+        else
+        {
+            LastExecutor = executor;
+            executor->ExecuteMulti(MKLOutputT, MKLInputT);
+        }
+        ResetCapture();
+    };
+    size_t next_op = 0;
+    for (size_t k = 0; k <= kernels.size(); ++k)
+    {
+        for (; next_op < ops.size() && ops[next_op].position == k; ++next_op)
+        {
+            const RecordedMatrixOp &op = ops[next_op];
+            if (MatrixOpAsKernels(op, kernels, outputs, inputs, MKLKernels, MKLOutputT, MKLInputT)) continue;
+            flush();
+            if (implementation != nullptr)
+            {
+                *implementation += "// batched matrix operation whose result no later kernel of the capture reads: runs on its own\n";
+                continue;
+            }
+            if (op.inverse != nullptr) SwitchToComputeLocation(*op.inverse);
+            if (op.determinant != nullptr) SwitchToComputeLocation(*op.determinant);
+            MoveToComputeLocation(*op.matrices);
+            if (op.inverse != nullptr && op.determinant != nullptr)
+                Ops->BatchMatrixInvDet(*op.inverse, *op.determinant, *op.matrices);
+            else if (op.inverse != nullptr)
+                Ops->BatchMatrixInverse(*op.inverse, *op.matrices);
+            else
+                Ops->BatchMatrixDet(*op.determinant, *op.matrices);
+        }
+        if (k < kernels.size())
+        {
+            MKLKernels.push_back(kernels[k]);
+            MKLOutputT.push_back(outputs[k]);
+            MKLInputT.push_back(inputs[k]);
+        }
+    }
+    flush();
 }
 
 std::string TensorEngine::GetImplementation(const std::string &kernel_str, Tensor *output,
@@ -196,8 +359,9 @@ std::string TensorEngine::EndMultiKernelLaunchGetImplementation()
 {
     ACROBATIC_ASSERT(IsMultiKernelLaunch, "Found and EndMultiKernelLaunch before a BeginMultiKernelLaunch!");
     IsMultiKernelLaunch = false;
-    if (MKLKernels.empty()) return "";
-    return GetAddKernelExecutor()->GetImplementation(MKLOutputT, MKLInputT);
+    std::string implementation;
+    FinishCapture(&implementation);
+    return implementation;
 }
 
 std::string TensorEngine::GetLastImplementation()
@@ -211,6 +375,16 @@ TensorKernel *TensorEngine::GetAddTensorKernel(const std::string &kernel_str)
     if (it != KernelMap.end()) return it->second;
     TensorKernel *kernel = new TensorKernel(kernel_str);
     KernelMap[kernel_str] = kernel;
+    return kernel;
+}
+
+TensorKernel *TensorEngine::GetAddTensorKernel(const std::string &kernel_str, const std::string &function)
+{
+    const std::string key = kernel_str + " #" + function;  // '#' cannot occur in a kernel string
+    auto it = KernelMap.find(key);
+    if (it != KernelMap.end()) return it->second;
+    TensorKernel *kernel = new TensorKernel(kernel_str, function);
+    KernelMap[key] = kernel;
     return kernel;
 }
 
@@ -273,6 +447,11 @@ void TensorEngine::BatchMatrixInverse(Tensor &Ainv, Tensor &A)
 {
     ACROBATIC_ASSERT(Ops != nullptr, "The executor type of this engine provides no non-contraction ops.");
     checkInverseShapes(Ainv, A);
+    if (IsMultiKernelLaunch)
+    {
+        MKLMatrixOps.push_back({MKLKernels.size(), &Ainv, nullptr, &A});
+        return;
+    }
     SwitchToComputeLocation(Ainv);
     MoveToComputeLocation(A);
     Ops->BatchMatrixInverse(Ainv, A);
@@ -282,6 +461,11 @@ void TensorEngine::BatchMatrixDet(Tensor &Adet, Tensor &A)
 {
     ACROBATIC_ASSERT(Ops != nullptr, "The executor type of this engine provides no non-contraction ops.");
     checkDetShapes(Adet, A);
+    if (IsMultiKernelLaunch)
+    {
+        MKLMatrixOps.push_back({MKLKernels.size(), nullptr, &Adet, &A});
+        return;
+    }
     SwitchToComputeLocation(Adet);
     MoveToComputeLocation(A);
     Ops->BatchMatrixDet(Adet, A);
@@ -292,6 +476,11 @@ void TensorEngine::BatchMatrixInvDet(Tensor &Ainv, Tensor &Adet, Tensor &A)
     ACROBATIC_ASSERT(Ops != nullptr, "The executor type of this engine provides no non-contraction ops.");
     checkInverseShapes(Ainv, A);
     checkDetShapes(Adet, A);
+    if (IsMultiKernelLaunch)
+    {
+        MKLMatrixOps.push_back({MKLKernels.size(), &Ainv, &Adet, &A});
+        return;
+    }
     SwitchToComputeLocation(Ainv);
     SwitchToComputeLocation(Adet);
     MoveToComputeLocation(A);

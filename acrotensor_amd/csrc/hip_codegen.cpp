@@ -47,7 +47,10 @@ struct Sub
     std::vector<int> tile;    // loop ids kept in registers by one work item
     bool loopMode = false;    // contraction as counted loops instead of unrolled code
     bool fusedWithPrev = false;
-    int forwardedInput = -1;  // input occurrence served from the previous kernel's registers
+    std::vector<char> forwardedIn;  // per input occurrence: served from the registers of an earlier kernel of the chain
+    // 0: contraction.  1: the output is the inverse of the operand's trailing matrix, 2: its determinant.
+    int matrixOp = 0;
+    int matrixN = 0;
     bool forwardedOld = false;  // the old value of a += / -= output is the previous kernel's result, in registers
     int phase = 0;              // barrier-separated phase the kernel runs in
     long laneCount = 1, tileCount = 1, contrCount = 1;
@@ -173,7 +176,7 @@ class Generator
             for (auto &s : subs)
             {
                 s.fusedWithPrev = false;
-                s.forwardedInput = -1;
+                s.forwardedIn.clear();
                 s.forwardedOld = false;
                 s.loopMode = false;
             }
@@ -190,7 +193,7 @@ class Generator
                 for (auto &s : subs)
                 {
                     s.fusedWithPrev = false;
-                    s.forwardedInput = -1;
+                    s.forwardedIn.clear();
                     s.forwardedOld = false;
                     s.loopMode = false;
                 }
@@ -302,12 +305,31 @@ class Generator
             }
             for (const auto &name : k->ContractionIndexNames) s.contr.push_back(mk.GetIndexLoopNum(name));
             s.contrCount = product(s.contr, extent);
+            if (!k->Function.empty())
+            {
+                s.matrixOp = k->Function == "inv" ? 1 : 2;
+                s.matrixN = s.in[0].ext.back();
+                ACROBATIC_ASSERT(s.in[0].ext[s.in[0].ext.size() - 2] == s.matrixN && s.matrixN <= 3,
+                                 "HIP generator: a matrix kernel needs square matrices of at most 3 x 3.");
+            }
         }
 
-        if (!mk.SharedOuterIndexNames.empty())
+        // The batch index: the largest index that every kernel carries and none contracts (they come sorted), but
+        // never a row or column index of a matrix kernel, whose matrices stay whole inside one work item.
+        for (const auto &name : mk.SharedOuterIndexNames)
         {
-            batch = mk.GetIndexLoopNum(mk.SharedOuterIndexNames[0]);
+            const int id = mk.GetIndexLoopNum(name);
+            bool matrixIndex = false;
+            for (const auto &s : subs)
+            {
+                if (s.matrixOp == 0) continue;
+                const std::vector<int> &ids = s.in[0].idx;
+                matrixIndex = matrixIndex || id == ids[ids.size() - 1] || id == ids[ids.size() - 2];
+            }
+            if (matrixIndex) continue;
+            batch = id;
             E = extent[batch];
+            break;
         }
 
         if (factorise && envInt("ACRO_HIP_FACTORISE") >= 0) FactoriseKernels();
@@ -806,7 +828,15 @@ class Generator
                 if (id != batch) mid.push_back(id);
             }
             const long nin = static_cast<long>(s.in.size());
-            if (s.contrCount > kMaxUnrolledContraction || s.contrCount * nin > kUnrollBudget)
+            if (s.matrixOp != 0)
+            {
+                // One work item per matrix: the inverse keeps its row and column index as the register tile, the
+                // determinant contracts them.
+                s.loopMode = false;
+                s.tile.clear();
+                if (s.matrixOp == 1) s.tile.assign(s.out.idx.end() - 2, s.out.idx.end());
+            }
+            else if (s.contrCount > kMaxUnrolledContraction || s.contrCount * nin > kUnrollBudget)
             {
                 s.loopMode = true;
                 s.tile.clear();
@@ -875,31 +905,118 @@ class Generator
         s.tileCount = product(s.tile, extent);
     }
 
+    // May operand r of a kernel with lane indices `lane` be taken from the registers in which kernel q left its
+    // output?  The work item must be the same (same index wherever q's output carries the batch or a lane index) and
+    // the entry must be named at generation time (a tile or contraction index of the reader elsewhere).
+    bool ForwardableFrom(const Sub &q, const VarRef &r, const std::vector<int> &lane) const
+    {
+        if (r.uvar != q.out.uvar || r.idx.size() != q.out.idx.size()) return false;
+        for (size_t d = 0; d < r.idx.size(); ++d)
+        {
+            const int pid = q.out.idx[d];
+            const bool itemDim = pid == batch || has(lane, pid);
+            if (itemDim ? r.idx[d] != pid : (r.idx[d] == batch || has(lane, r.idx[d]))) return false;
+        }
+        return true;
+    }
+
+    // A kernel whose work items can be those of the previous kernel and that reads results of that kernel (or of
+    // the kernels it is itself applied after) entry by entry is applied in the same registers: a pointwise kernel
+    // after a contraction ("U = D T3"), but also a small contraction over the register tile of its producer
+    // ("D_e_m_n_k = W_k Jdet_e_k Jinv_e_k_n_j Jinv_e_k_m_j" after the inverse and determinant of J_e_k_m_n: one
+    // work item per (e, k) holds the nine entries of Jinv).
+    void ForwardAlongChain(int k, int chainStart)
+    {
+        Sub &s = subs[k];
+        const Sub &p = subs[k - 1];
+        if (envInt("ACRO_HIP_FORWARD") < 0 || p.loopMode || s.loopMode || p.out.repeated || s.out.repeated) return;
+        if (s.matrixOp == 2 && p.matrixOp == 1 && s.in[0].uvar == p.in[0].uvar && s.in[0].idx == p.in[0].idx)
+        {
+            // the determinant of the matrix that the previous kernel inverted: that kernel has computed it
+            s.fusedWithPrev = true;
+            s.forwardedIn.assign(1, 0);
+            s.lane = p.lane;
+            s.laneCount = p.laneCount;
+            return;
+        }
+        for (int id : p.lane)
+        {
+            if (!has(s.outIdx, id)) return;
+        }
+        std::vector<int> tile;
+        for (int id : s.out.idx)
+        {
+            if (id != batch && !has(p.lane, id) && !has(tile, id)) tile.push_back(id);
+        }
+        if (s.matrixOp == 1 && tile != std::vector<int>(s.out.idx.end() - 2, s.out.idx.end())) return;
+        if (s.matrixOp == 2 && !tile.empty()) return;
+        const long tc = product(tile, extent);
+        if (tc > kMaxTile || tc * s.contrCount * static_cast<long>(s.in.size()) > kUnrollBudget) return;
+        std::vector<char> fwd(s.in.size(), 0);
+        bool any = false;
+        for (size_t v = 0; v < s.in.size(); ++v)
+        {
+            const VarRef &r = s.in[v];
+            for (int q = k - 1; q >= chainStart; --q)
+            {
+                if (!ViewsOverlap(subs[q].out.uvar, r.uvar)) continue;
+                if (!ForwardableFrom(subs[q], r, p.lane)) return;  // it would have to wait for the stored copy
+                fwd[v] = 1;
+                any = true;
+                break;
+            }
+        }
+        if (!any) return;
+        for (int q = chainStart; q < k; ++q)
+        {
+            if (ViewsOverlap(subs[q].out.uvar, s.out.uvar)) return;
+            for (const auto &r : subs[q].in)
+            {
+                if (ViewsOverlap(r.uvar, s.out.uvar)) return;  // other work items may still read what this one would overwrite
+            }
+        }
+        s.fusedWithPrev = true;
+        s.forwardedIn = fwd;
+        s.lane = p.lane;
+        s.laneCount = p.laneCount;
+        s.tile = tile;
+        s.tileCount = tc;
+    }
+
     void PlanFusion()
     {
         const int K = static_cast<int>(subs.size());
+        int chainStart = 0;
         for (int k = 1; k < K; ++k)
         {
             Sub &s = subs[k];
             const Sub &p = subs[k - 1];
-            if (!s.contr.empty() || p.loopMode || p.out.repeated || s.out.repeated) continue;
+            if (!p.fusedWithPrev) chainStart = k - 1;
+            if (s.matrixOp != 0 || p.matrixOp != 0 || !s.contr.empty() || p.loopMode || p.out.repeated || s.out.repeated)
+            {
+                ForwardAlongChain(k, chainStart);
+                continue;
+            }
             std::set<int> a(s.outIdx.begin(), s.outIdx.end()), b(p.outIdx.begin(), p.outIdx.end());
-            if (a != b) continue;
             int fwd = -1;
-            for (size_t v = 0; v < s.in.size(); ++v)
+            for (size_t v = 0; v < s.in.size() && a == b; ++v)
             {
                 if (s.in[v].uvar == p.out.uvar && s.in[v].idx == p.out.idx) fwd = static_cast<int>(v);
             }
-            if (fwd < 0) continue;
             // Every other use of the producer's variable in this kernel would need the stored copy.
             bool other_use = (s.out.uvar == p.out.uvar);
             for (size_t v = 0; v < s.in.size(); ++v)
             {
                 if (static_cast<int>(v) != fwd && s.in[v].uvar == p.out.uvar) other_use = true;
             }
-            if (other_use) continue;
+            if (fwd < 0 || other_use)
+            {
+                ForwardAlongChain(k, chainStart);
+                continue;
+            }
             s.fusedWithPrev = true;
-            s.forwardedInput = fwd;
+            s.forwardedIn.assign(s.in.size(), 0);
+            s.forwardedIn[fwd] = 1;
             s.tile = p.tile;
             s.lane = p.lane;
             s.laneCount = p.laneCount;
@@ -918,7 +1035,7 @@ class Generator
             for (const auto &r : s.in) reads_it = reads_it || uvars[r.uvar].storage == uvars[p.out.uvar].storage;
             if (reads_it) continue;
             s.fusedWithPrev = true;
-            s.forwardedInput = -1;
+            s.forwardedIn.clear();
             s.forwardedOld = true;
         }
         AssignPhases();
@@ -985,7 +1102,10 @@ class Generator
         }
     }
 
-    bool FromRegisters(int k, int v) const { return subs[k].fusedWithPrev && subs[k].forwardedInput == v; }
+    bool FromRegisters(int k, int v) const
+    {
+        return subs[k].fusedWithPrev && static_cast<size_t>(v) < subs[k].forwardedIn.size() && subs[k].forwardedIn[v] != 0;
+    }
 
     int PhaseOf(int k) const { return subs[k].phase; }
 
@@ -1501,6 +1621,9 @@ class Generator
         return base;
     }
 
+    // Results that the kernels of a chain have left in registers: (operand, literal offset) -> register name.
+    typedef std::map<std::pair<int, long>, std::string> ForwardMap;
+
     struct Body
     {
         std::vector<std::string> bases;    // run-time base offsets
@@ -1524,7 +1647,7 @@ class Generator
     }
 
     std::string OperandExpr(int k, int v, const std::vector<int> &value, Body &body,
-                            const std::map<long, std::string> &forwarded)
+                            const ForwardMap &forwarded)
     {
         const Sub &s = subs[k];
         const VarRef &r = s.in[v];
@@ -1532,8 +1655,9 @@ class Generator
         const std::string tag = "k" + str(k) + "v" + str(v);
         if (src == kFromRegisters)
         {
-            // Same index names in the same order as the producer's output: its literal offset names the value.
-            return forwarded.at(LiteralOffset(subs[k - 1].out, subs[k - 1], false, value));
+            // Same work item as the producer's: the literal part of the offset names the value.
+            if (s.matrixOp == 2 && r.uvar != subs[k - 1].out.uvar) return "det" + str(k - 1);
+            return forwarded.at(std::make_pair(r.uvar, LiteralOffset(r, s, false, value)));
         }
         if (src == kFromConstant)
         {
@@ -1563,7 +1687,7 @@ class Generator
     // Sum over the contraction indices deeper than `depth`, of the product of the factors that close at those
     // levels.  Returns the name of a temporary, or "" when the remaining sum is exactly one.
     std::string PartialSum(int k, int depth, std::vector<int> &value, Body &body, const std::vector<int> &level,
-                           const std::map<long, std::string> &forwarded)
+                           const ForwardMap &forwarded)
     {
         const Sub &s = subs[k];
         const int n = static_cast<int>(s.contr.size());
@@ -1789,7 +1913,7 @@ class Generator
 
     // Unrolled body of kernel k for one work item.  `forwarded` maps the literal output offsets of the previous
     // kernel to the registers holding them; on return it describes this kernel's outputs.
-    void EmitUnrolledBody(int k, std::map<long, std::string> &forwarded, std::vector<std::string> &lines,
+    void EmitUnrolledBody(int k, ForwardMap &forwarded, std::vector<std::string> &lines,
                           const std::map<std::string, std::string> *preloaded = nullptr,
                           std::vector<std::pair<std::string, std::string>> *globalLoads = nullptr)
     {
@@ -1808,7 +1932,21 @@ class Generator
             }
         }
 
-        std::map<long, std::string> produced;
+        if (s.matrixOp != 0)
+        {
+            EmitMatrixBody(k, body, forwarded);
+            // no multiply-add fusion: the results are bit-identical to the host formulas, as those of the precompiled
+            // batched matrix kernels are
+            lines.push_back("#pragma clang fp contract(off)");
+            lines.push_back("// " + s.text + (s.matrixOp == 1 ? "   (matrix inverse)" : "   (determinant)"));
+            for (const auto &l : body.bases) lines.push_back(l);
+            for (const auto &l : body.loads) lines.push_back(l);
+            for (const auto &l : body.compute) lines.push_back(l);
+            for (const auto &l : body.stores) lines.push_back(l);
+            if (globalLoads != nullptr) *globalLoads = body.globalLoads;
+            return;
+        }
+
         std::vector<int> value(nidx, 0);
         const long tc = s.tileCount;
         for (long t = 0; t < tc; ++t)
@@ -1848,21 +1986,112 @@ class Generator
             }
             else
             {
-                const std::string old = s.forwardedOld ? forwarded.at(goff) : (OldValueInLds(k) ? laddr : gaddr);
+                const std::string old = s.forwardedOld ? forwarded.at(std::make_pair(s.out.uvar, goff))
+                                                       : (OldValueInLds(k) ? laddr : gaddr);
                 body.compute.push_back("const double " + name + " = " + old + (s.op == '+' ? " + " : " - ") + rhs + ";");
             }
             if (NeedsLdsCopy(k)) body.stores.push_back(laddr + " = " + name + ";");
             if (StoresToGlobal(k) && !CopiesOutFromLds(k)) body.stores.push_back(GlobalStore(k, gaddr, name));
-            produced[goff] = name;
+            forwarded[std::make_pair(s.out.uvar, goff)] = name;
         }
 
+        // The scope of a kernel applied after a matrix kernel is nested in that kernel's: back to the default there.
+        for (int q = k; q > 0 && subs[q].fusedWithPrev; --q)
+        {
+            if (subs[q - 1].matrixOp == 0) continue;
+            lines.push_back("#pragma clang fp contract(fast)");
+            break;
+        }
         lines.push_back("// " + s.text);
         for (const auto &l : body.bases) lines.push_back(l);
         for (const auto &l : body.loads) lines.push_back(l);
         for (const auto &l : body.compute) lines.push_back(l);
         for (const auto &l : body.stores) lines.push_back(l);
-        forwarded.swap(produced);
         if (globalLoads != nullptr) *globalLoads = body.globalLoads;
+    }
+
+    // One work item of a matrix kernel: the entries of the operand's matrix are loaded like any operand, the
+    // formulas are those of the reference's host implementation (ops/NativeCPUOps.hpp:38-86), term by term in the
+    // same order (the compiler may still fuse a multiply and an add): det = A0 A4 A8 + A1 A5 A6 + A2 A3 A7 - A6 A4 A2
+    // - A7 A5 A0 - A8 A3 A1 (row-major entries), inverse entry (i, j) = cofactor laid out as the reference lays it
+    // out, times 1.0 / det.
+    void EmitMatrixBody(int k, Body &body, ForwardMap &forwarded)
+    {
+        const Sub &s = subs[k];
+        const int n = s.matrixN;
+        const VarRef &r = s.in[0];
+        const int rowId = r.idx[r.idx.size() - 2], colId = r.idx[r.idx.size() - 1];
+        const std::string detName = "det" + str(k);
+        const bool reuse = s.matrixOp == 2 && s.fusedWithPrev && subs[k - 1].matrixOp == 1;
+        std::vector<std::string> a(n * n);
+        std::vector<int> value(nidx, 0);
+        if (!reuse)
+        {
+            for (int i = 0; i < n; ++i)
+            {
+                for (int j = 0; j < n; ++j)
+                {
+                    value[rowId] = i;
+                    value[colId] = j;
+                    a[i * n + j] = OperandExpr(k, 0, value, body, forwarded);
+                }
+            }
+        }
+        auto mul = [](const std::string &x, const std::string &y) { return x + " * " + y; };
+        if (reuse)
+            body.compute.push_back("const double " + detName + " = det" + str(k - 1) + ";");
+        else if (n == 1)
+            body.compute.push_back("const double " + detName + " = " + a[0] + ";");
+        else if (n == 2)
+            body.compute.push_back("const double " + detName + " = " + mul(a[0], a[3]) + " - " + mul(a[1], a[2]) + ";");
+        else
+            body.compute.push_back("const double " + detName + " = " + a[0] + " * " + a[4] + " * " + a[8] + " + " + a[1] + " * " +
+                                   a[5] + " * " + a[6] + " + " + a[2] + " * " + a[3] + " * " + a[7] + " - " + a[6] + " * " + a[4] +
+                                   " * " + a[2] + " - " + a[7] + " * " + a[5] + " * " + a[0] + " - " + a[8] + " * " + a[3] + " * " +
+                                   a[1] + ";");
+
+        std::vector<std::string> result;  // right-hand sides in tile order (row-major entries of the output)
+        if (s.matrixOp == 2)
+        {
+            result.push_back(detName);
+        }
+        else
+        {
+            const std::string inv = "inv" + str(k);
+            body.compute.push_back("const double " + inv + " = 1.0 / " + detName + ";");
+            if (n == 1)
+            {
+                result = {inv};
+            }
+            else if (n == 2)
+            {
+                result = {inv + " * " + a[3], "-" + inv + " * " + a[1], "-" + inv + " * " + a[2], inv + " * " + a[0]};
+            }
+            else
+            {
+                auto cof = [&](int p, int q, int u, int v) { return inv + " * (" + mul(a[p], a[q]) + " - " + mul(a[u], a[v]) + ")"; };
+                result = {cof(4, 8, 5, 7), cof(5, 6, 3, 8), cof(3, 7, 4, 6), cof(2, 7, 1, 8), cof(0, 8, 2, 6),
+                          cof(1, 6, 0, 7), cof(1, 5, 2, 4), cof(2, 3, 0, 5), cof(0, 4, 1, 3)};
+            }
+        }
+        for (size_t t = 0; t < result.size(); ++t)
+        {
+            std::fill(value.begin(), value.end(), 0);
+            if (s.matrixOp == 1)
+            {
+                value[s.tile[0]] = static_cast<int>(t) / n;
+                value[s.tile[1]] = static_cast<int>(t) % n;
+            }
+            const long goff = LiteralOffset(s.out, s, false, value);
+            const long loff = StoreOf(s.out.uvar).inLds ? LiteralOffset(s.out, s, true, value) : 0;
+            const std::string gaddr = PtrName(s.out.uvar) + "[o_k" + str(k) + "g + " + Lit(goff) + "]";
+            const std::string laddr = "lds[o_k" + str(k) + "l + " + str(loff) + "]";
+            const std::string name = "r" + str(k) + "_" + str(static_cast<long>(t));
+            body.compute.push_back("const double " + name + " = " + result[t] + ";");
+            if (NeedsLdsCopy(k)) body.stores.push_back(laddr + " = " + name + ";");
+            if (StoresToGlobal(k) && !CopiesOutFromLds(k)) body.stores.push_back(GlobalStore(k, gaddr, name));
+            forwarded[std::make_pair(s.out.uvar, goff)] = name;
+        }
     }
 
     // Counted-loop body (long contractions): one output per work item, no tile.
@@ -2396,7 +2625,7 @@ class Generator
             for (auto &c : ph.chains)
             {
                 c.loads.assign(c.last - c.first + 1, {});
-                std::map<long, std::string> forwarded;
+                ForwardMap forwarded;
                 long perPass = 0;
                 for (int kk = c.first; kk <= c.last; ++kk)
                 {
@@ -2531,7 +2760,7 @@ class Generator
             for (long j = 0; j < npass; ++j)
             {
                 emitItems(ph, ph.prefetched ? j : -1, [&](const Chain &c, const std::string &indent) {
-                    std::map<long, std::string> forwarded;
+                    ForwardMap forwarded;
                     for (int kk = c.first; kk <= c.last; ++kk)
                     {
                         std::vector<std::string> lines;

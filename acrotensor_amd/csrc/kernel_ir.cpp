@@ -97,6 +97,26 @@ TensorKernel::TensorKernel(const std::string &kernel) : KernelStr(kernel)
     ParseKernel();
 }
 
+TensorKernel::TensorKernel(const std::string &kernel, const std::string &function) : KernelStr(kernel), Function(function)
+{
+    ParseKernel();
+    ACROBATIC_ASSERT(Function.empty() || Function == "inv" || Function == "det", "Unknown kernel function:  " + Function);
+    if (Function.empty()) return;
+    ACROBATIC_ASSERT(InputVars.size() == 1 && EqOperator == "=", "A matrix kernel assigns a function of one operand:  " + KernelStr);
+    const std::vector<std::string> &in = InputVars[0].IndexNames, &out = OutputVar.IndexNames;
+    ACROBATIC_ASSERT(in.size() >= 2 && in[in.size() - 1] != in[in.size() - 2], "A matrix kernel needs two distinct trailing indices:  " + KernelStr);
+    const std::vector<std::string> lead(in.begin(), in.end() - 2);
+    for (size_t a = 0; a < in.size(); ++a)
+    {
+        for (size_t b = a + 1; b < in.size(); ++b)
+            ACROBATIC_ASSERT(in[a] != in[b], "A matrix kernel cannot repeat an index:  " + KernelStr);
+    }
+    if (Function == "inv")
+        ACROBATIC_ASSERT(out == in, "The inverse carries the indices of its operand:  " + KernelStr);
+    else
+        ACROBATIC_ASSERT(out == lead, "The determinant carries the leading indices of its operand:  " + KernelStr);
+}
+
 void TensorKernel::ParseKernel()
 {
     std::string text;
@@ -246,6 +266,7 @@ std::string TensorKernel::GetNameString() const
     };
     std::string name = spell(OutputVar);
     name += (EqOperator == "=") ? "eq" : (EqOperator == "+=") ? "pe" : "me";
+    if (!Function.empty()) name += "fn" + Function;
     for (const auto &var : InputVars) name += spell(var);
     return name;
 }
@@ -294,6 +315,7 @@ std::vector<int> TensorKernel::GetLoopIdxSizes(Tensor *output, std::vector<Tenso
 DimensionedKernel::DimensionedKernel(TensorKernel *kernel, Tensor *output, std::vector<Tensor *> &inputs)
 {
     KernelStr = kernel->KernelStr;
+    Function = kernel->Function;
     OutputVar = kernel->OutputVar;
     EqOperator = kernel->EqOperator;
     InputVars = kernel->InputVars;

@@ -112,6 +112,31 @@ def other_workload(at, workloads, args):
         points = E * Q * Q * Q
         abytes, flops = points * (9 + 1 + 1 + 9) * 8, points * 9 * 3 * 5
         units, unit_name = points, "Gpoints/s"
+    elif name == "jdsetup":
+        # the same geometric factors straight from the Jacobians: inverse, determinant and the contraction recorded as
+        # one launch, Jinv and Jdet transient (they never reach device memory)
+        E, Q = 16384, 10
+        W, C, J = at.Tensor(Q, Q, Q), at.Tensor(E, Q, Q, Q), at.Tensor(E, Q, Q, Q, 3, 3)
+        Jinv, Jdet, D = at.Tensor(E, Q, Q, Q, 3, 3), at.Tensor(E, Q, Q, Q), at.Tensor(E, 3, 3, Q, Q, Q)
+        W.data[...] = workloads.counter_uniform(0xAC28, 0, (Q, Q, Q), 0.1, 1.0)
+        C.data[...] = workloads.counter_uniform(0xAC28, 1, (E, Q, Q, Q), 0.5, 1.5)
+        J.data[...] = workloads.counter_uniform(0xAC28, 2, (E, Q, Q, Q, 3, 3), -0.1, 0.1)
+        J.data[...] += [[1.0, 0.0, 0.0], [0.0, 1.0, 0.0], [0.0, 0.0, 1.0]]
+        for t in (Jinv, Jdet):
+            t.SetTransient(True)
+        for t in (W, C, J, Jinv, Jdet, D):
+            t.MoveToGPU()
+        k = "D_e_m_n_k1_k2_k3 = W_k1_k2_k3 C_e_k1_k2_k3 Jdet_e_k1_k2_k3 Jinv_e_k1_k2_k3_n_j Jinv_e_k1_k2_k3_m_j"
+
+        def step():
+            engine.BeginMultiKernelLaunch()
+            engine.BatchMatrixInvDet(Jinv, Jdet, J)
+            engine(k, D, W, C, Jdet, Jinv, Jinv)
+            engine.EndMultiKernelLaunch()
+        label = "geometric factor setup D[16384,3,3,10,10,10] from J, C, W in one launch (inverse and determinant in registers)"
+        points = E * Q * Q * Q
+        abytes, flops = points * (9 + 1 + 9) * 8, points * (9 * 3 * 5 + 54)
+        units, unit_name = points, "Gpoints/s"
     elif name in ("scatter", "sumgather"):
         # node vector <-> element vector of the headline mesh size: 64^3 hex elements of degree 3
         import numpy as np
@@ -180,7 +205,7 @@ def main():
     ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store-all", action="store_true")
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup"],
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup"],
                     help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
                          "remaining baseline configurations at their full sizes and for the node-vector <-> "
                          "element-vector steps either side of the operator apply")

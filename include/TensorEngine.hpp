@@ -58,7 +58,10 @@ class TensorEngine
 
     void Clear();
     bool IsGPUAvailable() { return isHipReady(); }
-    // Kernels issued between Begin and End are captured and executed as ONE fused launch by End.
+    // Kernels issued between Begin and End are captured and executed as ONE fused launch by End.  Batched matrix
+    // inverses and determinants issued in between are captured too when a later kernel of the capture reads their
+    // result: they become kernels of the fused launch, and a result marked transient never reaches device memory.
+    // (The reference runs them at once, kernel/TensorEngine.cpp:627-671; the order of operations is the same.)
     void BeginMultiKernelLaunch();
     void EndMultiKernelLaunch();
 
@@ -76,6 +79,21 @@ class TensorEngine
     void SwitchToComputeLocation(Tensor &T);
     void MoveToComputeLocation(IndexMapping &M);
     void ResetCapture();
+    // A batched matrix operation recorded inside a multi-kernel launch, ahead of captured kernel number `position`.
+    struct RecordedMatrixOp
+    {
+        size_t position;
+        Tensor *inverse;      // null for a determinant alone
+        Tensor *determinant;  // null for an inverse alone
+        Tensor *matrices;
+    };
+    // Executes the capture (or, with `implementation` set, only describes it).
+    void FinishCapture(std::string *implementation);
+    bool MatrixOpAsKernels(const RecordedMatrixOp &op, const std::vector<DimensionedKernel *> &kernels,
+                           const std::vector<Tensor *> &outputs, const std::vector<std::vector<Tensor *>> &inputs,
+                           std::vector<DimensionedKernel *> &op_kernels, std::vector<Tensor *> &op_outputs,
+                           std::vector<std::vector<Tensor *>> &op_inputs);
+    TensorKernel *GetAddTensorKernel(const std::string &kernel_str, const std::string &function);
 
     std::string ExecutorType;
     std::unordered_map<std::string, TensorKernel *> KernelMap;
@@ -89,6 +107,7 @@ class TensorEngine
     std::vector<DimensionedKernel *> MKLKernels;
     std::vector<Tensor *> MKLOutputT;
     std::vector<std::vector<Tensor *>> MKLInputT;
+    std::vector<RecordedMatrixOp> MKLMatrixOps;
     KernelExecutor *LastExecutor;
 };
 

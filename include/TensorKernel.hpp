@@ -33,6 +33,9 @@ class TensorKernel
   public:
     explicit TensorKernel(const char *kernel);
     explicit TensorKernel(const std::string &kernel);
+    // A kernel whose right-hand side is not a product but a function of its single operand's trailing matrix
+    // (see Function below).  Used by the engine for batched matrix operations recorded in a multi-kernel launch.
+    TensorKernel(const std::string &kernel, const std::string &function);
     virtual ~TensorKernel() {}
 
     int GetNumIndices() const { return static_cast<int>(AllIndexNames.size()); }
@@ -72,6 +75,12 @@ class TensorKernel
     std::vector<int> GetLoopIdxSizes(Tensor *output, std::vector<Tensor *> &inputs) const;
 
     std::string KernelStr;
+    // "" for a contraction.  "inv": "Ainv_..._m_n = A_..._m_n" writes, for every leading index, the inverse of the
+    // trailing m x n matrix (m = n <= 3) laid out as the reference's batched inverse lays it out
+    // (ops/NativeCPUOps.hpp:38-67).  "det": "Adet_... = A_..._m_n" writes its determinant (ops/NativeCPUOps.hpp:70-86).
+    // The reference has no such kernels: its engine runs these operations outside the kernel machinery
+    // (kernel/TensorEngine.cpp:627-671).
+    std::string Function;
     KernelVar OutputVar;
     std::string EqOperator;
     std::vector<KernelVar> InputVars;

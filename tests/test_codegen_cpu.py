@@ -200,6 +200,60 @@ def generated_sources(TE):
         at.Tensor(4, 5, 5, 5, 3, 3))
     yield "one name, two tensors", TE.GetImplementation("A_m_n = B_m_j B_n_j", at.Tensor(3, 3), at.Tensor(3, 4), at.Tensor(3, 4))
     yield "repeated output index", TE.GetImplementation("A_i_i = B_i", at.Tensor(6, 6), at.Tensor(6))
+    for transient in (True, False):
+        yield "geometric factors from the Jacobians", geometric_factor_source(TE, 7, 4, 3, transient)
+    yield "geometric factors, 2 x 2", geometric_factor_source(TE, 7, 3, 2, True)
+
+
+GEOMETRIC_FACTORS = {
+    3: "D_e_m_n_k1_k2_k3 = W_k1_k2_k3 C_e_k1_k2_k3 Jdet_e_k1_k2_k3 Jinv_e_k1_k2_k3_n_j Jinv_e_k1_k2_k3_m_j",
+    2: "D_e_m_n_k1_k2 = W_k1_k2 C_e_k1_k2 Jdet_e_k1_k2 Jinv_e_k1_k2_n_j Jinv_e_k1_k2_m_j",
+}
+
+
+def geometric_factor_source(TE, E, Q, dim, transient):
+    """Inverse and determinant of the Jacobians and the contraction that turns them into the geometric factors of the
+    diffusion operator (reference unittest/kernel/test_TensorEngine.cpp:498-590), recorded as one launch."""
+    pts = (Q,) * dim
+    J, Jinv, Jdet = at.Tensor(E, *pts, dim, dim), at.Tensor(E, *pts, dim, dim), at.Tensor(E, *pts)
+    W, C, D = at.Tensor(*pts), at.Tensor(E, *pts), at.Tensor(E, dim, dim, *pts)
+    Jinv.SetTransient(transient)
+    Jdet.SetTransient(transient)
+    TE.BeginMultiKernelLaunch()
+    TE.BatchMatrixInvDet(Jinv, Jdet, J)
+    TE(GEOMETRIC_FACTORS[dim], D, W, C, Jdet, Jinv, Jinv)
+    return TE.EndMultiKernelLaunchGetImplementation()
+
+
+def test_matrix_operations_recorded_in_a_launch_are_fused_with_their_reader(TE):
+    src = geometric_factor_source(TE, 64, 10, 3, True)
+    assert src.count("__global__") == 1 and "__syncthreads" not in src
+    assert "(matrix inverse)" in src and "(determinant)" in src
+    # one work item per quadrature point holds the inverse, its determinant and the nine geometric factors
+    assert "lanes(k1,k2,k3)=1000 tile(n,j)=9" in src and "lanes(k1,k2,k3)=1000 tile(m,n)=9 contraction=3" in src
+    assert "Jdet<-registers Jinv<-registers Jinv<-registers" in src
+    assert "Jinv->\n" in src and "Jdet->\n" in src and "D->global" in src      # transient results are never stored
+    assert "const double det1 = det0;" in src                                      # the determinant is computed once
+    assert src.count("#pragma clang fp contract(off)") == 2 and src.count("#pragma clang fp contract(fast)") == 1
+    stored = geometric_factor_source(TE, 64, 10, 3, False)
+    assert "Jinv->global" in stored and "Jdet->global" in stored and "Jinv<-registers" in stored
+
+
+def test_matrix_operation_without_a_reader_in_the_launch_runs_on_its_own(TE):
+    J, Jinv, Jdet = at.Tensor(8, 3, 3), at.Tensor(8, 3, 3), at.Tensor(8)
+    A, B = at.Tensor(8, 4), at.Tensor(8, 4)
+    TE.BeginMultiKernelLaunch()
+    TE("A_e_i = B_e_i", A, B)
+    TE.BatchMatrixInvDet(Jinv, Jdet, J)
+    src = TE.EndMultiKernelLaunchGetImplementation()
+    assert src.count("__global__") == 1 and "runs on its own" in src and "matrix inverse" not in src
+    # ... and so does one whose result is its own operand
+    X, V = at.Tensor(8, 3), at.Tensor(8, 3)
+    TE.BeginMultiKernelLaunch()
+    TE.BatchMatrixInverse(J, J)
+    TE("X_e_i = J_e_i_j V_e_j", X, J, V)
+    src = TE.EndMultiKernelLaunchGetImplementation()
+    assert "runs on its own" in src and "matrix inverse" not in src
 
 
 def test_every_kind_of_generated_kernel_compiles_for_gfx950(TE, monkeypatch):
