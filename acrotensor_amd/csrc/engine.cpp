@@ -310,6 +310,35 @@ void TensorEngine::FinishCapture(std::string *implementation)
         }
         ResetCapture();
     };
+    // A capture that a matrix operation splits into several launches keeps nothing on chip across them: for its
+    // duration no tensor counts as transient (a transient result of one launch may be an operand of the next).
+    struct KeepEverything
+    {
+        std::vector<Tensor *> marked;
+        void Add(Tensor *t)
+        {
+            if (t == nullptr || !t->IsTransient()) return;
+            t->SetTransient(false);
+            marked.push_back(t);
+        }
+        ~KeepEverything()
+        {
+            for (Tensor *t : marked) t->SetTransient(true);
+        }
+    } keep;
+    auto keepAll = [&]() {
+        for (size_t k = 0; k < kernels.size(); ++k)
+        {
+            keep.Add(outputs[k]);
+            for (Tensor *t : inputs[k]) keep.Add(t);
+        }
+        for (const auto &op : ops)
+        {
+            keep.Add(op.inverse);
+            keep.Add(op.determinant);
+            keep.Add(op.matrices);
+        }
+    };
     size_t next_op = 0;
     for (size_t k = 0; k <= kernels.size(); ++k)
     {
@@ -317,6 +346,7 @@ void TensorEngine::FinishCapture(std::string *implementation)
         {
             const RecordedMatrixOp &op = ops[next_op];
             if (MatrixOpAsKernels(op, kernels, outputs, inputs, MKLKernels, MKLOutputT, MKLInputT)) continue;
+            keepAll();
             flush();
             if (implementation != nullptr)
             {

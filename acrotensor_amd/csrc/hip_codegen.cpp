@@ -920,6 +920,28 @@ class Generator
         return true;
     }
 
+    // Kernel k is about to join the chain that starts at chainStart, with lane indices `lane`: the kernels of a chain
+    // run one after the other in the same work item without a barrier, so every operand of k that a kernel of the
+    // chain writes must be the work item's own entry, taken from registers.  Marks those operands in `fwd`; false
+    // when some operand would need another work item's result.
+    bool ChainOperandsFromRegisters(int k, int chainStart, const std::vector<int> &lane, std::vector<char> &fwd) const
+    {
+        const Sub &s = subs[k];
+        fwd.assign(s.in.size(), 0);
+        for (size_t v = 0; v < s.in.size(); ++v)
+        {
+            const VarRef &r = s.in[v];
+            for (int q = k - 1; q >= chainStart; --q)
+            {
+                if (!ViewsOverlap(subs[q].out.uvar, r.uvar)) continue;
+                if (!ForwardableFrom(subs[q], r, lane)) return false;
+                fwd[v] = 1;
+                break;
+            }
+        }
+        return true;
+    }
+
     // A kernel whose work items can be those of the previous kernel and that reads results of that kernel (or of
     // the kernels it is itself applied after) entry by entry is applied in the same registers: a pointwise kernel
     // after a contraction ("U = D T3"), but also a small contraction over the register tile of its producer
@@ -952,21 +974,9 @@ class Generator
         if (s.matrixOp == 2 && !tile.empty()) return;
         const long tc = product(tile, extent);
         if (tc > kMaxTile || tc * s.contrCount * static_cast<long>(s.in.size()) > kUnrollBudget) return;
-        std::vector<char> fwd(s.in.size(), 0);
-        bool any = false;
-        for (size_t v = 0; v < s.in.size(); ++v)
-        {
-            const VarRef &r = s.in[v];
-            for (int q = k - 1; q >= chainStart; --q)
-            {
-                if (!ViewsOverlap(subs[q].out.uvar, r.uvar)) continue;
-                if (!ForwardableFrom(subs[q], r, p.lane)) return;  // it would have to wait for the stored copy
-                fwd[v] = 1;
-                any = true;
-                break;
-            }
-        }
-        if (!any) return;
+        std::vector<char> fwd;
+        if (!ChainOperandsFromRegisters(k, chainStart, p.lane, fwd)) return;
+        if (std::find(fwd.begin(), fwd.end(), 1) == fwd.end()) return;
         for (int q = chainStart; q < k; ++q)
         {
             if (ViewsOverlap(subs[q].out.uvar, s.out.uvar)) return;
@@ -983,45 +993,51 @@ class Generator
         s.tileCount = tc;
     }
 
+    int ChainStartOf(int k) const
+    {
+        while (k > 0 && subs[k].fusedWithPrev) --k;
+        return k;
+    }
+
     void PlanFusion()
     {
         const int K = static_cast<int>(subs.size());
-        int chainStart = 0;
         for (int k = 1; k < K; ++k)
         {
             Sub &s = subs[k];
             const Sub &p = subs[k - 1];
-            if (!p.fusedWithPrev) chainStart = k - 1;
-            if (s.matrixOp != 0 || p.matrixOp != 0 || !s.contr.empty() || p.loopMode || p.out.repeated || s.out.repeated)
+            const int chainStart = ChainStartOf(k - 1);
+            // A pointwise kernel over the previous kernel's outputs takes over its lanes and register tile as they are.
+            bool pointwise = s.matrixOp == 0 && p.matrixOp == 0 && s.contr.empty() && !p.loopMode && !p.out.repeated && !s.out.repeated;
+            if (pointwise)
             {
-                ForwardAlongChain(k, chainStart);
-                continue;
+                std::set<int> a(s.outIdx.begin(), s.outIdx.end()), b(p.outIdx.begin(), p.outIdx.end());
+                bool reads = false;
+                for (const auto &r : s.in) reads = reads || (r.uvar == p.out.uvar && r.idx == p.out.idx);
+                pointwise = a == b && reads && s.out.uvar != p.out.uvar;
             }
-            std::set<int> a(s.outIdx.begin(), s.outIdx.end()), b(p.outIdx.begin(), p.outIdx.end());
-            int fwd = -1;
-            for (size_t v = 0; v < s.in.size() && a == b; ++v)
+            std::vector<char> fwd;
+            if (pointwise && ChainOperandsFromRegisters(k, chainStart, p.lane, fwd))
             {
-                if (s.in[v].uvar == p.out.uvar && s.in[v].idx == p.out.idx) fwd = static_cast<int>(v);
+                bool overwrites = false;  // an earlier kernel of the chain reads or writes what this one writes
+                for (int q = chainStart; q < k; ++q)
+                {
+                    overwrites = overwrites || ViewsOverlap(subs[q].out.uvar, s.out.uvar);
+                    for (const auto &r : subs[q].in) overwrites = overwrites || ViewsOverlap(r.uvar, s.out.uvar);
+                }
+                if (!overwrites)
+                {
+                    s.fusedWithPrev = true;
+                    s.forwardedIn = fwd;
+                    s.tile = p.tile;
+                    s.lane = p.lane;
+                    s.laneCount = p.laneCount;
+                    s.tileCount = p.tileCount;
+                    s.loopMode = false;
+                    continue;
+                }
             }
-            // Every other use of the producer's variable in this kernel would need the stored copy.
-            bool other_use = (s.out.uvar == p.out.uvar);
-            for (size_t v = 0; v < s.in.size(); ++v)
-            {
-                if (static_cast<int>(v) != fwd && s.in[v].uvar == p.out.uvar) other_use = true;
-            }
-            if (fwd < 0 || other_use)
-            {
-                ForwardAlongChain(k, chainStart);
-                continue;
-            }
-            s.fusedWithPrev = true;
-            s.forwardedIn.assign(s.in.size(), 0);
-            s.forwardedIn[fwd] = 1;
-            s.tile = p.tile;
-            s.lane = p.lane;
-            s.laneCount = p.laneCount;
-            s.tileCount = p.tileCount;
-            s.loopMode = false;
+            ForwardAlongChain(k, chainStart);
         }
         // Accumulation chains ("Y = ...", "Y += ...", "Y += ..."): a kernel that adds into exactly what the previous
         // kernel produced, with the same pencil decomposition, takes the old value from that kernel's registers.
@@ -1031,11 +1047,10 @@ class Generator
             const Sub &p = subs[k - 1];
             if (s.fusedWithPrev || s.op == '=' || s.loopMode || p.loopMode || s.out.repeated) continue;
             if (s.out.uvar != p.out.uvar || s.out.idx != p.out.idx || s.tile != p.tile || s.lane != p.lane) continue;
-            bool reads_it = false;
-            for (const auto &r : s.in) reads_it = reads_it || uvars[r.uvar].storage == uvars[p.out.uvar].storage;
-            if (reads_it) continue;
+            std::vector<char> fwd;
+            if (!ChainOperandsFromRegisters(k, ChainStartOf(k - 1), p.lane, fwd)) continue;
             s.fusedWithPrev = true;
-            s.forwardedIn.clear();
+            s.forwardedIn = fwd;
             s.forwardedOld = true;
         }
         AssignPhases();
@@ -1901,6 +1916,7 @@ class Generator
         if (envInt("ACRO_HIP_LDS_COPY_OUT") < 0 || envInt("ACRO_HIP_PERSIST") > 0 || envInt("ACRO_HIP_LDS_PAD") > 0) return false;
         const Sub &s = subs[k];
         if (!NeedsLdsCopy(k) || !StoresToGlobal(k) || s.out.repeated) return false;
+        if (s.phase == subs.back().phase) return false;  // the copy runs after the barrier that ends the phase: the last has none
         const UVarInfo &u = uvars[s.out.uvar];
         const Storage &st = stores[u.storage];
         if (st.members.size() != 1 || st.batchDim != 0 || !u.fixed.empty() || u.viewOffset != 0) return false;

@@ -121,6 +121,62 @@ def test_random_chains_with_every_possible_kernel_reordered(at, engine, checker,
     run_random_chain(at, engine, checker, 7000 + seed)
 
 
+def forward_chain(rng):
+    """Random chain whose kernels all enumerate the same work items (the batch index e plus up to two more indices):
+    later kernels read earlier results entry by entry, under their own or other small index names, also twice and
+    also as the operand of a contraction, so the generator can apply them in the producer's registers.  Now and then
+    a batched matrix inverse or determinant of an earlier result joins the chain.
+    Returns (steps, shapes, produced names, names holding matrices); a step is (kernel string | "inv" | "det", out, ins)."""
+    items = ["e"] + list(rng.choice(["u", "v"], size=int(rng.integers(0, 3)), replace=False))
+    extent = {"e": int(rng.integers(1, 40)), "u": int(rng.integers(1, 7)), "v": int(rng.integers(1, 7))}
+    m = int(rng.integers(1, 4))                    # every small index has this extent, so that any may rename any
+    small = list("abcdfg")
+    for n in small:
+        extent[n] = m
+    shapes, produced, steps, mats = {}, [], [], set()
+    dims = {}                                       # produced name -> number of small dimensions
+    for k in range(int(rng.integers(2, 6))):
+        out = "R%d" % k
+        if rng.random() < 0.3:
+            # a well-conditioned matrix per work item (the fresh input is filled with identity + noise), copied by a
+            # kernel of the chain, then inverted and / or its determinant taken
+            idx = items + list(rng.choice(small, size=2, replace=False))
+            shapes["M%d" % k] = shapes[out] = tuple(extent[i] for i in idx)
+            mats.add("M%d" % k)
+            dims[out] = 2
+            steps.append((out + "_" + "_".join(idx) + " = M%d_" % k + "_".join(idx), out, ["M%d" % k]))
+            produced.append(out)
+            which = int(rng.integers(0, 3))
+            if which != 1:
+                shapes[out + "i"], dims[out + "i"] = shapes[out], 2
+                steps.append(("inv", out + "i", [out]))
+                produced.append(out + "i")
+            if which != 0:
+                shapes[out + "d"], dims[out + "d"] = shapes[out][:-2], 0
+                steps.append(("det", out + "d", [out]))
+                produced.append(out + "d")
+            continue
+        out_small = list(rng.choice(small, size=int(rng.integers(0, 3)), replace=False))
+        ins, names = [], []
+        for p in (rng.choice(produced, size=min(len(produced), int(rng.integers(1, 3))), replace=False) if produced else []):
+            for _ in range(int(rng.integers(1, 3))):
+                idx = items + list(rng.choice(small, size=dims[p], replace=False))
+                ins.append(str(p) + "_" + "_".join(idx))
+                names.append(str(p))
+        for f in range(int(rng.integers(1, 3))):
+            name = "F%d%d" % (k, f)
+            idx = list(rng.choice(items + small, size=int(rng.integers(1, 4)), replace=False))
+            shapes[name] = tuple(extent[i] for i in idx)
+            ins.append(name + "_" + "_".join(idx))
+            names.append(name)
+        op = "=" if rng.random() < 0.8 else "+="
+        shapes[out] = tuple(extent[i] for i in items + out_small)
+        dims[out] = len(out_small)
+        steps.append((out + "_" + "_".join(items + out_small) + " " + op + " " + " ".join(ins), out, names))
+        produced.append(out)
+    return steps, shapes, produced, mats
+
+
 def run_random_chain(at, engine, checker, seed):
     rng = np.random.default_rng(seed)
     strings, shapes, produced = random_chain(rng)
@@ -144,3 +200,47 @@ def run_random_chain(at, engine, checker, seed):
             continue
         tensors[n].MoveFromGPU()
         assert rel_err(tensors[n].data, expected[n]) <= TOL, n
+
+
+def run_forward_chain(at, engine, checker, seed):
+    rng = np.random.default_rng(seed)
+    steps, shapes, produced, mats = forward_chain(rng)
+    for s in steps:
+        print(s, flush=True)
+    arrays = {n: np.eye(shp[-1]) + 0.2 * rng.uniform(-1, 1, shp) if n in mats else rng.uniform(-1, 1, shp)
+              for n, shp in shapes.items()}
+    transient = [n for n in produced[:-1] if rng.random() < 0.5]
+    tensors = {n: to_tensor(at, a) for n, a in arrays.items()}
+    for n in transient:
+        tensors[n].SetTransient(True)
+    engine.BeginMultiKernelLaunch()
+    for s, out, ins in steps:
+        if s == "inv":
+            engine.BatchMatrixInverse(tensors[out], tensors[ins[0]])
+        elif s == "det":
+            engine.BatchMatrixDet(tensors[out], tensors[ins[0]])
+        else:
+            engine(s, tensors[out], *[tensors[i] for i in ins])
+    engine.EndMultiKernelLaunch()
+    expected = {n: a.copy() for n, a in arrays.items()}
+    for s, out, ins in steps:
+        if s == "inv":
+            expected[out][...] = checker.batch_matrix_inv_det(expected[ins[0]])[0]
+        elif s == "det":
+            expected[out][...] = checker.batch_matrix_inv_det(expected[ins[0]])[1]
+        else:
+            checker.contract(s, expected[out], *[expected[i] for i in ins])
+    for n in produced:
+        if n in transient:
+            continue
+        tensors[n].MoveFromGPU()
+        assert rel_err(tensors[n].data, expected[n]) <= 10 * TOL, n     # products of up to six factors
+    return engine.GetLastImplementation()
+
+
+@pytest.mark.parametrize("seed", range(45))
+def test_random_chains_over_the_same_work_items(at, engine, checker, seed):
+    # kernels applied in the registers of their producers, matrix inverses and determinants among them; seed 41 is a
+    # capture that a matrix operation without reader splits into three launches while a transient result of the
+    # first is an operand of the last
+    run_forward_chain(at, engine, checker, 90000 + seed)
