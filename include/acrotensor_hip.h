@@ -104,6 +104,9 @@ int acro_engine_set_executor_type(acro_engine *e, const char *exec_type);
 /* TensorEngine::operator()(kernel_str, out, inputs)  (kernel/TensorEngine.cpp:290-315) */
 int acro_engine_contract(acro_engine *e, const char *kernel, acro_tensor *out, acro_tensor *const *inputs,
                          int num_inputs);
+/* Between begin and end, acro_engine_batch_matrix_inverse / _det / _inv_det are recorded as well and run at end, in
+ * program order with the recorded kernels; an operation whose result a later recorded kernel reads is fused into the
+ * launch (the reference runs these operations at the call, kernel/TensorEngine.cpp:627-671). */
 int acro_engine_begin_multi_kernel_launch(acro_engine *e); /* kernel/TensorEngine.cpp:318-325 */
 int acro_engine_end_multi_kernel_launch(acro_engine *e);   /* kernel/TensorEngine.cpp:328-336 */
 /* TensorEngine::GetImplementation: copies the generated HIP source (NUL terminated, truncated to buflen) and
