@@ -262,6 +262,26 @@ static void gpuTests()
             for (int i = 0; i < 3; ++i)
                 for (int j = 0; j < 3; ++j) identity = identity && approx(I(b, i, j) + 1.0, (i == j ? 2.0 : 1.0));
         CHECK(identity);
+        // the same two steps recorded as one launch: the inverse becomes a kernel of the group and stays in registers
+        Tensor Ainv2(n, 3, 3), Adet2(n), I2(n, 3, 3);
+        Ainv2.SetTransient(true);
+        TE.BeginMultiKernelLaunch();
+        TE.BatchMatrixInvDet(Ainv2, Adet2, A);
+        TE("I_b_i_k = TI_b_j_i T_b_j_k", I2, Ainv2, A);
+        TE.EndMultiKernelLaunch();
+        CHECK(TE.GetLastImplementation().find("(matrix inverse)") != std::string::npos);
+        CHECK(TE.GetLastImplementation().find("TI<-registers") != std::string::npos);
+        I2.MoveFromGPU();
+        Adet2.MoveFromGPU();
+        Adet.MoveFromGPU();
+        bool same = true;
+        for (int b = 0; b < n; ++b)
+        {
+            same = same && Adet2(b) == Adet(b);
+            for (int i = 0; i < 3; ++i)
+                for (int j = 0; j < 3; ++j) same = same && I2(b, i, j) == I(b, i, j);
+        }
+        CHECK(same);
         Tensor bad(n, 4, 4);
         CHECK_THROWS(TE.BatchMatrixInverse(bad, bad));
 
