@@ -28,6 +28,8 @@
 //                               2: reorder whenever a chain is cheaper at all (default: only large kernels, 4x gain)
 //   ACRO_HIP_LDS_COPY_OUT=-1    stored results that also live in LDS are written by the lanes that computed them instead
 //                               of by the workgroup from the LDS tiles
+//   ACRO_HIP_FORWARD=-1         only a pointwise kernel directly after its producer is applied in that kernel's registers
+//                               (no contractions over the producer's register tile, no matrix kernels joined to readers)
 //   ACRO_HIP_RED_PENCIL=-1      split contractions: one lane per (slice, output entry) also when there are few outputs
 //   ACRO_HIP_ONE_PASS=1         split contractions: the workgroup that finishes last adds the per-workgroup partials
 //                               instead of a second kernel (measured 18.4 against 16.3 us: the device-scope release

@@ -176,3 +176,42 @@ def test_recorded_matrix_operations_replay_from_a_recorded_launch_sequence(at, e
         recording.launch()
         D.MoveFromGPU()
         assert rel_err(D.data, expected) <= TOL
+
+
+def test_geometric_factors_at_full_size(at, engine, checker):
+    # E = 16384 elements of 10^3 points (the size bench.py measures): a sample of elements against the checker, and
+    # on every point the symmetry of D and its closed form where the Jacobian is diagonal
+    E, Q = 16384, 10
+    rng = np.random.default_rng(77)
+    J = rng.uniform(-0.2, 0.2, (E, Q, Q, Q, 3, 3))
+    J[..., 0, 0] += 1.0
+    J[..., 1, 1] += 1.5
+    J[..., 2, 2] += 2.0
+    diagonal = np.arange(0, E, 97)                  # these elements get diagonal Jacobians
+    for a in range(3):
+        for b in range(3):
+            if a != b:
+                J[diagonal, ..., a, b] = 0.0
+    W, C = rng.uniform(0.1, 1.0, (Q, Q, Q)), rng.uniform(0.5, 1.5, (E, Q, Q, Q))
+    tJ, tW, tC = to_tensor(at, J), to_tensor(at, W), to_tensor(at, C)
+    Jinv, Jdet, D = at.Tensor(E, Q, Q, Q, 3, 3), at.Tensor(E, Q, Q, Q), at.Tensor(E, 3, 3, Q, Q, Q)
+    Jinv.SetTransient(True)
+    Jdet.SetTransient(True)
+    print("launch", flush=True)
+    engine.BeginMultiKernelLaunch()
+    engine.BatchMatrixInvDet(Jinv, Jdet, tJ)
+    engine(GEOMETRIC_FACTORS[3], D, tW, tC, Jdet, Jinv, Jinv)
+    engine.EndMultiKernelLaunch()
+    D.MoveFromGPU()
+    got = D.data
+    assert np.array_equal(got, got.transpose(0, 2, 1, 3, 4, 5))          # D_mn = D_nm, bit for bit
+    sample = np.unique(np.concatenate([[0, 1, E // 2, E - 1], rng.integers(0, E, 12)]))
+    _, _, expected = expected_factors(checker, 3, np.ascontiguousarray(J[sample]), W, np.ascontiguousarray(C[sample]))
+    assert rel_err(got[sample], expected) <= TOL
+    d = np.stack([J[diagonal, ..., a, a] for a in range(3)], axis=1)     # [elements, 3, Q, Q, Q]
+    closed = (W * C[diagonal] * d[:, 0] * d[:, 1] * d[:, 2])[:, None] / d ** 2
+    for a in range(3):
+        assert rel_err(got[diagonal, a, a], closed[:, a]) <= TOL
+        for b in range(3):
+            if a != b:
+                assert not got[diagonal, a, b].any()
