@@ -795,6 +795,48 @@ class Generator
         return perEntry <= 4096;
     }
 
+    // Loads per work item as LoadsPerItem counts them, except for streaming inputs (never written by the group,
+    // addressed through the batch index) whose lanes are far apart in memory: their loads are counted as the 16-byte
+    // instructions they become, each weighing as many times more as it touches more than 16 lines (four times what
+    // a coalesced one touches), if that is more than the plain count.  Measured with one lane per 4 x 4 matrix product against one lane per row: 44.6 against 88.7 % of the HBM
+    // peak; "A_e_i = B_e_i_j C_e_j" with 8 x 8: 38.1 against 75.8 %.
+    double AccessCostPerItem(const Sub &s, const std::vector<int> &tile) const
+    {
+        std::vector<int> lanes;
+        for (int id : s.out.idx)
+        {
+            if (id != batch && !has(tile, id) && !has(lanes, id)) lanes.push_back(id);
+        }
+        double cost = 0.0;
+        for (const auto &r : s.in)
+        {
+            if (IsUniform(s, r, tile)) continue;
+            std::set<int> seen;
+            long n = 1;
+            for (int id : r.idx)
+            {
+                if ((has(tile, id) || has(s.contr, id)) && seen.insert(id).second) n *= extent[id];
+            }
+            const bool streams = IsPureInput(r.uvar) && has(r.idx, batch);
+            if (!streams)
+            {
+                cost += static_cast<double>(n);
+                continue;
+            }
+            // trailing dimensions that the work item walks through are contiguous: pairs become 16-byte loads
+            long chunk = 1;
+            for (size_t d = r.idx.size(); d-- > 0;)
+            {
+                const int id = r.idx[d];
+                if (id == batch || has(lanes, id)) break;
+                chunk *= r.ext[d];
+            }
+            const double instructions = static_cast<double>(n) / chunk * ((chunk + 1) / 2);
+            cost += std::max(static_cast<double>(n), instructions * LinesPerInstruction(s, r, lanes) / 16.0);
+        }
+        return cost;
+    }
+
     long LoadsPerItem(const Sub &s, const std::vector<int> &tile) const
     {
         long loads = 0;
@@ -810,6 +852,80 @@ class Generator
             loads += n;
         }
         return loads;
+    }
+
+    // Doubles of streaming operands (inputs that carry the batch index) that one wavefront keeps coming back to: an
+    // operand whose fastest dimension is not a lane index is read by each lane in pieces, so the lines that one load
+    // instruction touches are touched again by the lane's next loads and have to stay in the CU's 32 KB vector cache
+    // in between.  ("A_e_i = B_e_i_j C_e_j" with one lane per entry: 64 lanes x 576 bytes.)
+    long WaveFootprint(const Sub &s, const std::vector<int> &tile) const
+    {
+        std::vector<int> lanes;
+        for (int id : s.outIdx)
+        {
+            if (id != batch && !has(tile, id)) lanes.push_back(id);
+        }
+        const long perEntry = std::max<long>(1, product(lanes, extent));
+        const long entriesPerWave = batch < 0 ? 1 : std::max<long>(1, 64 / perEntry);
+        long footprint = 0;
+        for (const auto &r : s.in)
+        {
+            if (!IsPureInput(r.uvar) || !has(r.idx, batch) || IsUniform(s, r, tile) || has(lanes, r.idx.back())) continue;
+            std::set<int> seen;
+            long perItem = 1, laneSpan = 1;
+            for (int id : r.idx)
+            {
+                if (id == batch || !seen.insert(id).second) continue;
+                (has(lanes, id) ? laneSpan : perItem) *= extent[id];
+            }
+            footprint += std::min<long>(64, laneSpan * entriesPerWave) * perItem;
+        }
+        return footprint;
+    }
+
+    // Average number of 128-byte lines that one load (or store) instruction of the first wavefront touches for
+    // occurrence r, the 64 work items being numbered as the emitted code numbers them (batch entries slowest, the
+    // last lane index fastest).  Four lines is a fully coalesced access; an operand read in pieces of 8 bytes at a
+    // stride of 72 touches 36, and the memory pipeline works through them one by one.
+    double LinesPerInstruction(const Sub &s, const VarRef &r, const std::vector<int> &lanes) const
+    {
+        std::vector<int> literal;  // tile and contraction indices of the occurrence
+        for (int id : r.idx)
+        {
+            if (id != batch && !has(lanes, id) && !has(literal, id)) literal.push_back(id);
+        }
+        const long combos = product(literal, extent), perEntry = std::max<long>(1, product(lanes, extent));
+        const long step = std::max<long>(1, combos / 32);  // a sample of the literal offsets is enough
+        std::vector<int> value(nidx, 0);
+        double total = 0.0;
+        long counted = 0;
+        for (long c = 0; c < combos; c += step, ++counted)
+        {
+            long rem = c;
+            for (int j = static_cast<int>(literal.size()) - 1; j >= 0; --j)
+            {
+                value[literal[j]] = static_cast<int>(rem % extent[literal[j]]);
+                rem /= extent[literal[j]];
+            }
+            std::set<long> lines;
+            for (long w = 0; w < 64; ++w)
+            {
+                const long b = w / perEntry;
+                if (b > 0 && (batch < 0 || b >= E)) break;
+                long rest = w % perEntry;
+                for (int j = static_cast<int>(lanes.size()) - 1; j >= 0; --j)
+                {
+                    value[lanes[j]] = static_cast<int>(rest % extent[lanes[j]]);
+                    rest /= extent[lanes[j]];
+                }
+                if (batch >= 0) value[batch] = static_cast<int>(b);
+                long a = 0;
+                for (size_t d = 0; d < r.idx.size(); ++d) a += static_cast<long>(value[r.idx[d]]) * r.stride[d];
+                lines.insert(a >> 4);
+            }
+            total += static_cast<double>(lines.size());
+        }
+        return counted > 0 ? total / static_cast<double>(counted) : 1.0;
     }
 
     static constexpr long kUnrollBudget = 8192;   // multiply-adds emitted per work item (before hoisting)
@@ -858,13 +974,25 @@ class Generator
                     const long loads = LoadsPerItem(s, t);
                     if (loads + tc > kMaxLiveValues && !t.empty()) continue;
                     // loads per produced output; a small bias keeps the tile short when nothing is gained
-                    double score = static_cast<double>(loads) / tc + 1e-3 * t.size() + 1e-6 * tc;
+                    const double cost = envInt("ACRO_HIP_FOOTPRINT") >= 0 ? AccessCostPerItem(s, t) : static_cast<double>(loads);
+                    double score = cost / tc + 1e-3 * t.size() + 1e-6 * tc;
+                    // ... unless the wavefront's working set of partly used lines outgrows its share of the vector cache
+                    const long footprint = WaveFootprint(s, t);
+                    if (footprint > 512 && envInt("ACRO_HIP_FOOTPRINT") >= 0) score *= static_cast<double>(footprint) / 512.0;
                     if (score < bestScore)
                     {
                         bestScore = score;
                         best = t;
                     }
                 }
+                // A kernel on its own whose batch entries are tiny (at most 32 outputs, every operand streaming):
+                // one output per lane.  The lanes of a wavefront then share the few lines of a handful of entries and
+                // every access is coalesced, which outweighs the extra loads (batched 4 x 4 matrix products: 88.7 %
+                // of the HBM peak against 55.5 % with a row per lane and 44.6 % with a product per lane; 3 x 3:
+                // 64.6 / 58.5 / 53.8 %).
+                bool streamingOnly = subs.size() == 1 && batch >= 0 && envInt("ACRO_HIP_FOOTPRINT") >= 0;
+                for (const auto &r : s.in) streamingOnly = streamingOnly && has(r.idx, batch) && !r.repeated;
+                if (streamingOnly && product(mid, extent) <= 32 && s.contrCount * nin <= 16) best.clear();
                 s.tile = best;
             }
             SetLanes(s);
