@@ -97,6 +97,7 @@ struct Storage
     int liveTo = -1;              // last kernel that reads the tile from LDS
     int phaseFrom = 0, phaseTo = 0;  // lifetime in barrier-separated phases (fused kernels share a phase)
     bool elide = false;           // no store to device memory
+    bool staged = false;          // small input without batch index: every workgroup copies it to LDS before it starts
 };
 
 long product(const std::vector<int> &ids, const std::vector<int> &extent)
@@ -1260,8 +1261,10 @@ class Generator
             st.wantLds = false;
             st.inLds = false;
             st.liveTo = -1;
+            st.staged = false;
         }
         if (batch < 0) return;
+        ChooseStagedInputs();
         for (size_t si = 0; si < stores.size(); ++si)
         {
             Storage &st = stores[si];
@@ -1288,6 +1291,71 @@ class Generator
         }
     }
 
+    // A small operand that does not depend on the batch entry but whose address depends on the lane
+    // ("A_e_i = B_i_j X_e_j" with one lane per i: lane i walks along row i of B, 512 bytes from its neighbour's) cannot
+    // be read with scalar loads, and read from device memory every load instruction touches 64 lines, which the
+    // memory pipeline works through one by one (measured 3 % of the HBM peak for that kernel with a 64 x 64 B).  Every
+    // workgroup copies such an operand into LDS once, with coalesced loads, and its lanes read it there; the stride of
+    // the lanes in LDS is made odd so that they fall into different banks.
+    static constexpr long kMaxStagedDoubles = 4096;
+
+    void ChooseStagedInputs()
+    {
+        if (envInt("ACRO_HIP_STAGE") < 0 || envInt("ACRO_HIP_PERSIST") > 0 || !opt.noalias) return;
+        const int K = static_cast<int>(subs.size());
+        for (size_t si = 0; si < stores.size(); ++si)
+        {
+            Storage &st = stores[si];
+            if (st.written || st.members.size() != 1 || st.anyRepeated) continue;
+            const UVarInfo &u = uvars[st.members[0]];
+            if (!u.consistent || !u.batchDims.empty() || !u.plainView || !u.fixed.empty() || u.isVirtual) continue;
+            if (u.size > kMaxStagedDoubles || u.size < 64) continue;
+            bool ok = true, farApart = false;
+            int first = -1, last = -1, laneDim = -1;
+            for (int k = 0; k < K && ok; ++k)
+            {
+                const Sub &sk = subs[k];
+                for (size_t v = 0; v < sk.in.size() && ok; ++v)
+                {
+                    const VarRef &r = sk.in[v];
+                    if (uvars[r.uvar].storage != static_cast<int>(si)) continue;
+                    if (sk.loopMode || sk.matrixOp != 0 || IsUniform(sk, r, sk.tile)) ok = false;
+                    if (!ok) break;
+                    if (first < 0)
+                    {
+                        first = k;
+                        for (size_t d = 0; d < r.idx.size(); ++d)
+                        {
+                            if (has(sk.lane, r.idx[d])) laneDim = static_cast<int>(d);  // fastest dimension that a lane index addresses
+                        }
+                    }
+                    last = k;
+                    farApart = farApart || LinesPerInstruction(sk, r, sk.lane) >= 16.0;
+                }
+                if (uvars[sk.out.uvar].storage == static_cast<int>(si)) ok = false;
+            }
+            if (!ok || !farApart || first < 0 || laneDim < 0) continue;
+            st.staged = true;
+            st.wantLds = true;
+            st.liveTo = last;
+            st.phaseFrom = 0;
+            st.phaseTo = PhaseOf(last);
+            // row-major, with the run of the dimensions faster than the lanes' made odd
+            long run = 1;
+            st.ldsStride.assign(st.dims.size(), 0);
+            for (int d = static_cast<int>(st.dims.size()) - 1; d >= 0; --d)
+            {
+                if (d == laneDim && run % 2 == 0) run += 1;
+                st.ldsStride[d] = static_cast<int>(run);
+                run *= st.dims[d];
+            }
+            st.tileSize = static_cast<int>(run);
+        }
+    }
+
+    // Doubles of LDS that a storage's tiles take in a workgroup of nb batch entries.
+    int LdsNeed(const Storage &st, int nb) const { return st.tileSize * (st.staged ? 1 : nb); }
+
     // First-fit placement of the tiles that are live at the same time; returns doubles needed for nb entries.
     int PlaceLds(int nb)
     {
@@ -1305,7 +1373,7 @@ class Generator
         for (int si : order)
         {
             Storage &u = stores[si];
-            const int need = u.tileSize * nb;
+            const int need = LdsNeed(u, nb);
             int offset = 0;
             bool moved = true;
             while (moved)
@@ -1315,7 +1383,7 @@ class Generator
                 {
                     const Storage &p = stores[pj];
                     const bool timeOverlap = !(p.phaseTo < u.phaseFrom || u.phaseTo < p.phaseFrom);
-                    const int pneed = p.tileSize * nb;
+                    const int pneed = LdsNeed(p, nb);
                     const bool spaceOverlap = !(p.ldsOffset + pneed <= offset || offset + need <= p.ldsOffset);
                     if (timeOverlap && spaceOverlap)
                     {
@@ -1458,10 +1526,33 @@ class Generator
         // statically; otherwise shrink the batch, and finally leave the largest tiles in device memory.
         const int budgetDoubles = 64 * 1024 / 8;
         for (auto &st : stores) st.inLds = st.wantLds;
+        // An operand staged in LDS is copied once per workgroup: the workgroup must serve enough batch entries for
+        // that copy to stay small against what the entries themselves move (one entry per 256 doubles staged).
+        if (opt.force_nb <= 0 && envInt("ACRO_HIP_NB") <= 0 && batch >= 0)
+        {
+            long staged = 0;
+            for (const auto &st : stores) staged += (st.staged && st.inLds) ? uvars[st.members[0]].size : 0;
+            const long wanted = std::min<long>(std::min<long>(E, 32), (staged + 255) / 256);
+            if (wanted > NB)
+            {
+                NB = static_cast<int>(wanted);
+                if (static_cast<long>(NB) * maxLane > 2L * NT) NT = 256;
+            }
+        }
         while (true)
         {
             ldsDoubles = PlaceLds(NB);
             if (ldsDoubles <= budgetDoubles) break;
+            bool dropped = false;  // staged operands are the first to go back to device memory
+            for (auto &st : stores)
+            {
+                if (st.staged && st.inLds && !dropped)
+                {
+                    st.inLds = false;
+                    dropped = true;
+                }
+            }
+            if (dropped) continue;
             if (NB > 1 && opt.force_nb <= 0)
             {
                 NB /= 2;
@@ -1631,7 +1722,7 @@ class Generator
         for (size_t si = 0; si < stores.size(); ++si)
         {
             Storage &st = stores[si];
-            if (!st.inLds) continue;
+            if (!st.inLds || st.staged) continue;
             const int ndim = static_cast<int>(st.dims.size()) - 1;
             std::vector<int> pad(ndim, 0), bestPad(ndim, 0);
             int bestEntry = 0;
@@ -1703,7 +1794,9 @@ class Generator
         const Storage &st = StoreOf(r.uvar);
         std::string expr;
         auto add = [&](const std::string &term) { expr += (expr.empty() ? "" : " + ") + term; };
-        if (lds)
+        if (lds && st.staged)
+            add(str(st.ldsOffset + LdsViewOffset(r.uvar)));
+        else if (lds)
             add(str(st.ldsOffset + LdsViewOffset(r.uvar)) + " + b * " + str(st.tileSize));
         else if (u.viewOffset != 0)
             add(Lit(u.viewOffset));
@@ -1748,7 +1841,7 @@ class Generator
         const Sub &s = subs[k];
         const VarRef &r = s.in[v];
         if (FromRegisters(k, v)) return kFromRegisters;
-        if (StoreOf(r.uvar).inLds && readCovered[k][v]) return kFromLds;
+        if (StoreOf(r.uvar).inLds && (readCovered[k][v] || StoreOf(r.uvar).staged)) return kFromLds;
         if (IsUniform(s, r, s.tile)) return kFromConstant;
         return kFromGlobal;
     }
@@ -2698,6 +2791,29 @@ class Generator
             out << "    const int e0 = blockIdx.x * " << NB << ";\n    {\n";
 
         const bool guardBatch = (E % NB) != 0;
+
+        bool anyStaged = false;
+        for (size_t si = 0; si < stores.size(); ++si)
+        {
+            const Storage &st = stores[si];
+            if (!st.staged || !st.inLds) continue;
+            anyStaged = true;
+            const UVarInfo &u = uvars[st.members[0]];
+            out << "    {   // " << u.name << ": device memory -> LDS, once per workgroup\n";
+            out << "        for (int i = tid; i < " << u.size << "; i += " << NT << ")\n        {\n";
+            out << "            int r_ = i, a = " << st.ldsOffset << ";\n";
+            long natural = u.size;
+            for (size_t d = 0; d < st.dims.size(); ++d)
+            {
+                natural /= st.dims[d];
+                if (d + 1 < st.dims.size())
+                    out << "            a += (r_ / " << natural << ") * " << st.ldsStride[d] << "; r_ %= " << natural << ";\n";
+                else
+                    out << "            a += r_ * " << st.ldsStride[d] << ";\n";
+            }
+            out << "            lds[a] = T" << si << "[" << Lit(u.viewOffset) << " + i];\n        }\n    }\n";
+        }
+        if (anyStaged) out << "    __syncthreads();\n";
 
         // Work-item header: batch entry and lane indices of item `w` of the phase that kernel `ks` opens.
         auto emitHeader = [&](const Sub &s, const std::string &indent) {

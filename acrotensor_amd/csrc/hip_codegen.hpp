@@ -30,6 +30,9 @@
 //                               of by the workgroup from the LDS tiles
 //   ACRO_HIP_FORWARD=-1         only a pointwise kernel directly after its producer is applied in that kernel's registers
 //                               (no contractions over the producer's register tile, no matrix kernels joined to readers)
+//   ACRO_HIP_FOOTPRINT=-1       register tiles by loads per output alone (no weight for uncoalesced streaming loads, no
+//                               cache-footprint term, no one-output-per-lane rule for tiny batch entries)
+//   ACRO_HIP_STAGE=-1           small invariant operands with lane-dependent addresses stay in device memory (not staged in LDS)
 //   ACRO_HIP_RED_PENCIL=-1      split contractions: one lane per (slice, output entry) also when there are few outputs
 //   ACRO_HIP_ONE_PASS=1         split contractions: the workgroup that finishes last adds the per-workgroup partials
 //                               instead of a second kernel (measured 18.4 against 16.3 us: the device-scope release

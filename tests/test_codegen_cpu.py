@@ -147,6 +147,30 @@ def test_diffusion_chain_batching_follows_the_contractions_not_the_pointwise_ker
     assert src.count("__syncthreads()") == 6
 
 
+def test_small_invariant_operand_read_by_rows_is_staged_in_lds(TE):
+    # lane i walks along row i of B: from device memory every load instruction would touch 64 lines; each workgroup
+    # copies B to LDS once (row stride 65, so that the lanes fall into different banks) and serves 16 entries
+    src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
+    assert "B<-lds" in src and "// B: device memory -> LDS, once per workgroup" in src
+    assert "a += (r_ / 64) * 65" in src and "16 per workgroup of 256 lanes" in src
+    assert src.index("__syncthreads()") < src.index("// A_e_i = B_i_j X_e_j")
+    # a table that the lanes read at unit stride, or one read through scalar loads, is left where it is
+    assert "<-lds" not in TE.GetImplementation("A_e_i = B_j_i X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
+    assert "B<-scalar" in TE.GetImplementation("A_e_q_j = B_q_i X_e_i_j", at.Tensor(500, 5, 16), at.Tensor(5, 4), at.Tensor(500, 4, 16))
+
+
+def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE):
+    # one lane per matrix product would read 128-byte pieces 128 bytes apart; tiny entries get one output per lane
+    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 4, 4), at.Tensor(4096, 4, 4), at.Tensor(4096, 4, 4))
+    assert "lanes(i,k)=16 tile()=1" in src
+    # one lane per entry would read 512-byte rows 512 bytes apart and overflow the vector cache: one lane per row
+    src = TE.GetImplementation("A_e_i = B_e_i_j C_e_j", at.Tensor(4096, 8), at.Tensor(4096, 8, 8), at.Tensor(4096, 8))
+    assert "lanes(i)=8 tile()=1" in src
+    # 8 x 8 products keep a row of outputs per lane
+    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 8, 8), at.Tensor(4096, 8, 8), at.Tensor(4096, 8, 8))
+    assert "tile(k)=8" in src or "tile(i)=8" in src
+
+
 def test_views_that_cannot_be_resolved_fall_back(TE):
     # the same parent viewed with the element index in two different positions cannot be fused
     T = at.Tensor(4, 4)
@@ -200,6 +224,7 @@ def generated_sources(TE):
         at.Tensor(4, 5, 5, 5, 3, 3))
     yield "one name, two tensors", TE.GetImplementation("A_m_n = B_m_j B_n_j", at.Tensor(3, 3), at.Tensor(3, 4), at.Tensor(3, 4))
     yield "repeated output index", TE.GetImplementation("A_i_i = B_i", at.Tensor(6, 6), at.Tensor(6))
+    yield "operand staged in LDS", TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
     for transient in (True, False):
         yield "geometric factors from the Jacobians", geometric_factor_source(TE, 7, 4, 3, transient)
     yield "geometric factors, 2 x 2", geometric_factor_source(TE, 7, 3, 2, True)

@@ -404,3 +404,18 @@ def test_slice_of_a_slice_inside_a_fused_launch(at, engine):
     expected[1, 2] = A.data
     assert np.array_equal(P.data, expected)
     assert rel_err(R.data, expected[1].sum(axis=2)) <= TOL
+
+
+@pytest.mark.parametrize("kernel,shapes", [
+    ("A_e_i = B_i_j X_e_j", [(64, 64), (1000, 64)]),             # B staged in LDS, 16 entries per workgroup, ragged end
+    ("A_e_i = B_i_j X_e_j", [(40, 24), (3, 24)]),                # fewer entries than a workgroup would take
+    ("A_e_i_k = B_i_j C_k_l X_e_j_l", [(12, 10), (9, 11), (77, 10, 11)]),   # two staged tables, reordered into steps
+    ("A_e_i_k = B_e_i_j C_e_j_k", [(1001, 4, 4), (1001, 4, 4)]), # one output per lane
+    ("A_e_i_k = B_e_i_j C_e_j_k", [(333, 3, 3), (333, 3, 3)]),
+    ("A_e_i = B_e_i_j C_e_j", [(515, 8, 8), (515, 8)]),          # one lane per row
+])
+def test_kernels_whose_schedule_follows_the_memory_access_pattern(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(len(kernel) + shapes[-1][0])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    got, expected = run_single(at, engine, checker, kernel, np.zeros(output_shape(kernel, shapes)), *ins)
+    assert rel_err(got, expected) <= TOL
