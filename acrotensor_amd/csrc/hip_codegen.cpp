@@ -51,6 +51,9 @@ struct Sub
     // 0: contraction.  1: the output is the inverse of the operand's trailing matrix, 2: its determinant.
     int matrixOp = 0;
     int matrixN = 0;
+    // > 0: the kernel has one output per batch entry; that many adjacent lanes share its contraction and add their
+    // partial sums through lane exchanges
+    int splitLanes = 0;
     bool forwardedOld = false;  // the old value of a += / -= output is the previous kernel's result, in registers
     int phase = 0;              // barrier-separated phase the kernel runs in
     long laneCount = 1, tileCount = 1, contrCount = 1;
@@ -993,10 +996,32 @@ class Generator
                 // 64.6 / 58.5 / 53.8 %).
                 bool streamingOnly = subs.size() == 1 && batch >= 0 && envInt("ACRO_HIP_FOOTPRINT") >= 0;
                 for (const auto &r : s.in) streamingOnly = streamingOnly && has(r.idx, batch) && !r.repeated;
-                if (streamingOnly && product(mid, extent) <= 32 && s.contrCount * nin <= 16) best.clear();
+                const long outputs = product(mid, extent), loadsPerOutput = s.contrCount * nin;
+                if (streamingOnly && ((outputs <= 32 && loadsPerOutput <= 16) || (outputs <= 64 && loadsPerOutput <= 4))) best.clear();
                 s.tile = best;
             }
             SetLanes(s);
+            // One output per batch entry ("A_e = B_e_i C_e_i", "A_e = B_e_n"): with one lane per entry every lane walks
+            // along its own rows, 8 bytes per line and load instruction (55 and 52 % of the HBM peak).  Instead a power
+            // of two of adjacent lanes shares the entry: lane c of them takes the terms c, c + lanes, ... of the
+            // flattened contraction, so that the lanes of a wavefront read consecutive addresses, and the partial sums
+            // are added in a butterfly of lane exchanges (a fixed order: results are reproducible).
+            if (subs.size() == 1 && batch >= 0 && mid.empty() && s.matrixOp == 0 && !s.out.repeated && s.contrCount >= 8 &&
+                envInt("ACRO_HIP_SPLIT_LANES") >= 0)
+            {
+                bool streams = false;  // some operand carries the batch index and the fastest contraction index last
+                for (const auto &r : s.in) streams = streams || (has(r.idx, batch) && r.idx.back() == s.contr.back());
+                if (streams)
+                {
+                    int lanes = 1;
+                    while (lanes * 2 <= 64 && lanes * 2 <= s.contrCount) lanes *= 2;
+                    s.splitLanes = lanes;
+                    s.loopMode = true;
+                    s.tile.clear();
+                    s.tileCount = 1;
+                    s.laneCount = lanes;
+                }
+            }
         }
     }
 
@@ -2332,9 +2357,78 @@ class Generator
     }
 
     // Counted-loop body (long contractions): one output per work item, no tile.
+    // One output per batch entry, its contraction shared by s.splitLanes adjacent lanes.
+    void EmitSplitLanesBody(int k, std::vector<std::string> &lines)
+    {
+        const Sub &s = subs[k];
+        Body body;
+        EmitBases(k, body);
+        const int L = s.splitLanes;
+        lines.push_back("// " + s.text + "   (contraction shared by " + str(L) + " lanes)");
+        for (const auto &l : body.bases) lines.push_back(l);
+        lines.push_back("const int cl = w & " + str(L - 1) + ";");
+        lines.push_back("double sum = 0.0;");
+        lines.push_back("#pragma unroll 4");
+        lines.push_back("for (int c = cl; c < " + str(s.contrCount) + "; c += " + str(L) + ")");
+        lines.push_back("{");
+        long st = s.contrCount;
+        for (size_t j = 0; j < s.contr.size(); ++j)
+        {
+            st /= extent[s.contr[j]];
+            const std::string name = IdxVar(s.contr[j]);
+            if (s.contr.size() == 1)
+                lines.push_back("    const int " + name + " = c;");
+            else if (j == 0)
+                lines.push_back("    const int " + name + " = c / " + str(st) + ";");
+            else
+                lines.push_back("    const int " + name + " = (c / " + str(st) + ") % " + str(extent[s.contr[j]]) + ";");
+        }
+        std::string prod;
+        for (size_t v = 0; v < s.in.size(); ++v)
+        {
+            const VarRef &r = s.in[v];
+            const Source src = SourceOf(k, static_cast<int>(v));
+            const bool lds = (src == kFromLds);
+            std::string off;
+            for (size_t d = 0; d < r.idx.size(); ++d)
+            {
+                const int id = r.idx[d];
+                if (!has(s.contr, id)) continue;
+                const long stride = lds ? LdsStride(r.uvar, d) : r.stride[d];
+                off += (off.empty() ? "" : " + ") + IdxVar(id) + " * " + (lds ? str(stride) : Lit(stride));
+            }
+            if (off.empty()) off = "0";
+            std::string opnd;
+            if (src == kFromConstant)
+                opnd = ConstPtrName(r.uvar) + "[" + ScalarBase(r) + Lit(uvars[r.uvar].viewOffset) + " + " + off + "]";
+            else if (lds)
+                opnd = "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
+            else
+                opnd = PtrName(r.uvar) + "[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
+            prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
+        }
+        lines.push_back("    sum += " + prod + ";");
+        lines.push_back("}");
+        // the lanes of an entry are adjacent and aligned, so every exchange partner works on the same entry
+        for (int m = L / 2; m >= 1; m /= 2) lines.push_back("sum += __shfl_xor(sum, " + str(m) + ", " + str(L) + ");");
+        const std::string gaddr = PtrName(s.out.uvar) + "[o_k" + str(k) + "g]";
+        lines.push_back("if (cl == 0)");
+        lines.push_back("{");
+        if (s.op == '=')
+            lines.push_back("    " + GlobalStore(k, gaddr, "sum"));
+        else
+            lines.push_back("    " + gaddr + " = " + gaddr + (s.op == '+' ? " + sum;" : " - sum;"));
+        lines.push_back("}");
+    }
+
     void EmitLoopBody(int k, std::vector<std::string> &lines)
     {
         const Sub &s = subs[k];
+        if (s.splitLanes > 0)
+        {
+            EmitSplitLanesBody(k, lines);
+            return;
+        }
         Body body;
         EmitBases(k, body);
         lines.push_back("// " + s.text + "   (contraction as counted loops)");

@@ -225,6 +225,7 @@ def generated_sources(TE):
     yield "one name, two tensors", TE.GetImplementation("A_m_n = B_m_j B_n_j", at.Tensor(3, 3), at.Tensor(3, 4), at.Tensor(3, 4))
     yield "repeated output index", TE.GetImplementation("A_i_i = B_i", at.Tensor(6, 6), at.Tensor(6))
     yield "operand staged in LDS", TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
+    yield "contraction shared by lanes", TE.GetImplementation("A_e += B_e_i_j C_j_i", at.Tensor(1000), at.Tensor(1000, 5, 7), at.Tensor(7, 5))
     for transient in (True, False):
         yield "geometric factors from the Jacobians", geometric_factor_source(TE, 7, 4, 3, transient)
     yield "geometric factors, 2 x 2", geometric_factor_source(TE, 7, 3, 2, True)

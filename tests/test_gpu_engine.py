@@ -419,3 +419,24 @@ def test_kernels_whose_schedule_follows_the_memory_access_pattern(at, engine, ch
     ins = [rng.uniform(-1, 1, s) for s in shapes]
     got, expected = run_single(at, engine, checker, kernel, np.zeros(output_shape(kernel, shapes)), *ins)
     assert rel_err(got, expected) <= TOL
+
+
+@pytest.mark.parametrize("kernel,shapes", [
+    ("A_e = B_e_i C_e_i", [(1003, 16), (1003, 16)]),             # 16 lanes per entry
+    ("A_e += B_e_i C_e_i", [(77, 9), (77, 9)]),                  # 8 lanes, 9 terms: lane 0 takes two
+    ("A_e -= B_e_n", [(301, 1000)]),                             # 64 lanes per entry
+    ("A_e = B_e_i_j C_j_i", [(130, 5, 7), (7, 5)]),              # two contraction indices, one operand transposed
+    ("A_e = B_e_i_j C_e_i_j D_j", [(64, 6, 4), (64, 6, 4), (4,)]),
+    ("A_e = B_i_e_j C_e_j", [(3, 50, 11), (50, 11)]),            # batch index in the middle of an operand
+])
+def test_one_output_per_batch_entry_shares_the_contraction_between_lanes(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(len(kernel) + shapes[0][0])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "contraction shared by" in engine.GetLastImplementation()
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected       # the checker adds for "-=", as the reference's interpreter does
+    assert rel_err(got, expected) <= TOL
+    again, _ = run_single(at, engine, checker, kernel, out0, *ins)
+    assert np.array_equal(got, again)                            # fixed order of the lane exchanges: reproducible
