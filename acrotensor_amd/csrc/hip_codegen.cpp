@@ -1005,21 +1005,38 @@ class Generator
             // along its own rows, 8 bytes per line and load instruction (55 and 52 % of the HBM peak).  Instead a power
             // of two of adjacent lanes shares the entry: lane c of them takes the terms c, c + lanes, ... of the
             // flattened contraction, so that the lanes of a wavefront read consecutive addresses, and the partial sums
-            // are added in a butterfly of lane exchanges (a fixed order: results are reproducible).
-            if (subs.size() == 1 && batch >= 0 && mid.empty() && s.matrixOp == 0 && !s.out.repeated && s.contrCount >= 8 &&
-                envInt("ACRO_HIP_SPLIT_LANES") >= 0)
+            // are added in a butterfly of lane exchanges (a fixed order: results are reproducible).  The same for a
+            // kernel with few outputs per entry and a contraction along the fastest dimension of a streaming operand
+            // ("A_e_i = B_e_i_n", "Y_e_i = M_e_i_j X_e_j" with an element matrix of 27 x 27).
+            const long splitFrom = envInt("ACRO_HIP_SPLIT_FROM") > 0 ? envInt("ACRO_HIP_SPLIT_FROM") : 8;
+            if (subs.size() == 1 && batch >= 0 && s.matrixOp == 0 && !s.out.repeated && envInt("ACRO_HIP_SPLIT_LANES") >= 0 &&
+                !s.contr.empty() && (mid.empty() ? s.contrCount >= 8 : (s.contrCount >= splitFrom && product(mid, extent) <= 64)))
             {
-                bool streams = false;  // some operand carries the batch index and the fastest contraction index last
-                for (const auto &r : s.in) streams = streams || (has(r.idx, batch) && r.idx.back() == s.contr.back());
+                // the operand that an entry reads most of carries the batch index and the fastest contraction index last
+                const VarRef *most = &s.in[0];
+                auto perEntry = [&](const VarRef &r) { return has(r.idx, batch) ? r.size / E : r.size; };
+                for (const auto &r : s.in)
+                {
+                    if (perEntry(r) > perEntry(*most)) most = &r;
+                }
+                const bool streams = has(most->idx, batch) && most->idx.back() == s.contr.back();
                 if (streams)
                 {
+                    // At most a row of 16 lanes: the exchanges inside a row are register moves, not LDS traffic.  With
+                    // several outputs per entry a lane should have at least four terms of its own, or the exchanges
+                    // outweigh the arithmetic (16 x 16 matrix-vector products with one term per lane: 47 % against
+                    // 59 % unsplit).
+                    const long atMost = mid.empty() ? s.contrCount : s.contrCount / 4;
                     int lanes = 1;
-                    while (lanes * 2 <= 64 && lanes * 2 <= s.contrCount) lanes *= 2;
-                    s.splitLanes = lanes;
-                    s.loopMode = true;
-                    s.tile.clear();
-                    s.tileCount = 1;
-                    s.laneCount = lanes;
+                    while (lanes * 2 <= 16 && lanes * 2 <= atMost) lanes *= 2;
+                    if (lanes >= (mid.empty() ? 2 : 4))
+                    {
+                        s.tile.clear();
+                        SetLanes(s);
+                        s.splitLanes = lanes;
+                        s.loopMode = true;
+                        s.laneCount *= lanes;
+                    }
                 }
             }
         }
@@ -2409,8 +2426,21 @@ class Generator
         }
         lines.push_back("    sum += " + prod + ";");
         lines.push_back("}");
-        // the lanes of an entry are adjacent and aligned, so every exchange partner works on the same entry
-        for (int m = L / 2; m >= 1; m /= 2) lines.push_back("sum += __shfl_xor(sum, " + str(m) + ", " + str(L) + ");");
+        // The lanes of an output are adjacent and aligned, so every exchange partner works on the same output.  Lanes
+        // 1 and 2 apart swap inside their quad; then every lane of a quad holds the same value and mirroring the
+        // half row (8 lanes), then the row (16 lanes), pairs each quad with the one it has not met yet.  Every lane
+        // ends up with the same sum, added in the same order.
+        static const char *const kDppControl[4] = {"0xB1", "0x4E", "0x141", "0x140"};  // quad_perm [1,0,3,2], [2,3,0,1], row_half_mirror, row_mirror
+        for (int step = 0; (1 << step) < L; ++step)
+        {
+            lines.push_back("{");
+            lines.push_back("    union { double d; int i[2]; } mine, other;");
+            lines.push_back("    mine.d = sum;");
+            lines.push_back(std::string("    other.i[0] = __builtin_amdgcn_update_dpp(0, mine.i[0], ") + kDppControl[step] + ", 0xF, 0xF, false);");
+            lines.push_back(std::string("    other.i[1] = __builtin_amdgcn_update_dpp(0, mine.i[1], ") + kDppControl[step] + ", 0xF, 0xF, false);");
+            lines.push_back("    sum += other.d;");
+            lines.push_back("}");
+        }
         const std::string gaddr = PtrName(s.out.uvar) + "[o_k" + str(k) + "g]";
         lines.push_back("if (cl == 0)");
         lines.push_back("{");

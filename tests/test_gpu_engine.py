@@ -428,6 +428,10 @@ def test_kernels_whose_schedule_follows_the_memory_access_pattern(at, engine, ch
     ("A_e = B_e_i_j C_j_i", [(130, 5, 7), (7, 5)]),              # two contraction indices, one operand transposed
     ("A_e = B_e_i_j C_e_i_j D_j", [(64, 6, 4), (64, 6, 4), (4,)]),
     ("A_e = B_i_e_j C_e_j", [(3, 50, 11), (50, 11)]),            # batch index in the middle of an operand
+    ("A_e_i = B_e_i_j C_e_j", [(203, 16, 16), (203, 16)]),       # element matrix times element vector: 4 lanes per row
+    ("A_e_i += B_e_i_j C_e_j", [(35, 27, 27), (35, 27)]),        # odd row length, lanes 0 - 2 take a seventh term
+    ("A_e_i = B_e_i_j C_e_j", [(9, 64, 64), (9, 64)]),           # 16 lanes per row, four passes per entry
+    ("A_e_i_k = B_e_i_k_n", [(21, 3, 5, 100)]),                  # two lane indices next to the shared contraction
 ])
 def test_one_output_per_batch_entry_shares_the_contraction_between_lanes(at, engine, checker, kernel, shapes):
     rng = np.random.default_rng(len(kernel) + shapes[0][0])
