@@ -1008,9 +1008,8 @@ class Generator
             // are added in a butterfly of lane exchanges (a fixed order: results are reproducible).  The same for a
             // kernel with few outputs per entry and a contraction along the fastest dimension of a streaming operand
             // ("A_e_i = B_e_i_n", "Y_e_i = M_e_i_j X_e_j" with an element matrix of 27 x 27).
-            const long splitFrom = envInt("ACRO_HIP_SPLIT_FROM") > 0 ? envInt("ACRO_HIP_SPLIT_FROM") : 8;
             if (subs.size() == 1 && batch >= 0 && s.matrixOp == 0 && !s.out.repeated && envInt("ACRO_HIP_SPLIT_LANES") >= 0 &&
-                !s.contr.empty() && (mid.empty() ? s.contrCount >= 8 : (s.contrCount >= splitFrom && product(mid, extent) <= 64)))
+                !s.contr.empty() && (mid.empty() ? s.contrCount >= 8 : (s.contrCount >= 16 && product(mid, extent) <= 64)))
             {
                 // the operand that an entry reads most of carries the batch index and the fastest contraction index last
                 const VarRef *most = &s.in[0];
