@@ -78,6 +78,71 @@ def cpu_baseline(workloads, sample_elems):
 FP64_PEAK_GFLOPS = 78600.0
 
 
+# Single kernels a user of the reference's API writes, at large batch sizes: (kernel, input shapes, output shape).
+KERNEL_SHAPES = [
+    ("A_e_i = B_e_i", [(1 << 22, 16)], (1 << 22, 16)),
+    ("A_e_i += B_e_i", [(1 << 22, 16)], (1 << 22, 16)),
+    ("A_e_i = B_e_i C_e_i D_e_i", [(1 << 22, 16)] * 3, (1 << 22, 16)),
+    ("A_e_i = B_e_i_j C_j", [(1 << 20, 8, 8), (8,)], (1 << 20, 8)),
+    ("A_e_i = B_e_i_j C_e_j", [(1 << 20, 8, 8), (1 << 20, 8)], (1 << 20, 8)),
+    ("A_e_i = B_e_i_j C_e_j", [(1 << 18, 16, 16), (1 << 18, 16)], (1 << 18, 16)),
+    ("A_e_i = B_e_i_j C_e_j", [(1 << 17, 27, 27), (1 << 17, 27)], (1 << 17, 27)),
+    ("A_e_i = B_e_i_j C_e_j", [(1 << 15, 64, 64), (1 << 15, 64)], (1 << 15, 64)),
+    ("A_e_i_k = B_e_i_j C_e_j_k", [(1 << 21, 3, 3), (1 << 21, 3, 3)], (1 << 21, 3, 3)),
+    ("A_e_i_k = B_e_i_j C_e_j_k", [(1 << 20, 4, 4), (1 << 20, 4, 4)], (1 << 20, 4, 4)),
+    ("A_e_i_k = B_e_i_j C_e_j_k", [(1 << 18, 8, 8), (1 << 18, 8, 8)], (1 << 18, 8, 8)),
+    ("A_e_i_k = B_e_i_j C_j_k", [(1 << 20, 8, 8), (8, 8)], (1 << 20, 8, 8)),
+    ("A_e = B_e_i C_e_i", [(1 << 21, 16), (1 << 21, 16)], (1 << 21,)),
+    ("A_e = B_e_n", [(1 << 16, 1024)], (1 << 16,)),
+    ("A_e_i = B_e_i_n", [(1 << 17, 4, 256)], (1 << 17, 4)),
+    ("A_e_i_j = B_e_i C_e_j", [(1 << 20, 8), (1 << 20, 8)], (1 << 20, 8, 8)),
+    ("A_e_i_j = B_e_j_i", [(1 << 20, 8, 8)], (1 << 20, 8, 8)),
+    ("A_e_i_j_k = B_e_k_j_i", [(1 << 16, 8, 8, 8)], (1 << 16, 8, 8, 8)),
+    ("A_e_i = B_e_i_i", [(1 << 20, 8, 8)], (1 << 20, 8)),
+    ("A_e_q_j_k = B_q_i X_e_i_j_k", [(5, 4), (1 << 19, 4, 4, 4)], (1 << 19, 5, 4, 4)),
+    ("A_e_i = B_i_j X_e_j", [(64, 64), (1 << 18, 64)], (1 << 18, 64)),
+    ("S_i = A_n_i", [(1 << 20, 64)], (64,)),
+    ("S_i = A_i_n", [(64, 1 << 20)], (64,)),
+    ("A_i_j = B_j_i", [(8192, 8192)], (8192, 8192)),
+]
+
+
+def kernel_shapes(at, args):
+    """One line for the whole list: per kernel the launch time by HIP events and algorithmic bytes / time against the
+    HBM peak; `value` is the geometric mean of those fractions."""
+    import math
+    import numpy as np
+    engine = at.TensorEngine("HIP")
+    steps = min(args.steps, 20)
+    results = []
+    for kernel, in_shapes, out_shape in KERNEL_SHAPES:
+        tensors = [at.Tensor(*s) for s in in_shapes] + [at.Tensor(*out_shape)]
+        for t in tensors:
+            t.SwitchToGPU()
+            t.Set(0.5)
+        step = lambda: engine(kernel, tensors[-1], *tensors[:-1])
+        for _ in range(5):
+            step()
+        at.synchronize()
+        with at.hip_event_timer() as ev:
+            for _ in range(steps):
+                step()
+        launch_s = ev.ms * 1e-3 / steps
+        abytes = sum(int(np.prod(s)) * 8 for s in in_shapes) + int(np.prod(out_shape)) * 8 * (2 if "+=" in kernel else 1)
+        results.append({"kernel": kernel, "inputs": [list(s) for s in in_shapes], "launch_us": launch_s * 1e6,
+                        "algorithmic_bytes": abytes, "frac": abytes / launch_s * 1e-9 / HBM_PEAK_GBS,
+                        "schedule": engine.GetLastImplementation().splitlines()[1][3:]})
+        del tensors
+    mean = math.exp(sum(math.log(r["frac"]) for r in results) / len(results))
+    total_s = sum(r["launch_us"] for r in results) * 1e-6
+    return {
+        "metric": "fraction of the HBM peak, geometric mean over %d single-kernel shapes (1 GPU)" % len(results),
+        "value": mean, "unit": "fraction of 8 TB/s", "n_gpus": 1, "steps": steps, "warmup": 5,
+        "ms_per_step": total_s * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
+        "data": "synthetic", "config": {"workload": "kernel shapes, one launch each per step"}, "kernels": results,
+    }
+
+
 def other_workload(at, workloads, args):
     """Same measurement for cfg1 / cfg2 / cfg3 / cfg5 at the sizes of the baseline configurations, and for
     FlatIndexedScatter / FlatIndexedSumGather on the headline mesh."""
@@ -205,7 +270,7 @@ def main():
     ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store-all", action="store_true")
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup"],
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "shapes"],
                     help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
                          "remaining baseline configurations at their full sizes and for the node-vector <-> "
                          "element-vector steps either side of the operator apply")
@@ -223,6 +288,9 @@ def main():
     if not at.is_hip_ready():
         sys.exit("bench.py needs a HIP device; there is no host fallback.")
 
+    if args.workload == "shapes":
+        print(json.dumps(kernel_shapes(at, args)))
+        return
     if args.workload != "cfg4":
         print(json.dumps(other_workload(at, workloads, args)))
         return
