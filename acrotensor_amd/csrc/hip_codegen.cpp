@@ -2940,7 +2940,12 @@ class Generator
 
         // Work-item header: batch entry and lane indices of item `w` of the phase that kernel `ks` opens.
         auto emitHeader = [&](const Sub &s, const std::string &indent) {
-            out << indent << "const int b = w / " << s.laneCount << ";\n";
+            // A wavefront whose 64 items belong to one batch entry: say so, and the compiler turns loads that depend
+            // on the entry alone into scalar loads.
+            if (s.laneCount % 64 == 0 && envInt("ACRO_HIP_WAVE_UNIFORM") >= 0)
+                out << indent << "const int b = __builtin_amdgcn_readfirstlane(w / " << s.laneCount << ");\n";
+            else
+                out << indent << "const int b = w / " << s.laneCount << ";\n";
             out << indent << "const int e = e0 + b;\n";
             if (!s.lane.empty())
             {
