@@ -13,6 +13,19 @@
 //  * An output that a later kernel of the group consumes stays in LDS (one tile per batch entry); its store to
 //    device memory is skipped when the tensor is marked transient.  A kernel without contraction whose operand
 //    was just produced with the same index set is applied in registers (no LDS round trip).
+//    More generally a kernel whose work items can be those of the previous kernel, and that reads that kernel's
+//    results (or those of the kernels it was applied after) entry by entry, runs in the same registers, also when it
+//    contracts over the producer's register tile.
+//  * A kernel with three or more operands written as one big sum is evaluated as a chain of smaller contractions
+//    (the cheapest elimination order whose partial results fit in LDS) when that saves at least 4x the multiply-adds.
+//  * Matrix kernels (TensorKernel::Function "inv" / "det": what the engine turns recorded batched inverses and
+//    determinants into) take one work item per matrix and follow the host formulas term by term.
+//  * Register tiles are chosen by loads per output, weighted by how the lanes reach device memory (lines touched per
+//    load instruction, cache footprint of a wavefront); batch entries with few outputs get one output per lane; a
+//    kernel whose dominant operand streams along the contraction shares each output between 2 - 16 lanes that add
+//    their partial sums by DPP exchanges; small invariant operands with lane-dependent addresses are staged in LDS.
+//  * A single kernel with few outputs and a long contraction runs the "reduction schedule": the contraction range
+//    is split over workgroups and lanes, partial sums are added in a fixed order by a second one-workgroup kernel.
 //  * Contractions too long to unroll fall back to counted loops with the same lane mapping.
 //
 // Experiment switches (environment, read when a kernel is generated; defaults are what measured best on MI355X):
