@@ -2600,14 +2600,25 @@ class Generator
         // instructions (A alone streamed at 6.1 TB/s that way, A and B together at 5.0 - 5.5 TB/s).
         const bool pencil = outputsFastest && O <= 16 && envInt("ACRO_HIP_RED_PENCIL") >= 0;
         const int NTr = kReductionLanes;
-        const long Sn = pencil ? NTr : NTr / O;  // contraction slices per workgroup and step
+        // Contraction index fastest and more than four outputs ("S_i = A_i_n" with 64 rows): with all outputs in every
+        // workgroup only NTr / O lanes would walk along a row (32-byte pieces of 64 different rows per load
+        // instruction).  Instead a workgroup takes four outputs, 64 adjacent lanes each, and the workgroups are dealt
+        // out over groups of outputs as well as over the contraction range.
+        const bool byRows = !pencil && !outputsFastest && O > 4 && NTr / O < 64 && envInt("ACRO_HIP_ONE_PASS") <= 0 &&
+                            envInt("ACRO_HIP_RED_ROWS") >= 0;
+        const long Sn = pencil ? NTr : (byRows ? 64 : NTr / O);  // contraction slices per workgroup and step
+        const long Ow = NTr / Sn, Go = byRows ? (O + Ow - 1) / Ow : 1;  // outputs per workgroup, groups of outputs
         // First-stage workgroups.  Pencil: one per CU (256 on this device) without unrolling, i.e. about 20 KB of
         // loads in flight per CU and one 4.7 MB window moving through the operands; more workgroups or deeper
         // unrolling measured slower at every n (n = 2^24: 206 us with 256 workgroups, 216 with 512, 252 with 2 048;
         // 214 / 263 us with the loop unrolled 2 / 4 times).  One lane per (slice, output entry): 8 bytes per lane
         // and load, so up to 512 workgroups and four loads in flight per lane (also swept: 256 - 8 192 workgroups,
         // unroll 1 - 8).
-        const long G = std::min<long>(pencil ? 256 : 512, std::max<long>(1, Nc / (Sn * (pencil ? 4 : 16))));
+        const long G = byRows ? std::min<long>(std::max<long>(1, 1024 / Go), std::max<long>(1, Nc / (Sn * 16)))
+                              : std::min<long>(pencil ? 256 : 512, std::max<long>(1, Nc / (Sn * (pencil ? 4 : 16))));
+        // G counts the shares of the contraction range (rows of partials in the scratch buffer); the grid has one
+        // workgroup per share and group of outputs.
+        const long gridG = G * Go;
         // Lanes of the finishing kernel: enough for every lane to have all its loads of partials in flight at once
         // (the kernel is a chain of memory latencies: launch, one round of loads, LDS; 1024 lanes instead of 256
         // measured 16.8 instead of 17.2 us for the pair of launches at n = 2^20), at most 1024.  The one-pass
@@ -2625,14 +2636,17 @@ class Generator
         std::snprintf(hex, sizeof(hex), "%016llx",
                       static_cast<unsigned long long>(hashString(dimName + "/reduction/" + (opt.noalias ? "n" : "a") +
                                                                  (Positional() ? "p" : "u") +
-                                                                 (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "2" : "1") + "/" + str(envInt("ACRO_HIP_RED_PENCIL")))));
+                                                                 (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "2" : "1") + "/" + str(envInt("ACRO_HIP_RED_PENCIL")) +
+                                                                 (byRows ? "/rows" : ""))));
         plan.module_name = std::string("acro_red_") + hex;
         const std::string fPartial = plan.module_name + "_partial", fFinal = plan.module_name + "_final";
 
         std::ostringstream sched;
         sched << "reduction schedule: " << O << " output entries, contraction of " << Nc << " terms split over " << G
               << " workgroups x " << Sn << " slices ("
-              << (pencil ? "a lane owns whole slices" : (outputsFastest ? "output entries on adjacent lanes" : "slices on adjacent lanes"))
+              << (pencil ? "a lane owns whole slices"
+                         : (byRows ? "four outputs per workgroup, 64 adjacent lanes along each"
+                                   : (outputsFastest ? "output entries on adjacent lanes" : "slices on adjacent lanes")))
               << "), partials added in a fixed order by "
               << (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "a second kernel" : "the workgroup that finishes last") << "\n  [0] " << s.text << "\n";
         plan.schedule = sched.str();
@@ -2663,7 +2677,7 @@ class Generator
         // ---- stage 1: per-workgroup partial sums
         out << "\nextern \"C\" __global__ __launch_bounds__(" << NTr << ") void " << fPartial << "(" << ParamList()
             << ", double *__restrict__ scratch)\n{\n";
-        out << "    __shared__ double red[" << (pencil ? NTr * O : NTr) << "];\n";
+        out << "    __shared__ double red[" << (pencil ? NTr * O : (byRows ? NTr + Ow * 16 : NTr)) << "];\n";
         if (!twoKernels) out << "    __shared__ int isLast;\n";
         out << "    const int lane = threadIdx.x;\n";
         // Workgroups interleave: in every step the G workgroups together read one contiguous window of the
@@ -2735,6 +2749,32 @@ class Generator
             out << "    if (lane < " << O << ")\n    {\n        double t = 0.0;\n";
             out << "        for (int k = 0; k < 64; ++k) t += red[k * " << O << " + lane];\n";
         }
+        else if (byRows)
+        {
+            out << "    const int og = blockIdx.x % " << Go << ", gc = blockIdx.x / " << Go << ";\n";
+            out << "    const int o = og * " << Ow << " + lane / " << Sn << ", sl = lane % " << Sn << ";\n";
+            out << "    double sum = 0.0;\n";
+            out << "    if (o < " << O << ")\n    {\n";
+            decompose(s.outIdx, "o", "        ");
+            out << "#pragma unroll 4\n";
+            out << "        for (long c = (long)gc * " << Sn << " + sl; c < " << Nc << "; c += " << G * Sn << ")\n        {\n";
+            decompose(s.contr, "c", "            ");
+            std::string prod;
+            for (const auto &r : s.in)
+            {
+                const std::string opnd = PtrName(r.uvar) + "[" + FullOffset(r) + "]";
+                prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
+            }
+            out << "            sum += " << prod << ";\n        }\n    }\n";
+            out << "    red[lane] = sum;\n    __syncthreads();\n";
+            // 16 lanes per output add four slices each, then one lane adds the 16: a fixed order
+            out << "    if (lane < " << Ow * 16 << ")\n    {\n        double t = 0.0;\n";
+            out << "        for (int k = 0; k < " << Sn / 16 << "; ++k) t += red[(lane / 16) * " << Sn << " + (lane % 16) * " << Sn / 16 << " + k];\n";
+            out << "        red[" << NTr << " + lane] = t;\n    }\n    __syncthreads();\n";
+            out << "    if (lane < " << Ow << " && og * " << Ow << " + lane < " << O << ")\n    {\n        double t = 0.0;\n";
+            out << "        for (int k = 0; k < 16; ++k) t += red[" << NTr << " + lane * 16 + k];\n";
+            out << "        scratch[(long)gc * " << O << " + og * " << Ow << " + lane] = t;\n    }\n}\n";
+        }
         else
         {
             if (outputsFastest)
@@ -2760,7 +2800,11 @@ class Generator
             out << "        for (int k = 0; k < " << Sn << "; ++k) t += red["
                 << (outputsFastest ? "k * " + str(O) + " + lane" : "lane * " + str(Sn) + " + k") << "];\n";
         }
-        if (twoKernels)
+        if (byRows)
+        {
+            // written above
+        }
+        else if (twoKernels)
             out << "        scratch[(long)blockIdx.x * " << O << " + lane] = t;\n    }\n}\n";
         else
             out << "        __hip_atomic_store(&scratch[(long)blockIdx.x * " << O
@@ -2825,7 +2869,7 @@ class Generator
         const int S = static_cast<int>(stores.size());
         HipLaunch partial;
         partial.function_name = fPartial;
-        partial.grid = static_cast<unsigned>(G);
+        partial.grid = static_cast<unsigned>(gridG);
         partial.block = NTr;
         for (int si = 0; si < S; ++si) partial.params.push_back(si);
         partial.params.push_back(-1);

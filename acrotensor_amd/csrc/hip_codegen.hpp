@@ -49,6 +49,7 @@
 //   ACRO_HIP_SPLIT_LANES=-1     one lane per batch entry also for kernels with one output per entry (no lane exchanges)
 //   ACRO_HIP_WAVE_UNIFORM=-1    no readfirstlane on the batch entry of wavefronts that hold items of one entry only
 //   ACRO_HIP_RED_PENCIL=-1      split contractions: one lane per (slice, output entry) also when there are few outputs
+//   ACRO_HIP_RED_ROWS=-1        split contractions of few long rows: all outputs in every workgroup, NT / outputs lanes along a row
 //   ACRO_HIP_ONE_PASS=1         split contractions: the workgroup that finishes last adds the per-workgroup partials
 //                               instead of a second kernel (measured 18.4 against 16.3 us: the device-scope release
 //                               writes back the XCD's L2 once per workgroup)

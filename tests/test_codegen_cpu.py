@@ -103,10 +103,17 @@ def test_split_contraction_with_few_outputs_gives_a_lane_whole_slices(TE, monkey
     assert "a lane owns whole slices" in src and "split over 256 workgroups" in src
     assert src.count("double acc") == 9 and src.count("T2[ob1") == 1      # B is loaded once per slice, not per output
     assert src.count("__global__") == 2 and "atomic" not in src            # second kernel adds the partials
-    # many outputs, or outputs that are not the fastest dimension of the big operand: one lane per (slice, output)
+    # outputs that are not the fastest dimension of the big operand: 64 adjacent lanes walk along each row, four
+    # rows per workgroup, and the grid covers groups of rows as well as shares of the contraction
     S2, A2 = at.Tensor(40), at.Tensor(40, 1 << 14)
     src = TE.GetImplementation("S_i = A_i_n B_n", S2, A2, at.Tensor(1 << 14))
+    assert "four outputs per workgroup, 64 adjacent lanes along each" in src and "blockIdx.x % 10" in src
+    # at most four such outputs: all of them in every workgroup
+    src = TE.GetImplementation("S_i = A_i_n B_n", at.Tensor(4), at.Tensor(4, 1 << 14), at.Tensor(1 << 14))
     assert "slices on adjacent lanes" in src
+    # many outputs that are the fastest dimension: one lane per (slice, output)
+    src = TE.GetImplementation("S_i = A_n_i B_n", at.Tensor(40), at.Tensor(1 << 14, 40), at.Tensor(1 << 14))
+    assert "output entries on adjacent lanes" in src
     monkeypatch.setenv("ACRO_HIP_ONE_PASS", "1")
     src = TE.GetImplementation("S_i_j = A_n_i_j B_n", S, at.Tensor((1 << 18) + 1, 3, 3), at.Tensor((1 << 18) + 1))
     assert src.count("__global__") == 1 and "__hip_atomic_fetch_add" in src
@@ -225,6 +232,7 @@ def generated_sources(TE):
     yield "one name, two tensors", TE.GetImplementation("A_m_n = B_m_j B_n_j", at.Tensor(3, 3), at.Tensor(3, 4), at.Tensor(3, 4))
     yield "repeated output index", TE.GetImplementation("A_i_i = B_i", at.Tensor(6, 6), at.Tensor(6))
     yield "operand staged in LDS", TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
+    yield "split contraction, few long rows", TE.GetImplementation("S_i += A_i_n B_n", at.Tensor(6), at.Tensor(6, 9000), at.Tensor(9000))
     yield "contraction shared by lanes", TE.GetImplementation("A_e += B_e_i_j C_j_i", at.Tensor(1000), at.Tensor(1000, 5, 7), at.Tensor(7, 5))
     for transient in (True, False):
         yield "geometric factors from the Jacobians", geometric_factor_source(TE, 7, 4, 3, transient)

@@ -444,3 +444,20 @@ def test_one_output_per_batch_entry_shares_the_contraction_between_lanes(at, eng
     assert rel_err(got, expected) <= TOL
     again, _ = run_single(at, engine, checker, kernel, out0, *ins)
     assert np.array_equal(got, again)                            # fixed order of the lane exchanges: reproducible
+
+
+@pytest.mark.parametrize("kernel,shapes,out", [
+    ("S_i = A_i_n", [(64, 70001)], (64,)),                       # four rows per workgroup, 64 lanes along each
+    ("S_i += A_i_n B_n", [(6, 9000), (9000,)], (6,)),            # last group of outputs half empty
+    ("S_i_j = A_i_j_n", [(5, 7, 4099)], (5, 7)),
+    ("S_i = A_i_m_n B_m", [(9, 3, 3001), (3,)], (9,)),           # two contraction indices
+])
+def test_split_contraction_of_few_long_rows(at, engine, checker, kernel, shapes, out):
+    rng = np.random.default_rng(shapes[0][-1])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, out)
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "64 adjacent lanes along each" in engine.GetLastImplementation()
+    assert rel_err(got, expected) <= TOL
+    again, _ = run_single(at, engine, checker, kernel, out0, *ins)
+    assert np.array_equal(got, again)
