@@ -942,6 +942,7 @@ class Generator
     {
         for (auto &s : subs)
         {
+            s.splitLanes = 0;
             std::vector<int> mid;
             for (int id : s.outIdx)
             {
