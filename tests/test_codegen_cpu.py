@@ -233,6 +233,7 @@ def generated_sources(TE):
     yield "repeated output index", TE.GetImplementation("A_i_i = B_i", at.Tensor(6, 6), at.Tensor(6))
     yield "operand staged in LDS", TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
     yield "split contraction, few long rows", TE.GetImplementation("S_i += A_i_n B_n", at.Tensor(6), at.Tensor(6, 9000), at.Tensor(9000))
+    yield "transpose through LDS tiles", TE.GetImplementation("A_i_e_j -= B_j_e_i", at.Tensor(100, 3, 70), at.Tensor(70, 3, 100))
     yield "contraction shared by lanes", TE.GetImplementation("A_e += B_e_i_j C_j_i", at.Tensor(1000), at.Tensor(1000, 5, 7), at.Tensor(7, 5))
     for transient in (True, False):
         yield "geometric factors from the Jacobians", geometric_factor_source(TE, 7, 4, 3, transient)
