@@ -296,9 +296,11 @@ void TensorEngine::FinishCapture(std::string *implementation)
     std::vector<RecordedMatrixOp> ops;
     ops.swap(MKLMatrixOps);
 
+    std::vector<GatheredInput> gathered;  // results of recorded scatters that the kernels read through the maps
     auto flush = [&]() {
         if (MKLKernels.empty()) return;
         KernelExecutor *executor = GetAddKernelExecutor();
+        executor->SetGatheredInputs(gathered);
         if (implementation != nullptr)
         {
             *implementation += executor->GetImplementation(MKLOutputT, MKLInputT);
@@ -309,6 +311,31 @@ void TensorEngine::FinishCapture(std::string *implementation)
             executor->ExecuteMulti(MKLOutputT, MKLInputT);
         }
         ResetCapture();
+    };
+    // A recorded scatter need not run when its result is transient, nothing else in the capture writes the result
+    // or the source, no kernel recorded before it reads the result, and a kernel recorded after it does.
+    auto readThroughMap = [&](const RecordedMatrixOp &op) {
+        if (!op.scatter_out->IsTransient() || op.scatter_out == op.scatter_in) return false;
+        bool read_later = false;
+        for (size_t k = 0; k < kernels.size(); ++k)
+        {
+            if (outputs[k] == op.scatter_out || outputs[k] == op.scatter_in) return false;
+            for (Tensor *t : inputs[k])
+            {
+                if (t != op.scatter_out) continue;
+                if (k < op.position) return false;
+                read_later = true;
+            }
+        }
+        for (const auto &other : ops)
+        {
+            if (&other == &op) continue;
+            for (Tensor *t : {other.inverse, other.determinant, other.matrices, other.scatter_out, other.scatter_in})
+            {
+                if (t == op.scatter_out || (t == op.scatter_in && t != other.scatter_in && t != other.matrices)) return false;
+            }
+        }
+        return read_later;
     };
     // A capture that a matrix operation splits into several launches keeps nothing on chip across them: for its
     // duration no tensor counts as transient (a transient result of one launch may be an operand of the next).
@@ -337,6 +364,10 @@ void TensorEngine::FinishCapture(std::string *implementation)
             keep.Add(op.inverse);
             keep.Add(op.determinant);
             keep.Add(op.matrices);
+            keep.Add(op.scatter_in);
+            bool through_map = false;  // a result that is read through its map stays transient: it is never written
+            for (const auto &g : gathered) through_map = through_map || g.operand == op.scatter_out;
+            if (!through_map) keep.Add(op.scatter_out);
         }
     };
     size_t next_op = 0;
@@ -345,6 +376,26 @@ void TensorEngine::FinishCapture(std::string *implementation)
         for (; next_op < ops.size() && ops[next_op].position == k; ++next_op)
         {
             const RecordedMatrixOp &op = ops[next_op];
+            if (op.scatter_out != nullptr)
+            {
+                if (readThroughMap(op))
+                {
+                    gathered.push_back({op.scatter_out, op.scatter_in, op.map});
+                    continue;
+                }
+                keepAll();
+                flush();
+                if (implementation != nullptr)
+                {
+                    *implementation += "// scatter whose result is not transient, or not only read by the kernels after it: runs on its own\n";
+                    continue;
+                }
+                SwitchToComputeLocation(*op.scatter_out);
+                MoveToComputeLocation(*op.scatter_in);
+                MoveToComputeLocation(*op.map);
+                Ops->FlatIndexedScatter(*op.scatter_out, *op.scatter_in, *op.map);
+                continue;
+            }
             if (MatrixOpAsKernels(op, kernels, outputs, inputs, MKLKernels, MKLOutputT, MKLInputT)) continue;
             keepAll();
             flush();
@@ -479,7 +530,7 @@ void TensorEngine::BatchMatrixInverse(Tensor &Ainv, Tensor &A)
     checkInverseShapes(Ainv, A);
     if (IsMultiKernelLaunch)
     {
-        MKLMatrixOps.push_back({MKLKernels.size(), &Ainv, nullptr, &A});
+        MKLMatrixOps.push_back({MKLKernels.size(), &Ainv, nullptr, &A, nullptr, nullptr, nullptr});
         return;
     }
     SwitchToComputeLocation(Ainv);
@@ -493,7 +544,7 @@ void TensorEngine::BatchMatrixDet(Tensor &Adet, Tensor &A)
     checkDetShapes(Adet, A);
     if (IsMultiKernelLaunch)
     {
-        MKLMatrixOps.push_back({MKLKernels.size(), nullptr, &Adet, &A});
+        MKLMatrixOps.push_back({MKLKernels.size(), nullptr, &Adet, &A, nullptr, nullptr, nullptr});
         return;
     }
     SwitchToComputeLocation(Adet);
@@ -508,7 +559,7 @@ void TensorEngine::BatchMatrixInvDet(Tensor &Ainv, Tensor &Adet, Tensor &A)
     checkDetShapes(Adet, A);
     if (IsMultiKernelLaunch)
     {
-        MKLMatrixOps.push_back({MKLKernels.size(), &Ainv, &Adet, &A});
+        MKLMatrixOps.push_back({MKLKernels.size(), &Ainv, &Adet, &A, nullptr, nullptr, nullptr});
         return;
     }
     SwitchToComputeLocation(Ainv);
@@ -522,6 +573,11 @@ void TensorEngine::FlatIndexedScatter(Tensor &Aout, Tensor &Ain, IndexMapping &M
     ACROBATIC_ASSERT(Ops != nullptr, "The executor type of this engine provides no non-contraction ops.");
     ACROBATIC_ASSERT(Aout.GetSize() == static_cast<size_t>(M.GetRangeSize()), "IndexMapping RangeSize does not match the output Tensor size.");
     ACROBATIC_ASSERT(Ain.GetSize() == static_cast<size_t>(M.GetDomainSize()), "IndexMapping DomainSize does not match the input Tensor size.");
+    if (IsMultiKernelLaunch && ExecutorType == "HIP")
+    {
+        MKLMatrixOps.push_back({MKLKernels.size(), nullptr, nullptr, nullptr, &Aout, &Ain, &M});
+        return;
+    }
     SwitchToComputeLocation(Aout);
     MoveToComputeLocation(Ain);
     MoveToComputeLocation(M);

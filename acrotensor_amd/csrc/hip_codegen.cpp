@@ -787,7 +787,7 @@ class Generator
     // depend on the lane (only on tile / contraction indices, which are literals or uniform loop counters).
     bool IsUniform(const Sub &s, const VarRef &r, const std::vector<int> &tile) const
     {
-        if (!opt.noalias || !IsPureInput(r.uvar)) return false;
+        if (!opt.noalias || !IsPureInput(r.uvar) || GatherSlot(r.uvar) >= 0) return false;
         bool carriesBatch = false;
         for (int id : r.idx)
         {
@@ -1356,6 +1356,7 @@ class Generator
             if (st.written || st.members.size() != 1 || st.anyRepeated) continue;
             const UVarInfo &u = uvars[st.members[0]];
             if (!u.consistent || !u.batchDims.empty() || !u.plainView || !u.fixed.empty() || u.isVirtual) continue;
+            if (GatherSlot(st.members[0]) >= 0) continue;
             if (u.size > kMaxStagedDoubles || u.size < 64) continue;
             bool ok = true, farApart = false;
             int first = -1, last = -1, laneDim = -1;
@@ -1819,6 +1820,24 @@ class Generator
 
     // Kernel parameters are storages; an operand addresses its storage at viewOffset.
     std::string PtrName(int uvar) const { return "T" + str(uvars[uvar].storage); }
+    // Pair number of an operand that is read through an index map instead of from its own memory, or -1.
+    int GatherSlot(int uvar) const
+    {
+        return static_cast<size_t>(uvar) < opt.gathered.size() ? opt.gathered[uvar] : -1;
+    }
+    int NumGatherSlots() const
+    {
+        int n = 0;
+        for (int g : opt.gathered) n = std::max(n, g + 1);
+        return n;
+    }
+    // Read of entry `offset` of an operand from device memory.
+    std::string GlobalRead(int uvar, const std::string &offset) const
+    {
+        const int g = GatherSlot(uvar);
+        if (g < 0) return PtrName(uvar) + "[" + offset + "]";
+        return "G" + str(g) + "s[G" + str(g) + "m[" + offset + "]]";
+    }
     std::string ConstPtrName(int uvar) const { return "C" + str(uvars[uvar].storage); }
     const Storage &StoreOf(int uvar) const { return stores[uvars[uvar].storage]; }
     // LDS stride of a view dimension, and the constant LDS offset of the view inside the storage's tile
@@ -1962,7 +1981,7 @@ class Generator
         }
         else
         {
-            const std::string rhs = PtrName(r.uvar) + "[" + base + " + " + Lit(off) + "]";
+            const std::string rhs = GlobalRead(r.uvar, base + " + " + Lit(off));
             body.loads.push_back("const double " + name + " = " + rhs + ";");
             if (Prefetchable(k, v)) body.globalLoads.push_back(std::make_pair(key, rhs));
         }
@@ -2429,7 +2448,7 @@ class Generator
             else if (lds)
                 opnd = "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
             else
-                opnd = PtrName(r.uvar) + "[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
+                opnd = GlobalRead(r.uvar, "o_k" + str(k) + "v" + str(v) + " + " + off);
             prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
         }
         lines.push_back("    sum += " + prod + ";");
@@ -2502,7 +2521,7 @@ class Generator
             else if (lds)
                 opnd = "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
             else
-                opnd = PtrName(r.uvar) + "[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
+                opnd = GlobalRead(r.uvar, "o_k" + str(k) + "v" + str(v) + " + " + off);
             prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
         }
         lines.push_back(indent + "sum += " + prod + ";");
@@ -2535,7 +2554,7 @@ class Generator
 
     bool UseReductionSchedule() const
     {
-        if (subs.size() != 1) return false;
+        if (subs.size() != 1 || NumGatherSlots() > 0) return false;
         const Sub &s = subs[0];
         if (s.out.repeated) return false;
         return s.contrCount >= kReductionMinContraction && product(s.outIdx, extent) <= kReductionMaxOutputs;
@@ -2586,6 +2605,8 @@ class Generator
             p += std::string(si ? ", " : "") + (stores[si].written ? "double *" : "const double *") +
                  (opt.noalias ? "__restrict__ " : "") + "T" + str(static_cast<long>(si));
         }
+        for (int g = 0; g < NumGatherSlots(); ++g)
+            p += ", const int *__restrict__ G" + str(g) + "m, const double *__restrict__ G" + str(g) + "s";
         return p;
     }
 
@@ -2904,7 +2925,7 @@ class Generator
     // that the transposed read is free of bank conflicts.
     bool UseTransposeSchedule() const
     {
-        if (subs.size() != 1 || envInt("ACRO_HIP_TRANSPOSE") < 0 || !opt.noalias) return false;
+        if (subs.size() != 1 || envInt("ACRO_HIP_TRANSPOSE") < 0 || !opt.noalias || NumGatherSlots() > 0) return false;
         const Sub &s = subs[0];
         if (s.matrixOp != 0 || s.in.size() != 1 || !s.contr.empty() || s.out.repeated || s.in[0].repeated) return false;
         if (s.in[0].uvar == s.out.uvar || s.in[0].idx.size() != s.out.idx.size() || s.out.idx.size() < 2) return false;
@@ -3010,6 +3031,7 @@ class Generator
                               "/" + str(envInt("ACRO_HIP_PERSIST"));
         for (const auto &st : stores) variant += st.elide ? "e" : (st.inLds ? "l" : "g");
         for (int u = 0; u < U; ++u) variant += "s" + str(uvars[u].storage) + "@" + str(uvars[u].viewOffset);
+        for (int g : opt.gathered) variant += "g" + str(g);
         char hex[32];
         std::snprintf(hex, sizeof(hex), "%016llx", static_cast<unsigned long long>(hashString(dimName + variant)));
         plan.module_name = std::string("acro_mk_") + hex;
@@ -3030,7 +3052,9 @@ class Generator
             for (size_t v = 0; v < s.in.size(); ++v)
             {
                 static const char *const names[] = {"registers", "scalar", "lds", "global"};
-                sched << " " << uvars[s.in[v].uvar].name << "<-" << names[SourceOf(k, static_cast<int>(v))];
+                const Source src = SourceOf(k, static_cast<int>(v));
+                sched << " " << uvars[s.in[v].uvar].name << "<-"
+                      << (src == kFromGlobal && GatherSlot(s.in[v].uvar) >= 0 ? "gathered" : names[src]);
             }
             const UVarInfo &uo = uvars[s.out.uvar];
             const bool elided = !StoresToGlobal(k);
@@ -3334,6 +3358,12 @@ class Generator
         launch.grid_y = static_cast<unsigned>(splitY);
         launch.block = static_cast<unsigned>(NT);
         for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
+        for (int g = 0; g < NumGatherSlots(); ++g)
+        {
+            launch.params.push_back(-2 - 2 * g);
+            launch.params.push_back(-3 - 2 * g);
+        }
+        plan.gathers_applied = NumGatherSlots() > 0;
         plan.launches.push_back(launch);
         plan.nb = NB;
         plan.lds_bytes = ldsDoubles * 8;

@@ -92,10 +92,16 @@ struct HipCodegenOptions
     bool positional = false;
     int force_nb = 0;  // 0 = choose
     int force_nt = 0;  // 0 = choose
+    // Per operand (empty: none): >= 0 says that the operand is never materialised: entry i of it is entry map[i] of a
+    // source vector (a FlatIndexedScatter recorded in the same multi-kernel launch whose result is transient).  The
+    // value numbers the (map, source) pair among the extra kernel parameters.  Only for operands that are read, never
+    // written, by the group, and not in positional mode.
+    std::vector<int> gathered;
 };
 
 // One kernel launch of a plan.  params: >= 0 is an index into HipKernelPlan::param_occurrence (a storage's device
-// pointer), -1 is the plan's scratch buffer.
+// pointer), -1 is the plan's scratch buffer, -2 - 2 g the index map (const int *) and -3 - 2 g the source vector
+// (const double *) of gathered-operand pair g.
 struct HipLaunch
 {
     std::string function_name;
@@ -133,6 +139,7 @@ struct HipKernelPlan
     std::vector<ZeroFill> zero_fills;
     int lds_bytes = 0;
     int nb = 0;
+    bool gathers_applied = false;  // the source reads gathered operands through their maps (HipCodegenOptions::gathered)
     std::string schedule;          // human readable schedule summary (also a comment in the source)
 };
 

@@ -12,7 +12,9 @@
 #include <memory>
 
 #include "HipRuntime.hpp"
+#include "IndexMapping.hpp"
 #include "KernelExecutor.hpp"
+#include "NonContractionOps.hpp"
 #include "SliceTensor.hpp"
 #include "hip_codegen.hpp"
 #include "hip_kernel.hpp"
@@ -40,7 +42,9 @@ class HipExecutor : public KernelExecutor
     {
         HipCodegenOptions options;
         bool fallback = false;
-        Bind(outputs, inputs, options, fallback);
+        std::vector<GatheredInput> gathered;
+        gathered.swap(Gathered);  // this call only
+        Bind(outputs, inputs, gathered, options, fallback);
         if (fallback) return "// not fused (overlapping or re-bound variables): one launch per kernel\n";
         return Describe(GetVariant(options));
     }
@@ -85,6 +89,7 @@ class HipExecutor : public KernelExecutor
     {
         std::string key = std::string(options.noalias ? "n" : "a") + (options.positional ? "p" : "u");
         for (bool t : options.transient) key += t ? '1' : '0';
+        for (int g : options.gathered) key += "g" + std::to_string(g);
         for (const auto &v : options.views)
         {
             key += "|" + std::to_string(v.storage) + "@" + std::to_string(v.offset);
@@ -108,8 +113,8 @@ class HipExecutor : public KernelExecutor
     // analysis: two different operands that overlap in memory, one of them written, forbid restrict / scalar
     // reads (single kernel) or fusion (group).  Host buffers mirror device buffers one to one, so the analysis
     // works before anything is mapped to the device.
-    void Bind(std::vector<Tensor *> &outputs, std::vector<std::vector<Tensor *>> &inputs, HipCodegenOptions &options,
-              bool &fallback)
+    void Bind(std::vector<Tensor *> &outputs, std::vector<std::vector<Tensor *>> &inputs,
+              const std::vector<GatheredInput> &gathered, HipCodegenOptions &options, bool &fallback)
     {
         const int K = MultiKernel->GetNumKernels();
         ACROBATIC_ASSERT(static_cast<int>(outputs.size()) == K && static_cast<int>(inputs.size()) == K,
@@ -193,6 +198,40 @@ class HipExecutor : public KernelExecutor
         }
         fallback = K > 1 && (hazard || rebound);
         options.noalias = !hazard;
+        // Operands that are read through an index map: whole tensors that the group only reads.
+        if (!gathered.empty() && !options.positional && !fallback && !hazard)
+        {
+            options.gathered.assign(n, -1);
+            for (size_t g = 0; g < gathered.size(); ++g)
+            {
+                for (size_t a = 0; a < n; ++a)
+                {
+                    if (operand[a] != gathered[g].operand) continue;
+                    bool alone = !written[a] && root[a] == operand[a];
+                    for (size_t b = 0; b < n; ++b) alone = alone && (b == a || root[b] != root[a]);
+                    if (alone) options.gathered[a] = static_cast<int>(g);
+                }
+            }
+        }
+    }
+
+    // Runs the scatters whose results the kernels of this call do not read through the maps (`applied`: per operand
+    // the pair number the generated code reads, or null when it reads none).
+    static void MaterialiseGathered(const std::vector<GatheredInput> &gathered, const std::vector<int> *applied)
+    {
+        for (size_t g = 0; g < gathered.size(); ++g)
+        {
+            bool through_map = false;
+            if (applied != nullptr)
+            {
+                for (int slot : *applied) through_map = through_map || slot == static_cast<int>(g);
+            }
+            if (through_map) continue;
+            gathered[g].operand->SwitchToGPU();
+            gathered[g].source->MoveToGPU();
+            gathered[g].map->MoveToGPU();
+            HipGPUOps().FlatIndexedScatter(*gathered[g].operand, *gathered[g].source, *gathered[g].map);
+        }
     }
 
     void Execute(std::vector<Tensor *> &outputs, std::vector<std::vector<Tensor *>> &inputs)
@@ -200,13 +239,18 @@ class HipExecutor : public KernelExecutor
         const int K = MultiKernel->GetNumKernels();
         ACROBATIC_ASSERT(static_cast<int>(outputs.size()) == K && static_cast<int>(inputs.size()) == K,
                          "Number of tensor lists does not match the number of kernels.");
+        std::vector<GatheredInput> gathered;
+        gathered.swap(Gathered);  // this call only
+        // a gathered operand is the result of a scatter: nothing to copy to the device for it
+        for (const auto &g : gathered) g.operand->SwitchToGPU();
         for (int ki = 0; ki < K; ++ki) MoveTensorsToGPU(outputs[ki], inputs[ki]);
 
         HipCodegenOptions options;
         bool fallback = false;
-        Bind(outputs, inputs, options, fallback);
+        Bind(outputs, inputs, gathered, options, fallback);
         if (fallback)
         {
+            MaterialiseGathered(gathered, nullptr);
             KernelExecutor::ExecuteMulti(outputs, inputs);
             return;
         }
@@ -214,8 +258,22 @@ class HipExecutor : public KernelExecutor
         if (!v.plan.fusable)
         {
             ACROBATIC_ASSERT(K > 1, "Internal error: a single kernel must always be executable.");
+            MaterialiseGathered(gathered, nullptr);
             KernelExecutor::ExecuteMulti(outputs, inputs);
             return;
+        }
+        MaterialiseGathered(gathered, v.plan.gathers_applied ? &options.gathered : nullptr);
+        std::vector<const int *> gatherMap(gathered.size(), nullptr);
+        std::vector<const double *> gatherSource(gathered.size(), nullptr);
+        if (v.plan.gathers_applied)
+        {
+            for (size_t g = 0; g < gathered.size(); ++g)
+            {
+                gathered[g].source->MoveToGPU();
+                gathered[g].map->MoveToGPU();
+                gatherMap[g] = gathered[g].map->GetMap().GetDeviceData();
+                gatherSource[g] = gathered[g].source->GetDeviceData();
+            }
         }
         const size_t nparam = v.plan.param_occurrence.size();
         std::vector<double *> ptr(nparam);
@@ -240,7 +298,15 @@ class HipExecutor : public KernelExecutor
             std::vector<void *> args(launch.params.size());
             for (size_t i = 0; i < args.size(); ++i)
             {
-                args[i] = launch.params[i] < 0 ? static_cast<void *>(&v.scratch) : static_cast<void *>(&ptr[launch.params[i]]);
+                const int code = launch.params[i];
+                if (code >= 0)
+                    args[i] = static_cast<void *>(&ptr[code]);
+                else if (code == -1)
+                    args[i] = static_cast<void *>(&v.scratch);
+                else if ((-code - 2) % 2 == 0)
+                    args[i] = static_cast<void *>(&gatherMap[(-code - 2) / 2]);
+                else
+                    args[i] = static_cast<void *>(&gatherSource[(-code - 2) / 2]);
             }
             v.kernel->Launch(launch.function_name, launch.grid, launch.grid_y, launch.block, args.data());
         }

@@ -202,6 +202,43 @@ def other_workload(at, workloads, args):
         points = E * Q * Q * Q
         abytes, flops = points * (9 + 1 + 9) * 8, points * (9 * 3 * 5 + 54)
         units, unit_name = points, "Gpoints/s"
+    elif name in ("scatter_apply", "scatter_then_apply"):
+        # node vector -> element vector -> p=3 mass apply on the headline mesh (64^3 elements).  scatter_apply records
+        # the scatter in the multi-kernel launch with a transient element vector, so the chain reads the node vector
+        # through the element-to-node map and the element vector never exists; scatter_then_apply runs the two steps
+        # one after the other.
+        import numpy as np
+        wl = workloads.config4(E=262144)
+        tensors = workloads.bind_to_engine(wl, at, transient=True)
+        dofs, nodes = workloads.hex_mesh_dof_map(64, 64, 64, 3)
+        M = at.IndexMapping(nodes, dofs.size)
+        M.map[:] = dofs.ravel()
+        L = at.Tensor(nodes)
+        L.data[...] = workloads.counter_uniform(0xAC29, 0, (nodes,), -1.0, 1.0)
+        tensors["X"].SetTransient(name == "scatter_apply")
+        for t in list(tensors.values()) + [L]:
+            t.MoveToGPU()
+        engine.FlatIndexedScatter(tensors["X"], L, M)        # moves the map to the device
+
+        def step():
+            if name == "scatter_apply":
+                engine.BeginMultiKernelLaunch()
+                engine.FlatIndexedScatter(tensors["X"], L, M)
+            else:
+                engine.FlatIndexedScatter(tensors["X"], L, M)
+                engine.BeginMultiKernelLaunch()
+            for k, out, ins in wl.kernels:
+                engine(k, tensors[out], *[tensors[i] for i in ins])
+            engine.EndMultiKernelLaunch()
+        label = ("node vector [7189057] -> p=3 mass apply on 262144 elements, " +
+                 ("element vector read through the map in one launch" if name == "scatter_apply"
+                  else "scatter and apply as two steps"))
+        E = 262144
+        abytes = dofs.size * 4 + nodes * 8 + E * (1000 + 512)
+        if name == "scatter_then_apply":
+            abytes += 2 * dofs.size * 8                      # the element vector written, then read
+        flops = wl.flops
+        units, unit_name = wl.dof, "GDOF/s"
     elif name in ("scatter", "sumgather"):
         # node vector <-> element vector of the headline mesh size: 64^3 hex elements of degree 3
         import numpy as np
@@ -270,7 +307,7 @@ def main():
     ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store-all", action="store_true")
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "shapes"],
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "scatter_apply", "scatter_then_apply", "shapes"],
                     help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
                          "remaining baseline configurations at their full sizes and for the node-vector <-> "
                          "element-vector steps either side of the operator apply")

@@ -13,6 +13,17 @@
 namespace acro
 {
 
+class IndexMapping;
+
+// An operand of the next launch that need not exist in memory: entry i of `operand` is entry map[i] of `source`
+// (a FlatIndexedScatter that the engine recorded in a multi-kernel launch, with a transient result).
+struct GatheredInput
+{
+    Tensor *operand;
+    Tensor *source;
+    IndexMapping *map;
+};
+
 class KernelExecutor
 {
   public:
@@ -33,6 +44,10 @@ class KernelExecutor
         return GetImplementation();
     }
     virtual std::string GetExecType() = 0;
+    // Applies to the next ExecuteMulti / GetImplementation(tensors) call only.  A policy that cannot read an operand
+    // through its map must produce the operand first; the default keeps the list for the sequential fallback below.
+    // No counterpart in the reference, whose engine runs a scatter at the call (kernel/TensorEngine.cpp:673-689).
+    virtual void SetGatheredInputs(const std::vector<GatheredInput> &gathered) { Gathered = gathered; }
     virtual void ExecuteSingle(Tensor *output, std::vector<Tensor *> &inputs) = 0;
     // Default: one single-kernel executor per kernel, run in order
     virtual void ExecuteMulti(std::vector<Tensor *> &output, std::vector<std::vector<Tensor *>> &inputs);
@@ -42,6 +57,7 @@ class KernelExecutor
     void MoveTensorsToGPU(Tensor *output, std::vector<Tensor *> &inputs);
     void MoveTensorsToOutputLocation(Tensor *output, std::vector<Tensor *> &inputs);
 
+    std::vector<GatheredInput> Gathered;
     DimensionedMultiKernel *MultiKernel;
     DimensionedKernel *FirstKernel;
     std::vector<DimensionedMultiKernel *> SubKernels;

@@ -58,6 +58,8 @@ class TensorEngine
 
     void Clear();
     bool IsGPUAvailable() { return isHipReady(); }
+    // A FlatIndexedScatter issued in between whose result is marked transient and is only read by the kernels that
+    // follow is not run at all: those kernels read the source vector through the index map.
     // Kernels issued between Begin and End are captured and executed as ONE fused launch by End.  Batched matrix
     // inverses and determinants issued in between are captured too when a later kernel of the capture reads their
     // result: they become kernels of the fused launch, and a result marked transient never reaches device memory.
@@ -86,6 +88,10 @@ class TensorEngine
         Tensor *inverse;      // null for a determinant alone
         Tensor *determinant;  // null for an inverse alone
         Tensor *matrices;
+        // a recorded FlatIndexedScatter instead (the three above are null then)
+        Tensor *scatter_out;
+        Tensor *scatter_in;
+        IndexMapping *map;
     };
     // Executes the capture (or, with `implementation` set, only describes it).
     void FinishCapture(std::string *implementation);

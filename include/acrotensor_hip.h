@@ -106,7 +106,9 @@ int acro_engine_contract(acro_engine *e, const char *kernel, acro_tensor *out, a
                          int num_inputs);
 /* Between begin and end, acro_engine_batch_matrix_inverse / _det / _inv_det are recorded as well and run at end, in
  * program order with the recorded kernels; an operation whose result a later recorded kernel reads is fused into the
- * launch (the reference runs these operations at the call, kernel/TensorEngine.cpp:627-671). */
+ * launch (the reference runs these operations at the call, kernel/TensorEngine.cpp:627-671).  The same for
+ * acro_engine_flat_indexed_scatter: with a transient result that only later recorded kernels read, those kernels read the
+ * source through the map and the result is never written. */
 int acro_engine_begin_multi_kernel_launch(acro_engine *e); /* kernel/TensorEngine.cpp:318-325 */
 int acro_engine_end_multi_kernel_launch(acro_engine *e);   /* kernel/TensorEngine.cpp:328-336 */
 /* TensorEngine::GetImplementation: copies the generated HIP source (NUL terminated, truncated to buflen) and

@@ -178,6 +178,30 @@ def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE):
     assert "tile(k)=8" in src or "tile(i)=8" in src
 
 
+def scatter_then_mass_apply_source(TE, transient_x):
+    wl = workloads.config4(E=27)
+    tensors = workloads.bind_to_engine(wl, at, transient=True)
+    dofs, nodes = workloads.hex_mesh_dof_map(3, 3, 3, 3)
+    M, L = at.IndexMapping(nodes, dofs.size), at.Tensor(nodes)
+    M.map[:] = dofs.ravel()
+    tensors["X"].SetTransient(transient_x)
+    TE.BeginMultiKernelLaunch()
+    TE.FlatIndexedScatter(tensors["X"], L, M)
+    for k, out, ins in wl.kernels:
+        TE(k, tensors[out], *[tensors[n] for n in ins])
+    return TE.EndMultiKernelLaunchGetImplementation()
+
+
+def test_recorded_scatter_with_transient_result_is_read_through_its_map(TE):
+    src = scatter_then_mass_apply_source(TE, True)
+    assert src.count("__global__") == 1 and "X<-gathered" in src
+    assert "const int *__restrict__ G0m, const double *__restrict__ G0s" in src and "G0s[G0m[o_k0v1 + 0]]" in src
+    assert "runs on its own" not in src
+    # an element vector that has to exist afterwards: the scatter runs, the chain reads what it wrote
+    src = scatter_then_mass_apply_source(TE, False)
+    assert "runs on its own" in src and "gathered" not in src and "X<-global" in src
+
+
 def test_views_that_cannot_be_resolved_fall_back(TE):
     # the same parent viewed with the element index in two different positions cannot be fused
     T = at.Tensor(4, 4)
@@ -234,6 +258,7 @@ def generated_sources(TE):
     yield "operand staged in LDS", TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
     yield "split contraction, few long rows", TE.GetImplementation("S_i += A_i_n B_n", at.Tensor(6), at.Tensor(6, 9000), at.Tensor(9000))
     yield "transpose through LDS tiles", TE.GetImplementation("A_i_e_j -= B_j_e_i", at.Tensor(100, 3, 70), at.Tensor(70, 3, 100))
+    yield "operand read through an index map", scatter_then_mass_apply_source(TE, True)
     yield "contraction shared by lanes", TE.GetImplementation("A_e += B_e_i_j C_j_i", at.Tensor(1000), at.Tensor(1000, 5, 7), at.Tensor(7, 5))
     for transient in (True, False):
         yield "geometric factors from the Jacobians", geometric_factor_source(TE, 7, 4, 3, transient)
