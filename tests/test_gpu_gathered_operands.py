@@ -133,3 +133,35 @@ def test_full_mesh_apply_through_the_map_equals_scatter_then_apply(at, engine):
 
     fused, separate = apply(True), apply(False)
     assert np.abs(separate).max() > 0.0 and np.array_equal(fused, separate)
+
+
+def test_apply_through_the_map_replays_from_a_recorded_launch_sequence(at, engine, checker):
+    dofs, nodes, M = mesh(at, 4, 3)
+    wl = workloads.config4(E=dofs.shape[0])
+    tensors = workloads.bind_to_engine(wl, at, transient=True)
+    tensors["X"].SetTransient(True)
+    rng = np.random.default_rng(12)
+    L = to_tensor(at, rng.uniform(-1, 1, nodes))
+
+    def step():
+        engine.BeginMultiKernelLaunch()
+        engine.FlatIndexedScatter(tensors["X"], L, M)
+        for k, out, ins in wl.kernels:
+            engine(k, tensors[out], *[tensors[i] for i in ins])
+        engine.EndMultiKernelLaunch()
+
+    step()
+    with at.recorded_launches() as recording:
+        step()
+    for _ in range(3):
+        L.Mult(-0.5)                                      # eager work between the replays: a new node vector
+        at.synchronize()
+        recording.launch()
+        tensors["Y"].MoveFromGPU()
+        replayed = tensors["Y"].data.copy()
+        tensors["Y"].MoveToGPU()
+        tensors["Y"].Set(0.0)
+        step()
+        tensors["Y"].MoveFromGPU()
+        assert np.abs(replayed).max() > 0.0 and np.array_equal(replayed, tensors["Y"].data)
+        tensors["Y"].MoveToGPU()
