@@ -297,6 +297,16 @@ static void gpuTests()
         TE.FlatIndexedSumGather(back, big, M);
         back.MoveFromGPU();
         CHECK(back(1) == 9.0 && back(3) == 12.0 && back(5) == 6.0);
+        // a scatter recorded in a multi-kernel launch, result transient: the kernel reads `small` through the map
+        Tensor gathered(8), squares(8);
+        gathered.SetTransient(true);
+        TE.BeginMultiKernelLaunch();
+        TE.FlatIndexedScatter(gathered, small, M);
+        TE("Q_i = G_i G_i", squares, gathered, gathered);
+        TE.EndMultiKernelLaunch();
+        CHECK(TE.GetLastImplementation().find("G<-gathered") != std::string::npos);
+        squares.MoveFromGPU();
+        CHECK(squares(0) == 0.0 && squares(5) == 2500.0 && squares(6) == 100.0 && squares(7) == 900.0);
     }
 
     std::printf("gpu: externally owned device memory\n");
