@@ -173,6 +173,11 @@ class Generator
             EmitTranspose(plan);
             return plan;
         }
+        if (UseOperatorSchedule())
+        {
+            EmitOperator(plan);
+            return plan;
+        }
         ChooseTiles();
         PlanFusion();
         ChooseBatching();
@@ -3018,6 +3023,132 @@ class Generator
         launch.function_name = plan.module_name;
         launch.grid = static_cast<unsigned>(groups);
         launch.block = 256;
+        for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
+        plan.launches.push_back(launch);
+    }
+
+    // ------------------------------------------------------------------------------ operator schedule
+    // One dense operator applied to every batch entry: "A_e_i = B_i_j X_e_j" with B too large for scalar operands or a
+    // register tile (16 <= rows, columns; at most 4 096 entries), also with several row or column indices
+    // ("A_e_i1_i2 = B_i1_i2_j1_j2 X_e_j1_j2").  The generic schedule stages B in LDS and gives a lane one row and one
+    // entry, which is bound by the 64 LDS reads per output (17 % of the HBM peak for 64 x 64).  Here a lane keeps its
+    // row for four entries at a time, so one LDS read feeds four multiply-adds; the entry number is uniform in a
+    // wavefront, so X is read with scalar loads, and the lanes of a wavefront write consecutive outputs (38 %).
+    // Taking the entries' vectors into registers first and handing them round with readlane was slower (216 us).
+    static constexpr int kOperatorEntriesPerLane = 4;
+
+    bool OperatorPattern(const VarRef *&op, const VarRef *&x) const
+    {
+        if (subs.size() != 1 || batch < 0 || !opt.noalias || NumGatherSlots() > 0 || envInt("ACRO_HIP_OPERATOR") < 0) return false;
+        const Sub &s = subs[0];
+        if (s.matrixOp != 0 || s.in.size() != 2 || s.contr.empty() || s.out.repeated) return false;
+        op = has(s.in[0].idx, batch) ? &s.in[1] : &s.in[0];
+        x = has(s.in[0].idx, batch) ? &s.in[0] : &s.in[1];
+        if (op->repeated || x->repeated || has(op->idx, batch) || !has(x->idx, batch)) return false;
+        if (op->uvar == s.out.uvar || x->uvar == s.out.uvar || !IsPureInput(op->uvar) || !IsPureInput(x->uvar)) return false;
+        // out = (e, I...), X = (e, J...), B = (I..., J...) with the same orders
+        if (s.out.idx.empty() || s.out.idx[0] != batch || x->idx[0] != batch) return false;
+        const std::vector<int> rows(s.out.idx.begin() + 1, s.out.idx.end()), cols(x->idx.begin() + 1, x->idx.end());
+        if (rows.empty() || cols.empty()) return false;
+        std::vector<int> both = rows;
+        both.insert(both.end(), cols.begin(), cols.end());
+        if (op->idx != both) return false;
+        for (int id : cols)
+        {
+            if (!has(s.contr, id)) return false;
+        }
+        if (cols.size() != s.contr.size()) return false;
+        const long nI = product(rows, extent), nJ = product(cols, extent);
+        return nI >= 16 && nJ >= 16 && nI <= 1024 && nI * nJ <= 4096;
+    }
+
+    bool UseOperatorSchedule() const
+    {
+        const VarRef *op = nullptr, *x = nullptr;
+        return OperatorPattern(op, x);
+    }
+
+    void EmitOperator(HipKernelPlan &plan)
+    {
+        const Sub &s = subs[0];
+        const VarRef *opr = nullptr, *x = nullptr;
+        OperatorPattern(opr, x);
+        const long nJ = x->size / E, nI = s.out.size / E;
+        const int R = kOperatorEntriesPerLane;
+        const long LI = (nI + 63) / 64 * 64;             // lanes per group of R entries: whole wavefronts
+        // 512 lanes: the operator's copy in LDS allows four workgroups per CU, and the scalar loads of X come straight
+        // from device memory, so the wavefronts in flight are what hides their latency (64 x 64: 104 us with 256
+        // lanes, 87 us with 512, 93 us with 1 024).
+        const int NTo = static_cast<int>(std::max<long>(512, LI));
+        const long rowStride = nJ % 2 == 0 ? nJ + 1 : nJ;  // odd: the lanes' rows start in different LDS banks
+        // Entries per workgroup: enough for the copy of B to stay small against what the entries move.
+        // (64 x 64: 143 us with 16 entries per workgroup, 104 us with 64, the same with 128.)
+        long groupsPerBlock = std::max<long>(1, (nI * nJ / 64 + R - 1) / R);
+        groupsPerBlock = std::max<long>(groupsPerBlock, NTo / LI);
+        const long NBo = groupsPerBlock * R;
+        const long blocks = (E + NBo - 1) / NBo;
+        for (const auto &st : stores)
+        {
+            long entries = 1;
+            for (int d : st.dims) entries *= d;
+            if (entries >= (1L << 31) - 1) wide = true;
+        }
+
+        const std::string dimName = mk.GetDimensionedNameString();
+        char hex[32];
+        std::snprintf(hex, sizeof(hex), "%016llx",
+                      static_cast<unsigned long long>(hashString(dimName + "/operator/" + (Positional() ? "p" : "u"))));
+        plan.module_name = std::string("acro_op_") + hex;
+        std::ostringstream sched;
+        sched << "operator schedule: " << nI << " x " << nJ << " operator in LDS (row stride " << rowStride << "), " << NBo
+              << " entries per workgroup of " << NTo << " lanes, a lane keeps its row for " << R << " entries\n  [0] " << s.text << "\n";
+        plan.schedule = sched.str();
+
+        out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
+        {
+            std::istringstream lines(plan.schedule);
+            std::string l;
+            while (std::getline(lines, l)) out << "// " << l << "\n";
+        }
+        const std::string B = PtrName(opr->uvar), X = PtrName(x->uvar), A = PtrName(s.out.uvar);
+        const char *assign = s.op == '=' ? " = " : (s.op == '+' ? " += " : " -= ");
+        out << "typedef const __attribute__((address_space(4))) double *acro_scalar_ptr;\n";
+        out << "\nextern \"C\" __global__ __launch_bounds__(" << NTo << ") void " << plan.module_name << "(" << ParamList() << ")\n{\n";
+        out << "    __shared__ double rows[" << nI * rowStride << "];\n";
+        out << "    const int tid = threadIdx.x;\n";
+        out << "    for (int i = tid; i < " << nI * nJ << "; i += " << NTo << ") rows[(i / " << nJ << ") * " << rowStride << " + i % " << nJ
+            << "] = " << B << "[" << Lit(uvars[opr->uvar].viewOffset) << " + i];\n";
+        out << "    __syncthreads();\n";
+        out << "    const long e0 = (long)blockIdx.x * " << NBo << ";\n";
+        out << "    for (int w = tid; w < " << groupsPerBlock * LI << "; w += " << NTo << ")\n    {\n";
+        out << "        const int g = __builtin_amdgcn_readfirstlane(w / " << LI << ");  // whole wavefronts share the entries\n";
+        out << "        const int i = w - g * " << LI << ";\n";
+        out << "        const long e = e0 + g * " << R << ";\n";
+        out << "        if (i >= " << nI << " || e >= " << E << ") continue;\n";
+        out << "        const double *row = rows + i * " << rowStride << ";\n";
+        out << "        const acro_scalar_ptr x = (acro_scalar_ptr)(" << X << " + " << Lit(uvars[x->uvar].viewOffset) << " + e * " << nJ
+            << ");  // uniform: scalar loads\n";
+        out << "        double *a = " << A << " + " << Lit(uvars[s.out.uvar].viewOffset) << " + e * " << nI << " + i;\n";
+        out << "        if (e + " << R << " <= " << E << ")\n        {\n";
+        for (int r = 0; r < R; ++r) out << "            double s" << r << " = 0.0;\n";
+        out << "#pragma unroll 4\n";
+        out << "            for (int j = 0; j < " << nJ << "; ++j)\n            {\n                const double b = row[j];\n";
+        for (int r = 0; r < R; ++r) out << "                s" << r << " += b * x[" << r * nJ << " + j];\n";
+        out << "            }\n";
+        for (int r = 0; r < R; ++r) out << "            a[" << r * nI << "]" << assign << "s" << r << ";\n";
+        out << "        }\n        else\n        {\n";
+        out << "            for (int r = 0; e + r < " << E << "; ++r)\n            {\n                double sum = 0.0;\n";
+        out << "                for (int j = 0; j < " << nJ << "; ++j) sum += row[j] * x[r * " << nJ << " + j];\n";
+        out << "                a[r * " << nI << "]" << assign << "sum;\n            }\n        }\n    }\n}\n";
+
+        plan.source = out.str();
+        plan.nb = static_cast<int>(NBo);
+        plan.lds_bytes = static_cast<int>(nI * rowStride * 8);
+        FillParams(plan, false);
+        HipLaunch launch;
+        launch.function_name = plan.module_name;
+        launch.grid = static_cast<unsigned>(blocks);
+        launch.block = static_cast<unsigned>(NTo);
         for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
         plan.launches.push_back(launch);
     }

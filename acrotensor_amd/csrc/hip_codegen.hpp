@@ -28,6 +28,8 @@
 //    is split over workgroups and lanes, partial sums are added in a fixed order by a second one-workgroup kernel.
 //  * A single kernel that only permutes the dimensions of one operand, with different long fastest dimensions on the
 //    two sides, moves tiles of 32 x 32 entries through LDS ("transpose schedule").
+//  * A dense operator of up to 4 096 entries applied to every batch entry ("A_e_i = B_i_j X_e_j") runs the "operator
+//    schedule": operator rows in LDS, a lane keeps its row for four entries, the entries' vectors come in by scalar loads.
 //  * Contractions too long to unroll fall back to counted loops with the same lane mapping.
 //
 // Experiment switches (environment, read when a kernel is generated; defaults are what measured best on MI355X):
@@ -51,6 +53,8 @@
 //   ACRO_HIP_SPLIT_LANES=-1     one lane per batch entry also for kernels with one output per entry (no lane exchanges)
 //   ACRO_HIP_WAVE_UNIFORM=-1    no readfirstlane on the batch entry of wavefronts that hold items of one entry only
 //   ACRO_HIP_TRANSPOSE=-1       permutations with long fastest dimensions on both sides run as ordinary kernels (no LDS tiles)
+//   ACRO_HIP_OPERATOR=-1        a dense operator applied to every batch entry runs through the generic schedule (operator staged
+//                               in LDS, one entry per lane) instead of the operator schedule
 //   ACRO_HIP_RED_PENCIL=-1      split contractions: one lane per (slice, output entry) also when there are few outputs
 //   ACRO_HIP_RED_ROWS=-1        split contractions of few long rows: all outputs in every workgroup, NT / outputs lanes along a row
 //   ACRO_HIP_ONE_PASS=1         split contractions: the workgroup that finishes last adds the per-workgroup partials

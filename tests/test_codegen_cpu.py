@@ -157,13 +157,28 @@ def test_diffusion_chain_batching_follows_the_contractions_not_the_pointwise_ker
 def test_small_invariant_operand_read_by_rows_is_staged_in_lds(TE):
     # lane i walks along row i of B: from device memory every load instruction would touch 64 lines; each workgroup
     # copies B to LDS once (row stride 65, so that the lanes fall into different banks) and serves 16 entries
-    src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
+    src = TE.GetImplementation("A_e_i = B_i_j X_e_j W_e", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64), at.Tensor(1000))
     assert "B<-lds" in src and "// B: device memory -> LDS, once per workgroup" in src
     assert "a += (r_ / 64) * 65" in src and "16 per workgroup of 256 lanes" in src
-    assert src.index("__syncthreads()") < src.index("// A_e_i = B_i_j X_e_j")
+    assert src.index("__syncthreads()") < src.index("// A_e_i = B_i_j X_e_j W_e")
     # a table that the lanes read at unit stride, or one read through scalar loads, is left where it is
     assert "<-lds" not in TE.GetImplementation("A_e_i = B_j_i X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
     assert "B<-scalar" in TE.GetImplementation("A_e_q_j = B_q_i X_e_i_j", at.Tensor(500, 5, 16), at.Tensor(5, 4), at.Tensor(500, 4, 16))
+
+
+def test_dense_operator_per_entry_uses_the_operator_schedule(TE):
+    src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
+    assert "operator schedule: 64 x 64 operator in LDS (row stride 65), 64 entries per workgroup of 512 lanes" in src
+    assert "__builtin_amdgcn_readfirstlane" in src and "acro_scalar_ptr x" in src and src.count("+= b * x[") == 4
+    # several row and column indices, operands in the other order, -=
+    src = TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(77, 5, 6), at.Tensor(77, 4, 7), at.Tensor(5, 6, 4, 7))
+    assert "operator schedule: 30 x 28 operator" in src and "] -= s3;" in src
+    # not this schedule: few rows (a register tile with scalar operands serves them), transposed operator, third operand
+    for kernel, shapes in (("A_e_i = B_i_j X_e_j", [(500, 4), (4, 64), (500, 64)]),
+                           ("A_e_i = B_j_i X_e_j", [(500, 64), (64, 64), (500, 64)]),
+                           ("A_e_i = B_i_j X_e_j W_e", [(500, 64), (64, 64), (500, 64), (500,)])):
+        tensors = [at.Tensor(*shp) for shp in shapes]
+        assert "operator schedule" not in TE.GetImplementation(kernel, *tensors)
 
 
 def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE):
@@ -255,7 +270,8 @@ def generated_sources(TE):
         at.Tensor(4, 5, 5, 5, 3, 3))
     yield "one name, two tensors", TE.GetImplementation("A_m_n = B_m_j B_n_j", at.Tensor(3, 3), at.Tensor(3, 4), at.Tensor(3, 4))
     yield "repeated output index", TE.GetImplementation("A_i_i = B_i", at.Tensor(6, 6), at.Tensor(6))
-    yield "operand staged in LDS", TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
+    yield "operand staged in LDS", TE.GetImplementation("A_e_i = B_i_j X_e_j W_e", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64), at.Tensor(1000))
+    yield "operator schedule", TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(77, 5, 6), at.Tensor(77, 4, 7), at.Tensor(5, 6, 4, 7))
     yield "split contraction, few long rows", TE.GetImplementation("S_i += A_i_n B_n", at.Tensor(6), at.Tensor(6, 9000), at.Tensor(9000))
     yield "transpose through LDS tiles", TE.GetImplementation("A_i_e_j -= B_j_e_i", at.Tensor(100, 3, 70), at.Tensor(70, 3, 100))
     yield "operand read through an index map", scatter_then_mass_apply_source(TE, True)

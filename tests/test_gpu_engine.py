@@ -407,8 +407,8 @@ def test_slice_of_a_slice_inside_a_fused_launch(at, engine):
 
 
 @pytest.mark.parametrize("kernel,shapes", [
-    ("A_e_i = B_i_j X_e_j", [(64, 64), (1000, 64)]),             # B staged in LDS, 16 entries per workgroup, ragged end
-    ("A_e_i = B_i_j X_e_j", [(40, 24), (3, 24)]),                # fewer entries than a workgroup would take
+    ("A_e_i = B_i_j X_e_j W_e", [(64, 64), (1000, 64), (1000,)]),   # B staged in LDS, 16 entries per workgroup, ragged end
+    ("A_e_i = B_i_j X_e_j W_e", [(40, 24), (3, 24), (3,)]),      # fewer entries than a workgroup would take
     ("A_e_i_k = B_i_j C_k_l X_e_j_l", [(12, 10), (9, 11), (77, 10, 11)]),   # two staged tables, reordered into steps
     ("A_e_i_k = B_e_i_j C_e_j_k", [(1001, 4, 4), (1001, 4, 4)]), # one output per lane
     ("A_e_i_k = B_e_i_j C_e_j_k", [(333, 3, 3), (333, 3, 3)]),
@@ -480,3 +480,23 @@ def test_permutations_with_long_fastest_dimensions_go_through_lds_tiles(at, engi
     if "-=" in kernel:
         expected = 2.0 * out0 - expected
     assert np.array_equal(got, expected)             # moves (and one addition): bit for bit
+
+
+@pytest.mark.parametrize("kernel,shapes", [
+    ("A_e_i = B_i_j X_e_j", [(64, 64), (1000, 64)]),
+    ("A_e_i -= B_i_j X_e_j", [(40, 30), (1001, 30)]),                     # ragged: 1001 entries, rows of 30
+    ("A_e_i += X_e_j B_i_j", [(20, 17), (23, 17)]),                       # operands the other way round, 23 entries
+    ("A_e_i1_i2 = B_i1_i2_j1_j2 X_e_j1_j2", [(5, 6, 4, 7), (77, 4, 7)]),  # several row and column indices
+    ("A_e_i = B_i_j X_e_j", [(1000, 4), (9, 4)]),                         # 1000 rows of 4: not this schedule
+])
+def test_dense_operator_applied_to_every_entry(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(shapes[0][0])
+    if kernel.startswith("A_e_i += X"):
+        shapes = [shapes[1], shapes[0]]
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert ("operator schedule" in engine.GetLastImplementation()) == (shapes[0] != (1000, 4))
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
