@@ -3030,50 +3030,88 @@ class Generator
     // ------------------------------------------------------------------------------ operator schedule
     // One dense operator applied to every batch entry: "A_e_i = B_i_j X_e_j" with B too large for scalar operands or a
     // register tile (16 <= rows, columns; at most 4 096 entries), also with several row or column indices
-    // ("A_e_i1_i2 = B_i1_i2_j1_j2 X_e_j1_j2").  The generic schedule stages B in LDS and gives a lane one row and one
-    // entry, which is bound by the 64 LDS reads per output (17 % of the HBM peak for 64 x 64).  Here a lane keeps its
+    // ("A_e_i1_i2 = B_i1_i2_j1_j2 X_e_j1_j2") and with several leading indices numbering the entries
+    // ("A_e_q_i = B_i_j X_e_q_j").  The generic schedule stages B in LDS and gives a lane one row and one
+    // entry, which is bound by the 64 LDS reads per output (17 % of the HBM peak for 64 x 64).  Two variants:
+    // rows a multiple of 16 and columns a multiple of 8 go to the FP64 matrix cores (EmitOperatorMatrixCores, 72 %;
+    // the operator may then also be stored transposed, "B_j_i").  Otherwise a lane keeps its
     // row for four entries at a time, so one LDS read feeds four multiply-adds; the entry number is uniform in a
-    // wavefront, so X is read with scalar loads, and the lanes of a wavefront write consecutive outputs (38 %).
+    // wavefront, so X is read with scalar loads, and the lanes of a wavefront write consecutive outputs (43 %).
     // Taking the entries' vectors into registers first and handing them round with readlane was slower (216 us).
     static constexpr int kOperatorEntriesPerLane = 4;
 
-    bool OperatorPattern(const VarRef *&op, const VarRef *&x) const
+    struct OperatorShape
+    {
+        const VarRef *op = nullptr, *x = nullptr;
+        long rows = 0, cols = 0, entries = 0;
+        bool transposed = false;   // the operator is stored with the contracted indices first: "B_j_i"
+        bool cores = false;        // sizes and alignment suit the FP64 matrix cores
+    };
+
+    bool OperatorPattern(OperatorShape &o) const
     {
         if (subs.size() != 1 || batch < 0 || !opt.noalias || NumGatherSlots() > 0 || envInt("ACRO_HIP_OPERATOR") < 0) return false;
         const Sub &s = subs[0];
         if (s.matrixOp != 0 || s.in.size() != 2 || s.contr.empty() || s.out.repeated) return false;
-        op = has(s.in[0].idx, batch) ? &s.in[1] : &s.in[0];
-        x = has(s.in[0].idx, batch) ? &s.in[0] : &s.in[1];
-        if (op->repeated || x->repeated || has(op->idx, batch) || !has(x->idx, batch)) return false;
-        if (op->uvar == s.out.uvar || x->uvar == s.out.uvar || !IsPureInput(op->uvar) || !IsPureInput(x->uvar)) return false;
-        // out = (e, I...), X = (e, J...), B = (I..., J...) with the same orders
-        if (s.out.idx.empty() || s.out.idx[0] != batch || x->idx[0] != batch) return false;
-        const std::vector<int> rows(s.out.idx.begin() + 1, s.out.idx.end()), cols(x->idx.begin() + 1, x->idx.end());
+        o.op = has(s.in[0].idx, batch) ? &s.in[1] : &s.in[0];
+        o.x = has(s.in[0].idx, batch) ? &s.in[0] : &s.in[1];
+        if (o.op->repeated || o.x->repeated || has(o.op->idx, batch) || !has(o.x->idx, batch)) return false;
+        if (o.op->uvar == s.out.uvar || o.x->uvar == s.out.uvar || !IsPureInput(o.op->uvar) || !IsPureInput(o.x->uvar)) return false;
+        // out = (e..., I...), X = (e..., J...), B = (I..., J...) or (J..., I...): the leading indices that the result
+        // and X share, the batch index first, number the entries
+        if (s.out.idx.empty() || s.out.idx[0] != batch || o.x->idx[0] != batch) return false;
+        size_t shared = 0;
+        while (shared < s.out.idx.size() && shared < o.x->idx.size() && s.out.idx[shared] == o.x->idx[shared] &&
+               !has(o.op->idx, s.out.idx[shared]))
+            ++shared;
+        const std::vector<int> lead(s.out.idx.begin(), s.out.idx.begin() + shared);
+        const std::vector<int> rows(s.out.idx.begin() + shared, s.out.idx.end()), cols(o.x->idx.begin() + shared, o.x->idx.end());
         if (rows.empty() || cols.empty()) return false;
-        std::vector<int> both = rows;
-        both.insert(both.end(), cols.begin(), cols.end());
-        if (op->idx != both) return false;
+        std::vector<int> plain = rows, swapped = cols;
+        plain.insert(plain.end(), cols.begin(), cols.end());
+        swapped.insert(swapped.end(), rows.begin(), rows.end());
+        if (o.op->idx != plain && o.op->idx != swapped) return false;
+        o.transposed = o.op->idx != plain;
         for (int id : cols)
         {
             if (!has(s.contr, id)) return false;
         }
         if (cols.size() != s.contr.size()) return false;
-        const long nI = product(rows, extent), nJ = product(cols, extent);
-        return nI >= 16 && nJ >= 16 && nI <= 1024 && nI * nJ <= 4096;
+        o.rows = product(rows, extent);
+        o.cols = product(cols, extent);
+        o.entries = product(lead, extent);
+        if (o.rows > 1024 || o.rows * o.cols > 4096) return false;
+        o.cores = envInt("ACRO_HIP_OPERATOR_MFMA") >= 0;
+        if (!o.cores) return o.rows >= 16 && o.cols >= 16 && !o.transposed;  // (its lanes walk the operator's rows)
+        // Small operators: the generic schedule (operator in scalar registers, an entry or an output per lane) reads
+        // and writes short pieces per lane and reaches 40 - 65 % of the HBM peak; 16 entries per wavefront on the
+        // matrix cores reach 70 - 88 % as long as the entries' vectors come in 16-byte loads (even length) and five
+        // or more rows fill the stores, or the vectors are long.  Measured wins: 8 x 4 53 -> 73 %, 16 x 4 43 -> 84 %,
+        // 8 x 8 61 -> 85 %, 10 x 10 52 -> 81 %, 8 x 16 62 -> 85 %, 3 x 27 41 -> 73 %; losses, hence excluded:
+        // 4 x 4 65 -> 49 %, 4 x 8 82 -> 77 %, 7 x 9 62 -> 57 %, 27 x 3 36 -> 28 %; 20 x 5 a tie.
+        const bool pairs = o.cols % 2 == 0 && uvars[o.x->uvar].viewOffset % 2 == 0;
+        return pairs ? (o.rows >= 5 && o.cols >= 4) : o.cols >= 16;
     }
 
     bool UseOperatorSchedule() const
     {
-        const VarRef *op = nullptr, *x = nullptr;
-        return OperatorPattern(op, x);
+        OperatorShape o;
+        return OperatorPattern(o);
     }
 
     void EmitOperator(HipKernelPlan &plan)
     {
         const Sub &s = subs[0];
-        const VarRef *opr = nullptr, *x = nullptr;
-        OperatorPattern(opr, x);
-        const long nJ = x->size / E, nI = s.out.size / E;
+        OperatorShape shape;
+        OperatorPattern(shape);
+        const VarRef *opr = shape.op, *x = shape.x;
+        const long nJ = shape.cols, nI = shape.rows;
+        const long E = shape.entries;        // entries of this schedule: all leading indices together
+        if (shape.cores)
+        {
+            EmitOperatorMatrixCores(plan, shape);
+            return;
+        }
         const int R = kOperatorEntriesPerLane;
         const long LI = (nI + 63) / 64 * 64;             // lanes per group of R entries: whole wavefronts
         // 512 lanes: the operator's copy in LDS allows four workgroups per CU, and the scalar loads of X come straight
@@ -3131,7 +3169,9 @@ class Generator
         out << "        double *a = " << A << " + " << Lit(uvars[s.out.uvar].viewOffset) << " + e * " << nI << " + i;\n";
         out << "        if (e + " << R << " <= " << E << ")\n        {\n";
         for (int r = 0; r < R; ++r) out << "            double s" << r << " = 0.0;\n";
-        out << "#pragma unroll 4\n";
+        // Eight terms per trip: the entry's operand words of one trip arrive in one scalar load per entry, and two
+        // trips' worth in flight hide the scalar cache's latency (measured: 119 / 87 / 79 / 78 us at 2 / 4 / 8 / 16).
+        out << "#pragma unroll 8\n";
         out << "            for (int j = 0; j < " << nJ << "; ++j)\n            {\n                const double b = row[j];\n";
         for (int r = 0; r < R; ++r) out << "                s" << r << " += b * x[" << r * nJ << " + j];\n";
         out << "            }\n";
@@ -3149,6 +3189,137 @@ class Generator
         launch.function_name = plan.module_name;
         launch.grid = static_cast<unsigned>(blocks);
         launch.block = static_cast<unsigned>(NTo);
+        for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
+        plan.launches.push_back(launch);
+    }
+
+    // The same on the FP64 matrix cores: a wavefront takes 16 entries at a time and forms their nI outputs with
+    // v_mfma_f64_16x16x4 (16 entries x 16 outputs x 4 terms per instruction).  The entries' vectors are the
+    // instruction's first operand, read with ordinary 16-byte vector loads (lane = entry + 16 * term group); the
+    // operator sits in LDS in the order the second operand wants it, one conflict-free 8-byte read per lane and
+    // instruction; a lane holds outputs (entry 4r + lane / 16, output lane % 16) in register r, so one store
+    // instruction writes four runs of 128 bytes.  The order of the terms inside a step is free as long as both
+    // operands agree: term group g of step s stands for j = 8 (s / 2) + 2 g + s % 2, which makes the entry's two
+    // doubles of a 16-byte load the operands of two successive steps.  MI355X's vector and matrix FP64 peaks are the
+    // same; what the matrix cores save is operand delivery: no scalar loads and 1/16 of the LDS reads.
+    // 64 x 64 on 2^18 entries: 47 - 51 us against 79 us with scalar loads (512 workgroups; 58 us with 1 024, 76 us
+    // with 2 048; loading the next 16 entries ahead of the arithmetic made no difference).
+    void EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape &shape)
+    {
+        const Sub &s = subs[0];
+        const VarRef &opr = *shape.op, &x = *shape.x;
+        const long nI = shape.rows, nJ = shape.cols, E = shape.entries;
+        // Sizes that the instruction's 16 x 4 blocks do not divide: the operator's copy in LDS is padded with zero
+        // rows and columns, the entries' vectors read as zero past their end, outputs past the last row are not
+        // stored.  Pairs of doubles (16-byte loads) need an even row length and an even first element.
+        const bool pairs = nJ % 2 == 0 && uvars[x.uvar].viewOffset % 2 == 0;
+        const long nIp = (nI + 15) / 16 * 16, nJp = pairs ? (nJ + 7) / 8 * 8 : (nJ + 3) / 4 * 4;
+        const long tilesN = nIp / 16, steps = nJp / 4;
+        const long tiles = (E + 15) / 16;
+        const bool ragged = E % 16 != 0;
+        // Equal work per CU matters more than the number of wavefronts: 256 CUs, one or two workgroups each.
+        // (Small operators, 8 x 8 to 32 x 32: the same with 512, 1 024, 2 048 or 4 096 workgroups.)
+        const long blocks = std::max<long>(1, std::min<long>(512, (tiles + 3) / 4));
+        for (const auto &st : stores)
+        {
+            long entries = 1;
+            for (int d : st.dims) entries *= d;
+            if (entries >= (1L << 31) - 1) wide = true;
+        }
+        const std::string dimName = mk.GetDimensionedNameString();
+        char hex[32];
+        std::snprintf(hex, sizeof(hex), "%016llx",
+                      static_cast<unsigned long long>(hashString(dimName + "/operator-mfma/" + (Positional() ? "p" : "u") + (pairs ? "2" : "1"))));
+        plan.module_name = std::string("acro_op_") + hex;
+        std::ostringstream sched;
+        sched << "operator schedule on the FP64 matrix cores: " << nI << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator")
+              << " in LDS in operand order";
+        if (nIp != nI || nJp != nJ) sched << " (padded to " << nIp << " x " << nJp << ")";
+        sched << ", " << E << " entries, 16 per wavefront and trip, "
+              << tilesN * steps << " v_mfma_f64_16x16x4 per trip, " << blocks << " workgroups of 256 lanes\n  [0] " << s.text << "\n";
+        plan.schedule = sched.str();
+
+        out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
+        {
+            std::istringstream lines(plan.schedule);
+            std::string l;
+            while (std::getline(lines, l)) out << "// " << l << "\n";
+        }
+        const std::string B = PtrName(opr.uvar), X = PtrName(x.uvar), A = PtrName(s.out.uvar);
+        const bool stream = s.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0;
+        // term group g (lane / 16) of step s stands for this j
+        const std::string termOf = pairs ? "8 * (step >> 1) + 2 * (l >> 4) + (step & 1)" : "4 * step + (l >> 4)";
+        out << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
+        out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << plan.module_name << "(" << ParamList() << ")\n{\n";
+        out << "    __shared__ double frag[" << nIp * nJp << "];\n";
+        out << "    for (int f = threadIdx.x; f < " << nIp * nJp << "; f += 256)\n    {\n";
+        out << "        const int l = f & 63, step = (f >> 6) % " << steps << ", t = (f >> 6) / " << steps << ";\n";
+        out << "        const int row = 16 * t + (l & 15), j = " << termOf << ";\n";
+        const std::string element = B + "[" + Lit(uvars[opr.uvar].viewOffset) + (shape.transposed ? " + j * " + str(nI) + " + row]" : " + row * " + str(nJ) + " + j]");
+        if (nIp != nI || nJp != nJ)
+            out << "        frag[f] = row < " << nI << " && j < " << nJ << " ? " << element << " : 0.0;\n    }\n";
+        else
+            out << "        frag[f] = " << element << ";\n    }\n";
+        out << "    __syncthreads();\n";
+        out << "    const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;\n";
+        out << "    const long waves = (long)gridDim.x * 4;\n";
+        out << "    for (long tile = (long)blockIdx.x * 4 + (threadIdx.x >> 6); tile < " << tiles << "; tile += waves)\n    {\n";
+        if (ragged)
+            out << "        const long ex = tile * 16 + c < " << E << " ? tile * 16 + c : " << E - 1 << ";  // past the end: any valid entry, never stored\n";
+        else
+            out << "        const long ex = tile * 16 + c;\n";
+        if (pairs)
+        {
+            out << "        const double *x = " << X << " + " << Lit(uvars[x.uvar].viewOffset) << " + ex * " << nJ << " + 2 * g;\n";
+            out << "        double2 xv[" << nJp / 8 << "];\n";
+            out << "#pragma unroll\n";
+            out << "        for (int q = 0; q < " << nJp / 8 << "; ++q) xv[q] = ";
+            if (nJp != nJ) out << "8 * q + 2 * g >= " << nJ << " ? double2{0.0, 0.0} : ";
+            out << "*reinterpret_cast<const double2 *>(x + 8 * q);\n";
+        }
+        else
+        {
+            out << "        const double *x = " << X << " + " << Lit(uvars[x.uvar].viewOffset) << " + ex * " << nJ << " + g;\n";
+            out << "        double xv[" << steps << "];\n";
+            out << "#pragma unroll\n";
+            out << "        for (int q = 0; q < " << steps << "; ++q) xv[q] = ";
+            if (nJp != nJ) out << "4 * q + g >= " << nJ << " ? 0.0 : ";
+            out << "x[4 * q];\n";
+        }
+        out << "        acro_double4 acc[" << tilesN << "];\n";
+        out << "#pragma unroll\n";
+        out << "        for (int t = 0; t < " << tilesN << "; ++t) acc[t] = acro_double4{0.0, 0.0, 0.0, 0.0};\n";
+        out << "#pragma unroll\n";
+        out << "        for (int step = 0; step < " << steps << "; ++step)\n        {\n";
+        if (pairs)
+            out << "            const double xs = (step & 1) ? xv[step >> 1].y : xv[step >> 1].x;\n";
+        else
+            out << "            const double xs = xv[step];\n";
+        out << "#pragma unroll\n";
+        out << "            for (int t = 0; t < " << tilesN << "; ++t)\n";
+        out << "                acc[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(xs, frag[(t * " << steps << " + step) * 64 + lane], acc[t], 0, 0, 0);\n";
+        out << "        }\n";
+        out << "        double *a = " << A << " + " << Lit(uvars[s.out.uvar].viewOffset) << " + (tile * 16 + g) * " << nI << " + c;\n";
+        out << "#pragma unroll\n";
+        out << "        for (int r = 0; r < 4; ++r)\n        {\n";
+        if (ragged) out << "            if (tile * 16 + g + 4 * r >= " << E << ") continue;\n";
+        out << "#pragma unroll\n";
+        out << "            for (int t = 0; t < " << tilesN << "; ++t)\n";
+        std::string guard = nIp != nI ? "if (16 * t + c < " + str(nI) + ") " : "";
+        if (stream)
+            out << "                " << guard << "__builtin_nontemporal_store(acc[t][r], a + 4 * r * " << nI << " + 16 * t);\n";
+        else
+            out << "                " << guard << "a[4 * r * " << nI << " + 16 * t]" << (s.op == '=' ? " = " : (s.op == '+' ? " += " : " -= ")) << "acc[t][r];\n";
+        out << "        }\n    }\n}\n";
+
+        plan.source = out.str();
+        plan.nb = 64;
+        plan.lds_bytes = static_cast<int>(nIp * nJp * 8);
+        FillParams(plan, false);
+        HipLaunch launch;
+        launch.function_name = plan.module_name;
+        launch.grid = static_cast<unsigned>(blocks);
+        launch.block = 256;
         for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
         plan.launches.push_back(launch);
     }

@@ -166,19 +166,40 @@ def test_small_invariant_operand_read_by_rows_is_staged_in_lds(TE):
     assert "B<-scalar" in TE.GetImplementation("A_e_q_j = B_q_i X_e_i_j", at.Tensor(500, 5, 16), at.Tensor(5, 4), at.Tensor(500, 4, 16))
 
 
-def test_dense_operator_per_entry_uses_the_operator_schedule(TE):
+def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
+    # FP64 matrix cores, 16 entries per wavefront and trip
     src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
-    assert "operator schedule: 64 x 64 operator in LDS (row stride 65), 64 entries per workgroup of 512 lanes" in src
-    assert "__builtin_amdgcn_readfirstlane" in src and "acro_scalar_ptr x" in src and src.count("+= b * x[") == 4
-    # several row and column indices, operands in the other order, -=
+    assert "operator schedule on the FP64 matrix cores: 64 x 64 operator in LDS in operand order, 1000 entries" in src
+    assert "__builtin_amdgcn_mfma_f64_16x16x4f64(xs, frag[(t * 16 + step) * 64 + lane], acc[t], 0, 0, 0)" in src
+    assert "j = 8 * (step >> 1) + 2 * (l >> 4) + (step & 1);" in src and "a + 4 * r * 64 + 16 * t" in src
+    assert "tile * 16 + c < 1000 ? tile * 16 + c : 999" in src and "if (tile * 16 + g + 4 * r >= 1000) continue;" in src
+    src = TE.GetImplementation("A_e_i += B_i_j X_e_j", at.Tensor(1024, 32), at.Tensor(32, 24), at.Tensor(1024, 24))
+    assert "32 x 24 operator" in src and "padded" not in src and "a[4 * r * 32 + 16 * t] += acc[t][r];" in src and "continue" not in src
+    # the operator stored transposed, and two leading indices that number the entries
+    src = TE.GetImplementation("A_e_q_i = B_j_i X_e_q_j", at.Tensor(100, 7, 32), at.Tensor(24, 32), at.Tensor(100, 7, 24))
+    assert "32 x 24 operator (stored transposed) in LDS in operand order, 700 entries" in src
+    assert "T1[0 + j * 32 + row]" in src and "tile * 16 + c < 700" in src
+    # sizes that 16 x 4 blocks do not divide: zero rows and columns in LDS, guarded loads and stores; an odd row
+    # length means single 8-byte loads of the entries' vectors
     src = TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(77, 5, 6), at.Tensor(77, 4, 7), at.Tensor(5, 6, 4, 7))
-    assert "operator schedule: 30 x 28 operator" in src and "] -= s3;" in src
-    # not this schedule: few rows (a register tile with scalar operands serves them), transposed operator, third operand
+    assert "30 x 28 operator in LDS in operand order (padded to 32 x 32)" in src
+    assert "frag[f] = row < 30 && j < 28 ? T2[0 + row * 28 + j] : 0.0;" in src
+    assert "8 * q + 2 * g >= 28 ? double2{0.0, 0.0} :" in src and "if (16 * t + c < 30) a[4 * r * 30 + 16 * t] -= acc[t][r];" in src
+    src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 30), at.Tensor(30, 27), at.Tensor(1000, 27))
+    assert "(padded to 32 x 28)" in src and "j = 4 * step + (l >> 4);" in src and "xv[q] = 4 * q + g >= 27 ? 0.0 : x[4 * q];" in src
+    # not this schedule: few rows (a register tile with scalar operands serves them), third operand
     for kernel, shapes in (("A_e_i = B_i_j X_e_j", [(500, 4), (4, 64), (500, 64)]),
-                           ("A_e_i = B_j_i X_e_j", [(500, 64), (64, 64), (500, 64)]),
                            ("A_e_i = B_i_j X_e_j W_e", [(500, 64), (64, 64), (500, 64), (500,)])):
         tensors = [at.Tensor(*shp) for shp in shapes]
         assert "operator schedule" not in TE.GetImplementation(kernel, *tensors)
+    # without the matrix cores: a lane keeps its row for four entries, whose vectors come through scalar loads
+    monkeypatch.setenv("ACRO_HIP_OPERATOR_MFMA", "-1")
+    src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 60), at.Tensor(60, 60), at.Tensor(1000, 60))
+    assert "operator schedule: 60 x 60 operator in LDS (row stride 61), 56 entries per workgroup of 512 lanes" in src
+    assert "__builtin_amdgcn_readfirstlane" in src and "acro_scalar_ptr x" in src and src.count("+= b * x[") == 4
+    src = TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(78, 5, 6), at.Tensor(78, 4, 7), at.Tensor(5, 6, 4, 7))
+    assert "operator schedule: 30 x 28 operator" in src and "] -= s3;" in src
+    assert "operator schedule" not in TE.GetImplementation("A_e_i = B_j_i X_e_j", at.Tensor(500, 64), at.Tensor(64, 64), at.Tensor(500, 64))
 
 
 def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE):
@@ -272,6 +293,8 @@ def generated_sources(TE):
     yield "repeated output index", TE.GetImplementation("A_i_i = B_i", at.Tensor(6, 6), at.Tensor(6))
     yield "operand staged in LDS", TE.GetImplementation("A_e_i = B_i_j X_e_j W_e", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64), at.Tensor(1000))
     yield "operator schedule", TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(77, 5, 6), at.Tensor(77, 4, 7), at.Tensor(5, 6, 4, 7))
+    yield "operator schedule, no padding", TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(77, 8, 6), at.Tensor(77, 4, 10), at.Tensor(8, 6, 4, 10))
+    yield "operator schedule, odd row length", TE.GetImplementation("A_e_i = B_j_i X_e_j", at.Tensor(500, 17), at.Tensor(33, 17), at.Tensor(500, 33))
     yield "split contraction, few long rows", TE.GetImplementation("S_i += A_i_n B_n", at.Tensor(6), at.Tensor(6, 9000), at.Tensor(9000))
     yield "transpose through LDS tiles", TE.GetImplementation("A_i_e_j -= B_j_e_i", at.Tensor(100, 3, 70), at.Tensor(70, 3, 100))
     yield "operand read through an index map", scatter_then_mass_apply_source(TE, True)
@@ -340,6 +363,9 @@ def test_every_kind_of_generated_kernel_compiles_for_gfx950(TE, monkeypatch):
     monkeypatch.setenv("ACRO_HIP_ONE_PASS", "1")
     sources.append(("split contraction, one launch",
                     TE.GetImplementation("S_i_j = A_n_i_j B_n", at.Tensor(3, 3), at.Tensor(70001, 3, 3), at.Tensor(70001))))
+    monkeypatch.setenv("ACRO_HIP_OPERATOR_MFMA", "-1")
+    sources.append(("operator schedule through scalar loads",
+                    TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(79, 5, 6), at.Tensor(79, 4, 7), at.Tensor(5, 6, 4, 7))))
     for name, src in sources:
         assert "__global__" in src, name
         size = ctypes.c_size_t(0)

@@ -487,7 +487,27 @@ def test_permutations_with_long_fastest_dimensions_go_through_lds_tiles(at, engi
     ("A_e_i -= B_i_j X_e_j", [(40, 30), (1001, 30)]),                     # ragged: 1001 entries, rows of 30
     ("A_e_i += X_e_j B_i_j", [(20, 17), (23, 17)]),                       # operands the other way round, 23 entries
     ("A_e_i1_i2 = B_i1_i2_j1_j2 X_e_j1_j2", [(5, 6, 4, 7), (77, 4, 7)]),  # several row and column indices
-    ("A_e_i = B_i_j X_e_j", [(1000, 4), (9, 4)]),                         # 1000 rows of 4: not this schedule
+    ("A_e_i = B_i_j X_e_j", [(1000, 4), (9, 4)]),                         # 1000 rows for 9 entries: not this schedule
+    # rows a multiple of 16, columns a multiple of 8: nothing to pad for the FP64 matrix cores
+    ("A_e_i -= B_i_j X_e_j", [(48, 40), (1001, 40)]),                     # ragged: 9 entries in the last trip
+    ("A_e_i += X_e_j B_i_j", [(16, 16), (23, 16)]),                       # operands the other way round, two trips
+    ("A_e_i = B_i_j X_e_j", [(32, 24), (4096, 24)]),                      # whole trips only
+    ("A_e_i = B_i_j X_e_j", [(16, 16), (40007, 16)]),                     # more trips than wavefronts
+    ("A_e_i = B_i_j X_e_j", [(16, 256), (300, 256)]),                     # 64 terms steps, one output tile
+    ("A_e_i = B_i_j X_e_j", [(256, 16), (300, 16)]),                      # 16 output tiles
+    ("A_e_i1_i2 -= B_i1_i2_j1_j2 X_e_j1_j2", [(8, 6, 4, 10), (77, 4, 10)]),
+    ("A_e_i = B_j_i X_e_j", [(40, 48), (1001, 40)]),                      # the operator stored transposed
+    ("A_e_q_i += B_j_i X_e_q_j", [(24, 32), (100, 7, 24)]),               # 700 entries numbered by two indices
+    ("A_e_q_i = B_i_j X_e_q_j", [(30, 20), (100, 7, 20)]),                # padded to 32 x 24
+    ("A_e_i = B_j_i X_e_j", [(33, 17), (500, 33)]),                       # odd row length: 8-byte loads, padded to 32 x 36
+    # small operators: with vectors of even length from five rows on, with odd length from 16 columns on
+    ("A_e_i = B_i_j X_e_j", [(8, 8), (5000, 8)]),
+    ("A_e_i -= B_i_j X_e_j", [(8, 4), (5001, 4)]),
+    ("A_e_i += B_i_j X_e_j", [(10, 10), (777, 10)]),
+    ("A_e_i = B_i_j X_e_j", [(3, 27), (900, 27)]),
+    ("A_e_i_k = B_e_i_j C_j_k", [(600, 8, 8), (8, 8)]),                   # entries (e, i), operator stored transposed
+    ("A_e_i = B_i_j X_e_j", [(4, 8), (5000, 8)]),                         # four rows: not this schedule
+    ("A_e_i = B_i_j X_e_j", [(7, 9), (5000, 9)]),                         # odd and short: not this schedule
 ])
 def test_dense_operator_applied_to_every_entry(at, engine, checker, kernel, shapes):
     rng = np.random.default_rng(shapes[0][0])
@@ -496,7 +516,54 @@ def test_dense_operator_applied_to_every_entry(at, engine, checker, kernel, shap
     ins = [rng.uniform(-1, 1, s) for s in shapes]
     out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
     got, expected = run_single(at, engine, checker, kernel, out0, *ins)
-    assert ("operator schedule" in engine.GetLastImplementation()) == (shapes[0] != (1000, 4))
+    if kernel == "A_e_i_k = B_e_i_j C_j_k":
+        rows, cols = 8, 8
+    else:
+        operator = ins[1] if kernel.startswith("A_e_i += X") else ins[0]
+        lead = 2 if "_q_" in kernel else 1
+        rows = int(np.prod(out0.shape[lead:]))
+        cols = operator.size // rows
+    chosen = (rows >= 5 and cols >= 4) if cols % 2 == 0 else cols >= 16
+    chosen = chosen and shapes[0] != (1000, 4)           # (there the batch index is i, which the operator carries)
+    assert ("operator schedule on the FP64 matrix cores" in engine.GetLastImplementation()) == chosen
+    needs_padding = rows % 16 != 0 or cols % (8 if cols % 2 == 0 else 4) != 0
+    assert ("padded" in engine.GetLastImplementation()) == (chosen and needs_padding)
     if "-=" in kernel:
         expected = 2.0 * out0 - expected
     assert rel_err(got, expected) <= TOL
+
+
+@pytest.mark.parametrize("kernel,shapes", [
+    ("A_e_i = B_i_j X_e_j", [(64, 64), (999, 64)]),
+    ("A_e_i -= B_i_j X_e_j", [(40, 30), (1003, 30)]),
+    ("A_e_q_i += B_i_j X_e_q_j", [(30, 20), (101, 7, 20)]),
+])
+def test_dense_operator_through_scalar_loads(at, engine, checker, monkeypatch, kernel, shapes):
+    """The variant of the operator schedule that does without the matrix cores."""
+    monkeypatch.setenv("ACRO_HIP_OPERATOR_MFMA", "-1")
+    rng = np.random.default_rng(shapes[1][0])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "a lane keeps its row for 4 entries" in engine.GetLastImplementation()
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
+
+
+def test_dense_operator_applied_to_slices(at, engine, checker):
+    """The entries' vectors and the results are slices of larger tensors (a slice starts at a whole number of rows,
+    so the 16-byte loads of the entries' vectors stay aligned)."""
+    rng = np.random.default_rng(5)
+    B = rng.uniform(-1, 1, (16, 24))
+    for entries in (50, 51):
+        X = rng.uniform(-1, 1, (3, entries, 24))
+        A0 = rng.uniform(-1, 1, (2, entries, 16))
+        tX, tA, tB = to_tensor(at, X), to_tensor(at, A0), to_tensor(at, B)
+        tA.MoveToGPU()
+        engine("A_e_i = B_i_j X_e_j", at.SliceTensor(tA, 1), tB, at.SliceTensor(tX, 1))
+        assert "matrix cores" in engine.GetLastImplementation()
+        tA.MoveFromGPU()
+        expected = np.zeros((entries, 16))
+        checker.contract("A_e_i = B_i_j X_e_j", expected, B, np.ascontiguousarray(X[1]))
+        assert rel_err(tA.data[1], expected) <= TOL and np.array_equal(tA.data[0], A0[0])
