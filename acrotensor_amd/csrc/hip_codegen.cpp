@@ -258,6 +258,7 @@ class Generator
     bool extentsConsistent = true;
     bool batchUniform = false;  // one batch entry per workgroup: the batch index is a scalar
     double busyLanes = 1.0;     // share of busy lanes in the wavefronts that the chosen batching issues
+    bool lightWorkgroups = false;  // the batch was raised because a workgroup would have moved too few bytes
     bool wide = false;          // 64-bit device-memory offsets
 
     // Literal of a device-memory stride or offset, and the type such offsets are computed in.
@@ -1578,6 +1579,44 @@ class Generator
             busyLanes = utilisation(NB, NT);
         }
 
+        // A streaming group (one phase, nothing in LDS) whose workgroups move very little is bound by the rate at
+        // which workgroups start, not by memory: with 1 - 2 KB per workgroup a copy reaches 72 % of the HBM peak and
+        // an outer product 64 %.  Such groups take more batch entries per workgroup, in several passes of its lanes,
+        // until a workgroup moves 8 KB (copy 72 -> 79 %, outer product 64 -> 88 %, batched 8 x 8 transpose 70 -> 77 %,
+        // batched dot product 71 -> 74 %).  From 3 KB per workgroup on the same change measured slower
+        // (`A_e_i += B_e_i` 77 -> 75 %, three-operand product 78 -> 75 %), hence the threshold.
+        lightWorkgroups = false;
+        if (opt.force_nb <= 0 && opt.force_nt <= 0 && envInt("ACRO_HIP_NB") <= 0 && envInt("ACRO_HIP_NT") <= 0 && batch >= 0 &&
+            envInt("ACRO_HIP_LIGHT") >= 0)
+        {
+            bool streaming = subs.back().phase == 0;
+            for (const auto &st : stores) streaming = streaming && !st.wantLds && !st.staged;
+            for (const auto &s : subs) streaming = streaming && s.splitLanes == 0 && !s.loopMode && s.matrixOp == 0 && has(s.out.idx, batch);
+            double perEntry = 0.0;
+            std::set<int> counted;
+            for (const auto &s : subs)
+            {
+                for (const auto &v : s.in)
+                {
+                    if (has(v.idx, batch) && counted.insert(v.uvar).second) perEntry += 8.0 * static_cast<double>(v.size) / static_cast<double>(E);
+                }
+                const double written = 8.0 * static_cast<double>(s.out.size) / static_cast<double>(E);
+                if (s.op != '=' && !counted.count(s.out.uvar)) perEntry += written;  // the old value is read first
+                if (counted.insert(s.out.uvar).second) perEntry += written;
+            }
+            if (streaming && perEntry > 0.0 && NB * perEntry < 2560.0)
+            {
+                long nb = NB;
+                while (nb * perEntry < 8192.0 && nb * 2 <= E && nb < 256) nb *= 2;
+                if (nb > NB)
+                {
+                    NB = static_cast<int>(nb);
+                    if (static_cast<long>(NB) * maxLane >= 512) NT = std::max(NT, 256);
+                    lightWorkgroups = true;
+                }
+            }
+        }
+
         // Everything that wants LDS gets it while the workgroup stays within the 64 KB a workgroup may declare
         // statically; otherwise shrink the batch, and finally leave the largest tiles in device memory.
         const int budgetDoubles = 64 * 1024 / 8;
@@ -1657,7 +1696,7 @@ class Generator
         // the upper half idle, which halves the residency.  Measured: p=2 mass assembly 37.2 -> 34.3 us, p=3 mass
         // apply with all intermediates stored 355 -> 335 us; the same change costs the read-dominated p=3 mass
         // apply with transient intermediates 8 % (86.4 -> 93.6 us), hence the condition.
-        if (NT == 128 && opt.force_nt <= 0 && envInt("ACRO_HIP_NT") <= 0 && batch >= 0)
+        if (NT == 128 && !lightWorkgroups && opt.force_nt <= 0 && envInt("ACRO_HIP_NT") <= 0 && batch >= 0)
         {
             double stored = 0.0, loaded = 0.0;
             std::set<int> counted;

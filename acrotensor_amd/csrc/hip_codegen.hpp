@@ -55,6 +55,8 @@
 //   ACRO_HIP_TRANSPOSE=-1       permutations with long fastest dimensions on both sides run as ordinary kernels (no LDS tiles)
 //   ACRO_HIP_OPERATOR=-1        a dense operator applied to every batch entry runs through the generic schedule (operator staged
 //                               in LDS, one entry per lane) instead of the operator schedule
+//   ACRO_HIP_LIGHT=-1           streaming groups whose workgroups move less than 2.5 KB keep their batch size (no extra
+//                               passes to bring a workgroup to 8 KB)
 //   ACRO_HIP_OPERATOR_MFMA=-1   the operator schedule never uses the FP64 matrix cores (a lane keeps its row for four entries,
 //                               whose vectors come through scalar loads, whatever the operator's sizes)
 //   ACRO_HIP_RED_PENCIL=-1      split contractions: one lane per (slice, output entry) also when there are few outputs

@@ -166,6 +166,21 @@ def test_small_invariant_operand_read_by_rows_is_staged_in_lds(TE):
     assert "B<-scalar" in TE.GetImplementation("A_e_q_j = B_q_i X_e_i_j", at.Tensor(500, 5, 16), at.Tensor(5, 4), at.Tensor(500, 4, 16))
 
 
+def test_streaming_kernels_with_light_workgroups_take_more_entries(TE, monkeypatch):
+    E = 100000
+    # 2 entries x (8 + 8 + 64) doubles = 1.3 KB per workgroup: raised to 16 entries in four passes of 256 lanes
+    outer = lambda: TE.GetImplementation("A_e_i_j = B_e_i C_e_j", at.Tensor(E, 8, 8), at.Tensor(E, 8), at.Tensor(E, 8))
+    assert "16 per workgroup of 256 lanes" in outer() and "w0 < 1024; w0 += 256" in outer()
+    assert "32 per workgroup of 256 lanes" in TE.GetImplementation("A_e_i = B_e_i", at.Tensor(E, 16), at.Tensor(E, 16))
+    # 3 KB per workgroup and more stay as they are (the old value of += counts)
+    assert "8 per workgroup of 128 lanes" in TE.GetImplementation("A_e_i += B_e_i", at.Tensor(E, 16), at.Tensor(E, 16))
+    assert "8 per workgroup of 128 lanes" in TE.GetImplementation("A_e_i = B_e_i C_e_i D_e_i", *[at.Tensor(E, 16)] * 4)
+    # few entries: never more than there are
+    assert "batch index e extent 9, 8 per workgroup" in TE.GetImplementation("A_e_i_j = B_e_i C_e_j", at.Tensor(9, 8, 8), at.Tensor(9, 8), at.Tensor(9, 8))
+    monkeypatch.setenv("ACRO_HIP_LIGHT", "-1")     # (other sizes: the engine keeps what it generated for the sizes above)
+    assert "2 per workgroup of 256 lanes" in TE.GetImplementation("A_e_i_j = B_e_i C_e_j", at.Tensor(E + 1, 8, 8), at.Tensor(E + 1, 8), at.Tensor(E + 1, 8))
+
+
 def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     # FP64 matrix cores, 16 entries per wavefront and trip
     src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
