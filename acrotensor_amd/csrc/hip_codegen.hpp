@@ -28,8 +28,11 @@
 //    is split over workgroups and lanes, partial sums are added in a fixed order by a second one-workgroup kernel.
 //  * A single kernel that only permutes the dimensions of one operand, with different long fastest dimensions on the
 //    two sides, moves tiles of 32 x 32 entries through LDS ("transpose schedule").
-//  * A dense operator of up to 4 096 entries applied to every batch entry ("A_e_i = B_i_j X_e_j") runs the "operator
-//    schedule": operator rows in LDS, a lane keeps its row for four entries, the entries' vectors come in by scalar loads.
+//  * A dense operator of up to 4 096 entries applied to every batch entry ("A_e_i = B_i_j X_e_j", also stored
+//    transposed or with several leading indices numbering the entries) runs the "operator schedule" on the FP64
+//    matrix cores: 16 entries per wavefront and trip through v_mfma_f64_16x16x4, the operator in LDS in operand order
+//    and padded with zeros to whole 16 x 4 blocks.
+//  * A streaming group whose workgroups would move less than 2.5 KB takes more batch entries per workgroup.
 //  * Contractions too long to unroll fall back to counted loops with the same lane mapping.
 //
 // Experiment switches (environment, read when a kernel is generated; defaults are what measured best on MI355X):
