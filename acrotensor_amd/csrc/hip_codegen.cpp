@@ -3085,17 +3085,38 @@ class Generator
         long rows = 0, cols = 0, entries = 0;
         bool transposed = false;   // the operator is stored with the contracted indices first: "B_j_i"
         bool cores = false;        // sizes and alignment suit the FP64 matrix cores
+        bool pairs = false;        // the entries' vectors (and weights of their shape) come in 16-byte loads
+        // Pointwise factors beside the operator and the vectors (matrix-core variant only): one value per entry
+        // "W_e", per output "W_e_i", per row "W_i" scale the result; per vector element "W_e_j" or per column
+        // "W_j" scale the entries' vectors as they are loaded.
+        std::vector<const VarRef *> perEntry, perOutput, perRow, perElement, perColumn;
     };
 
     bool OperatorPattern(OperatorShape &o) const
     {
         if (subs.size() != 1 || batch < 0 || !opt.noalias || NumGatherSlots() > 0 || envInt("ACRO_HIP_OPERATOR") < 0) return false;
         const Sub &s = subs[0];
-        if (s.matrixOp != 0 || s.in.size() != 2 || s.contr.empty() || s.out.repeated) return false;
-        o.op = has(s.in[0].idx, batch) ? &s.in[1] : &s.in[0];
-        o.x = has(s.in[0].idx, batch) ? &s.in[0] : &s.in[1];
-        if (o.op->repeated || o.x->repeated || has(o.op->idx, batch) || !has(o.x->idx, batch)) return false;
-        if (o.op->uvar == s.out.uvar || o.x->uvar == s.out.uvar || !IsPureInput(o.op->uvar) || !IsPureInput(o.x->uvar)) return false;
+        if (s.matrixOp != 0 || s.in.size() < 2 || s.contr.empty() || s.out.repeated) return false;
+        // the operator: the one operand without the batch index that carries contracted and free indices;
+        // the vectors: the first operand with the batch index that carries every contracted index
+        for (const auto &v : s.in)
+        {
+            bool contracted = false, free = false, all = true;
+            for (int id : v.idx) (has(s.contr, id) ? contracted : free) = true;
+            for (int id : s.contr) all = all && has(v.idx, id);
+            if (!has(v.idx, batch) && contracted && free)
+            {
+                if (o.op) return false;
+                o.op = &v;
+            }
+            else if (has(v.idx, batch) && all && !o.x)
+                o.x = &v;
+        }
+        if (!o.op || !o.x) return false;
+        for (const auto &v : s.in)
+        {
+            if (v.repeated || v.uvar == s.out.uvar || !IsPureInput(v.uvar)) return false;
+        }
         // out = (e..., I...), X = (e..., J...), B = (I..., J...) or (J..., I...): the leading indices that the result
         // and X share, the batch index first, number the entries
         if (s.out.idx.empty() || s.out.idx[0] != batch || o.x->idx[0] != batch) return false;
@@ -3121,15 +3142,31 @@ class Generator
         o.entries = product(lead, extent);
         if (o.rows > 1024 || o.rows * o.cols > 4096) return false;
         o.cores = envInt("ACRO_HIP_OPERATOR_MFMA") >= 0;
-        if (!o.cores) return o.rows >= 16 && o.cols >= 16 && !o.transposed;  // (its lanes walk the operator's rows)
+        o.pairs = o.cols % 2 == 0 && uvars[o.x->uvar].viewOffset % 2 == 0;
+        std::vector<int> outRows = lead;
+        outRows.insert(outRows.end(), rows.begin(), rows.end());
+        for (const auto &v : s.in)
+        {
+            if (&v == o.op || &v == o.x) continue;
+            if (v.idx == lead) o.perEntry.push_back(&v);
+            else if (v.idx == outRows) o.perOutput.push_back(&v);
+            else if (v.idx == rows) o.perRow.push_back(&v);
+            else if (v.idx == cols) o.perColumn.push_back(&v);
+            else if (v.idx == o.x->idx)
+            {
+                o.perElement.push_back(&v);
+                o.pairs = o.pairs && uvars[v.uvar].viewOffset % 2 == 0;
+            }
+            else return false;
+        }
+        if (!o.cores) return o.rows >= 16 && o.cols >= 16 && !o.transposed && s.in.size() == 2;  // (its lanes walk the operator's rows)
         // Small operators: the generic schedule (operator in scalar registers, an entry or an output per lane) reads
         // and writes short pieces per lane and reaches 40 - 65 % of the HBM peak; 16 entries per wavefront on the
         // matrix cores reach 70 - 88 % as long as the entries' vectors come in 16-byte loads (even length) and five
         // or more rows fill the stores, or the vectors are long.  Measured wins: 8 x 4 53 -> 73 %, 16 x 4 43 -> 84 %,
         // 8 x 8 61 -> 85 %, 10 x 10 52 -> 81 %, 8 x 16 62 -> 85 %, 3 x 27 41 -> 73 %; losses, hence excluded:
         // 4 x 4 65 -> 49 %, 4 x 8 82 -> 77 %, 7 x 9 62 -> 57 %, 27 x 3 36 -> 28 %; 20 x 5 a tie.
-        const bool pairs = o.cols % 2 == 0 && uvars[o.x->uvar].viewOffset % 2 == 0;
-        return pairs ? (o.rows >= 5 && o.cols >= 4) : o.cols >= 16;
+        return o.pairs ? (o.rows >= 5 && o.cols >= 4) : o.cols >= 16;
     }
 
     bool UseOperatorSchedule() const
@@ -3251,7 +3288,7 @@ class Generator
         // Sizes that the instruction's 16 x 4 blocks do not divide: the operator's copy in LDS is padded with zero
         // rows and columns, the entries' vectors read as zero past their end, outputs past the last row are not
         // stored.  Pairs of doubles (16-byte loads) need an even row length and an even first element.
-        const bool pairs = nJ % 2 == 0 && uvars[x.uvar].viewOffset % 2 == 0;
+        const bool pairs = shape.pairs;
         const long nIp = (nI + 15) / 16 * 16, nJp = pairs ? (nJ + 7) / 8 * 8 : (nJ + 3) / 4 * 4;
         const long tilesN = nIp / 16, steps = nJp / 4;
         const long tiles = (E + 15) / 16;
@@ -3319,6 +3356,22 @@ class Generator
             out << "        for (int q = 0; q < " << nJp / 8 << "; ++q) xv[q] = ";
             if (nJp != nJ) out << "8 * q + 2 * g >= " << nJ << " ? double2{0.0, 0.0} : ";
             out << "*reinterpret_cast<const double2 *>(x + 8 * q);\n";
+            for (const VarRef *w : shape.perElement)
+            {
+                out << "#pragma unroll\n";
+                out << "        for (int q = 0; q < " << nJp / 8 << "; ++q)\n        {\n";
+                if (nJp != nJ) out << "            if (8 * q + 2 * g >= " << nJ << ") continue;\n";
+                out << "            const double2 f = *reinterpret_cast<const double2 *>(" << PtrName(w->uvar) << " + " << Lit(uvars[w->uvar].viewOffset)
+                    << " + ex * " << nJ << " + 2 * g + 8 * q);\n            xv[q].x *= f.x;\n            xv[q].y *= f.y;\n        }\n";
+            }
+            for (const VarRef *w : shape.perColumn)
+            {
+                out << "#pragma unroll\n";
+                out << "        for (int q = 0; q < " << nJp / 8 << "; ++q)\n        {\n";
+                if (nJp != nJ) out << "            if (8 * q + 2 * g >= " << nJ << ") continue;\n";
+                out << "            const double *f = " << PtrName(w->uvar) << " + " << Lit(uvars[w->uvar].viewOffset)
+                    << " + 2 * g + 8 * q;\n            xv[q].x *= f[0];\n            xv[q].y *= f[1];\n        }\n";
+            }
         }
         else
         {
@@ -3328,6 +3381,20 @@ class Generator
             out << "        for (int q = 0; q < " << steps << "; ++q) xv[q] = ";
             if (nJp != nJ) out << "4 * q + g >= " << nJ << " ? 0.0 : ";
             out << "x[4 * q];\n";
+            for (const VarRef *w : shape.perElement)
+            {
+                out << "#pragma unroll\n";
+                out << "        for (int q = 0; q < " << steps << "; ++q) ";
+                if (nJp != nJ) out << "if (4 * q + g < " << nJ << ") ";
+                out << "xv[q] *= " << PtrName(w->uvar) << "[" << Lit(uvars[w->uvar].viewOffset) << " + ex * " << nJ << " + g + 4 * q];\n";
+            }
+            for (const VarRef *w : shape.perColumn)
+            {
+                out << "#pragma unroll\n";
+                out << "        for (int q = 0; q < " << steps << "; ++q) ";
+                if (nJp != nJ) out << "if (4 * q + g < " << nJ << ") ";
+                out << "xv[q] *= " << PtrName(w->uvar) << "[" << Lit(uvars[w->uvar].viewOffset) << " + g + 4 * q];\n";
+            }
         }
         out << "        acro_double4 acc[" << tilesN << "];\n";
         out << "#pragma unroll\n";
@@ -3346,13 +3413,29 @@ class Generator
         out << "#pragma unroll\n";
         out << "        for (int r = 0; r < 4; ++r)\n        {\n";
         if (ragged) out << "            if (tile * 16 + g + 4 * r >= " << E << ") continue;\n";
+        // the result's pointwise factors
+        std::string value = "acc[t][r]";
+        const bool scaled = !shape.perEntry.empty() || !shape.perOutput.empty() || !shape.perRow.empty();
+        if (scaled) out << "            const long en = tile * 16 + g + 4 * r;\n";
+        if (!shape.perEntry.empty())
+        {
+            out << "            const double se = ";
+            for (size_t i = 0; i < shape.perEntry.size(); ++i)
+                out << (i ? " * " : "") << PtrName(shape.perEntry[i]->uvar) << "[" << Lit(uvars[shape.perEntry[i]->uvar].viewOffset) << " + en]";
+            out << ";\n";
+            value += " * se";
+        }
+        for (const VarRef *w : shape.perOutput)
+            value += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + " + en * " + str(nI) + " + 16 * t + c]";
+        for (const VarRef *w : shape.perRow)
+            value += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + " + 16 * t + c]";
         out << "#pragma unroll\n";
         out << "            for (int t = 0; t < " << tilesN << "; ++t)\n";
         std::string guard = nIp != nI ? "if (16 * t + c < " + str(nI) + ") " : "";
         if (stream)
-            out << "                " << guard << "__builtin_nontemporal_store(acc[t][r], a + 4 * r * " << nI << " + 16 * t);\n";
+            out << "                " << guard << "__builtin_nontemporal_store(" << value << ", a + 4 * r * " << nI << " + 16 * t);\n";
         else
-            out << "                " << guard << "a[4 * r * " << nI << " + 16 * t]" << (s.op == '=' ? " = " : (s.op == '+' ? " += " : " -= ")) << "acc[t][r];\n";
+            out << "                " << guard << "a[4 * r * " << nI << " + 16 * t]" << (s.op == '=' ? " = " : (s.op == '+' ? " += " : " -= ")) << value << ";\n";
         out << "        }\n    }\n}\n";
 
         plan.source = out.str();

@@ -31,7 +31,8 @@
 //  * A dense operator of up to 4 096 entries applied to every batch entry ("A_e_i = B_i_j X_e_j", also stored
 //    transposed or with several leading indices numbering the entries) runs the "operator schedule" on the FP64
 //    matrix cores: 16 entries per wavefront and trip through v_mfma_f64_16x16x4, the operator in LDS in operand order
-//    and padded with zeros to whole 16 x 4 blocks.
+//    and padded with zeros to whole 16 x 4 blocks; pointwise factors per entry, output, row, vector element or
+//    column stay in the same launch.
 //  * A streaming group whose workgroups would move less than 2.5 KB takes more batch entries per workgroup.
 //  * Contractions too long to unroll fall back to counted loops with the same lane mapping.
 //

@@ -157,10 +157,10 @@ def test_diffusion_chain_batching_follows_the_contractions_not_the_pointwise_ker
 def test_small_invariant_operand_read_by_rows_is_staged_in_lds(TE):
     # lane i walks along row i of B: from device memory every load instruction would touch 64 lines; each workgroup
     # copies B to LDS once (row stride 65, so that the lanes fall into different banks) and serves 16 entries
-    src = TE.GetImplementation("A_e_i = B_i_j X_e_j W_e", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64), at.Tensor(1000))
+    src = TE.GetImplementation("A_e_i = B_i_j X_e_k_j W_e_k", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 2, 64), at.Tensor(1000, 2))
     assert "B<-lds" in src and "// B: device memory -> LDS, once per workgroup" in src
     assert "a += (r_ / 64) * 65" in src and "16 per workgroup of 256 lanes" in src
-    assert src.index("__syncthreads()") < src.index("// A_e_i = B_i_j X_e_j W_e")
+    assert src.index("__syncthreads()") < src.index("// A_e_i = B_i_j X_e_k_j W_e_k")
     # a table that the lanes read at unit stride, or one read through scalar loads, is left where it is
     assert "<-lds" not in TE.GetImplementation("A_e_i = B_j_i X_e_j", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64))
     assert "B<-scalar" in TE.GetImplementation("A_e_q_j = B_q_i X_e_i_j", at.Tensor(500, 5, 16), at.Tensor(5, 4), at.Tensor(500, 4, 16))
@@ -202,9 +202,15 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     assert "8 * q + 2 * g >= 28 ? double2{0.0, 0.0} :" in src and "if (16 * t + c < 30) a[4 * r * 30 + 16 * t] -= acc[t][r];" in src
     src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 30), at.Tensor(30, 27), at.Tensor(1000, 27))
     assert "(padded to 32 x 28)" in src and "j = 4 * step + (l >> 4);" in src and "xv[q] = 4 * q + g >= 27 ? 0.0 : x[4 * q];" in src
+    # pointwise factors: per entry, per output and per row on the result, per element and per column on the vectors
+    src = TE.GetImplementation("A_e_i -= B_i_j X_e_j W_e D_e_j R_i F_e_i C_j", at.Tensor(1000, 10), at.Tensor(10, 12), at.Tensor(1000, 12),
+                               at.Tensor(1000), at.Tensor(1000, 12), at.Tensor(10), at.Tensor(1000, 10), at.Tensor(12))
+    assert "operator schedule on the FP64 matrix cores: 10 x 12 operator" in src and "const double se = T3[0 + en];" in src
+    assert "-= acc[t][r] * se * T6[0 + en * 10 + 16 * t + c] * T5[0 + 16 * t + c];" in src
+    assert "const double2 f = *reinterpret_cast<const double2 *>(T4 + 0 + ex * 12 + 2 * g + 8 * q);" in src and "const double *f = T7 + 0 + 2 * g + 8 * q;" in src
     # not this schedule: few rows (a register tile with scalar operands serves them), third operand
     for kernel, shapes in (("A_e_i = B_i_j X_e_j", [(500, 4), (4, 64), (500, 64)]),
-                           ("A_e_i = B_i_j X_e_j W_e", [(500, 64), (64, 64), (500, 64), (500,)])):
+                           ("A_e_i = B_i_j X_e_k_j W_e_k", [(500, 64), (64, 64), (500, 2, 64), (500, 2)])):
         tensors = [at.Tensor(*shp) for shp in shapes]
         assert "operator schedule" not in TE.GetImplementation(kernel, *tensors)
     # without the matrix cores: a lane keeps its row for four entries, whose vectors come through scalar loads
@@ -306,7 +312,11 @@ def generated_sources(TE):
         at.Tensor(4, 5, 5, 5, 3, 3))
     yield "one name, two tensors", TE.GetImplementation("A_m_n = B_m_j B_n_j", at.Tensor(3, 3), at.Tensor(3, 4), at.Tensor(3, 4))
     yield "repeated output index", TE.GetImplementation("A_i_i = B_i", at.Tensor(6, 6), at.Tensor(6))
-    yield "operand staged in LDS", TE.GetImplementation("A_e_i = B_i_j X_e_j W_e", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 64), at.Tensor(1000))
+    yield "operand staged in LDS", TE.GetImplementation("A_e_i = B_i_j X_e_k_j W_e_k", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 2, 64), at.Tensor(1000, 2))
+    yield "operator schedule with pointwise factors", TE.GetImplementation("A_e_i -= B_i_j X_e_j W_e D_e_j R_i F_e_i C_j", at.Tensor(1000, 10), at.Tensor(10, 12),
+                                                                         at.Tensor(1000, 12), at.Tensor(1000), at.Tensor(1000, 12), at.Tensor(10), at.Tensor(1000, 10), at.Tensor(12))
+    yield "operator schedule with pointwise factors, odd length", TE.GetImplementation("A_e_i = B_i_j X_e_j D_e_j C_j W_e", at.Tensor(1000, 20), at.Tensor(20, 17),
+                                                                                     at.Tensor(1000, 17), at.Tensor(1000, 17), at.Tensor(17), at.Tensor(1000))
     yield "operator schedule", TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(77, 5, 6), at.Tensor(77, 4, 7), at.Tensor(5, 6, 4, 7))
     yield "operator schedule, no padding", TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(77, 8, 6), at.Tensor(77, 4, 10), at.Tensor(8, 6, 4, 10))
     yield "operator schedule, odd row length", TE.GetImplementation("A_e_i = B_j_i X_e_j", at.Tensor(500, 17), at.Tensor(33, 17), at.Tensor(500, 33))

@@ -407,8 +407,8 @@ def test_slice_of_a_slice_inside_a_fused_launch(at, engine):
 
 
 @pytest.mark.parametrize("kernel,shapes", [
-    ("A_e_i = B_i_j X_e_j W_e", [(64, 64), (1000, 64), (1000,)]),   # B staged in LDS, 16 entries per workgroup, ragged end
-    ("A_e_i = B_i_j X_e_j W_e", [(40, 24), (3, 24), (3,)]),      # fewer entries than a workgroup would take
+    ("A_e_i = B_i_j X_e_k_j W_e_k", [(64, 64), (1000, 2, 64), (1000, 2)]),   # B staged in LDS, 16 entries per workgroup, ragged end
+    ("A_e_i = B_i_j X_e_k_j W_e_k", [(40, 24), (3, 2, 24), (3, 2)]),      # fewer entries than a workgroup would take
     ("A_e_i_k = B_i_j C_k_l X_e_j_l", [(12, 10), (9, 11), (77, 10, 11)]),   # two staged tables, reordered into steps
     ("A_e_i_k = B_e_i_j C_e_j_k", [(1001, 4, 4), (1001, 4, 4)]), # one output per lane
     ("A_e_i_k = B_e_i_j C_e_j_k", [(333, 3, 3), (333, 3, 3)]),
@@ -528,6 +528,28 @@ def test_dense_operator_applied_to_every_entry(at, engine, checker, kernel, shap
     assert ("operator schedule on the FP64 matrix cores" in engine.GetLastImplementation()) == chosen
     needs_padding = rows % 16 != 0 or cols % (8 if cols % 2 == 0 else 4) != 0
     assert ("padded" in engine.GetLastImplementation()) == (chosen and needs_padding)
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
+
+
+@pytest.mark.parametrize("kernel,shapes", [
+    ("A_e_i = B_i_j X_e_j W_e", [(64, 64), (1000, 64), (1000,)]),                    # one factor per entry
+    ("A_e_i += B_i_j X_e_j W_e", [(40, 24), (43, 24), (43,)]),                       # three trips, the last with 11 entries
+    ("A_e_k = B_k_i X_e_i D_e_k", [(12, 10), (5003, 10), (5003, 12)]),               # interpolate, then weights per output
+    ("A_e_i = B_k_i U_e_k D_e_k", [(12, 10), (5003, 12), (5003, 12)]),               # weights per element, transposed operator
+    ("A_e_i -= B_i_j X_e_j W_e D_e_j R_i F_e_i C_j", [(10, 12), (1000, 12), (1000,), (1000, 12), (10,), (1000, 10), (12,)]),
+    ("A_e_i = B_i_j X_e_j D_e_j C_j W_e", [(20, 17), (777, 17), (777, 17), (17,), (777,)]),   # odd length: 8-byte loads
+    ("A_e_q_i = W_e_q B_i_j X_e_q_j", [(601, 3), (16, 8), (601, 3, 8)]),            # the factor first, two entry indices
+])
+def test_dense_operator_with_pointwise_factors(at, engine, checker, kernel, shapes):
+    """Factors beside the operator and the vectors: the result is scaled per entry, per output or per row as it is
+    stored, the vectors per element or per column as they are loaded (reference semantics: one product per term)."""
+    rng = np.random.default_rng(len(kernel) + shapes[1][0])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "operator schedule on the FP64 matrix cores" in engine.GetLastImplementation()
     if "-=" in kernel:
         expected = 2.0 * out0 - expected
     assert rel_err(got, expected) <= TOL
