@@ -239,6 +239,18 @@ def other_workload(at, workloads, args):
             abytes += 2 * dofs.size * 8                      # the element vector written, then read
         flops = wl.flops
         units, unit_name = wl.dof, "GDOF/s"
+    elif name == "operator":
+        # one dense 64 x 64 operator applied to 2^18 vectors: the one GEMM-shaped kernel of this engine (FP64 matrix cores)
+        E, n = 1 << 18, 64
+        B, X, A = at.Tensor(n, n), at.Tensor(E, n), at.Tensor(E, n)
+        B.data[...] = workloads.counter_uniform(0xAC28, 0, (n, n), -1.0, 1.0)
+        X.data[...] = workloads.counter_uniform(0xAC28, 1, (E, n), -1.0, 1.0)
+        for t in (B, X, A):
+            t.MoveToGPU()
+        step = lambda: engine("A_e_i = B_i_j X_e_j", A, B, X)
+        label = "A[262144,64] = B[64,64] X[262144,64], one dense operator applied to every vector"
+        abytes, flops = (2 * E * n + n * n) * 8, 2 * E * n * n
+        units, unit_name = E * n, "GDOF/s"
     elif name in ("scatter", "sumgather"):
         # node vector <-> element vector of the headline mesh size: 64^3 hex elements of degree 3
         import numpy as np
@@ -307,7 +319,7 @@ def main():
     ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store-all", action="store_true")
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "scatter_apply", "scatter_then_apply", "shapes"],
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "scatter_apply", "scatter_then_apply", "operator", "shapes"],
                     help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
                          "remaining baseline configurations at their full sizes and for the node-vector <-> "
                          "element-vector steps either side of the operator apply")
