@@ -3086,6 +3086,7 @@ class Generator
         bool transposed = false;   // the operator is stored with the contracted indices first: "B_j_i"
         bool cores = false;        // sizes and alignment suit the FP64 matrix cores
         bool pairs = false;        // the entries' vectors (and weights of their shape) come in 16-byte loads
+        bool trailing = false;     // the entries are the fastest dimension: "A_i_e = B_i_j X_j_e"
         // Pointwise factors beside the operator and the vectors (matrix-core variant only): one value per entry
         // "W_e", per output "W_e_i", per row "W_i" scale the result; per vector element "W_e_j" or per column
         // "W_j" scale the entries' vectors as they are loaded.
@@ -3119,13 +3120,32 @@ class Generator
         }
         // out = (e..., I...), X = (e..., J...), B = (I..., J...) or (J..., I...): the leading indices that the result
         // and X share, the batch index first, number the entries
-        if (s.out.idx.empty() || s.out.idx[0] != batch || o.x->idx[0] != batch) return false;
-        size_t shared = 0;
-        while (shared < s.out.idx.size() && shared < o.x->idx.size() && s.out.idx[shared] == o.x->idx[shared] &&
-               !has(o.op->idx, s.out.idx[shared]))
-            ++shared;
-        const std::vector<int> lead(s.out.idx.begin(), s.out.idx.begin() + shared);
-        const std::vector<int> rows(s.out.idx.begin() + shared, s.out.idx.end()), cols(o.x->idx.begin() + shared, o.x->idx.end());
+        if (s.out.idx.empty()) return false;
+        std::vector<int> lead, rows, cols;
+        if (s.out.idx[0] == batch && o.x->idx[0] == batch)
+        {
+            size_t shared = 0;
+            while (shared < s.out.idx.size() && shared < o.x->idx.size() && s.out.idx[shared] == o.x->idx[shared] &&
+                   !has(o.op->idx, s.out.idx[shared]))
+                ++shared;
+            lead.assign(s.out.idx.begin(), s.out.idx.begin() + shared);
+            rows.assign(s.out.idx.begin() + shared, s.out.idx.end());
+            cols.assign(o.x->idx.begin() + shared, o.x->idx.end());
+        }
+        else
+        {
+            // or the trailing ones, the entries being the fastest dimension of the result and of X
+            size_t shared = 0;
+            const size_t no = s.out.idx.size(), nx = o.x->idx.size();
+            while (shared < no && shared < nx && s.out.idx[no - 1 - shared] == o.x->idx[nx - 1 - shared] &&
+                   !has(o.op->idx, s.out.idx[no - 1 - shared]))
+                ++shared;
+            lead.assign(s.out.idx.end() - shared, s.out.idx.end());
+            rows.assign(s.out.idx.begin(), s.out.idx.end() - shared);
+            cols.assign(o.x->idx.begin(), o.x->idx.end() - shared);
+            o.trailing = true;
+            if (!has(lead, batch)) return false;
+        }
         if (rows.empty() || cols.empty()) return false;
         std::vector<int> plain = rows, swapped = cols;
         plain.insert(plain.end(), cols.begin(), cols.end());
@@ -3142,24 +3162,42 @@ class Generator
         o.entries = product(lead, extent);
         if (o.rows > 1024 || o.rows * o.cols > 4096) return false;
         o.cores = envInt("ACRO_HIP_OPERATOR_MFMA") >= 0;
-        o.pairs = o.cols % 2 == 0 && uvars[o.x->uvar].viewOffset % 2 == 0;
-        std::vector<int> outRows = lead;
-        outRows.insert(outRows.end(), rows.begin(), rows.end());
+        // 16-byte loads: along the vectors, or along the entries where those are the fastest dimension
+        o.pairs = (o.trailing ? o.entries % 2 == 0 && uvars[s.out.uvar].viewOffset % 2 == 0 : o.cols % 2 == 0) &&
+                  uvars[o.x->uvar].viewOffset % 2 == 0;
         for (const auto &v : s.in)
         {
             if (&v == o.op || &v == o.x) continue;
-            if (v.idx == lead) o.perEntry.push_back(&v);
-            else if (v.idx == outRows) o.perOutput.push_back(&v);
+            const bool even = uvars[v.uvar].viewOffset % 2 == 0;
+            if (v.idx == lead)
+            {
+                o.perEntry.push_back(&v);
+                if (o.trailing) o.pairs = o.pairs && even;
+            }
+            else if (v.idx == s.out.idx)
+            {
+                o.perOutput.push_back(&v);
+                if (o.trailing) o.pairs = o.pairs && even;
+            }
             else if (v.idx == rows) o.perRow.push_back(&v);
             else if (v.idx == cols) o.perColumn.push_back(&v);
             else if (v.idx == o.x->idx)
             {
                 o.perElement.push_back(&v);
-                o.pairs = o.pairs && uvars[v.uvar].viewOffset % 2 == 0;
+                o.pairs = o.pairs && even;
             }
             else return false;
         }
-        if (!o.cores) return o.rows >= 16 && o.cols >= 16 && !o.transposed && s.in.size() == 2;  // (its lanes walk the operator's rows)
+        if (!o.cores) return o.rows >= 16 && o.cols >= 16 && !o.transposed && !o.trailing && s.in.size() == 2;  // (its lanes walk the operator's rows)
+        if (o.trailing)
+        {
+            // Entries fastest: the generic schedule (one entry per lane, operator in scalar registers) streams whole
+            // lines already; it falls behind as the operator grows (generic -> matrix cores: 8 x 8 86 -> 85 %,
+            // 16 x 16 82 -> 84 %, 27 x 27 64 -> 78 %, 32 x 32 72 -> 80 %, 64 x 64 3 -> 65 %).  Two entries per lane
+            // cost a large operator its registers (64 x 64: 72 us against 52 us with one entry per lane).
+            if (o.rows * o.cols >= 2048) o.pairs = false;
+            return o.rows * o.cols >= 512;
+        }
         // Small operators: the generic schedule (operator in scalar registers, an entry or an output per lane) reads
         // and writes short pieces per lane and reaches 40 - 65 % of the HBM peak; 16 entries per wavefront on the
         // matrix cores reach 70 - 88 % as long as the entries' vectors come in 16-byte loads (even length) and five
@@ -3185,7 +3223,10 @@ class Generator
         const long E = shape.entries;        // entries of this schedule: all leading indices together
         if (shape.cores)
         {
-            EmitOperatorMatrixCores(plan, shape);
+            if (shape.trailing)
+                EmitOperatorEntriesFastest(plan, shape);
+            else
+                EmitOperatorMatrixCores(plan, shape);
             return;
         }
         const int R = kOperatorEntriesPerLane;
@@ -3437,6 +3478,140 @@ class Generator
         else
             out << "                " << guard << "a[4 * r * " << nI << " + 16 * t]" << (s.op == '=' ? " = " : (s.op == '+' ? " += " : " -= ")) << value << ";\n";
         out << "        }\n    }\n}\n";
+
+        plan.source = out.str();
+        plan.nb = 64;
+        plan.lds_bytes = static_cast<int>(nIp * nJp * 8);
+        FillParams(plan, false);
+        HipLaunch launch;
+        launch.function_name = plan.module_name;
+        launch.grid = static_cast<unsigned>(blocks);
+        launch.block = 256;
+        for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
+        plan.launches.push_back(launch);
+    }
+
+    // The same with the entries as the fastest dimension ("A_i_e = B_i_j X_j_e"): the roles of the instruction's operands
+    // are exchanged.  The operator is the first operand (16 rows x 4 terms per instruction, from LDS in operand order),
+    // the entries' vectors the second: lane = entry + 16 * term group reads X[j][e], 16 consecutive entries per term, and
+    // result register r of a lane holds row 4r + lane / 16 of its entry, so loads and stores run along the entries.
+    // With an even number of entries a wavefront takes 32 entries per trip: a lane loads two neighbouring entries in
+    // 16 bytes, which feed two accumulator sets (even and odd entries), and stores its two results together.
+    void EmitOperatorEntriesFastest(HipKernelPlan &plan, const OperatorShape &shape)
+    {
+        const Sub &s = subs[0];
+        const VarRef &opr = *shape.op, &x = *shape.x;
+        const long nI = shape.rows, nJ = shape.cols, E = shape.entries;
+        const bool pairs = shape.pairs;
+        const int per = pairs ? 32 : 16;
+        const long nIp = (nI + 15) / 16 * 16, nJp = (nJ + 3) / 4 * 4;
+        const long tilesM = nIp / 16, steps = nJp / 4;
+        const long trips = (E + per - 1) / per;
+        const bool ragged = E % per != 0;
+        const long blocks = std::max<long>(1, std::min<long>(512, (trips + 3) / 4));
+        for (const auto &st : stores)
+        {
+            long entries = 1;
+            for (int d : st.dims) entries *= d;
+            if (entries >= (1L << 31) - 1) wide = true;
+        }
+        const std::string dimName = mk.GetDimensionedNameString();
+        char hex[32];
+        std::snprintf(hex, sizeof(hex), "%016llx",
+                      static_cast<unsigned long long>(hashString(dimName + "/operator-mfma-t/" + (Positional() ? "p" : "u") + (pairs ? "2" : "1"))));
+        plan.module_name = std::string("acro_op_") + hex;
+        std::ostringstream sched;
+        sched << "operator schedule on the FP64 matrix cores, entries fastest: " << nI << " x " << nJ
+              << (shape.transposed ? " operator (stored transposed)" : " operator") << " in LDS in operand order";
+        if (nIp != nI || nJp != nJ) sched << " (padded to " << nIp << " x " << nJp << ")";
+        sched << ", " << E << " entries, " << per << " per wavefront and trip, " << tilesM * steps * (pairs ? 2 : 1)
+              << " v_mfma_f64_16x16x4 per trip, " << blocks << " workgroups of 256 lanes\n  [0] " << s.text << "\n";
+        plan.schedule = sched.str();
+
+        out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
+        {
+            std::istringstream lines(plan.schedule);
+            std::string l;
+            while (std::getline(lines, l)) out << "// " << l << "\n";
+        }
+        const std::string B = PtrName(opr.uvar), X = PtrName(x.uvar), A = PtrName(s.out.uvar);
+        const bool stream = s.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0;
+        const std::string vt = pairs ? "acro_double2" : "double";
+        auto offsetOf = [&](const VarRef &v) { return Lit(uvars[v.uvar].viewOffset); };
+        out << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
+        out << "typedef double acro_double2 __attribute__((ext_vector_type(2)));\n";
+        out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << plan.module_name << "(" << ParamList() << ")\n{\n";
+        out << "    __shared__ double frag[" << nIp * nJp << "];\n";
+        out << "    for (int f = threadIdx.x; f < " << nIp * nJp << "; f += 256)\n    {\n";
+        out << "        const int l = f & 63, step = (f >> 6) % " << steps << ", t = (f >> 6) / " << steps << ";\n";
+        out << "        const int row = 16 * t + (l & 15), j = 4 * step + (l >> 4);\n";
+        const std::string element = B + "[" + offsetOf(opr) + (shape.transposed ? " + j * " + str(nI) + " + row]" : " + row * " + str(nJ) + " + j]");
+        if (nIp != nI || nJp != nJ)
+            out << "        frag[f] = row < " << nI << " && j < " << nJ << " ? " << element << " : 0.0;\n    }\n";
+        else
+            out << "        frag[f] = " << element << ";\n    }\n";
+        out << "    __syncthreads();\n";
+        out << "    const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;\n";
+        out << "    const long waves = (long)gridDim.x * 4;\n";
+        out << "    for (long trip = (long)blockIdx.x * 4 + (threadIdx.x >> 6); trip < " << trips << "; trip += waves)\n    {\n";
+        out << "        const long e = trip * " << per << " + " << (pairs ? "2 * c" : "c") << ";\n";
+        if (ragged)
+            out << "        const long ex = e < " << E << " ? e : " << E - (pairs ? 2 : 1) << ";  // past the end: any valid entry, never stored\n";
+        else
+            out << "        const long ex = e;\n";
+        out << "        " << vt << " xv[" << steps << "];\n";
+        out << "#pragma unroll\n";
+        out << "        for (int step = 0; step < " << steps << "; ++step)\n        {\n";
+        out << "            const int j = 4 * step + g;\n";
+        if (nJp != nJ) out << "            if (j >= " << nJ << ") { xv[step] = " << (pairs ? "acro_double2{0.0, 0.0}" : "0.0") << "; continue; }\n";
+        out << "            xv[step] = *reinterpret_cast<const " << vt << " *>(" << X << " + " << offsetOf(x) << " + j * " << E << " + ex);\n";
+        for (const VarRef *w : shape.perElement)
+            out << "            xv[step] *= *reinterpret_cast<const " << vt << " *>(" << PtrName(w->uvar) << " + " << offsetOf(*w) << " + j * " << E << " + ex);\n";
+        for (const VarRef *w : shape.perColumn)
+            out << "            xv[step] *= " << PtrName(w->uvar) << "[" << offsetOf(*w) << " + j];\n";
+        out << "        }\n";
+        out << "        acro_double4 acc0[" << tilesM << "]" << (pairs ? ", acc1[" + str(tilesM) + "]" : "") << ";\n";
+        out << "#pragma unroll\n";
+        out << "        for (int t = 0; t < " << tilesM << "; ++t) acc0[t] = " << (pairs ? "acc1[t] = " : "") << "acro_double4{0.0, 0.0, 0.0, 0.0};\n";
+        out << "#pragma unroll\n";
+        out << "        for (int step = 0; step < " << steps << "; ++step)\n        {\n";
+        out << "#pragma unroll\n";
+        out << "            for (int t = 0; t < " << tilesM << "; ++t)\n            {\n";
+        out << "                const double b = frag[(t * " << steps << " + step) * 64 + lane];\n";
+        if (pairs)
+        {
+            out << "                acc0[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(b, xv[step].x, acc0[t], 0, 0, 0);\n";
+            out << "                acc1[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(b, xv[step].y, acc1[t], 0, 0, 0);\n";
+        }
+        else
+            out << "                acc0[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(b, xv[step], acc0[t], 0, 0, 0);\n";
+        out << "            }\n        }\n";
+        if (ragged) out << "        if (e >= " << E << ") continue;\n";
+        if (!shape.perEntry.empty())
+        {
+            out << "        const " << vt << " se = ";
+            for (size_t i = 0; i < shape.perEntry.size(); ++i)
+                out << (i ? " * " : "") << "*reinterpret_cast<const " << vt << " *>(" << PtrName(shape.perEntry[i]->uvar) << " + " << offsetOf(*shape.perEntry[i]) << " + e)";
+            out << ";\n";
+        }
+        out << "#pragma unroll\n";
+        out << "        for (int t = 0; t < " << tilesM << "; ++t)\n";
+        out << "#pragma unroll\n";
+        out << "            for (int r = 0; r < 4; ++r)\n            {\n";
+        out << "                const int i = 16 * t + 4 * r + g;\n";
+        if (nIp != nI) out << "                if (i >= " << nI << ") continue;\n";
+        out << "                " << vt << " v = " << (pairs ? "acro_double2{acc0[t][r], acc1[t][r]}" : "acc0[t][r]") << ";\n";
+        if (!shape.perEntry.empty()) out << "                v *= se;\n";
+        for (const VarRef *w : shape.perOutput)
+            out << "                v *= *reinterpret_cast<const " << vt << " *>(" << PtrName(w->uvar) << " + " << offsetOf(*w) << " + i * " << E << " + e);\n";
+        for (const VarRef *w : shape.perRow)
+            out << "                v *= " << PtrName(w->uvar) << "[" << offsetOf(*w) << " + i];\n";
+        out << "                " << vt << " *a = reinterpret_cast<" << vt << " *>(" << A << " + " << offsetOf(s.out) << " + i * " << E << " + e);\n";
+        if (stream)
+            out << "                __builtin_nontemporal_store(v, a);\n";
+        else
+            out << "                *a " << (s.op == '=' ? "= " : (s.op == '+' ? "+= " : "-= ")) << "v;\n";
+        out << "            }\n    }\n}\n";
 
         plan.source = out.str();
         plan.nb = 64;

@@ -29,7 +29,8 @@
 //  * A single kernel that only permutes the dimensions of one operand, with different long fastest dimensions on the
 //    two sides, moves tiles of 32 x 32 entries through LDS ("transpose schedule").
 //  * A dense operator of up to 4 096 entries applied to every batch entry ("A_e_i = B_i_j X_e_j", also stored
-//    transposed or with several leading indices numbering the entries) runs the "operator schedule" on the FP64
+//    transposed, with several leading indices numbering the entries, or with the entries as the fastest dimension,
+//    "A_i_e = B_i_j X_j_e") runs the "operator schedule" on the FP64
 //    matrix cores: 16 entries per wavefront and trip through v_mfma_f64_16x16x4, the operator in LDS in operand order
 //    and padded with zeros to whole 16 x 4 blocks; pointwise factors per entry, output, row, vector element or
 //    column stay in the same launch.

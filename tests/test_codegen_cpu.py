@@ -208,6 +208,13 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     assert "operator schedule on the FP64 matrix cores: 10 x 12 operator" in src and "const double se = T3[0 + en];" in src
     assert "-= acc[t][r] * se * T6[0 + en * 10 + 16 * t + c] * T5[0 + 16 * t + c];" in src
     assert "const double2 f = *reinterpret_cast<const double2 *>(T4 + 0 + ex * 12 + 2 * g + 8 * q);" in src and "const double *f = T7 + 0 + 2 * g + 8 * q;" in src
+    # the entries as the fastest dimension: the operator becomes the instruction's first operand
+    src = TE.GetImplementation("A_i_e -= B_i_j X_j_e W_e", at.Tensor(30, 1002), at.Tensor(30, 27), at.Tensor(27, 1002), at.Tensor(1002))
+    assert "matrix cores, entries fastest: 30 x 27 operator in LDS in operand order (padded to 32 x 28), 1002 entries, 32 per wavefront" in src
+    assert "acc1[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(b, xv[step].y, acc1[t], 0, 0, 0);" in src and "const long ex = e < 1002 ? e : 1000;" in src
+    src = TE.GetImplementation("A_i_e = B_i_j X_j_e", at.Tensor(64, 1001), at.Tensor(64, 64), at.Tensor(64, 1001))
+    assert "1001 entries, 16 per wavefront and trip" in src and "__builtin_nontemporal_store(v, a);" in src and "acc1" not in src
+    assert "operator schedule" not in TE.GetImplementation("A_i_e = B_i_j X_j_e", at.Tensor(16, 3000), at.Tensor(16, 16), at.Tensor(16, 3000))
     # not this schedule: few rows (a register tile with scalar operands serves them), third operand
     for kernel, shapes in (("A_e_i = B_i_j X_e_j", [(500, 4), (4, 64), (500, 64)]),
                            ("A_e_i = B_i_j X_e_k_j W_e_k", [(500, 64), (64, 64), (500, 2, 64), (500, 2)])):
@@ -315,6 +322,9 @@ def generated_sources(TE):
     yield "operand staged in LDS", TE.GetImplementation("A_e_i = B_i_j X_e_k_j W_e_k", at.Tensor(1000, 64), at.Tensor(64, 64), at.Tensor(1000, 2, 64), at.Tensor(1000, 2))
     yield "operator schedule with pointwise factors", TE.GetImplementation("A_e_i -= B_i_j X_e_j W_e D_e_j R_i F_e_i C_j", at.Tensor(1000, 10), at.Tensor(10, 12),
                                                                          at.Tensor(1000, 12), at.Tensor(1000), at.Tensor(1000, 12), at.Tensor(10), at.Tensor(1000, 10), at.Tensor(12))
+    yield "operator schedule, entries fastest", TE.GetImplementation("A_i_e -= B_i_j X_j_e W_e D_j_e R_i F_i_e C_j", at.Tensor(30, 1002), at.Tensor(30, 27),
+                                                                   at.Tensor(27, 1002), at.Tensor(1002), at.Tensor(27, 1002), at.Tensor(30), at.Tensor(30, 1002), at.Tensor(27))
+    yield "operator schedule, entries fastest, one per lane", TE.GetImplementation("A_i_e = B_j_i X_j_e F_i_e", at.Tensor(64, 1001), at.Tensor(64, 64), at.Tensor(64, 1001), at.Tensor(64, 1001))
     yield "operator schedule with pointwise factors, odd length", TE.GetImplementation("A_e_i = B_i_j X_e_j D_e_j C_j W_e", at.Tensor(1000, 20), at.Tensor(20, 17),
                                                                                      at.Tensor(1000, 17), at.Tensor(1000, 17), at.Tensor(17), at.Tensor(1000))
     yield "operator schedule", TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(77, 5, 6), at.Tensor(77, 4, 7), at.Tensor(5, 6, 4, 7))

@@ -573,6 +573,26 @@ def test_dense_operator_through_scalar_loads(at, engine, checker, monkeypatch, k
     assert rel_err(got, expected) <= TOL
 
 
+@pytest.mark.parametrize("kernel,shapes", [
+    ("A_i_e = B_i_j X_j_e", [(64, 64), (64, 1000)]),                                 # 16 entries per trip
+    ("A_i_e -= B_i_j X_j_e", [(30, 27), (27, 1002)]),                                # 32 per trip, ragged end, padded to 32 x 28
+    ("A_i_e += B_j_i X_j_e", [(27, 30), (27, 1001)]),                                # odd number of entries: one per lane
+    ("A_i1_i2_e_q = X_j_e_q B_i1_i2_j", [(40, 7, 9), (6, 5, 40)]),                   # 63 entries numbered by two indices
+    ("A_i_e -= B_i_j X_j_e W_e D_j_e R_i F_i_e C_j", [(30, 27), (27, 1002), (1002,), (27, 1002), (30,), (30, 1002), (27,)]),
+    ("A_k_e = B_k_i X_i_e D_k_e", [(24, 22), (22, 5003), (24, 5003)]),
+    ("A_i_e = B_i_j X_j_e", [(16, 16), (16, 3000)]),                                 # small operator: not this schedule
+])
+def test_dense_operator_with_the_entries_as_the_fastest_dimension(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(len(kernel) + shapes[1][-1])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert ("matrix cores, entries fastest" in engine.GetLastImplementation()) == (shapes[0] != (16, 16))
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
+
+
 def test_dense_operator_applied_to_slices(at, engine, checker):
     """The entries' vectors and the results are slices of larger tensors (a slice starts at a whole number of rows,
     so the 16-byte loads of the entries' vectors stay aligned)."""
