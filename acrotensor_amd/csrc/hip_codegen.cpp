@@ -3204,7 +3204,8 @@ class Generator
         // or more rows fill the stores, or the vectors are long.  Measured wins: 8 x 4 53 -> 73 %, 16 x 4 43 -> 84 %,
         // 8 x 8 61 -> 85 %, 10 x 10 52 -> 81 %, 8 x 16 62 -> 85 %, 3 x 27 41 -> 73 %; losses, hence excluded:
         // 4 x 4 65 -> 49 %, 4 x 8 82 -> 77 %, 7 x 9 62 -> 57 %, 27 x 3 36 -> 28 %; 20 x 5 a tie.
-        return o.pairs ? (o.rows >= 5 && o.cols >= 4) : o.cols >= 16;
+        // (odd lengths: 9 x 9 47 -> 59 %, 25 x 25 45 -> 68 %, 27 x 27 46 -> 66 %; 5 x 5 63 -> 58 %)
+        return o.pairs ? (o.rows >= 5 && o.cols >= 4) : (o.cols >= 16 || (o.cols >= 9 && o.rows >= 8));
     }
 
     bool UseOperatorSchedule() const
@@ -3330,6 +3331,9 @@ class Generator
         // rows and columns, the entries' vectors read as zero past their end, outputs past the last row are not
         // stored.  Pairs of doubles (16-byte loads) need an even row length and an even first element.
         const bool pairs = shape.pairs;
+        // (Vectors of odd length come in 8-byte loads, 32-byte pieces per entry.  Reading the 16 vectors of a trip as
+        // one contiguous range into a per-wavefront piece of LDS first measured slower: 17 x 17 70 -> 58 %,
+        // 33 x 33 63 -> 41 %, 9 x 9 59 -> 39 %; only 27 x 27 gained, 66 -> 70 %.)
         const long nIp = (nI + 15) / 16 * 16, nJp = pairs ? (nJ + 7) / 8 * 8 : (nJ + 3) / 4 * 4;
         const long tilesN = nIp / 16, steps = nJp / 4;
         const long tiles = (E + 15) / 16;

@@ -506,6 +506,7 @@ def test_permutations_with_long_fastest_dimensions_go_through_lds_tiles(at, engi
     ("A_e_i += B_i_j X_e_j", [(10, 10), (777, 10)]),
     ("A_e_i = B_i_j X_e_j", [(3, 27), (900, 27)]),
     ("A_e_i_k = B_e_i_j C_j_k", [(600, 8, 8), (8, 8)]),                   # entries (e, i), operator stored transposed
+    ("A_e_i = B_i_j X_e_j", [(9, 9), (5000, 9)]),
     ("A_e_i = B_i_j X_e_j", [(4, 8), (5000, 8)]),                         # four rows: not this schedule
     ("A_e_i = B_i_j X_e_j", [(7, 9), (5000, 9)]),                         # odd and short: not this schedule
 ])
@@ -523,7 +524,7 @@ def test_dense_operator_applied_to_every_entry(at, engine, checker, kernel, shap
         lead = 2 if "_q_" in kernel else 1
         rows = int(np.prod(out0.shape[lead:]))
         cols = operator.size // rows
-    chosen = (rows >= 5 and cols >= 4) if cols % 2 == 0 else cols >= 16
+    chosen = (rows >= 5 and cols >= 4) if cols % 2 == 0 else (cols >= 16 or (cols >= 9 and rows >= 8))
     chosen = chosen and shapes[0] != (1000, 4)           # (there the batch index is i, which the operator carries)
     assert ("operator schedule on the FP64 matrix cores" in engine.GetLastImplementation()) == chosen
     needs_padding = rows % 16 != 0 or cols % (8 if cols % 2 == 0 else 4) != 0
