@@ -3189,6 +3189,9 @@ class Generator
             else return false;
         }
         if (!o.cores) return o.rows >= 16 && o.cols >= 16 && !o.transposed && !o.trailing && s.in.size() == 2;  // (its lanes walk the operator's rows)
+        // A lane holds cols / 4 vector elements and rows / 4 results; the padded operator must fit the 64 KB of LDS
+        // that a workgroup may declare.
+        if (o.rows > 256 || o.cols > 256 || ((o.rows + 15) / 16 * 16) * ((o.cols + 7) / 8 * 8) > 8192) return false;
         if (o.trailing)
         {
             // Entries fastest: the generic schedule (one entry per lane, operator in scalar registers) streams whole

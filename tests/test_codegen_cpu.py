@@ -215,6 +215,9 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     src = TE.GetImplementation("A_i_e = B_i_j X_j_e", at.Tensor(64, 1001), at.Tensor(64, 64), at.Tensor(64, 1001))
     assert "1001 entries, 16 per wavefront and trip" in src and "__builtin_nontemporal_store(v, a);" in src and "acc1" not in src
     assert "operator schedule" not in TE.GetImplementation("A_i_e = B_i_j X_j_e", at.Tensor(16, 3000), at.Tensor(16, 16), at.Tensor(16, 3000))
+    # very long vectors or very many rows would not fit a lane's registers: not this schedule
+    assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 5), at.Tensor(5, 818), at.Tensor(900, 818))
+    assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 300), at.Tensor(300, 12), at.Tensor(900, 12))
     # not this schedule: few rows (a register tile with scalar operands serves them), third operand
     for kernel, shapes in (("A_e_i = B_i_j X_e_j", [(500, 4), (4, 64), (500, 64)]),
                            ("A_e_i = B_i_j X_e_k_j W_e_k", [(500, 64), (64, 64), (500, 2, 64), (500, 2)])):

@@ -495,6 +495,7 @@ def test_permutations_with_long_fastest_dimensions_go_through_lds_tiles(at, engi
     ("A_e_i = B_i_j X_e_j", [(16, 16), (40007, 16)]),                     # more trips than wavefronts
     ("A_e_i = B_i_j X_e_j", [(16, 256), (300, 256)]),                     # 64 terms steps, one output tile
     ("A_e_i = B_i_j X_e_j", [(256, 16), (300, 16)]),                      # 16 output tiles
+    ("A_e_i = B_i_j X_e_j", [(17, 240), (300, 240)]),                     # padded to 32 x 240: 60 KB of LDS
     ("A_e_i1_i2 -= B_i1_i2_j1_j2 X_e_j1_j2", [(8, 6, 4, 10), (77, 4, 10)]),
     ("A_e_i = B_j_i X_e_j", [(40, 48), (1001, 40)]),                      # the operator stored transposed
     ("A_e_q_i += B_j_i X_e_q_j", [(24, 32), (100, 7, 24)]),               # 700 entries numbered by two indices
