@@ -1583,7 +1583,7 @@ class Generator
         // which workgroups start, not by memory: with 1 - 2 KB per workgroup a copy reaches 72 % of the HBM peak and
         // an outer product 64 %.  Such groups take more batch entries per workgroup, in several passes of its lanes,
         // until a workgroup moves 8 KB (copy 72 -> 79 %, outer product 64 -> 88 %, batched 8 x 8 transpose 70 -> 77 %,
-        // batched dot product 71 -> 74 %).  From 3 KB per workgroup on the same change measured slower
+        // batched dot product 71 -> 76 %).  From 3 KB per workgroup on the same change measured slower
         // (`A_e_i += B_e_i` 77 -> 75 %, three-operand product 78 -> 75 %), hence the threshold.
         lightWorkgroups = false;
         if (opt.force_nb <= 0 && opt.force_nt <= 0 && envInt("ACRO_HIP_NB") <= 0 && envInt("ACRO_HIP_NT") <= 0 && batch >= 0 &&
@@ -1591,7 +1591,13 @@ class Generator
         {
             bool streaming = subs.back().phase == 0;
             for (const auto &st : stores) streaming = streaming && !st.wantLds && !st.staged;
-            for (const auto &s : subs) streaming = streaming && s.splitLanes == 0 && !s.loopMode && s.matrixOp == 0 && has(s.out.idx, batch);
+            bool shared = false;   // outputs shared by lanes: their workgroups keep 128 lanes (batched dot product with
+                                   // 16 entries per workgroup: 76 % in 128 lanes, 66 % in 256)
+            for (const auto &s : subs)
+            {
+                streaming = streaming && (!s.loopMode || s.splitLanes != 0) && s.matrixOp == 0 && has(s.out.idx, batch);
+                shared = shared || s.splitLanes != 0;
+            }
             double perEntry = 0.0;
             std::set<int> counted;
             for (const auto &s : subs)
@@ -1611,7 +1617,7 @@ class Generator
                 if (nb > NB)
                 {
                     NB = static_cast<int>(nb);
-                    if (static_cast<long>(NB) * maxLane >= 512) NT = std::max(NT, 256);
+                    if (static_cast<long>(NB) * maxLane >= 512 && !shared) NT = std::max(NT, 256);
                     lightWorkgroups = true;
                 }
             }
