@@ -2462,7 +2462,8 @@ class Generator
         for (const auto &l : body.bases) lines.push_back(l);
         lines.push_back("const int cl = w & " + str(L - 1) + ";");
         lines.push_back("double sum = 0.0;");
-        lines.push_back("#pragma unroll 4");
+        // eight loads in flight per lane (row sums of 1 024 terms: 69 % of the HBM peak with 4, 75 % with 8, 73 % with 16)
+        lines.push_back("#pragma unroll 8");
         lines.push_back("for (int c = cl; c < " + str(s.contrCount) + "; c += " + str(L) + ")");
         lines.push_back("{");
         long st = s.contrCount;
@@ -2836,7 +2837,7 @@ class Generator
             out << "    double sum = 0.0;\n";
             out << "    if (o < " << O << ")\n    {\n";
             decompose(s.outIdx, "o", "        ");
-            out << "#pragma unroll 4\n";
+            out << "#pragma unroll 4\n";   // (8: 77 -> 71 % of the HBM peak for 64 rows of 2^20 terms)
             out << "        for (long c = (long)gc * " << Sn << " + sl; c < " << Nc << "; c += " << G * Sn << ")\n        {\n";
             decompose(s.contr, "c", "            ");
             std::string prod;
@@ -2865,7 +2866,7 @@ class Generator
             out << "    if (lane < " << Sn * O << ")\n    {\n";
             decompose(s.outIdx, "o", "        ");
             out << "        const long g = " << gExpr << ";\n";
-            out << "#pragma unroll 4\n";
+            out << "#pragma unroll 8\n";   // (4: 71 %, 8: 75 %, 16: 74 % of the HBM peak for 64 column sums over 2^20 rows)
             out << "        for (long c = g * " << Sn << " + sl; c < " << Nc << "; c += " << G * Sn << ")\n        {\n";
             decompose(s.contr, "c", "            ");
             std::string prod;
