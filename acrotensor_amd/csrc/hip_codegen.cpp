@@ -3104,10 +3104,11 @@ class Generator
         std::vector<const VarRef *> perEntry, perOutput, perRow, perElement, perColumn;
     };
 
-    bool OperatorPattern(OperatorShape &o) const
+    // `k`: the kernel of the group; `alone`: it is the whole group (inputs are then never written in the launch).
+    bool OperatorPattern(OperatorShape &o, int k = 0, bool alone = true) const
     {
-        if (subs.size() != 1 || batch < 0 || !opt.noalias || NumGatherSlots() > 0 || envInt("ACRO_HIP_OPERATOR") < 0) return false;
-        const Sub &s = subs[0];
+        if ((alone && subs.size() != 1) || batch < 0 || !opt.noalias || NumGatherSlots() > 0 || envInt("ACRO_HIP_OPERATOR") < 0) return false;
+        const Sub &s = subs[k];
         if (s.matrixOp != 0 || s.in.size() < 2 || s.contr.empty() || s.out.repeated) return false;
         // the operator: the one operand without the batch index that carries contracted and free indices;
         // the vectors: the first operand with the batch index that carries every contracted index
@@ -3127,7 +3128,8 @@ class Generator
         if (!o.op || !o.x) return false;
         for (const auto &v : s.in)
         {
-            if (v.repeated || v.uvar == s.out.uvar || !IsPureInput(v.uvar)) return false;
+            if (v.repeated || v.uvar == s.out.uvar || uvars[v.uvar].storage == uvars[s.out.uvar].storage) return false;
+            if (alone && !IsPureInput(v.uvar)) return false;
         }
         // out = (e..., I...), X = (e..., J...), B = (I..., J...) or (J..., I...): the leading indices that the result
         // and X share, the batch index first, number the entries
@@ -3222,14 +3224,56 @@ class Generator
         return o.pairs ? (o.rows >= 5 && o.cols >= 4) : (o.cols >= 16 || (o.cols >= 9 && o.rows >= 8));
     }
 
+    // A group of several kernels each of which is a large dense operator applied to every entry ("U = B X D" followed
+    // by "Y = Bt U": a dense element operator applied and applied back) runs as one matrix-core launch per kernel,
+    // in order on the stream, with the intermediates in device memory.  The fused chain schedule keeps the
+    // intermediates on chip but gives a lane one entry and one row, which for large operators is bound by LDS reads:
+    // 64 x 64, 2^18 entries: 400 us fused against 134 us for the two launches; 27 x 27: 241 against 143 us; small
+    // operators stay fused (8 x 8 with a transient intermediate: 156 against 227 us; 12 x 10: 124 against 165 us).
+    bool UseOperatorSequence() const
+    {
+        if (subs.size() < 2 || envInt("ACRO_HIP_OPERATOR_SEQUENCE") < 0) return false;
+        for (size_t k = 0; k < subs.size(); ++k)
+        {
+            OperatorShape o;
+            if (!OperatorPattern(o, static_cast<int>(k), false) || !o.cores || o.rows * o.cols < 512) return false;
+        }
+        return true;
+    }
+
     bool UseOperatorSchedule() const
     {
         OperatorShape o;
-        return OperatorPattern(o);
+        return OperatorPattern(o) || UseOperatorSequence();
     }
+
+    int opSub = 0;            // the kernel that the operator emitters work on
+    bool opSequence = false;  // ... as one of several launches
 
     void EmitOperator(HipKernelPlan &plan)
     {
+        if (subs.size() > 1)
+        {
+            opSequence = true;
+            std::string schedule;
+            int lds = 0;
+            for (size_t k = 0; k < subs.size(); ++k)
+            {
+                opSub = static_cast<int>(k);
+                OperatorShape shape;
+                OperatorPattern(shape, opSub, false);
+                if (shape.trailing)
+                    EmitOperatorEntriesFastest(plan, shape);
+                else
+                    EmitOperatorMatrixCores(plan, shape);
+                schedule += plan.schedule;
+                lds = std::max(lds, plan.lds_bytes);
+            }
+            plan.schedule = schedule;
+            plan.lds_bytes = lds;
+            plan.module_name = plan.launches.front().function_name;
+            return;
+        }
         const Sub &s = subs[0];
         OperatorShape shape;
         OperatorPattern(shape);
@@ -3338,7 +3382,7 @@ class Generator
     // with 2 048; loading the next 16 entries ahead of the arithmetic made no difference).
     void EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape &shape)
     {
-        const Sub &s = subs[0];
+        const Sub &s = subs[opSub];
         const VarRef &opr = *shape.op, &x = *shape.x;
         const long nI = shape.rows, nJ = shape.cols, E = shape.entries;
         // Sizes that the instruction's 16 x 4 blocks do not divide: the operator's copy in LDS is padded with zero
@@ -3367,17 +3411,17 @@ class Generator
         const std::string dimName = mk.GetDimensionedNameString();
         char hex[32];
         std::snprintf(hex, sizeof(hex), "%016llx",
-                      static_cast<unsigned long long>(hashString(dimName + "/operator-mfma/" + (Positional() ? "p" : "u") + (pairs ? "2" : "1"))));
+                      static_cast<unsigned long long>(hashString(dimName + "/operator-mfma/" + str(opSub) + "/" + (Positional() ? "p" : "u") + (pairs ? "2" : "1"))));
         plan.module_name = std::string("acro_op_") + hex;
         std::ostringstream sched;
         sched << "operator schedule on the FP64 matrix cores: " << nI << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator")
               << " in LDS in operand order";
         if (nIp != nI || nJp != nJ) sched << " (padded to " << nIp << " x " << nJp << ")";
         sched << ", " << E << " entries, 16 per wavefront and trip, "
-              << tilesN * steps << " v_mfma_f64_16x16x4 per trip, " << blocks << " workgroups of 256 lanes\n  [0] " << s.text << "\n";
+              << tilesN * steps << " v_mfma_f64_16x16x4 per trip, " << blocks << " workgroups of 256 lanes\n  [" << opSub << "] " << s.text << "\n";
         plan.schedule = sched.str();
 
-        out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
+        if (opSub == 0) out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
         {
             std::istringstream lines(plan.schedule);
             std::string l;
@@ -3387,7 +3431,7 @@ class Generator
         const bool stream = s.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0;
         // term group g (lane / 16) of step s stands for this j
         const std::string termOf = pairs ? "8 * (step >> 1) + 2 * (l >> 4) + (step & 1)" : "4 * step + (l >> 4)";
-        out << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
+        out << (opSub == 0 ? "" : "\n") << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
         out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << plan.module_name << "(" << ParamList() << ")\n{\n";
         out << "    __shared__ double frag[" << nIp * nJp << "];\n";
         out << "    for (int f = threadIdx.x; f < " << nIp * nJp << "; f += 256)\n    {\n";
@@ -3517,7 +3561,7 @@ class Generator
     // 16 bytes, which feed two accumulator sets (even and odd entries), and stores its two results together.
     void EmitOperatorEntriesFastest(HipKernelPlan &plan, const OperatorShape &shape)
     {
-        const Sub &s = subs[0];
+        const Sub &s = subs[opSub];
         const VarRef &opr = *shape.op, &x = *shape.x;
         const long nI = shape.rows, nJ = shape.cols, E = shape.entries;
         const bool pairs = shape.pairs;
@@ -3536,17 +3580,17 @@ class Generator
         const std::string dimName = mk.GetDimensionedNameString();
         char hex[32];
         std::snprintf(hex, sizeof(hex), "%016llx",
-                      static_cast<unsigned long long>(hashString(dimName + "/operator-mfma-t/" + (Positional() ? "p" : "u") + (pairs ? "2" : "1"))));
+                      static_cast<unsigned long long>(hashString(dimName + "/operator-mfma-t/" + str(opSub) + "/" + (Positional() ? "p" : "u") + (pairs ? "2" : "1"))));
         plan.module_name = std::string("acro_op_") + hex;
         std::ostringstream sched;
         sched << "operator schedule on the FP64 matrix cores, entries fastest: " << nI << " x " << nJ
               << (shape.transposed ? " operator (stored transposed)" : " operator") << " in LDS in operand order";
         if (nIp != nI || nJp != nJ) sched << " (padded to " << nIp << " x " << nJp << ")";
         sched << ", " << E << " entries, " << per << " per wavefront and trip, " << tilesM * steps * (pairs ? 2 : 1)
-              << " v_mfma_f64_16x16x4 per trip, " << blocks << " workgroups of 256 lanes\n  [0] " << s.text << "\n";
+              << " v_mfma_f64_16x16x4 per trip, " << blocks << " workgroups of 256 lanes\n  [" << opSub << "] " << s.text << "\n";
         plan.schedule = sched.str();
 
-        out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
+        if (opSub == 0) out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
         {
             std::istringstream lines(plan.schedule);
             std::string l;
@@ -3556,7 +3600,7 @@ class Generator
         const bool stream = s.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0;
         const std::string vt = pairs ? "acro_double2" : "double";
         auto offsetOf = [&](const VarRef &v) { return Lit(uvars[v.uvar].viewOffset); };
-        out << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
+        out << (opSub == 0 ? "" : "\n") << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
         out << "typedef double acro_double2 __attribute__((ext_vector_type(2)));\n";
         out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << plan.module_name << "(" << ParamList() << ")\n{\n";
         out << "    __shared__ double frag[" << nIp * nJp << "];\n";

@@ -62,6 +62,8 @@
 //                               in LDS, one entry per lane) instead of the operator schedule
 //   ACRO_HIP_LIGHT=-1           streaming groups whose workgroups move less than 2.5 KB keep their batch size (no extra
 //                               passes to bring a workgroup to 8 KB)
+//   ACRO_HIP_OPERATOR_SEQUENCE=-1  groups of several large operator-shaped kernels run as one fused chain kernel instead of one
+//                               matrix-core launch per kernel
 //   ACRO_HIP_OPERATOR_MFMA=-1   the operator schedule never uses the FP64 matrix cores (a lane keeps its row for four entries,
 //                               whose vectors come through scalar loads, whatever the operator's sizes)
 //   ACRO_HIP_RED_PENCIL=-1      split contractions: one lane per (slice, output entry) also when there are few outputs

@@ -595,6 +595,33 @@ def test_dense_operator_with_the_entries_as_the_fastest_dimension(at, engine, ch
     assert rel_err(got, expected) <= TOL
 
 
+@pytest.mark.parametrize("nq,nd,entries,transient", [(32, 27, 1003, True), (32, 27, 1003, False), (64, 64, 517, True), (8, 8, 1000, True)])
+def test_dense_operator_applied_and_applied_back_in_one_capture(at, engine, checker, nq, nd, entries, transient):
+    """Y = Bt (D o (B X)) recorded as two kernels.  Large operators run as one matrix-core launch per kernel (the
+    intermediate goes through device memory even when it is marked transient), small ones as one fused kernel."""
+    rng = np.random.default_rng(nq * nd + entries)
+    B, X, D = rng.uniform(-1, 1, (nq, nd)), rng.uniform(-1, 1, (entries, nd)), rng.uniform(0.5, 1.5, (entries, nq))
+    Y0 = rng.uniform(-1, 1, (entries, nd))
+    tB, tX, tD, tY, tU = to_tensor(at, B), to_tensor(at, X), to_tensor(at, D), to_tensor(at, Y0), at.Tensor(entries, nq)
+    tU.SetTransient(transient)
+    print("operator chain", nq, nd, entries, transient, flush=True)
+    engine.BeginMultiKernelLaunch()
+    engine("U_e_k = B_k_j X_e_j D_e_k", tU, tB, tX, tD)
+    engine("Y_e_i += B_k_i U_e_k", tY, tB, tU)
+    engine.EndMultiKernelLaunch()
+    src = engine.GetLastImplementation()
+    assert (src.count("operator schedule on the FP64 matrix cores") == 2) == (nq * nd >= 512)
+    tY.MoveFromGPU()
+    U = np.zeros((entries, nq))
+    checker.contract("U_e_k = B_k_j X_e_j D_e_k", U, B, X, D)
+    expected = Y0.copy()
+    checker.contract("Y_e_i += B_k_i U_e_k", expected, B, U)
+    assert rel_err(tY.data, expected) <= TOL
+    if not transient:
+        tU.MoveFromGPU()
+        assert rel_err(tU.data, U) <= TOL
+
+
 def test_dense_operator_applied_to_slices(at, engine, checker):
     """The entries' vectors and the results are slices of larger tensors (a slice starts at a whole number of rows,
     so the 16-byte loads of the entries' vectors stay aligned)."""
