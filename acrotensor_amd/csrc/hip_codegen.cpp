@@ -3241,17 +3241,52 @@ class Generator
         return true;
     }
 
+    // Two operator-shaped kernels of which the second is applied to the first one's result, and that result is
+    // transient and read by nothing else: one kernel, the intermediate handed over through LDS.
+    bool OperatorPair(OperatorShape &first, OperatorShape &second) const
+    {
+        if (subs.size() != 2 || envInt("ACRO_HIP_OPERATOR_PAIR") < 0) return false;
+        if (!OperatorPattern(first, 0, false) || !OperatorPattern(second, 1, false)) return false;
+        if (!first.cores || !second.cores || first.trailing || second.trailing) return false;
+        const Sub &k0 = subs[0], &k1 = subs[1];
+        if (k0.op != '=' || second.x->uvar != k0.out.uvar || second.x->idx != k0.out.idx) return false;
+        if (!stores[uvars[k0.out.uvar].storage].transient || uvars[k1.out.uvar].storage == uvars[k0.out.uvar].storage) return false;
+        if (!second.perElement.empty() || !second.perColumn.empty()) return false;
+        for (const auto &v : k1.in)
+        {
+            if (&v != second.x && uvars[v.uvar].storage == uvars[k0.out.uvar].storage) return false;
+        }
+        if (first.entries != second.entries || first.rows != second.cols) return false;
+        // (2^19 - 2^22 entries, generic fused chain -> this kernel: 8 x 8 156 -> 142 us, 12 x 10 124 -> 93 us, 16 x 16 137 -> 61 us,
+        // 20 x 12 125 -> 64 us, 24 x 20 277 -> 169 us; against two launches: 27 x 27 143 -> 74 us, 32 x 27 112 -> 62 us,
+        // 64 x 27 190 -> 92 us)
+        if (first.rows * first.cols < 64 || second.rows * second.cols < 64) return false;
+        const long n1 = ((first.rows + 15) / 16 * 16) * (first.pairs ? (first.cols + 7) / 8 * 8 : (first.cols + 3) / 4 * 4);
+        const long n2 = ((second.rows + 15) / 16 * 16) * ((second.cols + 3) / 4 * 4);
+        return (n1 + n2 + 64 * (first.rows + 1)) * 8 <= 64 * 1024;
+    }
+
     bool UseOperatorSchedule() const
     {
-        OperatorShape o;
-        return OperatorPattern(o) || UseOperatorSequence();
+        OperatorShape o, o2;
+        return OperatorPattern(o) || OperatorPair(o, o2) || UseOperatorSequence();
     }
+
 
     int opSub = 0;            // the kernel that the operator emitters work on
     bool opSequence = false;  // ... as one of several launches
 
     void EmitOperator(HipKernelPlan &plan)
     {
+        {
+            OperatorShape first, second;
+            if (OperatorPair(first, second))
+            {
+                opSub = 0;
+                EmitOperatorMatrixCores(plan, first, &second, 1);
+                return;
+            }
+        }
         if (subs.size() > 1)
         {
             opSequence = true;
@@ -3380,7 +3415,10 @@ class Generator
     // same; what the matrix cores save is operand delivery: no scalar loads and 1/16 of the LDS reads.
     // 64 x 64 on 2^18 entries: 47 - 51 us against 79 us with scalar loads (512 workgroups; 58 us with 1 024, 76 us
     // with 2 048; loading the next 16 entries ahead of the arithmetic made no difference).
-    void EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape &shape)
+    // With `next` (and its kernel `nextSub`) the result of this operator never leaves the chip: it is scaled, written
+    // to a per-wavefront piece of LDS in the result layout (entry 4r + lane / 16, output lane % 16), read back in the
+    // operand layout (entry lane % 16, term group lane / 16) and multiplied by the second operator.
+    void EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape &shape, const OperatorShape *next = nullptr, int nextSub = -1)
     {
         const Sub &s = subs[opSub];
         const VarRef &opr = *shape.op, &x = *shape.x;
@@ -3394,6 +3432,8 @@ class Generator
         // 33 x 33 63 -> 41 %, 9 x 9 59 -> 39 %; only 27 x 27 gained, 66 -> 70 %.)
         const long nIp = (nI + 15) / 16 * 16, nJp = pairs ? (nJ + 7) / 8 * 8 : (nJ + 3) / 4 * 4;
         const long tilesN = nIp / 16, steps = nJp / 4;
+        const long steps2 = (nI + 3) / 4;                 // the second operator contracts over this one's rows
+        const long midStride = nI % 2 == 0 ? nI + 1 : nI; // odd: the lanes' rows of the hand-over buffer start in different banks
         const long tiles = (E + 15) / 16;
         const bool ragged = E % 16 != 0;
         // Equal work per CU matters more than the number of wavefronts: 256 CUs, one or two workgroups each.
@@ -3411,7 +3451,7 @@ class Generator
         const std::string dimName = mk.GetDimensionedNameString();
         char hex[32];
         std::snprintf(hex, sizeof(hex), "%016llx",
-                      static_cast<unsigned long long>(hashString(dimName + "/operator-mfma/" + str(opSub) + "/" + (Positional() ? "p" : "u") + (pairs ? "2" : "1"))));
+                      static_cast<unsigned long long>(hashString(dimName + "/operator-mfma/" + str(opSub) + "/" + (Positional() ? "p" : "u") + (pairs ? "2" : "1") + (next ? "+" : ""))));
         plan.module_name = std::string("acro_op_") + hex;
         std::ostringstream sched;
         sched << "operator schedule on the FP64 matrix cores: " << nI << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator")
@@ -3419,6 +3459,9 @@ class Generator
         if (nIp != nI || nJp != nJ) sched << " (padded to " << nIp << " x " << nJp << ")";
         sched << ", " << E << " entries, 16 per wavefront and trip, "
               << tilesN * steps << " v_mfma_f64_16x16x4 per trip, " << blocks << " workgroups of 256 lanes\n  [" << opSub << "] " << s.text << "\n";
+        if (next)
+            sched << "  [" << nextSub << "] " << subs[nextSub].text << " : " << next->rows << " x " << next->cols << (next->transposed ? " operator (stored transposed)" : " operator")
+                  << " applied to the first result on chip (handed over through " << 16 * midStride * 8 << " bytes of LDS per wavefront)\n";
         plan.schedule = sched.str();
 
         if (opSub == 0) out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
@@ -3442,6 +3485,18 @@ class Generator
             out << "        frag[f] = row < " << nI << " && j < " << nJ << " ? " << element << " : 0.0;\n    }\n";
         else
             out << "        frag[f] = " << element << ";\n    }\n";
+        if (next)
+        {
+            // the second operator: its columns are the first one's rows, terms in natural order
+            const long rows2P = (next->rows + 15) / 16 * 16;
+            out << "    __shared__ double frag2[" << rows2P * steps2 * 4 << "];\n";
+            out << "    __shared__ double stage[" << 4 * 16 * midStride << "];\n";
+            out << "    for (int f = threadIdx.x; f < " << rows2P * steps2 * 4 << "; f += 256)\n    {\n";
+            out << "        const int l = f & 63, step = (f >> 6) % " << steps2 << ", t = (f >> 6) / " << steps2 << ";\n";
+            out << "        const int row = 16 * t + (l & 15), j = 4 * step + (l >> 4);\n";
+            out << "        frag2[f] = row < " << next->rows << " && j < " << nI << " ? " << PtrName(next->op->uvar) << "[" << Lit(uvars[next->op->uvar].viewOffset)
+                << (next->transposed ? " + j * " + str(next->rows) + " + row]" : " + row * " + str(nI) + " + j]") << " : 0.0;\n    }\n";
+        }
         out << "    __syncthreads();\n";
         out << "    const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;\n";
         // (A contiguous range of trips per workgroup instead of this stride: the same or up to 8 % slower.)
@@ -3512,38 +3567,76 @@ class Generator
         out << "            for (int t = 0; t < " << tilesN << "; ++t)\n";
         out << "                acc[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(xs, frag[(t * " << steps << " + step) * 64 + lane], acc[t], 0, 0, 0);\n";
         out << "        }\n";
-        out << "        double *a = " << A << " + " << Lit(uvars[s.out.uvar].viewOffset) << " + (tile * 16 + g) * " << nI << " + c;\n";
-        out << "#pragma unroll\n";
-        out << "        for (int r = 0; r < 4; ++r)\n        {\n";
-        if (ragged) out << "            if (tile * 16 + g + 4 * r >= " << E << ") continue;\n";
-        // the result's pointwise factors
-        std::string value = "acc[t][r]";
-        const bool scaled = !shape.perEntry.empty() || !shape.perOutput.empty() || !shape.perRow.empty();
-        if (scaled) out << "            const long en = tile * 16 + g + 4 * r;\n";
-        if (!shape.perEntry.empty())
-        {
-            out << "            const double se = ";
-            for (size_t i = 0; i < shape.perEntry.size(); ++i)
-                out << (i ? " * " : "") << PtrName(shape.perEntry[i]->uvar) << "[" << Lit(uvars[shape.perEntry[i]->uvar].viewOffset) << " + en]";
-            out << ";\n";
-            value += " * se";
-        }
-        for (const VarRef *w : shape.perOutput)
-            value += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + " + en * " + str(nI) + " + 16 * t + c]";
-        for (const VarRef *w : shape.perRow)
-            value += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + " + 16 * t + c]";
-        out << "#pragma unroll\n";
-        out << "            for (int t = 0; t < " << tilesN << "; ++t)\n";
-        std::string guard = nIp != nI ? "if (16 * t + c < " + str(nI) + ") " : "";
-        if (stream)
-            out << "                " << guard << "__builtin_nontemporal_store(" << value << ", a + 4 * r * " << nI << " + 16 * t);\n";
+        // Stores of one operator's results (or, with toLds, their hand-over to the second operator).
+        auto emitResults = [&](const Sub &ks, const OperatorShape &sh, long rows, const std::string &accName, bool toLds) {
+            const long rowsP = (rows + 15) / 16 * 16;
+            const bool streams = ks.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0;
+            if (!toLds)
+                out << "        double *a = " << PtrName(ks.out.uvar) << " + " << Lit(uvars[ks.out.uvar].viewOffset) << " + (tile * 16 + g) * " << rows << " + c;\n";
+            out << "#pragma unroll\n";
+            out << "        for (int r = 0; r < 4; ++r)\n        {\n";
+            if (ragged) out << "            if (tile * 16 + g + 4 * r >= " << E << ") continue;\n";
+            // the result's pointwise factors
+            std::string value = accName + "[t][r]";
+            const bool scaled = !sh.perEntry.empty() || !sh.perOutput.empty() || !sh.perRow.empty();
+            if (scaled) out << "            const long en = tile * 16 + g + 4 * r;\n";
+            if (!sh.perEntry.empty())
+            {
+                out << "            const double se = ";
+                for (size_t i = 0; i < sh.perEntry.size(); ++i)
+                    out << (i ? " * " : "") << PtrName(sh.perEntry[i]->uvar) << "[" << Lit(uvars[sh.perEntry[i]->uvar].viewOffset) << " + en]";
+                out << ";\n";
+                value += " * se";
+            }
+            for (const VarRef *w : sh.perOutput)
+                value += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + " + en * " + str(rows) + " + 16 * t + c]";
+            for (const VarRef *w : sh.perRow)
+                value += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + " + 16 * t + c]";
+            out << "#pragma unroll\n";
+            out << "            for (int t = 0; t < " << rowsP / 16 << "; ++t)\n";
+            std::string guard = rowsP != rows ? "if (16 * t + c < " + str(rows) + ") " : "";
+            if (toLds)
+                out << "                " << guard << "mid[(4 * r + g) * " << midStride << " + 16 * t + c] = " << value << ";\n";
+            else if (streams)
+                out << "                " << guard << "__builtin_nontemporal_store(" << value << ", a + 4 * r * " << rows << " + 16 * t);\n";
+            else
+                out << "                " << guard << "a[4 * r * " << rows << " + 16 * t]" << (ks.op == '=' ? " = " : (ks.op == '+' ? " += " : " -= ")) << value << ";\n";
+            out << "        }\n";
+        };
+        (void)A;
+        (void)stream;
+        if (!next)
+            emitResults(s, shape, nI, "acc", false);
         else
-            out << "                " << guard << "a[4 * r * " << nI << " + 16 * t]" << (s.op == '=' ? " = " : (s.op == '+' ? " += " : " -= ")) << value << ";\n";
-        out << "        }\n    }\n}\n";
+        {
+            const long rows2 = next->rows, rows2P = (rows2 + 15) / 16 * 16;
+            out << "        double *mid = stage + (threadIdx.x >> 6) * " << 16 * midStride << ";\n";
+            out << "        {\n";
+            emitResults(s, shape, nI, "acc", true);
+            out << "        }\n";
+            // a wavefront's LDS accesses complete in program order: no barrier, only the compiler kept from reordering
+            out << "        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");\n        __builtin_amdgcn_wave_barrier();\n";
+            out << "        acro_double4 acc2[" << rows2P / 16 << "];\n";
+            out << "#pragma unroll\n";
+            out << "        for (int t = 0; t < " << rows2P / 16 << "; ++t) acc2[t] = acro_double4{0.0, 0.0, 0.0, 0.0};\n";
+            out << "#pragma unroll\n";
+            out << "        for (int step = 0; step < " << steps2 << "; ++step)\n        {\n";
+            out << "            const double us = ";
+            if (steps2 * 4 != nI) out << "4 * step + g >= " << nI << " ? 0.0 : ";
+            out << "mid[c * " << midStride << " + 4 * step + g];\n";
+            out << "#pragma unroll\n";
+            out << "            for (int t = 0; t < " << rows2P / 16 << "; ++t)\n";
+            out << "                acc2[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(us, frag2[(t * " << steps2 << " + step) * 64 + lane], acc2[t], 0, 0, 0);\n";
+            out << "        }\n";
+            out << "        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");\n        __builtin_amdgcn_wave_barrier();\n";
+            emitResults(subs[nextSub], *next, rows2, "acc2", false);
+        }
+        out << "    }\n}\n";
+
 
         plan.source = out.str();
         plan.nb = 64;
-        plan.lds_bytes = static_cast<int>(nIp * nJp * 8);
+        plan.lds_bytes = static_cast<int>((nIp * nJp + (next ? (next->rows + 15) / 16 * 16 * steps2 * 4 + 64 * midStride : 0)) * 8);
         FillParams(plan, false);
         HipLaunch launch;
         launch.function_name = plan.module_name;

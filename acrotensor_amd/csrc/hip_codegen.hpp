@@ -33,7 +33,8 @@
 //    "A_i_e = B_i_j X_j_e") runs the "operator schedule" on the FP64
 //    matrix cores: 16 entries per wavefront and trip through v_mfma_f64_16x16x4, the operator in LDS in operand order
 //    and padded with zeros to whole 16 x 4 blocks; pointwise factors per entry, output, row, vector element or
-//    column stay in the same launch.
+//    column stay in the same launch; a second operator applied to a transient result runs in the same kernel, the
+//    intermediate passing from the result layout to the operand layout through a per-wavefront piece of LDS.
 //  * A streaming group whose workgroups would move less than 2.5 KB takes more batch entries per workgroup.
 //  * Contractions too long to unroll fall back to counted loops with the same lane mapping.
 //
@@ -62,6 +63,7 @@
 //                               in LDS, one entry per lane) instead of the operator schedule
 //   ACRO_HIP_LIGHT=-1           streaming groups whose workgroups move less than 2.5 KB keep their batch size (no extra
 //                               passes to bring a workgroup to 8 KB)
+//   ACRO_HIP_OPERATOR_PAIR=-1   two operator-shaped kernels with a transient intermediate are not joined into one matrix-core kernel
 //   ACRO_HIP_OPERATOR_SEQUENCE=-1  groups of several large operator-shaped kernels run as one fused chain kernel instead of one
 //                               matrix-core launch per kernel
 //   ACRO_HIP_OPERATOR_MFMA=-1   the operator schedule never uses the FP64 matrix cores (a lane keeps its row for four entries,

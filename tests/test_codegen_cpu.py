@@ -328,7 +328,8 @@ def generated_sources(TE):
     yield "operator schedule, entries fastest", TE.GetImplementation("A_i_e -= B_i_j X_j_e W_e D_j_e R_i F_i_e C_j", at.Tensor(30, 1002), at.Tensor(30, 27),
                                                                    at.Tensor(27, 1002), at.Tensor(1002), at.Tensor(27, 1002), at.Tensor(30), at.Tensor(30, 1002), at.Tensor(27))
     yield "operator schedule, entries fastest, one per lane", TE.GetImplementation("A_i_e = B_j_i X_j_e F_i_e", at.Tensor(64, 1001), at.Tensor(64, 64), at.Tensor(64, 1001), at.Tensor(64, 1001))
-    yield "operator schedule, two launches", operator_chain_source(TE, 32, 27, 999)
+    yield "operator schedule, two launches", operator_chain_source(TE, 32, 27, 999, False)
+    yield "operator schedule, two operators in one kernel", operator_chain_source(TE, 30, 27, 998)
     yield "operator schedule with pointwise factors, odd length", TE.GetImplementation("A_e_i = B_i_j X_e_j D_e_j C_j W_e", at.Tensor(1000, 20), at.Tensor(20, 17),
                                                                                      at.Tensor(1000, 17), at.Tensor(1000, 17), at.Tensor(17), at.Tensor(1000))
     yield "operator schedule", TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(77, 5, 6), at.Tensor(77, 4, 7), at.Tensor(5, 6, 4, 7))
@@ -394,10 +395,10 @@ def test_matrix_operation_without_a_reader_in_the_launch_runs_on_its_own(TE):
     assert "runs on its own" in src and "matrix inverse" not in src
 
 
-def operator_chain_source(TE, nq, nd, entries=1000):
+def operator_chain_source(TE, nq, nd, entries=1000, transient=True):
     B, X, D = at.Tensor(nq, nd), at.Tensor(entries, nd), at.Tensor(entries, nq)
     U, Y = at.Tensor(entries, nq), at.Tensor(entries, nd)
-    U.SetTransient(True)
+    U.SetTransient(transient)
     TE.BeginMultiKernelLaunch()
     TE("U_e_k = B_k_j X_e_j D_e_k", U, B, X, D)
     TE("Y_e_i = B_k_i U_e_k", Y, B, U)
@@ -405,12 +406,18 @@ def operator_chain_source(TE, nq, nd, entries=1000):
 
 
 def test_large_dense_operators_in_a_capture_run_as_one_matrix_core_launch_each(TE):
-    src = operator_chain_source(TE, 32, 27)
+    src = operator_chain_source(TE, 32, 27, transient=False)
     assert src.count("__global__") == 2 and src.count("operator schedule on the FP64 matrix cores") == 2
     assert "[0] U_e_k = B_k_j X_e_j D_e_k" in src and "[1] Y_e_i = B_k_i U_e_k" in src and "(stored transposed)" in src
-    # small operators stay one fused kernel with the intermediate on chip
-    src = operator_chain_source(TE, 8, 8)
+    # a transient intermediate never leaves the chip: one kernel, handed over through LDS between the two products
+    src = operator_chain_source(TE, 32, 27, 1001)
+    assert src.count("__global__") == 1 and "applied to the first result on chip (handed over through 4224 bytes of LDS per wavefront)" in src
+    assert "mid[(4 * r + g) * 33 + 16 * t + c] = acc[t][r] * T3[0 + en * 32 + 16 * t + c];" in src
+    assert "const double us = mid[c * 33 + 4 * step + g];" in src and "T0[" not in src
+    # small operators whose intermediate is stored stay one kernel of the chain schedule
+    src = operator_chain_source(TE, 8, 8, transient=False)
     assert src.count("__global__") == 1 and "operator schedule" not in src
+    assert "applied to the first result on chip" in operator_chain_source(TE, 8, 8, 1002)
 
 
 def test_every_kind_of_generated_kernel_compiles_for_gfx950(TE, monkeypatch):
