@@ -251,6 +251,26 @@ def other_workload(at, workloads, args):
         label = "A[262144,64] = B[64,64] X[262144,64], one dense operator applied to every vector"
         abytes, flops = (2 * E * n + n * n) * 8, 2 * E * n * n
         units, unit_name = E * n, "GDOF/s"
+    elif name == "dense_apply":
+        # a dense element operator applied, weighted at the quadrature points and applied back: 27 dofs (p=2 hex),
+        # 64 points, both products in one matrix-core kernel, the intermediate transient
+        E, nd, nq = 1 << 19, 27, 64
+        B, X, D, U, Y = at.Tensor(nq, nd), at.Tensor(E, nd), at.Tensor(E, nq), at.Tensor(E, nq), at.Tensor(E, nd)
+        B.data[...] = workloads.counter_uniform(0xAC29, 0, (nq, nd), -1.0, 1.0)
+        X.data[...] = workloads.counter_uniform(0xAC29, 1, (E, nd), -1.0, 1.0)
+        D.data[...] = workloads.counter_uniform(0xAC29, 2, (E, nq), 0.5, 1.5)
+        U.SetTransient(True)
+        for t in (B, X, D, U, Y):
+            t.MoveToGPU()
+
+        def step():
+            engine.BeginMultiKernelLaunch()
+            engine("U_e_k = B_k_j X_e_j D_e_k", U, B, X, D)
+            engine("Y_e_i = B_k_i U_e_k", Y, B, U)
+            engine.EndMultiKernelLaunch()
+        label = "Y[524288,27] = Bt (D o (B X)), B[64,27], D[524288,64]: dense element operator in one launch"
+        abytes, flops = (E * (nd + nq + nd) + nq * nd) * 8, E * (4 * nq * nd + nq)
+        units, unit_name = E * nd, "GDOF/s"
     elif name in ("scatter", "sumgather"):
         # node vector <-> element vector of the headline mesh size: 64^3 hex elements of degree 3
         import numpy as np
@@ -319,7 +339,7 @@ def main():
     ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store-all", action="store_true")
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "scatter_apply", "scatter_then_apply", "operator", "shapes"],
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "scatter_apply", "scatter_then_apply", "operator", "dense_apply", "shapes"],
                     help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
                          "remaining baseline configurations at their full sizes and for the node-vector <-> "
                          "element-vector steps either side of the operator apply")
