@@ -3090,6 +3090,64 @@ class Generator
     // Taking the entries' vectors into registers first and handing them round with readlane was slower (216 us).
     static constexpr int kOperatorEntriesPerLane = 4;
 
+    // The kernels that the operator schedules see: the group's kernels, with pointwise kernels folded into the operator
+    // kernel whose transient result they rescale ("U = B X" followed by "V = U D" reads as "V = B X D").
+    mutable std::vector<Sub> opKernels;
+    mutable bool opKernelsReady = false;
+
+    void FoldPointwiseKernels() const
+    {
+        if (opKernelsReady) return;
+        opKernelsReady = true;
+        opKernels.clear();
+        for (size_t k = 0; k < subs.size(); ++k)
+        {
+            const Sub &p = subs[k];
+            bool folded = false;
+            if (!opKernels.empty() && p.contr.empty() && p.op == '=' && p.matrixOp == 0 && !p.out.repeated && envInt("ACRO_HIP_OPERATOR_FOLD") >= 0)
+            {
+                Sub &m = opKernels.back();
+                const int u = m.out.uvar;
+                int reads = 0;
+                bool sameShape = true;
+                for (const auto &v : p.in)
+                {
+                    if (uvars[v.uvar].storage != uvars[u].storage) continue;
+                    ++reads;
+                    sameShape = sameShape && v.uvar == u && v.idx == m.out.idx && !v.repeated;
+                }
+                bool readLater = false;
+                for (size_t j = k + 1; j < subs.size(); ++j)
+                {
+                    for (const auto &v : subs[j].in) readLater = readLater || uvars[v.uvar].storage == uvars[u].storage;
+                    readLater = readLater || uvars[subs[j].out.uvar].storage == uvars[u].storage;
+                }
+                if (reads == 1 && sameShape && !readLater && m.op == '=' && !m.contr.empty() && p.out.idx == m.out.idx &&
+                    stores[uvars[u].storage].transient && uvars[p.out.uvar].storage != uvars[u].storage)
+                {
+                    for (const auto &v : p.in)
+                    {
+                        if (v.uvar != u) m.in.push_back(v);
+                    }
+                    m.out = p.out;
+                    m.text += " ; " + p.text;
+                    folded = true;
+                }
+            }
+            if (!folded) opKernels.push_back(p);
+        }
+    }
+    int NumOpKernels() const
+    {
+        FoldPointwiseKernels();
+        return static_cast<int>(opKernels.size());
+    }
+    const Sub &OpKernel(int k) const
+    {
+        FoldPointwiseKernels();
+        return opKernels[k];
+    }
+
     struct OperatorShape
     {
         const VarRef *op = nullptr, *x = nullptr;
@@ -3107,8 +3165,8 @@ class Generator
     // `k`: the kernel of the group; `alone`: it is the whole group (inputs are then never written in the launch).
     bool OperatorPattern(OperatorShape &o, int k = 0, bool alone = true) const
     {
-        if ((alone && subs.size() != 1) || batch < 0 || !opt.noalias || NumGatherSlots() > 0 || envInt("ACRO_HIP_OPERATOR") < 0) return false;
-        const Sub &s = subs[k];
+        if ((alone && NumOpKernels() != 1) || batch < 0 || !opt.noalias || NumGatherSlots() > 0 || envInt("ACRO_HIP_OPERATOR") < 0) return false;
+        const Sub &s = OpKernel(k);
         if (s.matrixOp != 0 || s.in.size() < 2 || s.contr.empty() || s.out.repeated) return false;
         // the operator: the one operand without the batch index that carries contracted and free indices;
         // the vectors: the first operand with the batch index that carries every contracted index
@@ -3232,11 +3290,11 @@ class Generator
     // operators stay fused (8 x 8 with a transient intermediate: 156 against 227 us; 12 x 10: 124 against 165 us).
     bool UseOperatorSequence() const
     {
-        if (subs.size() < 2 || envInt("ACRO_HIP_OPERATOR_SEQUENCE") < 0) return false;
-        for (size_t k = 0; k < subs.size(); ++k)
+        if (NumOpKernels() < 2 || envInt("ACRO_HIP_OPERATOR_SEQUENCE") < 0) return false;
+        for (int k = 0; k < NumOpKernels(); ++k)
         {
             OperatorShape o;
-            if (!OperatorPattern(o, static_cast<int>(k), false) || !o.cores || o.rows * o.cols < 512) return false;
+            if (!OperatorPattern(o, k, false) || !o.cores || o.rows * o.cols < 512) return false;
         }
         return true;
     }
@@ -3245,10 +3303,10 @@ class Generator
     // transient and read by nothing else: one kernel, the intermediate handed over through LDS.
     bool OperatorPair(OperatorShape &first, OperatorShape &second) const
     {
-        if (subs.size() != 2 || envInt("ACRO_HIP_OPERATOR_PAIR") < 0) return false;
+        if (NumOpKernels() != 2 || envInt("ACRO_HIP_OPERATOR_PAIR") < 0) return false;
         if (!OperatorPattern(first, 0, false) || !OperatorPattern(second, 1, false)) return false;
         if (!first.cores || !second.cores || first.trailing || second.trailing) return false;
-        const Sub &k0 = subs[0], &k1 = subs[1];
+        const Sub &k0 = OpKernel(0), &k1 = OpKernel(1);
         if (k0.op != '=' || second.x->uvar != k0.out.uvar || second.x->idx != k0.out.idx) return false;
         if (!stores[uvars[k0.out.uvar].storage].transient || uvars[k1.out.uvar].storage == uvars[k0.out.uvar].storage) return false;
         if (!second.perElement.empty() || !second.perColumn.empty()) return false;
@@ -3287,14 +3345,14 @@ class Generator
                 return;
             }
         }
-        if (subs.size() > 1)
+        if (NumOpKernels() > 1)
         {
             opSequence = true;
             std::string schedule;
             int lds = 0;
-            for (size_t k = 0; k < subs.size(); ++k)
+            for (int k = 0; k < NumOpKernels(); ++k)
             {
-                opSub = static_cast<int>(k);
+                opSub = k;
                 OperatorShape shape;
                 OperatorPattern(shape, opSub, false);
                 if (shape.trailing)
@@ -3309,7 +3367,7 @@ class Generator
             plan.module_name = plan.launches.front().function_name;
             return;
         }
-        const Sub &s = subs[0];
+        const Sub &s = OpKernel(0);
         OperatorShape shape;
         OperatorPattern(shape);
         const VarRef *opr = shape.op, *x = shape.x;
@@ -3420,7 +3478,7 @@ class Generator
     // operand layout (entry lane % 16, term group lane / 16) and multiplied by the second operator.
     void EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape &shape, const OperatorShape *next = nullptr, int nextSub = -1)
     {
-        const Sub &s = subs[opSub];
+        const Sub &s = OpKernel(opSub);
         const VarRef &opr = *shape.op, &x = *shape.x;
         const long nI = shape.rows, nJ = shape.cols, E = shape.entries;
         // Sizes that the instruction's 16 x 4 blocks do not divide: the operator's copy in LDS is padded with zero
@@ -3460,7 +3518,7 @@ class Generator
         sched << ", " << E << " entries, 16 per wavefront and trip, "
               << tilesN * steps << " v_mfma_f64_16x16x4 per trip, " << blocks << " workgroups of 256 lanes\n  [" << opSub << "] " << s.text << "\n";
         if (next)
-            sched << "  [" << nextSub << "] " << subs[nextSub].text << " : " << next->rows << " x " << next->cols << (next->transposed ? " operator (stored transposed)" : " operator")
+            sched << "  [" << nextSub << "] " << OpKernel(nextSub).text << " : " << next->rows << " x " << next->cols << (next->transposed ? " operator (stored transposed)" : " operator")
                   << " applied to the first result on chip (handed over through " << 16 * midStride * 8 << " bytes of LDS per wavefront)\n";
         plan.schedule = sched.str();
 
@@ -3629,7 +3687,7 @@ class Generator
             out << "                acc2[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(us, frag2[(t * " << steps2 << " + step) * 64 + lane], acc2[t], 0, 0, 0);\n";
             out << "        }\n";
             out << "        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");\n        __builtin_amdgcn_wave_barrier();\n";
-            emitResults(subs[nextSub], *next, rows2, "acc2", false);
+            emitResults(OpKernel(nextSub), *next, rows2, "acc2", false);
         }
         out << "    }\n}\n";
 
@@ -3654,7 +3712,7 @@ class Generator
     // 16 bytes, which feed two accumulator sets (even and odd entries), and stores its two results together.
     void EmitOperatorEntriesFastest(HipKernelPlan &plan, const OperatorShape &shape)
     {
-        const Sub &s = subs[opSub];
+        const Sub &s = OpKernel(opSub);
         const VarRef &opr = *shape.op, &x = *shape.x;
         const long nI = shape.rows, nJ = shape.cols, E = shape.entries;
         const bool pairs = shape.pairs;

@@ -63,6 +63,7 @@
 //                               in LDS, one entry per lane) instead of the operator schedule
 //   ACRO_HIP_LIGHT=-1           streaming groups whose workgroups move less than 2.5 KB keep their batch size (no extra
 //                               passes to bring a workgroup to 8 KB)
+//   ACRO_HIP_OPERATOR_FOLD=-1   a pointwise kernel that rescales an operator kernel's transient result is not folded into it
 //   ACRO_HIP_OPERATOR_PAIR=-1   two operator-shaped kernels with a transient intermediate are not joined into one matrix-core kernel
 //   ACRO_HIP_OPERATOR_SEQUENCE=-1  groups of several large operator-shaped kernels run as one fused chain kernel instead of one
 //                               matrix-core launch per kernel

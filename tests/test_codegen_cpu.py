@@ -420,6 +420,23 @@ def test_large_dense_operators_in_a_capture_run_as_one_matrix_core_launch_each(T
     assert "applied to the first result on chip" in operator_chain_source(TE, 8, 8, 1002)
 
 
+def test_pointwise_kernel_after_an_operator_kernel_is_folded_into_it(TE):
+    E, nq, nd = 1005, 32, 27
+    B, X, D = at.Tensor(nq, nd), at.Tensor(E, nd), at.Tensor(E, nq)
+    U, V, Y = at.Tensor(E, nq), at.Tensor(E, nq), at.Tensor(E, nd)
+    for transient in (True, False):
+        U.SetTransient(transient)
+        V.SetTransient(True)
+        TE.BeginMultiKernelLaunch()
+        TE("U_e_k = B_k_j X_e_j", U, B, X)
+        TE("V_e_k = U_e_k D_e_k", V, U, D)
+        TE("Y_e_i = B_k_i V_e_k", Y, B, V)
+        src = TE.EndMultiKernelLaunchGetImplementation()
+        # a stored U must reach device memory: nothing is folded then, and the group is an ordinary chain
+        assert ("[0] U_e_k = B_k_j X_e_j ; V_e_k = U_e_k D_e_k" in src) == transient
+        assert ("applied to the first result on chip" in src) == transient
+
+
 def test_every_kind_of_generated_kernel_compiles_for_gfx950(TE, monkeypatch):
     import ctypes
     from acrotensor_amd import _capi

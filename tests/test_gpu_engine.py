@@ -632,6 +632,39 @@ def test_dense_operator_applied_and_applied_back_in_one_capture(at, engine, chec
         assert rel_err(tU.data, U) <= TOL
 
 
+@pytest.mark.parametrize("nq,nd,entries,three", [(32, 27, 1003, True), (64, 27, 700, True), (12, 10, 2001, True), (64, 64, 300, True), (32, 27, 1003, False)])
+def test_pointwise_kernels_between_dense_operators_are_folded_into_them(at, engine, checker, nq, nd, entries, three):
+    """U = B X, V = U o D, Y = Bt V written as three kernels (or the first two alone) with transient intermediates:
+    the pointwise kernel becomes a factor of the operator kernel before it."""
+    rng = np.random.default_rng(nq + nd + entries)
+    B, X, D = rng.uniform(-1, 1, (nq, nd)), rng.uniform(-1, 1, (entries, nd)), rng.uniform(0.5, 1.5, (entries, nq))
+    tB, tX, tD = to_tensor(at, B), to_tensor(at, X), to_tensor(at, D)
+    tU, tV, tY = at.Tensor(entries, nq), at.Tensor(entries, nq), at.Tensor(entries, nd)
+    tU.SetTransient(True)
+    tV.SetTransient(three)
+    print("folded chain", nq, nd, entries, three, flush=True)
+    engine.BeginMultiKernelLaunch()
+    engine("U_e_k = B_k_j X_e_j", tU, tB, tX)
+    engine("V_e_k = D_e_k U_e_k", tV, tD, tU)
+    if three:
+        engine("Y_e_i = B_k_i V_e_k", tY, tB, tV)
+    engine.EndMultiKernelLaunch()
+    src = engine.GetLastImplementation()
+    assert "[0] U_e_k = B_k_j X_e_j ; V_e_k = D_e_k U_e_k" in src
+    V = np.zeros((entries, nq))
+    checker.contract("V_e_k = B_k_j X_e_j D_e_k", V, B, X, D)
+    if three:
+        assert ("applied to the first result on chip" in src) == (nq < 64 or nd < 64)
+        expected = np.zeros((entries, nd))
+        checker.contract("Y_e_i = B_k_i V_e_k", expected, B, V)
+        tY.MoveFromGPU()
+        assert rel_err(tY.data, expected) <= TOL
+    else:
+        assert src.count("__global__") == 1
+        tV.MoveFromGPU()
+        assert rel_err(tV.data, V) <= TOL
+
+
 def test_dense_operator_applied_to_slices(at, engine, checker):
     """The entries' vectors and the results are slices of larger tensors (a slice starts at a whole number of rows,
     so the 16-byte loads of the entries' vectors stay aligned)."""
