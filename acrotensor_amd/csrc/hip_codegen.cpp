@@ -3299,8 +3299,8 @@ class Generator
         return true;
     }
 
-    // Two operator-shaped kernels of which the second is applied to the first one's result, and that result is
-    // transient and read by nothing else: one kernel, the intermediate handed over through LDS.
+    // Two operator-shaped kernels of which the second is applied to the first one's result: one kernel, the
+    // intermediate handed over through LDS (and stored as well unless it is transient).
     bool OperatorPair(OperatorShape &first, OperatorShape &second) const
     {
         if (NumOpKernels() != 2 || envInt("ACRO_HIP_OPERATOR_PAIR") < 0) return false;
@@ -3308,7 +3308,7 @@ class Generator
         if (!first.cores || !second.cores || first.trailing || second.trailing) return false;
         const Sub &k0 = OpKernel(0), &k1 = OpKernel(1);
         if (k0.op != '=' || second.x->uvar != k0.out.uvar || second.x->idx != k0.out.idx) return false;
-        if (!stores[uvars[k0.out.uvar].storage].transient || uvars[k1.out.uvar].storage == uvars[k0.out.uvar].storage) return false;
+        if (uvars[k1.out.uvar].storage == uvars[k0.out.uvar].storage) return false;
         if (!second.perElement.empty() || !second.perColumn.empty()) return false;
         for (const auto &v : k1.in)
         {
@@ -3672,6 +3672,13 @@ class Generator
             out << "        {\n";
             emitResults(s, shape, nI, "acc", true);
             out << "        }\n";
+            if (!stores[uvars[s.out.uvar].storage].transient)
+            {
+                // the first result is wanted in device memory as well
+                out << "        {\n";
+                emitResults(s, shape, nI, "acc", false);
+                out << "        }\n";
+            }
             // a wavefront's LDS accesses complete in program order: no barrier, only the compiler kept from reordering
             out << "        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");\n        __builtin_amdgcn_wave_barrier();\n";
             out << "        acro_double4 acc2[" << rows2P / 16 << "];\n";

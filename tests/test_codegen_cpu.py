@@ -406,7 +406,8 @@ def operator_chain_source(TE, nq, nd, entries=1000, transient=True):
 
 
 def test_large_dense_operators_in_a_capture_run_as_one_matrix_core_launch_each(TE):
-    src = operator_chain_source(TE, 32, 27, transient=False)
+    # two 64 x 64 operators and the hand-over buffer do not fit LDS together
+    src = operator_chain_source(TE, 64, 64, transient=False)
     assert src.count("__global__") == 2 and src.count("operator schedule on the FP64 matrix cores") == 2
     assert "[0] U_e_k = B_k_j X_e_j D_e_k" in src and "[1] Y_e_i = B_k_i U_e_k" in src and "(stored transposed)" in src
     # a transient intermediate never leaves the chip: one kernel, handed over through LDS between the two products
@@ -414,9 +415,10 @@ def test_large_dense_operators_in_a_capture_run_as_one_matrix_core_launch_each(T
     assert src.count("__global__") == 1 and "applied to the first result on chip (handed over through 4224 bytes of LDS per wavefront)" in src
     assert "mid[(4 * r + g) * 33 + 16 * t + c] = acc[t][r] * T3[0 + en * 32 + 16 * t + c];" in src
     assert "const double us = mid[c * 33 + 4 * step + g];" in src and "T0[" not in src
-    # small operators whose intermediate is stored stay one kernel of the chain schedule
-    src = operator_chain_source(TE, 8, 8, transient=False)
-    assert src.count("__global__") == 1 and "operator schedule" not in src
+    # an intermediate that is not transient is stored as well as handed over
+    src = operator_chain_source(TE, 32, 27, 1003, transient=False)
+    assert src.count("__global__") == 1 and "mid[(4 * r + g) * 33 + 16 * t + c] = " in src
+    assert "__builtin_nontemporal_store(acc[t][r] * T3[0 + en * 32 + 16 * t + c], a + 4 * r * 32 + 16 * t);" in src
     assert "applied to the first result on chip" in operator_chain_source(TE, 8, 8, 1002)
 
 

@@ -599,9 +599,9 @@ def test_dense_operator_with_the_entries_as_the_fastest_dimension(at, engine, ch
                                                      (30, 27, 1024, True), (27, 64, 700, True), (64, 27, 5000, True), (33, 17, 999, True),
                                                      (8, 8, 1000, False), (12, 10, 3001, True), (16, 16, 4096, True)])
 def test_dense_operator_applied_and_applied_back_in_one_capture(at, engine, checker, nq, nd, entries, transient):
-    """Y = Bt (D o (B X)) recorded as two kernels.  With a transient intermediate both products run in one matrix-core
-    kernel (the intermediate handed over through LDS); otherwise large operators run as one matrix-core launch per
-    kernel and small ones as one kernel of the chain schedule."""
+    """Y = Bt (D o (B X)) recorded as two kernels.  Both products run in one matrix-core kernel, the intermediate
+    handed over through LDS (and stored unless it is transient); operators too large for that run as one
+    matrix-core launch per kernel."""
     rng = np.random.default_rng(nq * nd + entries)
     B, X, D = rng.uniform(-1, 1, (nq, nd)), rng.uniform(-1, 1, (entries, nd)), rng.uniform(0.5, 1.5, (entries, nq))
     Y0 = rng.uniform(-1, 1, (entries, nd))
@@ -615,7 +615,7 @@ def test_dense_operator_applied_and_applied_back_in_one_capture(at, engine, chec
     src = engine.GetLastImplementation()
     cols = -(-nd // 8) * 8 if nd % 2 == 0 else -(-nd // 4) * 4
     fits = (-(-nq // 16) * 16 * cols + -(-nd // 16) * 16 * -(-nq // 4) * 4 + 64 * (nq + 1)) * 8 <= 65536
-    if transient and fits:
+    if fits:
         assert src.count("__global__") == 1 and "applied to the first result on chip" in src
     elif nq * nd >= 512:
         assert src.count("operator schedule on the FP64 matrix cores") == 2
