@@ -330,6 +330,7 @@ def generated_sources(TE):
     yield "operator schedule, entries fastest, one per lane", TE.GetImplementation("A_i_e = B_j_i X_j_e F_i_e", at.Tensor(64, 1001), at.Tensor(64, 64), at.Tensor(64, 1001), at.Tensor(64, 1001))
     yield "operator schedule, two launches", operator_chain_source(TE, 32, 27, 999, False)
     yield "operator schedule, two operators in one kernel", operator_chain_source(TE, 30, 27, 998)
+    yield "operator schedule, two operators in one kernel, 64 000 bytes of LDS", operator_chain_source(TE, 64, 27, 997, False)
     yield "operator schedule with pointwise factors, odd length", TE.GetImplementation("A_e_i = B_i_j X_e_j D_e_j C_j W_e", at.Tensor(1000, 20), at.Tensor(20, 17),
                                                                                      at.Tensor(1000, 17), at.Tensor(1000, 17), at.Tensor(17), at.Tensor(1000))
     yield "operator schedule", TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(77, 5, 6), at.Tensor(77, 4, 7), at.Tensor(5, 6, 4, 7))
