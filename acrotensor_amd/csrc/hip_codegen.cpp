@@ -3309,7 +3309,6 @@ class Generator
         const Sub &k0 = OpKernel(0), &k1 = OpKernel(1);
         if (k0.op != '=' || second.x->uvar != k0.out.uvar || second.x->idx != k0.out.idx) return false;
         if (uvars[k1.out.uvar].storage == uvars[k0.out.uvar].storage) return false;
-        if (!second.perElement.empty() || !second.perColumn.empty()) return false;
         for (const auto &v : k1.in)
         {
             if (&v != second.x && uvars[v.uvar].storage == uvars[k0.out.uvar].storage) return false;
@@ -3688,7 +3687,15 @@ class Generator
             out << "        for (int step = 0; step < " << steps2 << "; ++step)\n        {\n";
             out << "            const double us = ";
             if (steps2 * 4 != nI) out << "4 * step + g >= " << nI << " ? 0.0 : ";
-            out << "mid[c * " << midStride << " + 4 * step + g];\n";
+            out << "mid[c * " << midStride << " + 4 * step + g]";
+            // the second kernel's factors on its operand side: per element of the intermediate, or per column
+            const std::string inRange = steps2 * 4 != nI ? "(4 * step + g < " + str(nI) + " ? " : "";
+            const std::string otherwise = steps2 * 4 != nI ? " : 0.0)" : "";
+            for (const VarRef *w : next->perElement)
+                out << " * " << inRange << PtrName(w->uvar) << "[" << Lit(uvars[w->uvar].viewOffset) << " + ex * " << nI << " + 4 * step + g]" << otherwise;
+            for (const VarRef *w : next->perColumn)
+                out << " * " << inRange << PtrName(w->uvar) << "[" << Lit(uvars[w->uvar].viewOffset) << " + 4 * step + g]" << otherwise;
+            out << ";\n";
             out << "#pragma unroll\n";
             out << "            for (int t = 0; t < " << rows2P / 16 << "; ++t)\n";
             out << "                acc2[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(us, frag2[(t * " << steps2 << " + step) * 64 + lane], acc2[t], 0, 0, 0);\n";

@@ -665,6 +665,32 @@ def test_pointwise_kernels_between_dense_operators_are_folded_into_them(at, engi
         assert rel_err(tV.data, V) <= TOL
 
 
+@pytest.mark.parametrize("nq,nd,entries", [(30, 27, 1003), (64, 27, 512), (12, 10, 2001)])
+def test_second_operator_with_factors_on_the_intermediate(at, engine, checker, nq, nd, entries):
+    """U = B X, then Y = Bt (U o D o C) with the weights written into the second kernel: they are applied as the
+    intermediate is read back from LDS."""
+    rng = np.random.default_rng(nq * nd + entries)
+    B, X = rng.uniform(-1, 1, (nq, nd)), rng.uniform(-1, 1, (entries, nd))
+    D, C, W = rng.uniform(0.5, 1.5, (entries, nq)), rng.uniform(0.5, 1.5, nq), rng.uniform(0.5, 1.5, entries)
+    Y0 = rng.uniform(-1, 1, (entries, nd))
+    tB, tX, tD, tC, tW, tY = (to_tensor(at, a) for a in (B, X, D, C, W, Y0))
+    tU = at.Tensor(entries, nq)
+    tU.SetTransient(True)
+    print("operator pair with factors", nq, nd, entries, flush=True)
+    engine.BeginMultiKernelLaunch()
+    engine("U_e_k = B_k_j X_e_j", tU, tB, tX)
+    engine("Y_e_i -= B_k_i U_e_k D_e_k C_k W_e", tY, tB, tU, tD, tC, tW)
+    engine.EndMultiKernelLaunch()
+    assert "applied to the first result on chip" in engine.GetLastImplementation()
+    U = np.zeros((entries, nq))
+    checker.contract("U_e_k = B_k_j X_e_j", U, B, X)
+    expected = Y0.copy()
+    checker.contract("Y_e_i -= B_k_i U_e_k D_e_k C_k W_e", expected, B, U, D, C, W)
+    expected = 2.0 * Y0 - expected
+    tY.MoveFromGPU()
+    assert rel_err(tY.data, expected) <= TOL
+
+
 def test_dense_operator_applied_to_slices(at, engine, checker):
     """The entries' vectors and the results are slices of larger tensors (a slice starts at a whole number of rows,
     so the 16-byte loads of the entries' vectors stay aligned)."""
