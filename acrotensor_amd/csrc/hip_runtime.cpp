@@ -71,8 +71,29 @@ void *Stream()
 void SetStream(void *hip_stream)
 {
     notWhileCapturing("Changing the stream");
+    hipStream_t incoming = static_cast<hipStream_t>(hip_stream);
+    hipStream_t outgoing = static_cast<hipStream_t>(Stream());
+    if (incoming == nullptr)
+    {
+        // back to the library's own stream, created here if it never was
+        std::lock_guard<std::mutex> guard(g_lock);
+        if (g_own_stream == nullptr) ACRO_HIP_CHECK(hipStreamCreateWithFlags(&g_own_stream, hipStreamNonBlocking));
+        incoming = g_own_stream;
+    }
+    if (incoming != outgoing)
+    {
+        // Everything already queued on the outgoing stream (kernels, fills, a launched recorded sequence) is made
+        // to precede whatever is queued on the incoming stream from now on: tensors written before the switch may
+        // be read right after it.  The host does not wait.
+        hipEvent_t handover = nullptr;
+        ACRO_HIP_CHECK(hipEventCreateWithFlags(&handover, hipEventDisableTiming));
+        hipError_t err = hipEventRecord(handover, outgoing);
+        if (err == hipSuccess) err = hipStreamWaitEvent(incoming, handover, 0);
+        (void)hipEventDestroy(handover);  // released by the runtime once the event has completed
+        ACRO_HIP_CHECK(err);
+    }
     std::lock_guard<std::mutex> guard(g_lock);
-    g_adopted_stream = static_cast<hipStream_t>(hip_stream);
+    g_adopted_stream = (incoming == g_own_stream) ? nullptr : incoming;
 }
 
 void Synchronize()
