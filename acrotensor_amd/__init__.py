@@ -7,7 +7,8 @@ operations); every call goes through ``libacrotensor_hip.so``.  Errors that the 
 ``AcroError``.  There is no host compute path in this package.
 """
 from .api import (AcroError, IndexMapping, SliceTensor, Tensor, TensorEngine, describe_kernels, hip_event_timer,
-                  is_hip_ready, recorded_launches, set_pinned_host_allocation, synchronize)
+                  get_stream, is_hip_ready, recorded_launches, set_pinned_host_allocation, set_stream, synchronize)
 
 __all__ = ["AcroError", "IndexMapping", "SliceTensor", "Tensor", "TensorEngine", "describe_kernels",
-           "hip_event_timer", "is_hip_ready", "recorded_launches", "set_pinned_host_allocation", "synchronize"]
+           "get_stream", "hip_event_timer", "is_hip_ready", "recorded_launches", "set_pinned_host_allocation", "set_stream",
+           "synchronize"]

@@ -25,6 +25,16 @@ def is_hip_ready():
     return bool(_capi.load().acro_hip_is_ready())
 
 
+def set_stream(hip_stream):
+    """Adopt a caller's ``hipStream_t`` (an integer address or ``ctypes.c_void_p``); ``None`` hands it back and
+    returns to the library's own stream."""
+    _check(_capi.load().acro_hip_set_stream(hip_stream))
+
+
+def get_stream():
+    return _capi.load().acro_hip_get_stream()
+
+
 def synchronize():
     _check(_capi.load().acro_hip_synchronize())
 
