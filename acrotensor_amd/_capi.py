@@ -64,6 +64,7 @@ SIGNATURES = {
     "acro_engine_destroy": (ctypes.c_int, [handle]),
     "acro_engine_set_executor_type": (ctypes.c_int, [handle, ctypes.c_char_p]),
     "acro_engine_contract": (ctypes.c_int, [handle, ctypes.c_char_p, handle, handle_p, ctypes.c_int]),
+    "acro_engine_contract_no_alloc": (ctypes.c_int, [handle, ctypes.c_char_p, handle, handle_p, ctypes.c_int]),
     "acro_engine_begin_multi_kernel_launch": (ctypes.c_int, [handle]),
     "acro_engine_end_multi_kernel_launch": (ctypes.c_int, [handle]),
     "acro_engine_get_implementation": (ctypes.c_int, [handle, ctypes.c_char_p, handle, handle_p, ctypes.c_int,

@@ -216,6 +216,12 @@ class TensorEngine:
         arr, n = self._handles(inputs)
         _check(self._lib.acro_engine_contract(self._h, kernel.encode(), out._h, arr, n))
 
+    def contract_no_alloc(self, kernel, out, *inputs):
+        """The same as calling the engine, for callers that cannot allocate: tensors must be resident on the device
+        and the kernel must have run once through the ordinary call; scratch memory comes from a fixed array."""
+        arr, n = self._handles(inputs)
+        _check(self._lib.acro_engine_contract_no_alloc(self._h, kernel.encode(), out._h, arr, n))
+
     def GetImplementation(self, kernel, out, *inputs):
         arr, n = self._handles(inputs)
         return _fetch_string(lambda buf, size, needed: self._lib.acro_engine_get_implementation(

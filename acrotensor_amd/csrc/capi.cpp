@@ -3,7 +3,9 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <map>
 #include <memory>
+#include <mutex>
 #include <sstream>
 
 #include "AcroTensor.hpp"
@@ -391,6 +393,53 @@ int acro_engine_contract(acro_engine *e, const char *kernel, acro_tensor *out, a
     return guarded([&] {
         require(e != nullptr && kernel != nullptr && out != nullptr, "null argument");
         std::vector<Tensor *> in = unwrap(inputs, num_inputs);
+        e->te(std::string(kernel), out->t, in);
+    });
+}
+
+}  // extern "C"
+
+// ---- the one entry point that allocates nothing ----
+// Scratch memory of acro_engine_contract_no_alloc: the kernels of a split contraction keep their per-workgroup partial
+// sums (and an arrival counter) in device memory beyond their operands.  The ordinary entry point allocates such a
+// buffer per kernel; this array takes its place.  Every device the library runs on holds its own copy, at its own
+// address, until the process ends.
+#define ACRO_NO_ALLOC_SCRATCH_DOUBLES (ACRO_NO_ALLOC_SCRATCH_BYTES / sizeof(double))
+static __device__ __align__(256) double scratch[ACRO_NO_ALLOC_SCRATCH_DOUBLES];
+
+namespace
+{
+// Device address of `scratch` on the current device, looked up once per device.  The array's name means nothing as
+// a pointer in host code; only this address is ever handed to kernels and fills.
+double *scratchOnCurrentDevice()
+{
+    static std::mutex lock;
+    static std::map<int, double *> known;
+    int device = 0;
+    ACRO_HIP_CHECK(hipGetDevice(&device));
+    std::lock_guard<std::mutex> guard(lock);
+    auto it = known.find(device);
+    if (it == known.end())
+    {
+        void *address = nullptr;
+        ACRO_HIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+        require(address != nullptr, "the scratch array has no address on this device");
+        it = known.emplace(device, static_cast<double *>(address)).first;
+    }
+    return it->second;
+}
+}  // namespace
+
+extern "C" {
+
+int acro_engine_contract_no_alloc(acro_engine *e, const char *kernel, acro_tensor *out, acro_tensor *const *inputs,
+                                  int num_inputs)
+{
+    return guarded([&] {
+        require(e != nullptr && kernel != nullptr && out != nullptr, "null argument");
+        std::vector<Tensor *> in = unwrap(inputs, num_inputs);
+        double *ptr = scratchOnCurrentDevice();
+        hip::NoAllocation scope(ptr, ACRO_NO_ALLOC_SCRATCH_DOUBLES);
         e->te(std::string(kernel), out->t, in);
     });
 }

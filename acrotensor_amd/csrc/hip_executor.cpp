@@ -284,10 +284,22 @@ class HipExecutor : public KernelExecutor
             ACROBATIC_ASSERT(ptr[i] != nullptr, "Tensor has no device memory.");
             ptr[i] -= v.plan.param_offset[i];
         }
-        if (v.plan.scratch_doubles > 0 && v.scratch == nullptr)
+        double *scratch = nullptr;
+        if (v.plan.scratch_doubles > 0 && hip::NoAllocation::Active())
         {
-            v.scratch = static_cast<double *>(hip::Malloc(v.plan.scratch_doubles * sizeof(double)));
-            hip::FillDouble(v.scratch, 0.0, v.plan.scratch_doubles);  // on the stream, ahead of the first launch
+            // The caller's buffer is shared by every operation that runs this way and holds what the last one left
+            // there: the part this plan uses starts at zero every time, as a buffer of its own does the first time.
+            scratch = hip::NoAllocation::Scratch(v.plan.scratch_doubles);
+            hip::FillDouble(scratch, 0.0, v.plan.scratch_doubles);
+        }
+        else if (v.plan.scratch_doubles > 0)
+        {
+            if (v.scratch == nullptr)
+            {
+                v.scratch = static_cast<double *>(hip::Malloc(v.plan.scratch_doubles * sizeof(double)));
+                hip::FillDouble(v.scratch, 0.0, v.plan.scratch_doubles);  // on the stream, ahead of the first launch
+            }
+            scratch = v.scratch;
         }
         for (const auto &z : v.plan.zero_fills)
         {
@@ -302,7 +314,7 @@ class HipExecutor : public KernelExecutor
                 if (code >= 0)
                     args[i] = static_cast<void *>(&ptr[code]);
                 else if (code == -1)
-                    args[i] = static_cast<void *>(&v.scratch);
+                    args[i] = static_cast<void *>(&scratch);
                 else if ((-code - 2) % 2 == 0)
                     args[i] = static_cast<void *>(&gatherMap[(-code - 2) / 2]);
                 else

@@ -157,6 +157,10 @@ void HipKernel::Compile()
 void HipKernel::EnsureLoaded()
 {
     if (Module != nullptr) return;
+    // loading a code object allocates device memory for it
+    ACROBATIC_ASSERT(!hip::NoAllocation::Active(),
+                     "Kernel " + FunctionName + " is not loaded on the device yet, and a call that must not allocate "
+                     "cannot load it: run the same operation once through the ordinary entry point before.");
     hipModule_t module;
     hipError_t err = hipModuleLoadData(&module, CodeObject.data());
     if (err != hipSuccess && CacheHit)

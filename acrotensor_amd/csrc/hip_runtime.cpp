@@ -43,6 +43,17 @@ bool g_have_info = false;
 DeviceInfo g_info;
 bool g_capturing = false;
 
+thread_local double *t_no_alloc_scratch = nullptr;
+thread_local size_t t_no_alloc_doubles = 0;
+thread_local bool t_no_alloc = false;
+
+void notWithoutAllocation(const char *what)
+{
+    ACROBATIC_ASSERT(!t_no_alloc, std::string(what) +
+                                      " is not possible in a call that must not allocate: make the tensors resident "
+                                      "and run the same operation once through the ordinary entry point before.");
+}
+
 void notWhileCapturing(const char *what)
 {
     ACROBATIC_ASSERT(!g_capturing, std::string(what) +
@@ -104,6 +115,7 @@ void Synchronize()
 
 void *Malloc(size_t bytes)
 {
+    notWithoutAllocation("Allocating device memory");
     notWhileCapturing("Allocating device memory");
     void *p = nullptr;
     ACRO_HIP_CHECK(hipMalloc(&p, bytes));
@@ -121,6 +133,7 @@ void Free(void *dptr)
 
 void *HostMalloc(size_t bytes)
 {
+    notWithoutAllocation("Allocating page-locked host memory");
     void *p = nullptr;
     ACRO_HIP_CHECK(hipHostMalloc(&p, bytes, hipHostMallocDefault));
     return p;
@@ -131,6 +144,36 @@ void HostFree(void *hptr)
     if (hptr == nullptr) return;
     if (!g_capturing) ACRO_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(Stream())));
     ACRO_HIP_CHECK(hipHostFree(hptr));
+}
+
+NoAllocation::NoAllocation(double *scratch, size_t doubles)
+{
+    ACROBATIC_ASSERT(!t_no_alloc, "Calls that must not allocate do not nest.");
+    t_no_alloc = true;
+    t_no_alloc_scratch = scratch;
+    t_no_alloc_doubles = doubles;
+}
+
+NoAllocation::~NoAllocation()
+{
+    t_no_alloc = false;
+    t_no_alloc_scratch = nullptr;
+    t_no_alloc_doubles = 0;
+}
+
+bool NoAllocation::Active()
+{
+    return t_no_alloc;
+}
+
+double *NoAllocation::Scratch(size_t doubles)
+{
+    ACROBATIC_ASSERT(t_no_alloc, "Internal error: no provided scratch buffer outside a call that must not allocate.");
+    ACROBATIC_ASSERT(doubles <= t_no_alloc_doubles,
+                     "This operation needs " + std::to_string(doubles * sizeof(double)) +
+                         " bytes of scratch memory; a call that must not allocate has " +
+                         std::to_string(t_no_alloc_doubles * sizeof(double)) + " bytes.  Use the ordinary entry point.");
+    return t_no_alloc_scratch;
 }
 
 void CopyToDevice(void *dst, const void *src, size_t bytes)

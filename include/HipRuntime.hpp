@@ -50,6 +50,23 @@ bool Capturing();
 void Launch(Graph *graph);     // asynchronous, in stream order with everything else on Stream()
 void Destroy(Graph *graph);
 
+// Calls that must not allocate.  While a NoAllocation object lives on a thread, that thread's calls into the
+// library allocate no device or page-locked memory and load no code object: Malloc, HostMalloc and the first launch
+// of a kernel that is not loaded yet throw (Free only ever runs from destructors and is not reached), and launches
+// that need a scratch buffer take `doubles` entries at `scratch` (device memory the caller of this layer provides;
+// larger requests throw) instead of a buffer of their own.
+class NoAllocation
+{
+  public:
+    NoAllocation(double *scratch, size_t doubles);
+    ~NoAllocation();
+    NoAllocation(const NoAllocation &) = delete;
+    NoAllocation &operator=(const NoAllocation &) = delete;
+    static bool Active();
+    // The provided scratch buffer, after checking that `doubles` entries fit.  Only while Active().
+    static double *Scratch(size_t doubles);
+};
+
 // Multiprocessor count, LDS bytes per workgroup, wavefront size of the current device (cached).
 struct DeviceInfo
 {

@@ -104,6 +104,20 @@ int acro_engine_set_executor_type(acro_engine *e, const char *exec_type);
 /* TensorEngine::operator()(kernel_str, out, inputs)  (kernel/TensorEngine.cpp:290-315) */
 int acro_engine_contract(acro_engine *e, const char *kernel, acro_tensor *out, acro_tensor *const *inputs,
                          int num_inputs);
+/* The same operation as acro_engine_contract for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc); no counterpart in the reference, whose launches never allocate
+ * because its kernels have no scratch memory (exec/CudaExecutor.cpp:70-101).  This call allocates no device or
+ * page-locked memory and loads no code object: every tensor must already be resident on the device, and the same
+ * kernel string on tensors of the same extents must have run once through acro_engine_contract (which compiles and
+ * loads the kernel); otherwise the call fails with a message saying so.  Kernels that need scratch memory beyond
+ * their operands (split contractions such as "S_i_j = A_n_i_j B_n": per-workgroup partial sums) take it from one
+ * array of ACRO_NO_ALLOC_SCRATCH_BYTES that the library holds on every device it runs on until the process ends; a
+ * kernel that needs more is refused with a message.  All calls on a device share that array, which keeps the last
+ * call's contents (the part a call uses is cleared first, on the stream): calls that overlap on one device, from
+ * several threads or on several streams, race.  Results are bit-identical to acro_engine_contract's. */
+#define ACRO_NO_ALLOC_SCRATCH_BYTES (256u * 1024u)
+int acro_engine_contract_no_alloc(acro_engine *e, const char *kernel, acro_tensor *out, acro_tensor *const *inputs,
+                                  int num_inputs);
 /* Between begin and end, acro_engine_batch_matrix_inverse / _det / _inv_det are recorded as well and run at end, in
  * program order with the recorded kernels; an operation whose result a later recorded kernel reads is fused into the
  * launch (the reference runs these operations at the call, kernel/TensorEngine.cpp:627-671).  The same for
