@@ -45,9 +45,10 @@ def set_pinned_host_allocation(flag=True):
 
 
 class Tensor:
-    """Dense row-major fp64 tensor: ``Tensor(d0, d1, ...)``.  ``.data`` is a numpy view of the host buffer."""
+    """Dense row-major fp64 tensor: ``Tensor(d0, d1, ...)``.  ``.data`` is a numpy view of the host buffer.
+    ``hdata`` wraps a caller's numpy array, ``ddata`` / ``ongpu`` additionally a caller's device buffer."""
 
-    def __init__(self, *dims, hdata=None, _handle=None, _keep=None):
+    def __init__(self, *dims, hdata=None, ddata=None, ongpu=False, _handle=None, _keep=None):
         self._lib = _capi.load()
         self._keep = _keep            # objects that must outlive this tensor (external buffer, slice parent)
         self._h = ctypes.c_void_p()
@@ -63,9 +64,12 @@ class Tensor:
                     raise AcroError("hdata must be a C-contiguous float64 numpy array")
                 self._keep = hdata
                 hptr = hdata.ctypes.data_as(ctypes.c_void_p)
-            _check(self._lib.acro_tensor_create(n, arr, hptr, None, 0, ctypes.byref(self._h)))
+            # ddata: address of an existing device buffer of the caller (with hdata only), ongpu: it holds the
+            # current data (the reference's Tensor(dims, hdata, ddata, ongpu), tensor/Tensor.cpp:166-202)
+            dptr = ctypes.c_void_p(int(ddata)) if ddata else None
+            _check(self._lib.acro_tensor_create(n, arr, hptr, dptr, 1 if ongpu else 0, ctypes.byref(self._h)))
         else:
-            raise AcroError("Cant initilize tensor without any dimensions.")
+            raise AcroError("A tensor needs at least one dimension.")
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None

@@ -376,6 +376,22 @@ void TensorEngine::FinishCapture(std::string *implementation)
         for (; next_op < ops.size() && ops[next_op].position == k; ++next_op)
         {
             const RecordedMatrixOp &op = ops[next_op];
+            if (op.sum_gather)
+            {
+                // never part of a fused launch (its rows cross workgroups): runs on its own, at its place
+                keepAll();
+                flush();
+                if (implementation != nullptr)
+                {
+                    *implementation += "// sum-gather: runs on its own\n";
+                    continue;
+                }
+                SwitchToComputeLocation(*op.scatter_out);
+                MoveToComputeLocation(*op.scatter_in);
+                MoveToComputeLocation(*op.map);
+                Ops->FlatIndexedSumGather(*op.scatter_out, *op.scatter_in, *op.map);
+                continue;
+            }
             if (op.scatter_out != nullptr)
             {
                 if (readThroughMap(op))
@@ -590,6 +606,15 @@ void TensorEngine::FlatIndexedSumGather(Tensor &Aout, Tensor &Ain, IndexMapping 
     ACROBATIC_ASSERT(Aout.GetSize() == static_cast<size_t>(M.GetDomainSize()), "IndexMapping DomainSize does not match the output Tensor size.");
     ACROBATIC_ASSERT(Ain.GetSize() == static_cast<size_t>(M.GetRangeSize()), "IndexMapping RangeSize does not match the input Tensor size.");
     if (!M.IsInverseComputed()) M.ComputeInverse();
+    if (IsMultiKernelLaunch && ExecutorType == "HIP")
+    {
+        // Like every other operation of a capture it takes effect at End, at its place among the recorded kernels
+        // (run at once, it would gather an operand that the kernels recorded before it have not produced yet).
+        RecordedMatrixOp op{MKLKernels.size(), nullptr, nullptr, nullptr, &Aout, &Ain, &M};
+        op.sum_gather = true;
+        MKLMatrixOps.push_back(op);
+        return;
+    }
     SwitchToComputeLocation(Aout);
     MoveToComputeLocation(Ain);
     MoveToComputeLocation(M);

@@ -3532,6 +3532,10 @@ class Generator
         // term group g (lane / 16) of step s stands for this j
         const std::string termOf = pairs ? "8 * (step >> 1) + 2 * (l >> 4) + (step & 1)" : "4 * step + (l >> 4)";
         out << (opSub == 0 ? "" : "\n") << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
+        // Two doubles moved by one 16-byte instruction.  The type only promises the 8-byte alignment that every
+        // operand has (a caller's device buffer, a slice at an odd offset of it); the hardware takes such
+        // addresses for accesses to device memory.
+        out << "typedef double acro_pair __attribute__((ext_vector_type(2), aligned(8)));\n";
         out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << plan.module_name << "(" << ParamList() << ")\n{\n";
         out << "    __shared__ double frag[" << nIp * nJp << "];\n";
         out << "    for (int f = threadIdx.x; f < " << nIp * nJp << "; f += 256)\n    {\n";
@@ -3570,13 +3574,13 @@ class Generator
             out << "#pragma unroll\n";
             out << "        for (int q = 0; q < " << nJp / 8 << "; ++q) xv[q] = ";
             if (nJp != nJ) out << "8 * q + 2 * g >= " << nJ << " ? double2{0.0, 0.0} : ";
-            out << "*reinterpret_cast<const double2 *>(x + 8 * q);\n";
+            out << "[&] { const acro_pair t = *reinterpret_cast<const acro_pair *>(x + 8 * q); return double2{t.x, t.y}; }();\n";
             for (const VarRef *w : shape.perElement)
             {
                 out << "#pragma unroll\n";
                 out << "        for (int q = 0; q < " << nJp / 8 << "; ++q)\n        {\n";
                 if (nJp != nJ) out << "            if (8 * q + 2 * g >= " << nJ << ") continue;\n";
-                out << "            const double2 f = *reinterpret_cast<const double2 *>(" << PtrName(w->uvar) << " + " << Lit(uvars[w->uvar].viewOffset)
+                out << "            const acro_pair f = *reinterpret_cast<const acro_pair *>(" << PtrName(w->uvar) << " + " << Lit(uvars[w->uvar].viewOffset)
                     << " + ex * " << nJ << " + 2 * g + 8 * q);\n            xv[q].x *= f.x;\n            xv[q].y *= f.y;\n        }\n";
             }
             for (const VarRef *w : shape.perColumn)
@@ -3766,7 +3770,8 @@ class Generator
         const std::string vt = pairs ? "acro_double2" : "double";
         auto offsetOf = [&](const VarRef &v) { return Lit(uvars[v.uvar].viewOffset); };
         out << (opSub == 0 ? "" : "\n") << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
-        out << "typedef double acro_double2 __attribute__((ext_vector_type(2)));\n";
+        // only the 8-byte alignment that every operand has is promised (see acro_pair in the other operator kernel)
+        out << "typedef double acro_double2 __attribute__((ext_vector_type(2), aligned(8)));\n";
         out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << plan.module_name << "(" << ParamList() << ")\n{\n";
         out << "    __shared__ double frag[" << nIp * nJp << "];\n";
         out << "    for (int f = threadIdx.x; f < " << nIp * nJp << "; f += 256)\n    {\n";

@@ -111,8 +111,8 @@ class HipExecutor : public KernelExecutor
     // reference's exec/CudaExecutor.cpp:83-99; when one name is bound to two different tensors a group falls back
     // to one launch per kernel and a single kernel switches to one operand per occurrence.  Also the aliasing
     // analysis: two different operands that overlap in memory, one of them written, forbid restrict / scalar
-    // reads (single kernel) or fusion (group).  Host buffers mirror device buffers one to one, so the analysis
-    // works before anything is mapped to the device.
+    // reads (single kernel) or fusion (group).  Host buffers mirror library-allocated device buffers one to one, so
+    // the analysis works before anything is mapped to the device; device buffers that exist are compared as well.
     void Bind(std::vector<Tensor *> &outputs, std::vector<std::vector<Tensor *>> &inputs,
               const std::vector<GatheredInput> &gathered, HipCodegenOptions &options, bool &fallback)
     {
@@ -192,7 +192,11 @@ class HipExecutor : public KernelExecutor
             {
                 if (root[a] == root[b]) continue;
                 const double *pa = root[a]->GetData(), *pb = root[b]->GetData();
-                const bool overlap = pa < pb + root[b]->GetSize() && pb < pa + root[a]->GetSize();
+                bool overlap = pa < pb + root[b]->GetSize() && pb < pa + root[a]->GetSize();
+                // device buffers that callers handed in need not mirror the layout of the host buffers
+                const double *da = root[a]->GetDeviceData(), *db = root[b]->GetDeviceData();
+                if (da != nullptr && db != nullptr)
+                    overlap = overlap || (da < db + root[b]->GetSize() && db < da + root[a]->GetSize());
                 if (overlap && (written[a] || written[b])) hazard = true;
             }
         }

@@ -117,7 +117,9 @@ struct SmallMatrix<3>
 // The matrices of a workgroup are contiguous in memory, so the workgroup copies them to and from LDS as one
 // stream of 16-byte pieces (full-rate HBM access), and lane t works on matrix t out of LDS.  For 2x2 the lane
 // stride in LDS is padded from 4 to 5 doubles so that lanes fall into distinct banks; 9 and 1 are odd already.
-template <int M, bool WANT_INV, bool WANT_DET>
+// PAIRS: the matrices start at a multiple of 16 bytes and are read as pairs of doubles; otherwise (a slice at an odd
+// offset, a caller's device buffer) one double at a time.
+template <int M, bool WANT_INV, bool WANT_DET, bool PAIRS>
 __global__ __launch_bounds__(kMatLanes) void batchMatrixKernel(const double *__restrict__ A, double *__restrict__ Ainv,
                                                             double *__restrict__ Adet, size_t num_mat)
 {
@@ -130,11 +132,20 @@ __global__ __launch_bounds__(kMatLanes) void batchMatrixKernel(const double *__r
     const int ndbl = static_cast<int>(count) * MM;
     const double *src = A + first * MM;
 
-    // first * MM * 8 bytes is a multiple of 16 (kMatLanes is even), so pairs of doubles are aligned
+    // first * MM * 8 bytes is a multiple of 16 (kMatLanes is even), so pairs of doubles are aligned when A is
     const double2 *src2 = reinterpret_cast<const double2 *>(src);
     for (int i = threadIdx.x; i < ndbl / 2; i += kMatLanes)
     {
-        const double2 v = src2[i];
+        double2 v;
+        if (PAIRS)
+        {
+            v = src2[i];
+        }
+        else
+        {
+            v.x = src[2 * i];
+            v.y = src[2 * i + 1];
+        }
         if (LS == MM)
         {
             tile[2 * i] = v.x;
@@ -324,23 +335,29 @@ void launchBatchMatrix(int mdim, const double *A, double *Ainv, double *Adet, si
     const size_t groups = (num_mat + kMatLanes - 1) / kMatLanes;
     ACROBATIC_ASSERT(groups <= 0x7fffffffu, "Operand too large for a one-dimensional grid.");
     const unsigned grid = static_cast<unsigned>(groups == 0 ? 1 : groups);
+    const bool pairs = reinterpret_cast<uintptr_t>(A) % 16 == 0;
+#define ACRO_LAUNCH_BATCH_MATRIX(M)                                                                                   \
+    if (pairs)                                                                                                        \
+        hipLaunchKernelGGL((batchMatrixKernel<M, WANT_INV, WANT_DET, true>), dim3(grid), dim3(kMatLanes), 0, stream(), \
+                           A, Ainv, Adet, num_mat);                                                                   \
+    else                                                                                                              \
+        hipLaunchKernelGGL((batchMatrixKernel<M, WANT_INV, WANT_DET, false>), dim3(grid), dim3(kMatLanes), 0,          \
+                           stream(), A, Ainv, Adet, num_mat)
     switch (mdim)
     {
         case 1:
-            hipLaunchKernelGGL((batchMatrixKernel<1, WANT_INV, WANT_DET>), dim3(grid), dim3(kMatLanes), 0, stream(), A,
-                               Ainv, Adet, num_mat);
+            ACRO_LAUNCH_BATCH_MATRIX(1);
             break;
         case 2:
-            hipLaunchKernelGGL((batchMatrixKernel<2, WANT_INV, WANT_DET>), dim3(grid), dim3(kMatLanes), 0, stream(), A,
-                               Ainv, Adet, num_mat);
+            ACRO_LAUNCH_BATCH_MATRIX(2);
             break;
         case 3:
-            hipLaunchKernelGGL((batchMatrixKernel<3, WANT_INV, WANT_DET>), dim3(grid), dim3(kMatLanes), 0, stream(), A,
-                               Ainv, Adet, num_mat);
+            ACRO_LAUNCH_BATCH_MATRIX(3);
             break;
         default:
             ACROBATIC_ASSERT(false, "Batched matrix ops support 1x1, 2x2 and 3x3 matrices only.");
     }
+#undef ACRO_LAUNCH_BATCH_MATRIX
     ACRO_HIP_CHECK(hipGetLastError());
 }
 

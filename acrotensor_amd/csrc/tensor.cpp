@@ -34,8 +34,8 @@ bool Tensor::GetPinnedHostAllocation()
 }
 
 Tensor::Tensor()
-    : Size(0), Initialized(false), OwnsData(false), MappedToGPU(false), OnGPU(false), Transient(false),
-      Data(nullptr), DeviceData(nullptr)
+    : Size(0), Initialized(false), OwnsData(false), OwnsDeviceData(false), MappedToGPU(false), OnGPU(false),
+      Transient(false), Data(nullptr), DeviceData(nullptr)
 {
 }
 
@@ -46,17 +46,17 @@ Tensor::Tensor(const std::vector<int> &dims, double *hdata, double *ddata, bool 
 
 void Tensor::Init(const std::vector<int> &dims, double *hdata, double *ddata, bool ongpu)
 {
-    ACROBATIC_ASSERT(!IsInitialized(), "Can't initilize a tensor a second time.");
-    ACROBATIC_ASSERT(!dims.empty(), "Cant initilize tensor without any dimensions.");
+    ACROBATIC_ASSERT(!IsInitialized(), "A tensor can be initialized only once.");
+    ACROBATIC_ASSERT(!dims.empty(), "A tensor needs at least one dimension.");
     for (int d : dims)
     {
-        ACROBATIC_ASSERT(d > 0, "Can't initilize tensor with non-positive dimensions.");
+        ACROBATIC_ASSERT(d > 0, "Every dimension of a tensor must be positive.");
     }
     // External device memory is only accepted next to external host memory, and only a tensor that has a
     // device pointer can start out flagged as resident on the device (reference tensor/Tensor.cpp:189-200).
-    ACROBATIC_ASSERT(ddata == nullptr || hdata != nullptr, "Acrotensor does not currently support GPU only tensors.");
+    ACROBATIC_ASSERT(ddata == nullptr || hdata != nullptr, "A device buffer can only be supplied together with a host buffer (no device-only tensors).");
     ACROBATIC_ASSERT(ddata != nullptr || !ongpu,
-                     "Acrotensor cannot mark external data as on the GPU if no GPU pointer is provided.");
+                     "External data cannot be flagged as current on the device without a device pointer.");
 
     Dims = dims;
     UpdateStrides();
@@ -69,6 +69,7 @@ void Tensor::Init(const std::vector<int> &dims, double *hdata, double *ddata, bo
     else
         Data = OwnsData ? new double[Size] : hdata;
     DeviceData = ddata;
+    OwnsDeviceData = false;  // a device buffer handed in stays the caller's
     MappedToGPU = (ddata != nullptr);
     OnGPU = ongpu;
     Initialized = true;
@@ -76,8 +77,10 @@ void Tensor::Init(const std::vector<int> &dims, double *hdata, double *ddata, bo
 
 Tensor::~Tensor()
 {
-    if (!OwnsData) return;
-    if (PinnedData)
+    // Host and device buffers are released by whoever allocated them, independently of each other: a tensor over a
+    // caller's host buffer still owns the device mirror that MapToGPU allocated for it (the reference frees the
+    // mirror only together with an owned host buffer, tensor/Tensor.cpp:205-215, and leaks it otherwise).
+    if (OwnsData && PinnedData)
     {
         try
         {
@@ -87,11 +90,11 @@ Tensor::~Tensor()
         {
         }
     }
-    else
+    else if (OwnsData)
     {
         delete[] Data;
     }
-    if (MappedToGPU && DeviceData != nullptr)
+    if (OwnsDeviceData && DeviceData != nullptr)
     {
         try
         {
@@ -147,8 +150,15 @@ void Tensor::Reshape(const std::vector<int> &dims)
 void Tensor::Retarget(double *hdata, double *ddata)
 {
     ACROBATIC_ASSERT(!OwnsData);
+    if (OwnsDeviceData && DeviceData != ddata)
+    {
+        hip::Free(DeviceData);  // the mirror of the buffer that is being left
+        OwnsDeviceData = false;
+    }
     Data = hdata;
     DeviceData = ddata;
+    MappedToGPU = (ddata != nullptr);
+    if (!MappedToGPU) OnGPU = false;
 }
 
 void Tensor::Set(double val)
@@ -174,8 +184,9 @@ void Tensor::Mult(double c)
 
 void Tensor::MapToGPU()
 {
-    ACROBATIC_ASSERT(!IsMappedToGPU(), "Trying to map data to the GPU a second time.");
+    ACROBATIC_ASSERT(!IsMappedToGPU(), "The data already has a device mirror.");
     DeviceData = static_cast<double *>(hip::Malloc(GetByteSize()));
+    OwnsDeviceData = true;
     MappedToGPU = true;
 }
 
@@ -197,8 +208,9 @@ void Tensor::SwitchToGPU()
 
 void Tensor::UnmapFromGPU()
 {
-    ACROBATIC_ASSERT(IsMappedToGPU(), "Can't unmap data that is not mapped to the GPU.");
-    hip::Free(DeviceData);
+    ACROBATIC_ASSERT(IsMappedToGPU(), "There is no device mirror to release.");
+    if (OwnsDeviceData) hip::Free(DeviceData);  // a caller's device buffer is only let go of
+    OwnsDeviceData = false;
     DeviceData = nullptr;
     MappedToGPU = false;
     OnGPU = false;
@@ -234,7 +246,7 @@ void Tensor::Print()
 
 void SliceTensor::SliceInit(Tensor &T, const std::vector<int> &sind)
 {
-    ACROBATIC_ASSERT(T.IsInitialized(), "Can't slice an uninitilized tensor.");
+    ACROBATIC_ASSERT(T.IsInitialized(), "The tensor to slice is not initialized.");
     ACROBATIC_ASSERT(T.GetRank() > static_cast<int>(sind.size()), "Can't slice more dimensions than the tensor rank.");
     ACROBATIC_ASSERT(!sind.empty(), "Can't slice without any leading indices.");
     for (size_t d = 0; d < sind.size(); ++d)
@@ -310,7 +322,8 @@ bool SliceTensor::IsTransient() const
 // ----------------------------------------------------------------------------------------- IndexVector
 
 IndexVector::IndexVector()
-    : Size(0), Initialized(false), OwnsData(false), MappedToGPU(false), OnGPU(false), Data(nullptr), DeviceData(nullptr)
+    : Size(0), Initialized(false), OwnsData(false), OwnsDeviceData(false), MappedToGPU(false), OnGPU(false), Data(nullptr),
+      DeviceData(nullptr)
 {
 }
 
@@ -321,11 +334,11 @@ IndexVector::IndexVector(int dim, int *hdata, int *ddata, bool ongpu) : IndexVec
 
 void IndexVector::Init(int dim, int *hdata, int *ddata, bool ongpu)
 {
-    ACROBATIC_ASSERT(!IsInitialized(), "Can't initilize a vector a second time.");
-    ACROBATIC_ASSERT(dim > 0, "Cant initilize vector without any dimensions.");
-    ACROBATIC_ASSERT(ddata == nullptr || hdata != nullptr, "Acrotensor does not currently support GPU only vectors.");
+    ACROBATIC_ASSERT(!IsInitialized(), "An index vector can be initialized only once.");
+    ACROBATIC_ASSERT(dim > 0, "An index vector needs a positive length.");
+    ACROBATIC_ASSERT(ddata == nullptr || hdata != nullptr, "A device buffer can only be supplied together with a host buffer (no device-only index vectors).");
     ACROBATIC_ASSERT(ddata != nullptr || !ongpu,
-                     "Acrotensor cannot mark external data as on the GPU if no GPU pointer is provided.");
+                     "External data cannot be flagged as current on the device without a device pointer.");
     Size = static_cast<size_t>(dim);
     OwnsData = (hdata == nullptr);
     Data = OwnsData ? new int[Size] : hdata;
@@ -337,9 +350,8 @@ void IndexVector::Init(int dim, int *hdata, int *ddata, bool ongpu)
 
 IndexVector::~IndexVector()
 {
-    if (!OwnsData) return;
-    delete[] Data;
-    if (MappedToGPU && DeviceData != nullptr)
+    if (OwnsData) delete[] Data;
+    if (OwnsDeviceData && DeviceData != nullptr)
     {
         try
         {
@@ -354,14 +366,22 @@ IndexVector::~IndexVector()
 void IndexVector::Retarget(int *hdata, int *ddata)
 {
     ACROBATIC_ASSERT(!OwnsData);
+    if (OwnsDeviceData && DeviceData != ddata)
+    {
+        hip::Free(DeviceData);
+        OwnsDeviceData = false;
+    }
     Data = hdata;
     DeviceData = ddata;
+    MappedToGPU = (ddata != nullptr);
+    if (!MappedToGPU) OnGPU = false;
 }
 
 void IndexVector::MapToGPU()
 {
-    ACROBATIC_ASSERT(!IsMappedToGPU(), "Trying to map data to the GPU a second time.");
+    ACROBATIC_ASSERT(!IsMappedToGPU(), "The data already has a device mirror.");
     DeviceData = static_cast<int *>(hip::Malloc(Size * sizeof(int)));
+    OwnsDeviceData = true;
     MappedToGPU = true;
 }
 
@@ -383,8 +403,9 @@ void IndexVector::SwitchToGPU()
 
 void IndexVector::UnmapFromGPU()
 {
-    ACROBATIC_ASSERT(IsMappedToGPU(), "Can't unmap data that is not mapped to the GPU.");
-    hip::Free(DeviceData);
+    ACROBATIC_ASSERT(IsMappedToGPU(), "There is no device mirror to release.");
+    if (OwnsDeviceData) hip::Free(DeviceData);
+    OwnsDeviceData = false;
     DeviceData = nullptr;
     MappedToGPU = false;
     OnGPU = false;

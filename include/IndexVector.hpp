@@ -43,6 +43,7 @@ class IndexVector
     size_t Size;
     bool Initialized;
     bool OwnsData;
+    bool OwnsDeviceData;  // the device mirror was allocated by MapToGPU (not handed in by the caller)
     bool MappedToGPU;
     bool OnGPU;
     int *Data;

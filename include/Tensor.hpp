@@ -156,6 +156,7 @@ class Tensor
 
     bool Initialized;
     bool OwnsData;
+    bool OwnsDeviceData;  // the device mirror was allocated by MapToGPU (not handed in by the caller)
     bool PinnedData = false;  // the owned host buffer is page-locked
     bool MappedToGPU;
     bool OnGPU;

@@ -88,10 +88,11 @@ class TensorEngine
         Tensor *inverse;      // null for a determinant alone
         Tensor *determinant;  // null for an inverse alone
         Tensor *matrices;
-        // a recorded FlatIndexedScatter instead (the three above are null then)
+        // a recorded FlatIndexedScatter or FlatIndexedSumGather instead (the three above are null then)
         Tensor *scatter_out;
         Tensor *scatter_in;
         IndexMapping *map;
+        bool sum_gather = false;  // scatter_out / scatter_in are the sum-gather's result and operand
     };
     // Executes the capture (or, with `implementation` set, only describes it).
     void FinishCapture(std::string *implementation);

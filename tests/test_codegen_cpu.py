@@ -207,7 +207,7 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
                                at.Tensor(1000), at.Tensor(1000, 12), at.Tensor(10), at.Tensor(1000, 10), at.Tensor(12))
     assert "operator schedule on the FP64 matrix cores: 10 x 12 operator" in src and "const double se = T3[0 + en];" in src
     assert "-= acc[t][r] * se * T6[0 + en * 10 + 16 * t + c] * T5[0 + 16 * t + c];" in src
-    assert "const double2 f = *reinterpret_cast<const double2 *>(T4 + 0 + ex * 12 + 2 * g + 8 * q);" in src and "const double *f = T7 + 0 + 2 * g + 8 * q;" in src
+    assert "const acro_pair f = *reinterpret_cast<const acro_pair *>(T4 + 0 + ex * 12 + 2 * g + 8 * q);" in src and "const double *f = T7 + 0 + 2 * g + 8 * q;" in src
     # the entries as the fastest dimension: the operator becomes the instruction's first operand
     src = TE.GetImplementation("A_i_e -= B_i_j X_j_e W_e", at.Tensor(30, 1002), at.Tensor(30, 27), at.Tensor(27, 1002), at.Tensor(1002))
     assert "matrix cores, entries fastest: 30 x 27 operator in LDS in operand order (padded to 32 x 28), 1002 entries, 32 per wavefront" in src

@@ -707,3 +707,50 @@ def test_dense_operator_applied_to_slices(at, engine, checker):
         expected = np.zeros((entries, 16))
         checker.contract("A_e_i = B_i_j X_e_j", expected, B, np.ascontiguousarray(X[1]))
         assert rel_err(tA.data[1], expected) <= TOL and np.array_equal(tA.data[0], A0[0])
+
+
+@pytest.mark.parametrize("m", [1, 2, 3])
+def test_batched_matrices_at_odd_offsets(at, engine, checker, m):
+    # slices whose first entry is 8 but not 16 bytes into the allocation, and a caller's device buffer likewise
+    E = 5
+    rng = np.random.default_rng(40 + m)
+    J = np.eye(m) + 0.1 * rng.uniform(-1, 1, (3, E, m, m))
+    tJ, tI, tD = to_tensor(at, J), at.Tensor(*J.shape), at.Tensor(3, E)
+    for k in range(3):
+        engine.BatchMatrixInvDet(at.SliceTensor(tI, k), at.SliceTensor(tD, k), at.SliceTensor(tJ, k))
+    tI.MoveFromGPU()
+    tD.MoveFromGPU()
+    ri, rd = checker.batch_matrix_inv_det(J)
+    assert np.array_equal(tI.data, ri) and np.array_equal(tD.data, rd)
+    # a caller's device buffer one double into an allocation
+    pool = at.Tensor(2 * J[0].size + 8)
+    pool.MoveToGPU()
+    host = np.ascontiguousarray(J[1])
+    ext = at.Tensor(*host.shape, hdata=host, ddata=pool.GetDeviceData() + 8, ongpu=False)
+    ext.MoveToGPU()
+    inv, det = at.Tensor(*host.shape), at.Tensor(E)
+    engine.BatchMatrixInvDet(inv, det, ext)
+    inv.MoveFromGPU()
+    det.MoveFromGPU()
+    assert np.array_equal(inv.data, ri[1]) and np.array_equal(det.data, rd[1])
+
+
+def test_operator_kernels_on_buffers_that_are_only_8_byte_aligned(at, engine, checker):
+    # the operator schedule moves the entries' vectors with 16-byte instructions; a caller's device buffer one double
+    # into an allocation must work like any other
+    E, n = 300, 12
+    rng = np.random.default_rng(77)
+    B, X = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (E, n))
+    pool = at.Tensor(2 * X.size + 16)
+    pool.MoveToGPU()
+    base = pool.GetDeviceData()
+    hx, ha = X.copy(), np.zeros((E, n))
+    tX = at.Tensor(E, n, hdata=hx, ddata=base + 8, ongpu=False)
+    tA = at.Tensor(E, n, hdata=ha, ddata=base + 8 * (X.size + 3), ongpu=False)
+    tX.MoveToGPU()
+    engine("A_e_i = B_i_j X_e_j", tA, to_tensor(at, B), tX)
+    assert "matrix cores" in engine.GetLastImplementation()
+    tA.MoveFromGPU()
+    expected = np.zeros((E, n))
+    checker.contract("A_e_i = B_i_j X_e_j", expected, B, X)
+    assert rel_err(ha, expected) <= 1e-12

@@ -165,3 +165,32 @@ def test_apply_through_the_map_replays_from_a_recorded_launch_sequence(at, engin
         tensors["Y"].MoveFromGPU()
         assert np.abs(replayed).max() > 0.0 and np.array_equal(replayed, tensors["Y"].data)
         tensors["Y"].MoveToGPU()
+
+
+def test_sum_gather_recorded_in_a_capture_runs_at_its_place(at, engine, checker):
+    # node vector -> element vector -> mass apply -> node vector in ONE capture: the sum-gather is recorded like the
+    # scatter and the kernels and takes effect after the kernels recorded before it
+    dofs, nodes = workloads.hex_mesh_dof_map(3, 2, 2, 3)
+    E = dofs.shape[0]
+    for transient_x in (False, True):
+        wl = workloads.config4(E=E)
+        tensors = workloads.bind_to_engine(wl, at, transient=True)
+        tensors["X"].SetTransient(transient_x)
+        M = at.IndexMapping(nodes, dofs.size)
+        M.map[:] = dofs.ravel()
+        rng = np.random.default_rng(5)
+        Lv = rng.uniform(-1, 1, nodes)
+        L, Lout = to_tensor(at, Lv), at.Tensor(nodes)
+        Lout.data[...] = -7.0
+        engine.BeginMultiKernelLaunch()
+        engine.FlatIndexedScatter(tensors["X"], L, M)
+        for k, out, ins in wl.kernels:
+            engine(k, tensors[out], *[tensors[n] for n in ins])
+        engine.FlatIndexedSumGather(Lout, tensors["Y"], M)
+        engine.EndMultiKernelLaunch()
+        Lout.MoveFromGPU()
+        wl.arrays["X"][...] = Lv[dofs]
+        Y = workloads.run_on_checker(wl, checker)["Y"]
+        expected = np.zeros(nodes)
+        np.add.at(expected, dofs.ravel(), Y.ravel())
+        assert rel_err(Lout.data, expected) <= 1e-12, transient_x

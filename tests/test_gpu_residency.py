@@ -118,3 +118,51 @@ def test_page_locked_host_buffers_move_like_ordinary_ones(at):
         X.MoveFromGPU()
         assert np.array_equal(X.data, 2.0 * ref)
     del T, U
+
+
+def device_memory_in_use():
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return total.value - free.value
+
+
+def test_device_mirror_of_a_tensor_over_a_callers_host_buffer_is_released(at):
+    # the library allocated the mirror, so the library frees it, whoever owns the host buffer
+    host = np.ones(8 << 20)                              # 64 MiB
+    at.synchronize()
+    before = device_memory_in_use()
+    for _ in range(12):
+        T = at.Tensor(host.size, hdata=host)
+        T.MoveToGPU()
+        T.Mult(2.0)
+        T.MoveFromGPU()
+        del T
+    assert host[0] == 4096.0 and host[-1] == 4096.0
+    assert device_memory_in_use() - before < 3 * host.nbytes
+
+
+def test_callers_device_buffer_is_used_and_never_freed(at, engine):
+    # a tensor over a caller's host AND device buffer, the device buffer at an odd offset (8-byte aligned only) of an
+    # allocation that belongs to another tensor
+    n = 1001
+    pool = at.Tensor(4096)
+    pool.data[...] = 0.0
+    pool.MoveToGPU()
+    base = pool.GetDeviceData()
+    host = np.zeros(n)
+    V = at.Tensor(n, hdata=host, ddata=base + 8 * 3, ongpu=True)
+    assert V.IsMappedToGPU() and V.IsOnGPU() and V.GetDeviceData() == base + 24
+    V.Set(2.0)
+    X = to_tensor(at, np.arange(n, dtype=np.float64))
+    engine("V_i += X_i", V, X)
+    V.MoveFromGPU()
+    assert np.array_equal(host, 2.0 + np.arange(n))
+    V.UnmapFromGPU()                                     # lets go of the caller's buffer, does not free it
+    assert not V.IsMappedToGPU()
+    del V
+    pool.MoveFromGPU()
+    expected = np.zeros(4096)
+    expected[3:3 + n] = 2.0 + np.arange(n)
+    assert np.array_equal(pool.data, expected)
