@@ -11,24 +11,39 @@ import numpy as np
 _MASK = (1 << 64) - 1
 
 
-def _splitmix64(x):
-    """Vectorised splitmix64 finaliser on uint64 arrays."""
-    x = (x + np.uint64(0x9E3779B97F4A7C15)) & np.uint64(_MASK)
-    z = x
-    z = ((z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)) & np.uint64(_MASK)
-    z = ((z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)) & np.uint64(_MASK)
-    return z ^ (z >> np.uint64(31))
+def _splitmix64_inplace(z):
+    """splitmix64 finaliser applied in place to a uint64 array (arithmetic wraps modulo 2^64)."""
+    z += np.uint64(0x9E3779B97F4A7C15)
+    z ^= z >> np.uint64(30)
+    z *= np.uint64(0xBF58476D1CE4E5B9)
+    z ^= z >> np.uint64(27)
+    z *= np.uint64(0x94D049BB133111EB)
+    z ^= z >> np.uint64(31)
+    return z
 
 
 def counter_uniform(seed, tensor_id, shape, lo=0.0, hi=1.0, first=0):
     """fp64 array of ``shape``: entry with flat index i is uniform in [lo, hi), a pure function of (seed, tensor_id, first+i)."""
     n = int(np.prod(shape))
+    out = np.empty(n, dtype=np.float64)
     with np.errstate(over="ignore"):
-        base = _splitmix64(np.uint64(seed) * np.uint64(0x1000003) + np.uint64(tensor_id))
-        idx = np.arange(first, first + n, dtype=np.uint64)
-        bits = _splitmix64(base + idx * np.uint64(0x9E3779B97F4A7C15))
-    u = (bits >> np.uint64(11)).astype(np.float64) * (1.0 / 9007199254740992.0)
-    return (lo + (hi - lo) * u).reshape(shape)
+        base = _splitmix64_inplace(np.array([np.uint64(seed) * np.uint64(0x1000003) + np.uint64(tensor_id)],
+                                            dtype=np.uint64))[0]
+        chunk = 1 << 18                                   # a few passes over 2 MiB at a time stay in cache
+        for start in range(0, n, chunk):
+            stop = min(n, start + chunk)
+            bits = np.arange(first + start, first + stop, dtype=np.uint64)
+            bits *= np.uint64(0x9E3779B97F4A7C15)
+            bits += base
+            _splitmix64_inplace(bits)
+            bits >>= np.uint64(11)
+            u = out[start:stop]
+            u[...] = bits                                 # exact: 53 bits
+            u *= 1.0 / 9007199254740992.0
+            if not (lo == 0.0 and hi == 1.0):
+                u *= (hi - lo)
+                u += lo
+    return out.reshape(shape)
 
 
 class Workload:
@@ -46,6 +61,9 @@ class Workload:
         self.algorithmic_bytes = algorithmic_bytes
         self.flops = flops
         self.seed = seed
+        written = {out for _, out, _ in kernels}
+        written |= {self.slices[n][0] for n in written if n in self.slices}
+        self.inputs = tuple(n for n in arrays if n not in written)   # arrays that carry data into the first kernel
 
     def view(self, name, arrays=None):
         arrays = self.arrays if arrays is None else arrays
@@ -55,12 +73,54 @@ class Workload:
         return arrays[name]
 
 
-def bind_to_engine(workload, at, transient=True):
-    """Create engine tensors for a workload; returns name -> Tensor (slices as SliceTensor of their parent)."""
+def bind_to_engine(workload, at, transient=True, inputs_only=False):
+    """Create engine tensors for a workload; returns name -> Tensor (slices as SliceTensor of their parent).
+    ``inputs_only``: the host buffers of tensors that the kernels write are left as allocated (large benchmarks)."""
     tensors = {}
     for name, arr in workload.arrays.items():
         t = at.Tensor(*arr.shape)
-        t.data[...] = arr
+        if not inputs_only or name in workload.inputs:
+            t.data[...] = arr
+        tensors[name] = t
+    for name, (parent, idx) in workload.slices.items():
+        tensors[name] = at.SliceTensor(tensors[parent], *idx)
+    for name in workload.transient:
+        tensors[name].SetTransient(bool(transient))
+    return tensors
+
+
+def bind_to_engine_repeated(workload, at, engine, times, transient=True, index="e"):
+    """Engine tensors for ``times`` copies of the workload laid end to end along the index called ``index`` (the
+    element index), built on the device: inputs that carry the index are uploaded once and repeated there by a
+    broadcasting kernel, tensors that the kernels write only get device memory.  For benchmarks at sizes whose
+    inputs would take minutes to generate and upload (configs[4]: 4.7 GB of geometric factors); timings do not
+    depend on the values.  Returns name -> Tensor."""
+    axes = {}
+    for k, out, ins in workload.kernels:
+        lhs, rhs = k.replace("+=", "=").replace("-=", "=").split("=")
+        for token, name in zip([lhs.split()[0]] + rhs.split(), [out] + list(ins)):
+            axes[name] = token.split("_")[1:]
+    tensors = {}
+    for name, arr in workload.arrays.items():
+        names = axes.get(name)
+        if names is None or index not in names:
+            t = at.Tensor(*arr.shape)                        # invariant operand (basis matrices)
+            t.data[...] = arr
+            t.MoveToGPU()
+        elif name in workload.inputs:
+            if names.index(index) != 0:
+                raise ValueError("inputs must carry the repeated index first")
+            small = at.Tensor(*arr.shape)
+            small.data[...] = arr
+            t = at.Tensor(times, *arr.shape)
+            t.SwitchToGPU()
+            letters = ["a%d" % d for d in range(arr.ndim)]
+            engine("R_t_%s = S_%s" % ("_".join(letters), "_".join(letters)), t, small)
+            t.Reshape(times * arr.shape[0], *arr.shape[1:])
+        else:
+            axis = names.index(index)
+            t = at.Tensor(*[n * times if d == axis else n for d, n in enumerate(arr.shape)])
+            t.SwitchToGPU()
         tensors[name] = t
     for name, (parent, idx) in workload.slices.items():
         tensors[name] = at.SliceTensor(tensors[parent], *idx)

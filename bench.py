@@ -7,16 +7,24 @@ resident in HBM.  Prints ONE JSON line:
   value           GDOF/s over the timed steps, host-side TensorEngine overhead included (wall clock between two
                   device synchronisations)
   roofline        algorithmic bytes of one launch (X + D + Y = 2024 B per element) over the launch duration
-                  measured with HIP events on the library's stream, against the 8 TB/s HBM peak
+                  measured with HIP events on the library's stream, against the 8 TB/s HBM peak; `traffic` is the
+                  HBM traffic that hardware counters showed for exactly the kernel that ran (identified by name and
+                  a hash of its generated source), null for any other kernel
   cpu_baseline    the same chain on the host: the reference's own CPUInterpreted executor (oracle/_ref, kind
                   "reference") or, if that library is absent, the plain-C restatement (kind "port"), one thread,
                   on a bounded sample of elements
   store_all       the same launch when the six intermediates are ordinary (non-transient) tensors, i.e. also
-                  written to HBM as the reference's generated kernel always does
+                  written to HBM as the reference's generated kernel always does: what a caller gets who changes
+                  nothing but the policy string
+  all_configs     the other four baseline configurations at their full sizes, each with launch time by HIP
+                  events, algorithmic GB/s, fraction of the HBM peak, GFLOP/s and its own single-thread CPU
+                  baseline (on a stated sample where the host would take minutes)
 """
 import argparse
+import hashlib
 import json
 import os
+import re
 import sys
 import time
 
@@ -26,9 +34,24 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 METRIC = "GDOF/s + % HBM peak, p=3 sum-factorised hex mass apply fp64 (1 GPU)"
 
-# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a
-# copy kernel of known size); None until the profile summary under profiles/ has been taken for this kernel.
-MEASURED_TRAFFIC_BYTES = 541836805  # profiles/cfg4_mass_apply_hbm_traffic.md
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the same counter
+# reads for a copy kernel of known size), keyed by the kernel the counters were taken on: (name of its first
+# function, first 16 hex digits of the SHA-1 of the generated source).  A generator change that alters the source of
+# a kernel therefore drops its figure (the line then says null) until the counters are taken again.
+TRAFFIC_BY_KERNEL = {
+}
+
+
+def kernel_identity(engine):
+    """(function names, source hash) of the kernel(s) the engine's most recent launch used."""
+    src = engine.GetLastImplementation()
+    names = re.findall(r"__global__[^\n]*?\bvoid\s+(\w+)\s*\(", src)
+    return names, hashlib.sha1(src.encode()).hexdigest()[:16]
+
+
+def measured_traffic(engine):
+    names, digest = kernel_identity(engine)
+    return TRAFFIC_BY_KERNEL.get((names[0] if names else "", digest))
 
 
 def settle_clocks(at, workloads, wl, engine, tensors, seconds):
@@ -54,15 +77,18 @@ def time_steps(at, workloads, wl, engine, tensors, steps, warmup):
     return wall, ev.ms * 1e-3
 
 
-def cpu_baseline(workloads, sample_elems):
+def host_checker():
     sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import oracle  # tests/oracle.py - checker access, used here only for the reported CPU baseline
+    import oracle  # tests/oracle.py - checker access, used here only for the reported CPU baselines
 
-    wl = workloads.config4(E=sample_elems)
     if oracle.have_reference():
-        checker, kind = oracle.Reference(), "reference"
-    else:
-        checker, kind = oracle.Oracle(), "port"
+        return oracle.Reference(), "reference"
+    return oracle.Oracle(), "port"
+
+
+def cpu_baseline(workloads, sample_elems):
+    checker, kind = host_checker()
+    wl = workloads.config4(E=sample_elems)
     t0 = time.perf_counter()
     workloads.run_on_checker(wl, checker)
     dt = time.perf_counter() - t0
@@ -73,6 +99,40 @@ def cpu_baseline(workloads, sample_elems):
         "kind": kind,
         "sample": "%d of 262144 elements, whole 7-kernel chain, one pass, %.1f s" % (sample_elems, dt),
     }
+
+
+def cpu_baseline_for(name, workloads):
+    """Single-thread host figure for one of the other baseline configurations, in the unit of its GPU line."""
+    checker, kind = host_checker()
+    if name == "cfg1":
+        wl = workloads.config1()
+        t0 = time.perf_counter()
+        workloads.run_on_checker(wl, checker)
+        dt = time.perf_counter() - t0
+        value, unit, sample = wl.algorithmic_bytes / dt * 1e-9, "GB/s", "all 1048576 slices, one pass, %.2f s" % dt
+    elif name == "cfg2":
+        J = workloads.config2_inputs()
+        t0 = time.perf_counter()
+        checker.batch_matrix_inv_det(J)
+        dt = time.perf_counter() - t0
+        value, unit, sample = J.shape[0] * J.shape[1] / dt * 1e-9, "Gmatrices/s", "all 4194304 matrices, one pass, %.2f s" % dt
+    elif name == "cfg3":
+        n = 8192
+        wl = workloads.config3(E=n)
+        t0 = time.perf_counter()
+        workloads.run_on_checker(wl, checker)
+        dt = time.perf_counter() - t0
+        value, unit, sample = wl.algorithmic_bytes / dt * 1e-9, "GB/s", "%d of 32768 elements, kernel as written, one pass, %.1f s" % (n, dt)
+    elif name == "cfg5":
+        n = 4096
+        wl = workloads.config5(E=n)
+        t0 = time.perf_counter()
+        workloads.run_on_checker(wl, checker)
+        dt = time.perf_counter() - t0
+        value, unit, sample = wl.dof / dt * 1e-9, "GDOF/s", "%d of 65536 elements, whole 18-kernel chain, one pass, %.1f s" % (n, dt)
+    else:
+        raise ValueError(name)
+    return {"value": value, "unit": unit, "cores": 1, "kind": kind, "sample": sample}
 
 
 FP64_PEAK_GFLOPS = 78600.0
@@ -143,11 +203,11 @@ def kernel_shapes(at, args):
     }
 
 
-def other_workload(at, workloads, args):
-    """Same measurement for cfg1 / cfg2 / cfg3 / cfg5 at the sizes of the baseline configurations, and for
-    FlatIndexedScatter / FlatIndexedSumGather on the headline mesh."""
+def build_case(at, workloads, name):
+    """Tensors on the device and a step function for one workload: cfg1 / cfg2 / cfg3 / cfg5 at the sizes of the
+    baseline configurations, FlatIndexedScatter / FlatIndexedSumGather on the headline mesh, and the other pipelines.
+    Returns (engine, step, label, units per step, unit name, algorithmic bytes, flops as written)."""
     engine = at.TensorEngine("HIP")
-    name = args.workload
     if name == "cfg2":
         J = workloads.config2_inputs()
         E, Q = J.shape[:2]
@@ -291,20 +351,43 @@ def other_workload(at, workloads, args):
             label = "L-vector[7189057] = sum of E-vector[262144*64] entries through the element-to-node map"
             abytes = dofs.size * (4 + 8) + nodes * (4 + 8)    # inverse map + E-vector read + row offsets + L written
         units, unit_name, flops = dofs.size, "GDOF/s", dofs.size
+    elif name == "cfg5":
+        # inputs for 2048 elements, repeated 32 times along the element index on the device (generating and
+        # uploading all 4.7 GB of geometric factors from the host takes minutes; no timing depends on the values)
+        period, times = 2048, 32
+        small = workloads.config5(E=period)
+        tensors = workloads.bind_to_engine_repeated(small, at, engine, times, transient=True)
+        wl = small
+        step = lambda: workloads.launch(wl, engine, tensors)
+        label = ("configs[4]: p=7 hex diffusion apply, E=65536, 18-kernel multi-kernel launch, intermediates transient "
+                 "(input values repeat with a period of %d elements)" % period)
+        abytes, flops = small.algorithmic_bytes * times, small.flops * times
+        units, unit_name = small.dof * times, "GDOF/s"
     else:
-        wl = {"cfg1": workloads.config1, "cfg3": workloads.config3, "cfg5": workloads.config5}[name]()
-        tensors = workloads.bind_to_engine(wl, at, transient=True)
+        wl = {"cfg1": workloads.config1, "cfg3": workloads.config3}[name]()
+        tensors = workloads.bind_to_engine(wl, at, transient=True, inputs_only=True)
         for t in tensors.values():
             t.MoveToGPU()
         step = lambda: workloads.launch(wl, engine, tensors)
-        label = {"cfg1": "configs[0]: S_i_j = A_n_i_j B_n, n=2^20", "cfg3": "configs[2]: p=2 hex mass assembly, E=32768",
-                 "cfg5": "configs[4]: p=7 hex diffusion apply, E=65536"}[name]
+        label = {"cfg1": "configs[0]: S_i_j = A_n_i_j B_n, n=2^20", "cfg3": "configs[2]: p=2 hex mass assembly, E=32768"}[name]
         abytes, flops = wl.algorithmic_bytes, wl.flops
-        units, unit_name = (wl.dof, "GDOF/s") if wl.dof else (abytes, "GB/s")
-    steps, warmup = min(args.steps, 200), min(args.warmup, 20)
+        units, unit_name = abytes, "GB/s"
+    return engine, step, label, units, unit_name, abytes, flops
+
+
+def measure_case(at, engine, step, abytes, flops, steps, warmup, settle_seconds):
+    # sustained load before anything is timed (see settle_clocks): bursts of launches, not one launch per
+    # synchronisation, or the device drops back to idle clocks between them
+    step()
+    at.synchronize()
     t0 = time.perf_counter()
-    while time.perf_counter() - t0 < args.settle_seconds:
-        step()
+    step()
+    at.synchronize()
+    burst = max(1, min(100, int(2e-3 / max(time.perf_counter() - t0, 1e-6))))
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < settle_seconds:
+        for _ in range(burst):
+            step()
         at.synchronize()
     for _ in range(warmup):
         step()
@@ -317,15 +400,47 @@ def other_workload(at, workloads, args):
     wall = time.perf_counter() - t0
     launch_s = ev.ms * 1e-3 / steps
     achieved = abytes / launch_s * 1e-9
-    return {
+    names, digest = kernel_identity(engine)
+    roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(engine), "algorithmic_bytes": abytes,
+                "launch_us": launch_s * 1e6, "kernel": names[0] if names else None, "kernel_source_sha1_16": digest}
+    return wall, launch_s, roofline
+
+
+def all_configs(at, workloads, args):
+    """cfg1 / cfg2 / cfg3 / cfg5 at their full sizes, one after the other: GPU figures by HIP events and the host
+    baseline beside each."""
+    block = {}
+    for name in ("cfg1", "cfg2", "cfg3", "cfg5"):
+        engine, step, label, units, unit_name, abytes, flops = build_case(at, workloads, name)
+        steps = 50 if name == "cfg5" else 200
+        wall, launch_s, roofline = measure_case(at, engine, step, abytes, flops, steps, 10, args.settle_seconds)
+        block[name] = {
+            "workload": label, "launch_us": launch_s * 1e6, "steps": steps, "algorithmic_bytes": abytes,
+            "GBps": roofline["achieved"], "frac": roofline["frac"], "gflops_as_written": flops / launch_s * 1e-9,
+            "value": units / launch_s * 1e-9, "unit": unit_name, "traffic": roofline["traffic"],
+            "kernel": roofline["kernel"],
+        }
+        del engine, step
+        if not args.no_cpu_baseline:
+            block[name]["cpu_baseline"] = cpu_baseline_for(name, workloads)
+    return block
+
+
+def other_workload(at, workloads, args):
+    name = args.workload
+    engine, step, label, units, unit_name, abytes, flops = build_case(at, workloads, name)
+    steps, warmup = min(args.steps, 200), min(args.warmup, 20)
+    wall, launch_s, roofline = measure_case(at, engine, step, abytes, flops, steps, warmup, args.settle_seconds)
+    result = {
         "metric": "%s throughput (1 GPU)" % name, "value": units * steps / wall * 1e-9, "unit": unit_name, "n_gpus": 1,
         "steps": steps, "warmup": warmup, "ms_per_step": wall / steps * 1e3, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic", "config": {"workload": label},
-        "gflops_as_written": flops / launch_s * 1e-9,
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": abytes,
-                     "launch_us": launch_s * 1e6},
+        "gflops_as_written": flops / launch_s * 1e-9, "roofline": roofline,
     }
+    if name in ("cfg1", "cfg2", "cfg3", "cfg5") and not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_for(name, workloads)
+    return result
 
 
 def main():
@@ -339,6 +454,8 @@ def main():
     ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store-all", action="store_true")
+    ap.add_argument("--no-all-configs", action="store_true",
+                    help="leave out the block with the other four baseline configurations")
     ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "scatter_apply", "scatter_then_apply", "operator", "dense_apply", "shapes"],
                     help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
                          "remaining baseline configurations at their full sizes and for the node-vector <-> "
@@ -408,9 +525,11 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES,
+            "traffic": measured_traffic(engine),
             "algorithmic_bytes": wl.algorithmic_bytes,
             "launch_us": launch_s * 1e6,
+            "kernel": kernel_identity(engine)[0][0],
+            "kernel_source_sha1_16": kernel_identity(engine)[1],
         },
     }
 
@@ -420,16 +539,29 @@ def main():
         n2 = max(10, args.steps // 4)
         wall2, dev2 = time_steps(at, workloads, wl, engine, tensors, n2, max(5, args.warmup // 4))
         stored_bytes = args.elements * (64 + 125 + 64 + 610) * 8
+        moved = stored_bytes / (dev2 / n2) * 1e-9
         result["store_all"] = {
+            "what": "the same launch with T1..V2 as ordinary tensors: every intermediate is also written to HBM, "
+                    "as with the reference (what a caller gets who only changes the policy string)",
             "value": wl.dof * n2 / wall2 * 1e-9,
             "unit": "GDOF/s",
             "launch_us": dev2 / n2 * 1e6,
             "hbm_bytes_moved": stored_bytes,
-            "achieved_GBs_incl_intermediates": stored_bytes / (dev2 / n2) * 1e-9,
+            "achieved_GBs_incl_intermediates": moved,
+            "frac_of_hbm_peak_on_bytes_moved": moved / HBM_PEAK_GBS,
+            "traffic": measured_traffic(engine),
+            "kernel": kernel_identity(engine)[0][0],
+            "kernel_source_sha1_16": kernel_identity(engine)[1],
         }
+        for name in wl.transient:
+            tensors[name].SetTransient(True)
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(workloads, min(args.cpu_sample_elems, args.elements))
+
+    if not args.no_all_configs:
+        del tensors
+        result["all_configs"] = all_configs(at, workloads, args)
 
     print(json.dumps(result))
 
