@@ -5,6 +5,7 @@
 #include "hip_codegen.hpp"
 
 #include <algorithm>
+#include <cctype>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -1010,6 +1011,7 @@ class Generator
                 for (const auto &r : s.in) streamingOnly = streamingOnly && has(r.idx, batch) && !r.repeated;
                 const long outputs = product(mid, extent), loadsPerOutput = s.contrCount * nin;
                 if (streamingOnly && ((outputs <= 32 && loadsPerOutput <= 16) || (outputs <= 64 && loadsPerOutput <= 4))) best.clear();
+                ForcedTile(static_cast<int>(&s - subs.data()), mid, best);
                 s.tile = best;
             }
             SetLanes(s);
@@ -1053,6 +1055,32 @@ class Generator
         }
     }
 
+    // Experiment switch ACRO_HIP_FORCE_TILE="8:;3:q,r": kernel 8 of the group gets the empty register tile, kernel 3
+    // the tile (q, r), whatever the cost model says.  Names that are not output indices of the kernel are ignored.
+    void ForcedTile(int k, const std::vector<int> &mid, std::vector<int> &tile) const
+    {
+        const char *spec = std::getenv("ACRO_HIP_FORCE_TILE");
+        if (spec == nullptr) return;
+        std::istringstream all(spec);
+        std::string item;
+        while (std::getline(all, item, ';'))
+        {
+            const size_t colon = item.find(':');
+            if (colon == std::string::npos || std::atoi(item.substr(0, colon).c_str()) != k) continue;
+            if (!std::isdigit(static_cast<unsigned char>(item[0]))) continue;
+            tile.clear();
+            std::istringstream names(item.substr(colon + 1));
+            std::string name;
+            while (std::getline(names, name, ','))
+            {
+                for (int id : mid)
+                {
+                    if (idxName[id] == name && !has(tile, id)) tile.push_back(id);
+                }
+            }
+        }
+    }
+
     void SetLanes(Sub &s)
     {
         s.lane.clear();
@@ -1060,7 +1088,13 @@ class Generator
         // when it is stored to device memory, otherwise the largest operand read from device memory.
         const VarRef *order = &s.out;
         const UVarInfo &uo = uvars[s.out.uvar];
-        const bool out_stays_on_chip = stores[uo.storage].transient && uo.lastUse > uo.firstWrite;
+        // read again by a later kernel of the group, under this name or as a view of the same storage
+        bool readLater = uo.lastUse > uo.firstWrite;
+        for (size_t k2 = static_cast<size_t>(&s - subs.data()) + 1; k2 < subs.size() && !readLater; ++k2)
+        {
+            for (const auto &r : subs[k2].in) readLater = readLater || ViewsOverlap(r.uvar, s.out.uvar);
+        }
+        const bool out_stays_on_chip = stores[uo.storage].transient && readLater;
         if (out_stays_on_chip)
         {
             const VarRef *big = nullptr;
@@ -1919,6 +1953,8 @@ class Generator
             add(str(st.ldsOffset + LdsViewOffset(r.uvar)) + " + b * " + str(st.tileSize));
         else if (u.viewOffset != 0)
             add(Lit(u.viewOffset));
+        // Total stride of every lane index in this occurrence (an index may occur in two dimensions).
+        std::vector<long> laneStride(s.lane.size(), 0);
         for (size_t d = 0; d < r.idx.size(); ++d)
         {
             const int id = r.idx[d];
@@ -1926,11 +1962,55 @@ class Generator
             if (id == batch)
             {
                 if (!lds) add("e * " + Lit(stride));
+                continue;
             }
-            else if (has(s.lane, id))
+            for (size_t j = 0; j < s.lane.size(); ++j)
             {
-                add(IdxVar(id) + " * " + (lds ? str(stride) : Lit(stride)));
+                if (s.lane[j] == id) laneStride[j] += stride;
             }
+        }
+        // The work-item header splits the item number r_ into the lane indices, the last one fastest.  A run of
+        // consecutive lane indices that this occurrence lays out the same way (the stride of one is the stride of the
+        // next times its extent) needs no splitting: its terms add up to a single quotient of r_ times the last
+        // stride, and for an operand that follows the lanes' order throughout the offset is r_ times a constant.
+        // That spares the integer divisions and multiplications of every index in the run.
+        std::vector<long> divisor(s.lane.size(), 1);  // r_ / divisor[j] % extent = lane index j
+        {
+            long st = s.laneCount;
+            for (size_t j = 0; j < s.lane.size(); ++j)
+            {
+                st /= extent[s.lane[j]];
+                divisor[j] = st;
+            }
+        }
+        const bool collapse = envInt("ACRO_HIP_COLLAPSE") >= 0;
+        for (size_t j = 0; j < s.lane.size();)
+        {
+            if (laneStride[j] == 0)
+            {
+                ++j;
+                continue;
+            }
+            size_t k = j;
+            long span = extent[s.lane[j]];
+            while (collapse && k + 1 < s.lane.size() && laneStride[k + 1] != 0 &&
+                   laneStride[k] == laneStride[k + 1] * extent[s.lane[k + 1]])
+            {
+                ++k;
+                span *= extent[s.lane[k]];
+            }
+            const std::string factor = lds ? str(laneStride[k]) : Lit(laneStride[k]);
+            if (k == j)
+            {
+                add(IdxVar(s.lane[j]) + " * " + factor);
+            }
+            else
+            {
+                std::string q = divisor[k] == 1 ? std::string("r_") : "(r_ / " + str(divisor[k]) + ")";
+                if (j > 0) q = "(" + q + " % " + str(span) + ")";
+                add(q + " * " + factor);
+            }
+            j = k + 1;
         }
         return expr.empty() ? "0" : expr;
     }
@@ -3863,7 +3943,8 @@ class Generator
         const int U = static_cast<int>(uvars.size());
         const std::string dimName = mk.GetDimensionedNameString();
         std::string variant = str(NB) + "/" + str(NT) + "/" + (opt.noalias ? "n" : "a") + (Positional() ? "p" : "u") +
-                              "/" + str(envInt("ACRO_HIP_PERSIST"));
+                              "/" + str(envInt("ACRO_HIP_PERSIST")) + (envInt("ACRO_HIP_PIPELINE") > 0 ? "p" + str(envInt("ACRO_HIP_PIPELINE")) : "") +
+                              (envInt("ACRO_HIP_WAVES_PER_EU") > 0 ? "w" + str(envInt("ACRO_HIP_WAVES_PER_EU")) : "");
         for (const auto &st : stores) variant += st.elide ? "e" : (st.inLds ? "l" : "g");
         for (int u = 0; u < U; ++u) variant += "s" + str(uvars[u].storage) + "@" + str(uvars[u].viewOffset);
         for (int g : opt.gathered) variant += "g" + str(g);
@@ -3905,7 +3986,11 @@ class Generator
             while (std::getline(lines, l)) out << "// " << l << "\n";
         }
         out << "typedef const __attribute__((address_space(4))) double *acro_scalar_ptr;\n\n";
-        out << "extern \"C\" __global__ __launch_bounds__(" << NT << ") void " << function_name << "(";
+        out << "extern \"C\" __global__ __launch_bounds__(" << NT << ") ";
+        // experiment switch: ask the compiler for a register budget that lets this many wavefronts share a SIMD
+        if (envInt("ACRO_HIP_WAVES_PER_EU") > 0)
+            out << "__attribute__((amdgpu_waves_per_eu(" << envInt("ACRO_HIP_WAVES_PER_EU") << ", " << envInt("ACRO_HIP_WAVES_PER_EU") << "))) ";
+        out << "void " << function_name << "(";
         out << ParamList();
         out << ")\n{\n";
         if (ldsDoubles > 0) out << "    __shared__ double lds[" << ldsDoubles << "];\n";
@@ -3926,9 +4011,16 @@ class Generator
         const long persist = envInt("ACRO_HIP_PERSIST");
         const long gridGroups = persist > 0 ? std::min<long>(totalGroups, persist * 256) : totalGroups;
         const bool looped = gridGroups < totalGroups;
-        if (looped)
-            out << "    for (int e0 = blockIdx.x * " << NB << "; e0 < " << E << "; e0 += " << gridGroups * NB << ")\n    {\n";
-        else
+        // Pipelined form of the persistent loop (ACRO_HIP_PIPELINE=1): the streaming inputs of every phase, the first
+        // included, live in registers across iterations; a phase that has consumed its registers at once requests
+        // the next batch entries' values, so that a workgroup never waits for device memory at the top of an
+        // iteration and the memory system always holds requests of every resident workgroup.
+        const bool pipelined = looped && envInt("ACRO_HIP_PIPELINE") > 0;
+        const std::string loopHeader = "    for (int e0 = blockIdx.x * " + str(NB) + "; e0 < " + str(E) + "; e0 += " +
+                                       str(gridGroups * NB) + ")\n    {\n";
+        if (looped && !pipelined)
+            out << loopHeader;
+        else if (!looped)
             out << "    const int e0 = blockIdx.x * " << NB << ";\n    {\n";
 
         const bool guardBatch = (E % NB) != 0;
@@ -4000,6 +4092,7 @@ class Generator
             std::vector<Chain> chains;
             long slots = 0, passes = 1;
             bool prefetched = false;
+            bool carried = false;  // pipelined loop: the prefetched values are requested one iteration ahead
         };
         std::vector<Phase> phases;
         for (int k = 0; k < K;)
@@ -4023,7 +4116,7 @@ class Generator
         }
 
         long prefetchBudget = envInt("ACRO_HIP_PREFETCH") < 0 ? 0 : kPrefetchDoubles;
-        for (size_t pi = 1; pi < phases.size(); ++pi)
+        for (size_t pi = pipelined ? 0 : 1; pi < phases.size(); ++pi)
         {
             Phase &ph = phases[pi];
             long perLane = 0;  // registers one lane needs: a lane serves at most one chain per pass
@@ -4049,6 +4142,9 @@ class Generator
             if (!ok || perLane == 0 || perLane * ph.passes > prefetchBudget) continue;
             prefetchBudget -= perLane * ph.passes;
             ph.prefetched = true;
+            // ACRO_HIP_PIPELINE=<n>: phases that hold at most n doubles per lane are carried across iterations (the
+            // first phase always is: its inputs are what an iteration would otherwise start by waiting for)
+            ph.carried = pipelined && (pi == 0 || perLane * ph.passes <= envInt("ACRO_HIP_PIPELINE"));
         }
 
         // Emits, for pass j of a phase (or for the item loop when j < 0), the selection of the chain a lane works
@@ -4097,10 +4193,28 @@ class Generator
             out << "    }\n";
         };
 
+        // Requests the prefetched inputs of one phase for the batch entries that start at the `e0` in scope.
+        auto emitPrefetchLoads = [&](const Phase &ph) {
+            for (long j = 0; j < ph.passes; ++j)
+            {
+                emitItems(ph, j, [&](const Chain &c, const std::string &indent) {
+                    for (int kk = c.first; kk <= c.last; ++kk)
+                    {
+                        if (c.loads[kk - c.first].empty()) continue;
+                        Body bases;
+                        EmitBases(kk, bases);
+                        for (const auto &l : bases.bases) out << indent << l << "\n";
+                        for (const auto &ld : c.loads[kk - c.first])
+                            out << indent << c.names[kk - c.first][j].at(ld.first) << " = " << ld.second << ";\n";
+                    }
+                });
+            }
+        };
         for (auto &ph : phases)
         {
             if (!ph.prefetched) continue;
-            out << "    // streaming inputs of phase " << subs[ph.chains[0].first].phase << ", requested before the first phase\n";
+            out << "    // streaming inputs of phase " << subs[ph.chains[0].first].phase
+                << (pipelined ? ", held in registers across iterations\n" : ", requested before the first phase\n");
             for (auto &c : ph.chains)
                 c.names.assign(c.last - c.first + 1, std::vector<std::map<std::string, std::string>>(ph.passes));
             for (long j = 0; j < ph.passes; ++j)
@@ -4119,17 +4233,20 @@ class Generator
                 }
                 for (long n = 0; n < widest; ++n)
                     out << "    double pf" << subs[ph.chains[0].first].phase << "_" << j << "_" << n << " = 0.0;\n";
-                emitItems(ph, j, [&](const Chain &c, const std::string &indent) {
-                    for (int kk = c.first; kk <= c.last; ++kk)
-                    {
-                        if (c.loads[kk - c.first].empty()) continue;
-                        Body bases;
-                        EmitBases(kk, bases);
-                        for (const auto &l : bases.bases) out << indent << l << "\n";
-                        for (const auto &ld : c.loads[kk - c.first])
-                            out << indent << c.names[kk - c.first][j].at(ld.first) << " = " << ld.second << ";\n";
-                    }
-                });
+            }
+            if (!pipelined) emitPrefetchLoads(ph);
+        }
+        if (pipelined)
+        {
+            out << "    {   // the first batch entries of this workgroup\n    const int e0 = blockIdx.x * " << NB << ";\n";
+            for (const auto &ph : phases)
+            {
+                if (ph.carried) emitPrefetchLoads(ph);
+            }
+            out << "    }\n" << loopHeader;
+            for (const auto &ph : phases)
+            {
+                if (ph.prefetched && !ph.carried) emitPrefetchLoads(ph);  // requested at the top of every iteration
             }
         }
 
@@ -4181,6 +4298,14 @@ class Generator
                     }
                     for (int kk = c.first; kk <= c.last; ++kk) out << indent << "}\n";
                 });
+            }
+            if (ph.carried)
+            {
+                out << "    {   // the same inputs of this workgroup's next batch entries\n";
+                out << "    const int e0_next = e0 + " << gridGroups * NB << ";\n    if (e0_next < " << E << ")\n    {\n";
+                out << "    const int e0 = e0_next;\n";
+                emitPrefetchLoads(ph);
+                out << "    }\n    }\n";
             }
         }
         if (looped && ldsDoubles > 0) out << "    __syncthreads();\n";

@@ -47,6 +47,8 @@
 //   ACRO_HIP_PACK=1|-1          1: pick batch / workgroup size for wavefront utilisation also when one batch entry per
 //                               workgroup would do; -1: never (default: only for groups that batch several entries)
 //   ACRO_HIP_PERSIST=<n>        persistent grid of n workgroups per CU looping over the batch
+//   ACRO_HIP_PIPELINE=1         with ACRO_HIP_PERSIST: streaming inputs stay in registers across iterations and are
+//                               requested one iteration ahead
 //   ACRO_HIP_FACTORISE=-1|2     -1: evaluate multi-operand kernels as written instead of as a chain of steps;
 //                               2: reorder whenever a chain is cheaper at all (default: only large kernels, 4x gain)
 //   ACRO_HIP_LDS_COPY_OUT=-1    stored results that also live in LDS are written by the lanes that computed them instead
@@ -55,6 +57,9 @@
 //                               (no contractions over the producer's register tile, no matrix kernels joined to readers)
 //   ACRO_HIP_FOOTPRINT=-1       register tiles by loads per output alone (no weight for uncoalesced streaming loads, no
 //                               cache-footprint term, no one-output-per-lane rule for tiny batch entries)
+//   ACRO_HIP_FORCE_TILE="8:;3:q,r"  kernel 8 of the group takes the empty register tile, kernel 3 the tile (q, r)
+//   ACRO_HIP_COLLAPSE=-1        offsets are sums over every lane index (runs of lane indices that an operand lays out in
+//                               the lanes' own order are not collapsed into one multiple of the item number)
 //   ACRO_HIP_STAGE=-1           small invariant operands with lane-dependent addresses stay in device memory (not staged in LDS)
 //   ACRO_HIP_SPLIT_LANES=-1     one lane per batch entry also for kernels with one output per entry (no lane exchanges)
 //   ACRO_HIP_WAVE_UNIFORM=-1    no readfirstlane on the batch entry of wavefronts that hold items of one entry only

@@ -10,6 +10,7 @@
 #include <cstdlib>
 #include <fstream>
 #include <iostream>
+#include <sstream>
 
 #include "HipRuntime.hpp"
 
@@ -91,6 +92,19 @@ void rtcCheck(hiprtcResult r, const char *what)
 HipKernel::HipKernel(const std::string &module_name, const std::string &source)
     : FunctionName(module_name), Source(source), CacheHit(false), Module(nullptr)
 {
+    // Experiment hook: $ACRO_HIP_KERNEL_OVERRIDE_DIR/<module name>.hip, when it exists, is compiled in place of the
+    // generated source (same function names and parameters), e.g. a hand-edited copy of what GetImplementation printed.
+    if (const char *dir = std::getenv("ACRO_HIP_KERNEL_OVERRIDE_DIR"))
+    {
+        std::ifstream in(std::string(dir) + "/" + module_name + ".hip");
+        if (in)
+        {
+            std::ostringstream text;
+            text << in.rdbuf();
+            Source = text.str();
+            std::cerr << "acrotensor: " << module_name << " compiled from " << dir << "/" << module_name << ".hip" << std::endl;
+        }
+    }
     Compile();
 }
 
