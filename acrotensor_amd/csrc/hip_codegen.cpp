@@ -1752,7 +1752,30 @@ class Generator
                         loaded += static_cast<double>(s.in[v].size) / static_cast<double>(E);
                 }
             }
-            if (stored >= 3.0 * loaded && stored > 0.0) NT = 256;
+            if (stored >= 3.0 * loaded && stored > 0.0)
+            {
+                NT = 256;
+                // Results that leave through their LDS tiles are written as one contiguous range per tensor and
+                // workgroup.  Twice the batch entries in workgroups of twice the lanes keep as many entries in flight
+                // per CU and make those ranges twice as long (p=3 mass apply with all intermediates stored, 4 entries
+                // in 256 lanes -> 8 in 512: 336 -> 311 us; 8 in 256 lanes 332 us, 16 in 1 024 lanes 331 us).
+                bool throughLds = false;
+                for (int k = 0; k < K; ++k) throughLds = throughLds || CopiesOutFromLds(k);
+                if (throughLds && NB >= 2 && opt.force_nb <= 0 && envInt("ACRO_HIP_NB") <= 0 && 2L * NB <= E && envInt("ACRO_HIP_WRITE_BATCH") >= 0)
+                {
+                    const int wider = PlaceLds(2 * NB);
+                    if (wider <= budgetDoubles / 2)
+                    {
+                        NB *= 2;
+                        NT = 512;
+                        ldsDoubles = wider;
+                    }
+                    else
+                    {
+                        ldsDoubles = PlaceLds(NB);
+                    }
+                }
+            }
         }
     }
 
@@ -2797,7 +2820,7 @@ class Generator
         std::snprintf(hex, sizeof(hex), "%016llx",
                       static_cast<unsigned long long>(hashString(dimName + "/reduction/" + (opt.noalias ? "n" : "a") +
                                                                  (Positional() ? "p" : "u") +
-                                                                 (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "2" : "1") + "/" + str(envInt("ACRO_HIP_RED_PENCIL")) +
+                                                                 (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "2" : (envInt("ACRO_HIP_ONE_PASS") >= 2 ? "1l" : "1")) + "/" + str(envInt("ACRO_HIP_RED_PENCIL")) +
                                                                  (byRows ? "/rows" : ""))));
         plan.module_name = std::string("acro_red_") + hex;
         const std::string fPartial = plan.module_name + "_partial", fFinal = plan.module_name + "_final";
@@ -3009,10 +3032,15 @@ class Generator
         {
             // The partials were stored by the wavefront of lane 0 with device-scope atomic stores; its release on the
             // counter orders them before the arrival.  Only the last workgroup needs the acquire side.
+            // ACRO_HIP_ONE_PASS=2: the partials were written through to the device's point of coherence by the
+            // atomic stores; the storing wavefront only waits until they are acknowledged (a workgroup-scope release)
+            // and the arrival is counted without the device-scope release that writes back the XCD's L2.
+            const bool light = envInt("ACRO_HIP_ONE_PASS") >= 2;
+            if (light) out << "    __builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\");\n";
             out << "    __syncthreads();\n";
             out << "    if (lane == 0)\n    {\n";
             out << "        const unsigned int arrived = __hip_atomic_fetch_add(" << counter
-                << ", 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);\n";
+                << ", 1u, " << (light ? "__ATOMIC_RELAXED" : "__ATOMIC_RELEASE") << ", __HIP_MEMORY_SCOPE_AGENT);\n";
             out << "        isLast = (arrived == " << G - 1 << "u);\n    }\n";
             out << "    __syncthreads();\n";
             out << "    if (!isLast) return;\n";
@@ -4116,8 +4144,19 @@ class Generator
         }
 
         long prefetchBudget = envInt("ACRO_HIP_PREFETCH") < 0 ? 0 : kPrefetchDoubles;
-        for (size_t pi = pipelined ? 0 : 1; pi < phases.size(); ++pi)
+        // The first phase's own loads join the prefetch (ACRO_HIP_PREFETCH_FIRST=-1 switches that off): they are then
+        // requested ahead of the later phases' inputs, and since a wavefront's loads complete in the order they were
+        // issued, the first phase starts as soon as its own operands are there instead of after everything that was
+        // prefetched (p=7 diffusion apply: 960 -> 943 us).  Only when some later phase prefetches at all.
+        const bool firstToo = pipelined || envInt("ACRO_HIP_PREFETCH_FIRST") >= 0;
+        // Later phases first (they have the latency to hide), the first phase last, with what is left of the budget.
+        std::vector<size_t> phaseOrder;
+        for (size_t pi = 1; pi < phases.size(); ++pi) phaseOrder.push_back(pi);
+        if (firstToo && phases.size() > 1) phaseOrder.push_back(0);
+        bool anyLater = false;
+        for (size_t pi : phaseOrder)
         {
+            if (pi == 0 && !anyLater && !pipelined) break;
             Phase &ph = phases[pi];
             long perLane = 0;  // registers one lane needs: a lane serves at most one chain per pass
             bool ok = true;
@@ -4142,6 +4181,7 @@ class Generator
             if (!ok || perLane == 0 || perLane * ph.passes > prefetchBudget) continue;
             prefetchBudget -= perLane * ph.passes;
             ph.prefetched = true;
+            anyLater = anyLater || pi > 0;
             // ACRO_HIP_PIPELINE=<n>: phases that hold at most n doubles per lane are carried across iterations (the
             // first phase always is: its inputs are what an iteration would otherwise start by waiting for)
             ph.carried = pipelined && (pi == 0 || perLane * ph.passes <= envInt("ACRO_HIP_PIPELINE"));
@@ -4197,7 +4237,7 @@ class Generator
         auto emitPrefetchLoads = [&](const Phase &ph) {
             for (long j = 0; j < ph.passes; ++j)
             {
-                emitItems(ph, j, [&](const Chain &c, const std::string &indent) {
+                auto loadsOf = [&](const Chain &c, const std::string &indent) {
                     for (int kk = c.first; kk <= c.last; ++kk)
                     {
                         if (c.loads[kk - c.first].empty()) continue;
@@ -4207,7 +4247,22 @@ class Generator
                         for (const auto &ld : c.loads[kk - c.first])
                             out << indent << c.names[kk - c.first][j].at(ld.first) << " = " << ld.second << ";\n";
                     }
-                });
+                };
+                // A phase of one chain: lanes past the last work item request the last item's operands instead of
+                // nothing.  The requests then sit in straight-line code, and the compiler can count exactly how
+                // many loads were issued after the ones an earlier phase waits for (behind a branch it has to assume
+                // none, and that phase would wait for everything that was prefetched).
+                if (ph.chains.size() == 1 && !guardBatch && envInt("ACRO_HIP_PREFETCH_CLAMP") >= 0)
+                {
+                    const Chain &c = ph.chains[0];
+                    out << "    {\n        const int w0 = tid + " << j * NT << ";\n";
+                    out << "        const int w = w0 < " << c.W << " ? w0 : " << c.W - 1 << ";\n";
+                    emitHeader(subs[c.first], "        ");
+                    loadsOf(c, "        ");
+                    out << "    }\n";
+                    continue;
+                }
+                emitItems(ph, j, loadsOf);
             }
         };
         for (auto &ph : phases)

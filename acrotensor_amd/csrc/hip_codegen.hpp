@@ -60,6 +60,8 @@
 //   ACRO_HIP_FORCE_TILE="8:;3:q,r"  kernel 8 of the group takes the empty register tile, kernel 3 the tile (q, r)
 //   ACRO_HIP_COLLAPSE=-1        offsets are sums over every lane index (runs of lane indices that an operand lays out in
 //                               the lanes' own order are not collapsed into one multiple of the item number)
+//   ACRO_HIP_WRITE_BATCH=-1     write-heavy launches whose results leave through LDS tiles keep their batch size
+//                               (default: twice the batch entries in workgroups of 512 lanes)
 //   ACRO_HIP_STAGE=-1           small invariant operands with lane-dependent addresses stay in device memory (not staged in LDS)
 //   ACRO_HIP_SPLIT_LANES=-1     one lane per batch entry also for kernels with one output per entry (no lane exchanges)
 //   ACRO_HIP_WAVE_UNIFORM=-1    no readfirstlane on the batch entry of wavefronts that hold items of one entry only
