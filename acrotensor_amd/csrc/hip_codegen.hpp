@@ -62,6 +62,15 @@
 //                               the lanes' own order are not collapsed into one multiple of the item number)
 //   ACRO_HIP_WRITE_BATCH=-1     write-heavy launches whose results leave through LDS tiles keep their batch size
 //                               (default: twice the batch entries in workgroups of 512 lanes)
+//   ACRO_HIP_OPERATOR_COMPONENTS=-1  operators applied to vectors with trailing component indices ("A_e_i_k = B_i_j X_e_j_k")
+//                               run through the generic schedule, not on the matrix cores
+//   ACRO_HIP_COPY_OUT_TILE=-1   a kernel on its own whose lanes each write a long run of outputs stores them itself instead of
+//                               through an LDS tile that the workgroup writes out in whole lines
+//   ACRO_HIP_ROW_SUMS=-1        an element matrix times an element vector with rows that are no multiple of four doubles runs as
+//                               written (lanes along the rows) instead of as products into LDS followed by row sums
+//   ACRO_HIP_PREFETCH_FIRST=-1 / ACRO_HIP_PREFETCH_CLAMP=-1 / ACRO_HIP_PREFETCH_PASSES=-1
+//                               the first phase's operands are not requested ahead of the prefetched ones / prefetch loads of
+//                               partly filled passes stay behind a branch / a first phase of several passes keeps its item loop
 //   ACRO_HIP_STAGE=-1           small invariant operands with lane-dependent addresses stay in device memory (not staged in LDS)
 //   ACRO_HIP_SPLIT_LANES=-1     one lane per batch entry also for kernels with one output per entry (no lane exchanges)
 //   ACRO_HIP_WAVE_UNIFORM=-1    no readfirstlane on the batch entry of wavefronts that hold items of one entry only

@@ -165,6 +165,12 @@ KERNEL_SHAPES = [
     ("A_e_i = B_e_i_i", [(1 << 20, 8, 8)], (1 << 20, 8)),
     ("A_e_q_j_k = B_q_i X_e_i_j_k", [(5, 4), (1 << 19, 4, 4, 4)], (1 << 19, 5, 4, 4)),
     ("A_e_i = B_i_j X_e_j", [(64, 64), (1 << 18, 64)], (1 << 18, 64)),
+    ("A_e_i_k = B_i_j X_e_j_k", [(64, 64), (1 << 16, 64, 3)], (1 << 16, 64, 3)),
+    ("A_e_i_k = B_i_j X_e_j_k", [(16, 16), (1 << 18, 16, 3)], (1 << 18, 16, 3)),
+    ("A_e_i = B_i_j X_e_j", [(7, 9), (1 << 21, 9)], (1 << 21, 7)),
+    ("A_e_i = B_i_j X_e_j", [(20, 5), (1 << 21, 5)], (1 << 21, 20)),
+    ("A_e_i = B_i_j X_e_j", [(27, 3), (1 << 21, 3)], (1 << 21, 27)),
+    ("A_e_i = B_i_j X_e_j", [(27, 27), (1 << 19, 27)], (1 << 19, 27)),
     ("S_i = A_n_i", [(1 << 20, 64)], (64,)),
     ("S_i = A_i_n", [(64, 1 << 20)], (64,)),
     ("A_i_j = B_j_i", [(8192, 8192)], (8192, 8192)),

@@ -429,7 +429,7 @@ def test_kernels_whose_schedule_follows_the_memory_access_pattern(at, engine, ch
     ("A_e = B_e_i_j C_e_i_j D_j", [(64, 6, 4), (64, 6, 4), (4,)]),
     ("A_e = B_i_e_j C_e_j", [(3, 50, 11), (50, 11)]),            # batch index in the middle of an operand
     ("A_e_i = B_e_i_j C_e_j", [(203, 16, 16), (203, 16)]),       # element matrix times element vector: 4 lanes per row
-    ("A_e_i += B_e_i_j C_e_j", [(35, 27, 27), (35, 27)]),        # odd row length, lanes 0 - 2 take a seventh term
+    ("A_e_i += B_e_i_j C_e_j", [(35, 20, 20), (35, 20)]),        # 20 terms over 4 lanes (rows of odd length: two steps through LDS)
     ("A_e_i = B_e_i_j C_e_j", [(9, 64, 64), (9, 64)]),           # 16 lanes per row, four passes per entry
     ("A_e_i_k = B_e_i_k_n", [(21, 3, 5, 100)]),                  # two lane indices next to the shared contraction
 ])
@@ -754,3 +754,65 @@ def test_operator_kernels_on_buffers_that_are_only_8_byte_aligned(at, engine, ch
     expected = np.zeros((E, n))
     checker.contract("A_e_i = B_i_j X_e_j", expected, B, X)
     assert rel_err(ha, expected) <= 1e-12
+
+
+@pytest.mark.parametrize("kernel,shapes,matrix_cores", [
+    ("A_e_i_k = B_i_j X_e_j_k", [(64, 64), (333, 64, 3)], True),            # 999 entries (e, k): ragged last trip
+    ("A_e_i_k += B_i_j X_e_j_k", [(16, 16), (1000, 16, 3)], True),
+    ("A_e_i_k -= B_j_i X_e_j_k", [(33, 20), (77, 33, 2)], True),            # operator stored transposed, padded to 32 x 36
+    ("A_e_q_i_k = B_i_j X_e_q_j_k", [(30, 17), (50, 4, 17, 5)], True),      # two leading indices, five components
+    ("A_e_i_k_l = B_i_j X_e_j_k_l", [(24, 24), (101, 24, 2, 3)], True),     # two component indices
+    ("A_e_i_k = B_i_j X_e_j_k", [(8, 8), (1000, 8, 3)], False),             # small operator: the generic schedule
+    ("A_e_i_k = B_i_j X_e_j_k W_e", [(32, 32), (100, 32, 3), (100,)], False),  # with a factor: the generic schedule
+])
+def test_dense_operator_with_trailing_components(at, engine, checker, kernel, shapes, matrix_cores):
+    """The vectors and the results carry component indices behind the operator's ("A_e_i_k = B_i_j X_e_j_k", a vector
+    field interpolated component by component): entries (e, k) with their elements a stride apart."""
+    rng = np.random.default_rng(shapes[0][0] + shapes[1][0])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    src = engine.GetLastImplementation()
+    assert ("operator schedule on the FP64 matrix cores" in src and "components per vector element" in src) == matrix_cores
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
+    # integer data: exact whatever the order of the sums
+    ins = [rng.integers(-3, 4, s).astype(np.float64) for s in shapes]
+    got, expected = run_single(at, engine, checker, kernel.replace("+=", "=").replace("-=", "="), np.zeros_like(out0), *ins)
+    assert np.array_equal(got, expected)
+
+
+@pytest.mark.parametrize("kernel,shapes", [
+    ("A_e_i = B_i_j X_e_j", [(27, 3), (1000, 3)]),                # 27 results per lane: written out through an LDS tile
+    ("A_e_i = B_i_j X_e_j", [(20, 5), (777, 5)]),                 # even run, last workgroup partly filled
+    ("A_e_i_k = B_i_k_j X_e_j", [(5, 3, 3), (333, 3)]),           # the run spans two output dimensions
+    ("A_e_i = X_e_j B_j_i", [(2, 9), (130, 2)]),
+])
+def test_long_output_runs_leave_through_an_lds_tile(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(shapes[1][0])
+    if kernel.startswith("A_e_i = X"):
+        shapes = [shapes[1], shapes[0]]
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "LDS tiles -> device memory" in engine.GetLastImplementation()
+    assert rel_err(got, expected) <= TOL
+
+
+@pytest.mark.parametrize("kernel,shapes", [
+    ("A_e_i = B_e_i_j C_e_j", [(300, 27, 27), (300, 27)]),        # rows of 27: products into LDS, then row sums
+    ("A_e_i += B_e_i_j C_e_j", [(77, 9, 25), (77, 25)]),
+    ("A_e_i -= C_e_j B_e_i_j", [(50, 33), (50, 12, 33)]),
+    ("A_e_i = B_e_i_j_k C_e_j_k", [(40, 6, 3, 7), (40, 3, 7)]),   # two contraction indices, 21 terms
+    ("A_e_i = B_e_i_j C_j", [(200, 27, 27), (27,)]),              # the vector shared by all entries
+])
+def test_element_matrix_times_vector_with_odd_rows(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(shapes[0][0])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "steps of:" in engine.GetLastImplementation()
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
