@@ -1,0 +1,573 @@
+// Kernel code generator, the model of a kernel group: operands, storages and views, what each kernel reads of what earlier kernels wrote, contraction ordering.
+#include "hip_codegen_impl.hpp"
+
+namespace acro
+{
+namespace codegen
+{
+
+auto Generator::BuildModel() -> void
+{
+    nidx = static_cast<int>(mk.LoopIndices.size());
+    idxName = mk.LoopIndices;
+    extent.assign(nidx, 1);
+    for (int i = 0; i < nidx; ++i) extent[i] = mk.GetLoopDim(i);
+
+    uvars.resize(NumOperands());
+    const int K = mk.GetNumKernels();
+    subs.resize(K);
+    for (int ki = 0; ki < K; ++ki)
+    {
+        DimensionedKernel *k = mk.Kernels[ki];
+        Sub &s = subs[ki];
+        s.text = k->KernelStr;
+        s.op = k->EqOperator[0] == '=' ? '=' : k->EqOperator[0];
+        auto makeRef = [&](int vari) {
+            VarRef r;
+            r.uvar = OperandOf(ki, vari);
+            const KernelVar &kv = k->GetVar(vari);
+            const int rank = static_cast<int>(kv.IndexNames.size());
+            r.idx.resize(rank);
+            r.ext.resize(rank);
+            r.stride.assign(rank, 1);
+            for (int d = 0; d < rank; ++d)
+            {
+                r.idx[d] = mk.GetIndexLoopNum(kv.IndexNames[d]);
+                r.ext[d] = k->GetLoopDim(kv.IndexNames[d]);
+                if (r.ext[d] != extent[r.idx[d]]) extentsConsistent = false;
+            }
+            for (int d = rank - 2; d >= 0; --d) r.stride[d] = r.stride[d + 1] * r.ext[d + 1];
+            r.size = 1;
+            for (int d = 0; d < rank; ++d) r.size *= r.ext[d];
+            std::set<int> distinct(r.idx.begin(), r.idx.end());
+            r.repeated = static_cast<int>(distinct.size()) != rank;
+            return r;
+        };
+        s.out = makeRef(-1);
+        for (int vari = 0; vari < k->GetNumInputVars(); ++vari) s.in.push_back(makeRef(vari));
+        for (int id : s.out.idx)
+        {
+            if (!has(s.outIdx, id)) s.outIdx.push_back(id);
+        }
+        for (const auto &name : k->ContractionIndexNames) s.contr.push_back(mk.GetIndexLoopNum(name));
+        s.contrCount = product(s.contr, extent);
+        if (!k->Function.empty())
+        {
+            s.matrixOp = k->Function == "inv" ? 1 : 2;
+            s.matrixN = s.in[0].ext.back();
+            ACROBATIC_ASSERT(s.in[0].ext[s.in[0].ext.size() - 2] == s.matrixN && s.matrixN <= 3,
+                             "HIP generator: a matrix kernel needs square matrices of at most 3 x 3.");
+        }
+    }
+
+    // The batch index: the largest index that every kernel carries and none contracts (they come sorted), but
+    // never a row or column index of a matrix kernel, whose matrices stay whole inside one work item.
+    for (const auto &name : mk.SharedOuterIndexNames)
+    {
+        const int id = mk.GetIndexLoopNum(name);
+        bool matrixIndex = false;
+        for (const auto &s : subs)
+        {
+            if (s.matrixOp == 0) continue;
+            const std::vector<int> &ids = s.in[0].idx;
+            matrixIndex = matrixIndex || id == ids[ids.size() - 1] || id == ids[ids.size() - 2];
+        }
+        if (matrixIndex) continue;
+        batch = id;
+        E = extent[batch];
+        break;
+    }
+
+    if (factorise && envInt("ACRO_HIP_FACTORISE") >= 0) FactoriseKernels();
+
+    // Unique-variable facts, in program order (a kernel reads its inputs before it writes its output).
+    for (int ki = 0; ki < static_cast<int>(subs.size()); ++ki)
+    {
+        const Sub &s = subs[ki];
+        auto note = [&](const VarRef &r, bool is_write) {
+            UVarInfo &u = uvars[r.uvar];
+            std::vector<int> bd;
+            for (size_t d = 0; d < r.idx.size(); ++d)
+            {
+                if (r.idx[d] == batch) bd.push_back(static_cast<int>(d));
+            }
+            if (u.lastUse < 0 && u.dims.empty())
+            {
+                u.dims = r.ext;
+                u.size = r.size;
+                u.batchDims = bd;
+            }
+            else if (u.dims != r.ext || u.batchDims != bd)
+            {
+                u.consistent = false;
+            }
+            u.anyRepeated = u.anyRepeated || r.repeated;
+            u.lastUse = ki;
+            if (is_write)
+            {
+                if (!u.written) u.firstWrite = ki;
+                u.written = true;
+            }
+
+        };
+        for (const auto &r : s.in) note(r, false);
+        if (s.op != '=') note(s.out, false);
+        note(s.out, true);
+    }
+    for (int u = 0; u < NumOperands(); ++u)
+    {
+        auto first = FirstOccurrence(u);
+        uvars[u].name = mk.Kernels[first.first]->GetVarName(first.second);
+    }
+    BuildStorages();
+    AnalyseCoverage();
+    // Element offsets into device memory are 32-bit unless some tensor of the group reaches 2^31 entries
+    // (16 GiB of doubles; the device holds 288 GB): then every device-memory offset is computed in 64 bits.
+    for (const auto &st : stores)
+    {
+        long entries = 1;
+        for (int d : st.dims) entries *= d;
+        if (entries >= (1L << 31) - 1) wide = true;
+    }
+}
+
+auto Generator::NonBatchVolume(const std::set<int> &ids) const -> double
+{
+    double v = 1.0;
+    for (int id : ids)
+    {
+        if (id != batch) v *= extent[id];
+    }
+    return v;
+}
+
+auto Generator::FactoriseSearch(const Sub &orig, std::vector<int> &live, std::vector<std::vector<int>> &idxOf, std::vector<int> &remaining, double cost, std::vector<FactorStep> &steps, double &best, long &bestSlowest, std::vector<FactorStep> &bestSteps, long &visits) const -> void
+{
+    if (++visits > 20000) return;
+    // Finish here: one kernel over everything that is left.
+    {
+        std::set<int> all(orig.outIdx.begin(), orig.outIdx.end());
+        for (int o : live) all.insert(idxOf[o].begin(), idxOf[o].end());
+        const double total = cost + NonBatchVolume(all) * static_cast<double>(live.size());
+        // Among equally cheap orders prefer the one whose last kernel introduces the slowest-varying output
+        // indices: they become its register tile, and the lanes then follow the fast output dimensions, which
+        // keeps the stores of a wavefront contiguous.
+        long slowest = 0;
+        const int nin = static_cast<int>(orig.in.size());
+        for (size_t d = 0; d < orig.out.idx.size(); ++d)
+        {
+            const int id = orig.out.idx[d];
+            bool inIntermediate = false, inInput = false;
+            for (int o : live) (o >= nin ? inIntermediate : inInput) |= has(idxOf[o], id);
+            if (id != batch && inInput && !inIntermediate) slowest = slowest == 0 ? orig.out.stride[d] : std::min<long>(slowest, orig.out.stride[d]);
+        }
+        if (total < best * (1.0 - 1e-9) || (total <= best * (1.0 + 1e-9) && slowest > bestSlowest))
+        {
+            best = total;
+            bestSlowest = slowest;
+            bestSteps = steps;
+        }
+    }
+    for (size_t ci = 0; ci < remaining.size(); ++ci)
+    {
+        const int c = remaining[ci];
+        std::vector<int> group, rest;
+        for (int o : live) (has(idxOf[o], c) ? group : rest).push_back(o);
+        if (rest.empty() || group.empty()) continue;  // that is the final kernel
+        std::set<int> all;
+        for (int o : group) all.insert(idxOf[o].begin(), idxOf[o].end());
+        FactorStep st;
+        st.group = group;
+        for (int id : remaining)
+        {
+            if (all.count(id) == 0) continue;
+            bool outside = false;
+            for (int o : rest) outside = outside || has(idxOf[o], id);
+            if (!outside) st.summed.push_back(id);
+        }
+        std::set<int> kept = all;
+        for (int id : st.summed) kept.erase(id);
+        if (kept.count(batch) == 0 || NonBatchVolume(kept) > static_cast<double>(maxVirtualTile)) continue;
+        const double stepCost = cost + NonBatchVolume(all) * static_cast<double>(group.size());
+        if (stepCost > best) continue;
+        // Storage order of the result: batch index, the output's indices in the output's order, then the
+        // contraction indices still open (read by the next step as literal offsets, unit stride innermost).
+        st.result.push_back(batch);
+        for (int id : orig.outIdx)
+        {
+            if (id != batch && kept.count(id)) st.result.push_back(id);
+        }
+        for (int id : orig.contr)
+        {
+            if (kept.count(id)) st.result.push_back(id);
+        }
+        std::vector<int> nextLive = rest, nextRemaining;
+        nextLive.push_back(static_cast<int>(idxOf.size()));
+        for (int id : remaining)
+        {
+            if (!has(st.summed, id)) nextRemaining.push_back(id);
+        }
+        idxOf.push_back(st.result);
+        steps.push_back(st);
+        FactoriseSearch(orig, nextLive, idxOf, nextRemaining, stepCost, steps, best, bestSlowest, bestSteps, visits);
+        steps.pop_back();
+        idxOf.pop_back();
+    }
+}
+
+// Every kernel of the group that qualifies is replaced by its steps (a kernel of a multi-kernel launch just as
+// a kernel launched alone).
+auto Generator::FactoriseKernels() -> void
+{
+    std::vector<Sub> expanded;
+    int counter = 0;
+    for (size_t ki = 0; ki < subs.size(); ++ki)
+    {
+        if (subs.size() == 1 && ProductThenRowSums(static_cast<int>(ki), subs[ki], expanded, counter)) continue;
+        if (!FactoriseKernel(static_cast<int>(ki), subs[ki], subs.size() == 1, expanded, counter)) expanded.push_back(subs[ki]);
+    }
+    subs.swap(expanded);
+}
+
+// An element matrix applied to an element vector, "A_e_i = B_e_i_j C_e_j", whose rows are not a multiple of four
+// doubles long (27 x 27): with the lanes along the rows, whether one lane or a few per row, a wavefront reads its
+// matrices in pieces of a row, 216 bytes apart (47 - 53 % of the HBM peak).  Evaluated in two steps instead: the
+// products "_F1_e_i_j = B_e_i_j C_e_j" with the lanes along the matrix as it lies in memory, into a tile in LDS,
+// then the sums over j, one lane per row (a row stride that is odd spreads the lanes over the banks).
+auto Generator::ProductThenRowSums(int ki, const Sub &orig, std::vector<Sub> &result, int &counter) -> bool
+{
+    if (envInt("ACRO_HIP_ROW_SUMS") < 0 || batch < 0 || orig.in.size() != 2 || orig.contr.empty() || !opt.noalias) return false;
+    if (orig.out.repeated || orig.matrixOp != 0) return false;
+    const VarRef *matrix = nullptr, *vec = nullptr;
+    for (const auto &r : orig.in)
+    {
+        if (r.repeated || r.uvar == orig.out.uvar) return false;
+        bool all = has(r.idx, batch);
+        for (int id : orig.outIdx) all = all && has(r.idx, id);
+        for (int id : orig.contr) all = all && has(r.idx, id);
+        if (all && matrix == nullptr)
+            matrix = &r;
+        else
+            vec = &r;
+    }
+    if (matrix == nullptr || vec == nullptr || matrix == vec) return false;
+    // the contraction indices are the matrix's fastest dimensions, the vector carries nothing but them and the batch
+    const size_t nc = orig.contr.size();
+    if (matrix->idx.size() < nc + 2 || matrix->idx[0] != batch) return false;
+    for (size_t d = 0; d < nc; ++d)
+    {
+        if (!has(orig.contr, matrix->idx[matrix->idx.size() - 1 - d])) return false;
+    }
+    for (int id : vec->idx)
+    {
+        if (id != batch && !has(orig.contr, id)) return false;
+    }
+    const long rows = product(orig.outIdx, extent) / extent[batch], row = orig.contrCount;
+    if (row % 4 == 0 || row < 9 || rows < 4 || rows * row > 4096 || row > 512) return false;
+
+    DimensionedKernel *kernel = mk.Kernels[ki];
+    auto refText = [&](const std::string &name, const std::vector<int> &ids) {
+        std::string t = name;
+        for (int id : ids) t += "_" + idxName[id];
+        return t;
+    };
+    UVarInfo info;
+    info.isVirtual = true;
+    info.name = "_F" + str(static_cast<long>(++counter));
+    VarRef res;
+    res.uvar = static_cast<int>(uvars.size());
+    res.idx = matrix->idx;
+    res.ext = matrix->ext;
+    res.stride = matrix->stride;
+    res.size = matrix->size;
+    uvars.push_back(info);
+
+    Sub prod;
+    prod.op = '=';
+    prod.out = res;
+    prod.outIdx = res.idx;
+    prod.in = orig.in;
+    prod.contrCount = 1;
+    prod.flatItems = true;
+    prod.text = refText(info.name, res.idx) + " =";
+    for (size_t v = 0; v < orig.in.size(); ++v) prod.text += " " + refText(kernel->GetVarName(static_cast<int>(v)), orig.in[v].idx);
+    result.push_back(prod);
+
+    Sub fin = orig;
+    fin.in.assign(1, res);
+    fin.text = refText(kernel->GetVarName(-1), orig.out.idx) + " " + (orig.op == '=' ? "=" : std::string(1, orig.op) + "=") + " " +
+               refText(info.name, res.idx) + "   (steps of: " + orig.text + ")";
+    result.push_back(fin);
+    factorised = true;
+    return true;
+}
+
+// Appends the steps of kernel ki to `result` and returns true, or returns false when the kernel stays as written.
+auto Generator::FactoriseKernel(int ki, const Sub &orig, bool alone, std::vector<Sub> &result, int &counter) -> bool
+{
+    const int nin = static_cast<int>(orig.in.size());
+    if (batch < 0 || nin < 3 || orig.contr.empty() || !opt.noalias || orig.out.repeated) return false;
+    if (alone && orig.contrCount >= kReductionMinContraction && product(orig.outIdx, extent) <= kReductionMaxOutputs)
+        return false;  // the reduction schedule serves it
+    for (const auto &r : orig.in)
+    {
+        if (r.repeated || r.uvar == orig.out.uvar) return false;
+    }
+    std::vector<int> live;
+    std::vector<std::vector<int>> idxOf;
+    for (int v = 0; v < nin; ++v)
+    {
+        live.push_back(v);
+        idxOf.push_back(orig.in[v].idx);
+    }
+    std::vector<int> remaining = orig.contr;
+    std::vector<FactorStep> steps, bestSteps;
+    double best = 1e300;
+    long visits = 0, bestSlowest = -1;
+    std::set<int> all(orig.outIdx.begin(), orig.outIdx.end());
+    all.insert(orig.contr.begin(), orig.contr.end());
+    const double asWritten = NonBatchVolume(all) * static_cast<double>(nin);
+    FactoriseSearch(orig, live, idxOf, remaining, 0.0, steps, best, bestSlowest, bestSteps, visits);
+    // ACRO_HIP_FACTORISE=2 (tests): reorder whenever any chain is cheaper at all, however small the kernel.
+    const bool eager = envInt("ACRO_HIP_FACTORISE") >= 2;
+    if (bestSteps.empty()) return false;
+    if (!eager && (asWritten < kFactoriseMinWork || best * kFactoriseMinGain > asWritten)) return false;
+
+    DimensionedKernel *kernel = mk.Kernels[ki];
+    auto refText = [&](const std::string &name, const std::vector<int> &ids) {
+        std::string t = name;
+        for (int id : ids) t += "_" + idxName[id];
+        return t;
+    };
+    std::vector<VarRef> refOf(orig.in.begin(), orig.in.end());
+    std::vector<std::string> textOf;
+    for (int v = 0; v < nin; ++v) textOf.push_back(refText(kernel->GetVarName(v), orig.in[v].idx));
+    std::vector<bool> used(nin, false);
+    for (size_t t = 0; t < bestSteps.size(); ++t)
+    {
+        const FactorStep &st = bestSteps[t];
+        UVarInfo info;
+        info.isVirtual = true;
+        info.name = "_F" + str(static_cast<long>(++counter));
+        VarRef res;
+        res.uvar = static_cast<int>(uvars.size());
+        res.idx = st.result;
+        for (int id : st.result) res.ext.push_back(extent[id]);
+        res.stride.assign(res.idx.size(), 1);
+        for (int d = static_cast<int>(res.idx.size()) - 2; d >= 0; --d) res.stride[d] = res.stride[d + 1] * res.ext[d + 1];
+        for (int x : res.ext) res.size *= x;
+        uvars.push_back(info);
+
+        Sub s;
+        s.op = '=';
+        s.out = res;
+        s.outIdx = st.result;
+        s.contr = st.summed;
+        s.contrCount = product(s.contr, extent);
+        s.text = refText(info.name, st.result) + " =";
+        for (int o : st.group)
+        {
+            s.in.push_back(refOf[o]);
+            s.text += " " + textOf[o];
+            used[o] = true;
+        }
+        result.push_back(s);
+        refOf.push_back(res);
+        textOf.push_back(refText(info.name, st.result));
+        used.push_back(false);
+    }
+    Sub fin = orig;
+    fin.in.clear();
+    fin.contr.clear();
+    fin.text = refText(kernel->GetVarName(-1), orig.out.idx) + " " + (orig.op == '=' ? "=" : std::string(1, orig.op) + "=");
+    for (size_t o = 0; o < refOf.size(); ++o)
+    {
+        if (used[o]) continue;
+        fin.in.push_back(refOf[o]);
+        fin.text += " " + textOf[o];
+    }
+    for (int id : orig.contr)
+    {
+        bool summedEarlier = false;
+        for (const auto &st : bestSteps) summedEarlier = summedEarlier || has(st.summed, id);
+        if (!summedEarlier) fin.contr.push_back(id);
+    }
+    fin.contrCount = product(fin.contr, extent);
+    fin.text += "   (steps of: " + orig.text + ")";
+    result.push_back(fin);
+    factorised = true;
+    return true;
+}
+
+auto Generator::BuildStorages() -> void
+{
+    const int U = static_cast<int>(uvars.size());
+    int nstore = 0;
+    for (int u = 0; u < U; ++u)
+    {
+        UVarInfo &op = uvars[u];
+        if (static_cast<size_t>(u) < opt.views.size() && opt.views[u].storage >= 0)
+        {
+            op.storage = opt.views[u].storage;
+            op.viewOffset = opt.views[u].offset;
+        }
+        else
+        {
+            op.storage = -1 - u;  // renumbered below
+        }
+    }
+    // Dense storage numbers in order of first appearance.
+    std::map<int, int> renumber;
+    for (int u = 0; u < U; ++u)
+    {
+        auto it = renumber.find(uvars[u].storage);
+        if (it == renumber.end()) it = renumber.emplace(uvars[u].storage, nstore++).first;
+        uvars[u].storage = it->second;
+    }
+    stores.assign(nstore, Storage());
+    for (int u = 0; u < U; ++u)
+    {
+        UVarInfo &op = uvars[u];
+        Storage &st = stores[op.storage];
+        const bool hasView = static_cast<size_t>(u) < opt.views.size() && !opt.views[u].root_dims.empty();
+        if (st.dims.empty())
+        {
+            st.dims = hasView ? opt.views[u].root_dims : op.dims;
+            st.stride.assign(st.dims.size(), 1);
+            for (int d = static_cast<int>(st.dims.size()) - 2; d >= 0; --d)
+                st.stride[d] = st.stride[d + 1] * st.dims[d + 1];
+        }
+        st.members.push_back(u);
+        st.written = st.written || op.written;
+        st.anyRepeated = st.anyRepeated || op.anyRepeated;
+        const bool tr = op.isVirtual || (static_cast<size_t>(u) < opt.transient.size() && opt.transient[u]);
+        st.transient = st.transient && tr;
+        if (op.written && (st.firstWrite < 0 || op.firstWrite < st.firstWrite)) st.firstWrite = op.firstWrite;
+
+        // The view must be "leading indices fixed, trailing dimensions kept" to be resolved exactly.
+        const int nfixed = static_cast<int>(st.dims.size()) - static_cast<int>(op.dims.size());
+        op.plainView = nfixed >= 0;
+        if (op.plainView)
+        {
+            for (size_t d = 0; d < op.dims.size(); ++d) op.plainView = op.plainView && st.dims[d + nfixed] == op.dims[d];
+            long rest = op.viewOffset;
+            op.fixed.assign(nfixed, 0);
+            for (int d = 0; d < nfixed; ++d)
+            {
+                op.fixed[d] = static_cast<int>(rest / st.stride[d]);
+                rest -= op.fixed[d] * st.stride[d];
+                op.plainView = op.plainView && op.fixed[d] < st.dims[d];
+            }
+            op.plainView = op.plainView && rest == 0;
+        }
+        if (!op.plainView || !op.consistent || op.batchDims.size() != 1)
+        {
+            st.elementLocal = false;
+        }
+        else
+        {
+            const int bd = op.batchDims[0] + nfixed;
+            if (st.batchDim < 0) st.batchDim = bd;
+            if (st.batchDim != bd) st.elementLocal = false;
+        }
+    }
+    for (auto &st : stores)
+    {
+        if (batch < 0 || st.batchDim < 0) st.elementLocal = false;
+        if (!st.elementLocal) continue;
+        st.tileSize = 1;
+        st.ldsStride.assign(st.dims.size(), 0);
+        for (int d = static_cast<int>(st.dims.size()) - 1; d >= 0; --d)
+        {
+            if (d == st.batchDim) continue;
+            st.ldsStride[d] = st.tileSize;
+            st.tileSize *= st.dims[d];
+        }
+    }
+}
+
+// Is the region "storage at fixed leading indices `fixed`" contained in the union of the written regions?
+auto Generator::Covered(const Storage &st, const std::vector<int> &fixed, const std::vector<std::vector<int>> &written) const -> bool
+{
+    for (const auto &w : written)
+    {
+        if (w.size() <= fixed.size() && std::equal(w.begin(), w.end(), fixed.begin())) return true;
+    }
+    const int next = static_cast<int>(fixed.size());
+    if (next >= static_cast<int>(st.dims.size()) || next == st.batchDim) return false;
+    bool finer = false;
+    for (const auto &w : written)
+    {
+        if (w.size() > fixed.size() && std::equal(fixed.begin(), fixed.end(), w.begin())) finer = true;
+    }
+    if (!finer) return false;
+    std::vector<int> sub = fixed;
+    sub.push_back(0);
+    for (int v = 0; v < st.dims[next]; ++v)
+    {
+        sub.back() = v;
+        if (!Covered(st, sub, written)) return false;
+    }
+    return true;
+}
+
+auto Generator::AnalyseCoverage() -> void
+{
+    const int K = static_cast<int>(subs.size());
+    std::vector<std::vector<std::vector<int>>> written(stores.size());
+    readCovered.assign(K, std::vector<bool>());
+    oldCovered.assign(K, false);
+    for (int k = 0; k < K; ++k)
+    {
+        const Sub &s = subs[k];
+        readCovered[k].assign(s.in.size(), false);
+        for (size_t v = 0; v < s.in.size(); ++v)
+        {
+            const UVarInfo &op = uvars[s.in[v].uvar];
+            const Storage &st = stores[op.storage];
+            readCovered[k][v] = st.elementLocal && op.plainView && Covered(st, op.fixed, written[op.storage]);
+        }
+        const UVarInfo &oo = uvars[s.out.uvar];
+        const Storage &so = stores[oo.storage];
+        oldCovered[k] = so.elementLocal && oo.plainView && Covered(so, oo.fixed, written[oo.storage]);
+        if (so.elementLocal && oo.plainView && !s.out.repeated) written[oo.storage].push_back(oo.fixed);
+    }
+}
+
+auto Generator::CheckFusable(std::string &why) -> bool
+{
+    if (mk.GetNumKernels() == 1) return true;  // a single kernel always has a private batch index
+    for (const auto &s : subs)
+    {
+        if (s.out.repeated && s.op == '=')
+        {
+            why = "an assigned output repeats an index and needs a zero fill between kernels";
+            return false;
+        }
+    }
+    if (batch < 0)
+    {
+        why = "the kernels share no outer index";
+        return false;
+    }
+    if (!extentsConsistent)
+    {
+        why = "an index name has different extents in different kernels";
+        return false;
+    }
+    for (const auto &st : stores)
+    {
+        // Everything that touches a written tensor must address it through the batch index in one fixed
+        // position, or one workgroup would depend on another's results.
+        if (st.written && !st.elementLocal)
+        {
+            why = "variable " + uvars[st.members[0]].name +
+                  " is written and used with different shapes, element positions or an unresolvable view";
+            return false;
+        }
+    }
+    return true;
+}
+
+}  // namespace codegen
+}  // namespace acro
