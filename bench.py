@@ -39,6 +39,12 @@ METRIC = "GDOF/s + % HBM peak, p=3 sum-factorised hex mass apply fp64 (1 GPU)"
 # function, first 16 hex digits of the SHA-1 of the generated source).  A generator change that alters the source of
 # a kernel therefore drops its figure (the line then says null) until the counters are taken again.
 TRAFFIC_BY_KERNEL = {
+    ("acro_mk_4ceea56515f0c53c", "7b71a034a2a078a5"): 542071433,            # cfg4, intermediates transient
+    ("acro_mk_664cf228dc3d274e", "c11ed22788401073"): 1818141896,           # cfg4, every intermediate stored
+    ("acro_red_35ac69981569e511_partial", "1698cfe138e16625"): 83941812,    # cfg1 (first of its two launches)
+    ("batchMatrixKernel<3,inv,det>", "a58afa41f95bd93a"): 637578061,        # cfg2 (precompiled: hash of hip_ops.hip)
+    ("acro_mk_c7f1f43821aef74f", "19c88bbbd31b17c8"): 208703100,            # cfg3
+    ("acro_mk_e688ac87da28a7bd", "018c1f37edc57625"): 5258855302,           # cfg5
 }
 
 
@@ -441,6 +447,38 @@ def all_configs(at, workloads, args):
     return block
 
 
+def cfg1_sizes(at, args):
+    """The batched reduction of configs[0] at other lengths n: per-step time by HIP events (both launches of the
+    split contraction), algorithmic GB/s, and what is left over the time the bytes need at 6.5 TB/s (the rate the
+    same kernel reaches at n = 2^24).  At n = 2048 the bytes are negligible: that row is the cost of the two dependent
+    launches alone."""
+    engine = at.TensorEngine("HIP")
+    rows = []
+    for n in (2048, 16384, 65536, 262144, 524288, 1 << 20, 1 << 21, 1 << 22, 1 << 24):
+        A, B, S = at.Tensor(n, 3, 3), at.Tensor(n), at.Tensor(3, 3)
+        for t in (A, B, S):
+            t.SwitchToGPU()
+            t.Set(1.0)
+        step = lambda: engine("S_i_j = A_n_i_j B_n", S, A, B)
+        for _ in range(50):
+            step()
+        at.synchronize()
+        steps = 500 if n <= (1 << 21) else 100
+        with at.hip_event_timer() as ev:
+            for _ in range(steps):
+                step()
+        us = ev.ms * 1e3 / steps
+        nbytes = (n * 10 + 9) * 8
+        rows.append({"n": n, "us_per_step": us, "GBps": nbytes / us * 1e-3, "frac": nbytes / us * 1e-3 / HBM_PEAK_GBS,
+                     "us_of_bytes_at_6500_GBps": nbytes / 6.5e6, "us_beyond_that": us - nbytes / 6.5e6})
+        del A, B, S
+    at_full = [r for r in rows if r["n"] == 1 << 20][0]
+    return {"metric": "cfg1 batched reduction at other lengths (1 GPU)", "value": at_full["GBps"], "unit": "GB/s", "n_gpus": 1,
+            "steps": 500, "warmup": 50, "ms_per_step": at_full["us_per_step"] * 1e-3, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+            "config": {"workload": "S_i_j = A_n_i_j B_n for n = 2^11 .. 2^24; value is the n = 2^20 row"}, "sizes": rows}
+
+
 def other_workload(at, workloads, args):
     name = args.workload
     engine, step, label, units, unit_name, abytes, flops = build_case(at, workloads, name)
@@ -471,7 +509,7 @@ def main():
     ap.add_argument("--no-store-all", action="store_true")
     ap.add_argument("--no-all-configs", action="store_true",
                     help="leave out the block with the other four baseline configurations")
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "scatter_apply", "scatter_then_apply", "operator", "dense_apply", "shapes"],
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "scatter_apply", "scatter_then_apply", "operator", "dense_apply", "shapes", "cfg1_sizes"],
                     help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
                          "remaining baseline configurations at their full sizes and for the node-vector <-> "
                          "element-vector steps either side of the operator apply")
@@ -491,6 +529,9 @@ def main():
 
     if args.workload == "shapes":
         print(json.dumps(kernel_shapes(at, args)))
+        return
+    if args.workload == "cfg1_sizes":
+        print(json.dumps(cfg1_sizes(at, args)))
         return
     if args.workload != "cfg4":
         print(json.dumps(other_workload(at, workloads, args)))
