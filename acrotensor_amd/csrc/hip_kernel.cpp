@@ -28,6 +28,19 @@ const char *const kCompileOptions[] = {
 };
 constexpr int kNumCompileOptions = sizeof(kCompileOptions) / sizeof(kCompileOptions[0]);
 
+// Experiment hook: further options for the run-time compiler, separated by blanks (ACRO_HIP_COMPILE_OPTIONS="-mllvm
+// -amdgpu-..."); they are part of the key of the on-disk cache.
+std::vector<std::string> extraCompileOptions()
+{
+    std::vector<std::string> extra;
+    const char *env = std::getenv("ACRO_HIP_COMPILE_OPTIONS");
+    if (env == nullptr) return extra;
+    std::istringstream words(env);
+    std::string word;
+    while (words >> word) extra.push_back(word);
+    return extra;
+}
+
 uint64_t fnv1a(const std::string &s, uint64_t h = 1469598103934665603ull)
 {
     for (unsigned char c : s)
@@ -73,6 +86,7 @@ std::string cachePath(const std::string &name, const std::string &source)
     hiprtcVersion(&major, &minor);
     std::string salt = std::to_string(major) + "." + std::to_string(minor);
     for (int i = 0; i < kNumCompileOptions; ++i) salt += std::string(" ") + kCompileOptions[i];
+    for (const std::string &option : extraCompileOptions()) salt += " " + option;
     uint64_t h = fnv1a(source, fnv1a(salt + name));
     char hex[32];
     std::snprintf(hex, sizeof(hex), "%016llx", static_cast<unsigned long long>(h));
@@ -136,7 +150,10 @@ void HipKernel::Compile()
     hiprtcProgram prog;
     rtcCheck(hiprtcCreateProgram(&prog, Source.c_str(), (FunctionName + ".hip").c_str(), 0, nullptr, nullptr),
              "hiprtcCreateProgram");
-    hiprtcResult result = hiprtcCompileProgram(prog, kNumCompileOptions, const_cast<const char **>(kCompileOptions));
+    const std::vector<std::string> extra = extraCompileOptions();
+    std::vector<const char *> options(kCompileOptions, kCompileOptions + kNumCompileOptions);
+    for (const std::string &option : extra) options.push_back(option.c_str());
+    hiprtcResult result = hiprtcCompileProgram(prog, static_cast<int>(options.size()), options.data());
     if (result != HIPRTC_SUCCESS)
     {
         size_t log_size = 0;
