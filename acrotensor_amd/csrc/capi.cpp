@@ -437,6 +437,9 @@ int acro_engine_contract_no_alloc(acro_engine *e, const char *kernel, acro_tenso
 {
     return guarded([&] {
         require(e != nullptr && kernel != nullptr && out != nullptr, "null argument");
+        // Inside a multi-kernel launch the call would only be recorded; the launch at its end is an ordinary one.
+        require(!e->te.InMultiKernelLaunch(),
+                "acro_engine_contract_no_alloc cannot be used between BeginMultiKernelLaunch and EndMultiKernelLaunch");
         std::vector<Tensor *> in = unwrap(inputs, num_inputs);
         double *ptr = scratchOnCurrentDevice();
         hip::NoAllocation scope(ptr, ACRO_NO_ALLOC_SCRATCH_DOUBLES);

@@ -66,6 +66,8 @@ class TensorEngine
     // (The reference runs them at once, kernel/TensorEngine.cpp:627-671; the order of operations is the same.)
     void BeginMultiKernelLaunch();
     void EndMultiKernelLaunch();
+    // True between BeginMultiKernelLaunch and EndMultiKernelLaunch: calls are being recorded, not run.
+    bool InMultiKernelLaunch() const { return IsMultiKernelLaunch; }
 
     // Ends a capture started by BeginMultiKernelLaunch WITHOUT executing it and returns the implementation the
     // launch would have used (needs no device).

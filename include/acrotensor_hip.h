@@ -114,7 +114,9 @@ int acro_engine_contract(acro_engine *e, const char *kernel, acro_tensor *out, a
  * array of ACRO_NO_ALLOC_SCRATCH_BYTES that the library holds on every device it runs on until the process ends; a
  * kernel that needs more is refused with a message.  All calls on a device share that array, which keeps the last
  * call's contents (the part a call uses is cleared first, on the stream): calls that overlap on one device, from
- * several threads or on several streams, race.  Results are bit-identical to acro_engine_contract's. */
+ * several threads or on several streams, race.  Results are bit-identical to acro_engine_contract's.  Not available
+ * between acro_engine_begin_multi_kernel_launch and acro_engine_end_multi_kernel_launch (there a call is only
+ * recorded, and the launch at the end is an ordinary one). */
 #define ACRO_NO_ALLOC_SCRATCH_BYTES (256u * 1024u)
 int acro_engine_contract_no_alloc(acro_engine *e, const char *kernel, acro_tensor *out, acro_tensor *const *inputs,
                                   int num_inputs);

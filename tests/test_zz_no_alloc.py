@@ -89,3 +89,21 @@ def test_refuses_more_scratch_than_the_array_holds(at, engine):
     S.MoveFromGPU()
     assert np.array_equal(S.data, expected)
     assert np.abs(expected - A.data.sum(axis=0)).max() <= 1e-12 * np.abs(expected).max()
+
+
+def test_refused_inside_a_multi_kernel_launch(at, engine):
+    # between Begin and End a call is only recorded, and the launch at End is an ordinary one that may allocate
+    A, B = make(at, 3000, 16)
+    S = at.Tensor(3, 3)
+    for t in (A, B, S):
+        t.MoveToGPU()
+    engine(KERNEL, S, A, B)
+    engine.BeginMultiKernelLaunch()
+    try:
+        with pytest.raises(at.AcroError, match="between BeginMultiKernelLaunch and EndMultiKernelLaunch"):
+            engine.contract_no_alloc(KERNEL, S, A, B)
+    finally:
+        engine.EndMultiKernelLaunch()
+    engine.contract_no_alloc(KERNEL, S, A, B)
+    S.MoveFromGPU()
+    assert np.abs(S.data - np.einsum("nij,n->ij", A.data, B.data)).max() <= 1e-12 * np.abs(S.data).max()
