@@ -178,9 +178,9 @@ def config3(E=32768, seed=0xAC23):
                     algorithmic_bytes=E * (64 + 729) * 8 + 96, flops=E * 729 * 64 * 7, seed=seed)
 
 
-def config4(E=262144, seed=0xAC24):
-    """p=3 sum-factorised hex mass operator apply as a 7-kernel chain."""
-    Q, P = 5, 4
+def config4(E=262144, seed=0xAC24, Q=5, P=4):
+    """Sum-factorised hex mass operator apply as a 7-kernel chain (degree p = P - 1 with Q points per direction; the
+    baseline configuration is p=3: Q, P = 5, 4)."""
     arrays = {
         "B": counter_uniform(seed, 0, (Q, P), -1.0, 1.0),
         "X": counter_uniform(seed, 1, (E, P, P, P), -1.0, 1.0),
@@ -198,9 +198,10 @@ def config4(E=262144, seed=0xAC24):
         ("V2_e_i_j_s = B_r_j V1_e_i_r_s", "V2", ["B", "V1"]),
         ("Y_e_i_j_k = B_s_k V2_e_i_j_s", "Y", ["B", "V2"]),
     ]
-    return Workload("cfg4_mass_apply_p3", arrays, kernels, transient=("T1", "T2", "T3", "U", "V1", "V2"),
+    flops_per_element = 2 * Q * P * (P * P + Q * P + Q * Q) * 2 + Q ** 3    # three stages each way + the pointwise product
+    return Workload("cfg4_mass_apply_p%d" % (P - 1), arrays, kernels, transient=("T1", "T2", "T3", "U", "V1", "V2"),
                     outputs=("Y",), dof=E * P ** 3, algorithmic_bytes=E * (P ** 3 + Q ** 3 + P ** 3) * 8,
-                    flops=E * 5005, seed=seed)
+                    flops=E * flops_per_element, seed=seed)
 
 
 def config5(E=65536, seed=0xAC25, Q=10, P=8):

@@ -71,6 +71,20 @@ def test_config4_mass_apply(at, engine, checker, E, transient):
             assert rel_err(fetch(tensors, name), expected[name]) <= TOL, name
 
 
+@pytest.mark.parametrize("E,Q,P", [(61, 3, 2), (45, 4, 3), (131, 5, 4), (26, 6, 5), (13, 7, 6), (7, 8, 7), (5, 9, 8), (3, 10, 9)])
+@pytest.mark.parametrize("transient", [False, True])
+def test_mass_apply_at_other_degrees(at, engine, checker, E, Q, P, transient):
+    # the same 7-kernel chain at degrees 1 - 8: element counts that leave the last workgroup partly filled, every
+    # intermediate stored (the batches that leave through LDS tiles) and transient (the prefetch rules)
+    wl = workloads.config4(E=E, Q=Q, P=P)
+    tensors = run_workload(at, engine, wl, transient)
+    expected = workloads.run_on_checker(wl, checker)
+    assert rel_err(fetch(tensors, "Y"), expected["Y"]) <= TOL
+    if not transient:
+        for name in wl.transient:
+            assert rel_err(fetch(tensors, name), expected[name]) <= TOL, name
+
+
 @pytest.mark.parametrize("E,Q,P", [(1, 5, 4), (5, 5, 4), (3, 10, 8), (23, 3, 2), (19, 4, 3), (7, 6, 5), (3, 7, 6)])
 @pytest.mark.parametrize("transient", [False, True])
 def test_config5_diffusion_apply(at, engine, checker, E, Q, P, transient):
