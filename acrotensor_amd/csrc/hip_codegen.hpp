@@ -71,6 +71,8 @@
 //   ACRO_HIP_PREFETCH_FIRST=-1 / ACRO_HIP_PREFETCH_CLAMP=-1 / ACRO_HIP_PREFETCH_PASSES=-1
 //                               the first phase's operands are not requested ahead of the prefetched ones / prefetch loads of
 //                               partly filled passes stay behind a branch / a first phase of several passes keeps its item loop
+//   ACRO_HIP_LDS_BOTH_ENDS=-1   LDS tiles are always placed first-fit from the bottom (default: from both ends of the region
+//                               when that lets one more workgroup live on a compute unit)
 //   ACRO_HIP_STAGE=-1           small invariant operands with lane-dependent addresses stay in device memory (not staged in LDS)
 //   ACRO_HIP_SPLIT_LANES=-1     one lane per batch entry also for kernels with one output per entry (no lane exchanges)
 //   ACRO_HIP_WAVE_UNIFORM=-1    no readfirstlane on the batch entry of wavefronts that hold items of one entry only

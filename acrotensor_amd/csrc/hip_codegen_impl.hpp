@@ -275,6 +275,7 @@ class Generator
     // Doubles of LDS that a storage's tiles take in a workgroup of nb batch entries.
     int LdsNeed(const Storage &st, int nb) const { return st.tileSize * (st.staged ? 1 : nb); }
     int PlaceLds(int nb);
+    int PlaceLdsFromBothEnds(int nb);
     void ChooseBatching();
     static long ConflictCycles(const std::vector<long> &addr);
     std::vector<long> LaneAddresses(const Sub &s, const VarRef &r, int nb) const;
