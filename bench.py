@@ -39,12 +39,12 @@ METRIC = "GDOF/s + % HBM peak, p=3 sum-factorised hex mass apply fp64 (1 GPU)"
 # function, first 16 hex digits of the SHA-1 of the generated source).  A generator change that alters the source of
 # a kernel therefore drops its figure (the line then says null) until the counters are taken again.
 TRAFFIC_BY_KERNEL = {
-    ("acro_mk_4ceea56515f0c53c", "7b71a034a2a078a5"): 542071433,            # cfg4, intermediates transient
-    ("acro_mk_664cf228dc3d274e", "c11ed22788401073"): 1818141896,           # cfg4, every intermediate stored
-    ("acro_red_35ac69981569e511_partial", "1698cfe138e16625"): 83941812,    # cfg1 (first of its two launches)
-    ("batchMatrixKernel<3,inv,det>", "a58afa41f95bd93a"): 637578061,        # cfg2 (precompiled: hash of hip_ops.hip)
-    ("acro_mk_c7f1f43821aef74f", "19c88bbbd31b17c8"): 208703100,            # cfg3
-    ("acro_mk_e688ac87da28a7bd", "018c1f37edc57625"): 5258855302,           # cfg5
+    ("acro_mk_4ceea56515f0c53c", "7b71a034a2a078a5"): 542211446,            # cfg4, intermediates transient
+    ("acro_mk_664cf228dc3d274e", "c11ed22788401073"): 1817938170,           # cfg4, every intermediate stored
+    ("acro_red_35ac69981569e511_partial", "1698cfe138e16625"): 83941894,    # cfg1 (first of its two launches)
+    ("batchMatrixKernel<3,inv,det>", "a58afa41f95bd93a"): 637576860,        # cfg2 (precompiled: hash of hip_ops.hip)
+    ("acro_mk_c7f1f43821aef74f", "19c88bbbd31b17c8"): 208702980,            # cfg3
+    ("acro_mk_e688ac87da28a7bd", "018c1f37edc57625"): 5258894366,           # cfg5
 }
 
 
@@ -597,6 +597,10 @@ def main():
         for name in wl.transient:
             tensors[name].SetTransient(False)
         n2 = max(10, args.steps // 4)
+        # The first launch compiles the other kernel while the device idles: settle again before timing.
+        workloads.launch(wl, engine, tensors)
+        at.synchronize()
+        settle_clocks(at, workloads, wl, engine, tensors, args.settle_seconds)
         wall2, dev2 = time_steps(at, workloads, wl, engine, tensors, n2, max(5, args.warmup // 4))
         stored_bytes = args.elements * (64 + 125 + 64 + 610) * 8
         moved = stored_bytes / (dev2 / n2) * 1e-9
