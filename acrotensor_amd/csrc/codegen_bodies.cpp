@@ -343,7 +343,7 @@ auto Generator::WaveStoreLineCoverage(int k) const -> double
             rest /= extent[s.lane[j]];
         }
         if (batch >= 0) value[batch] = static_cast<int>(w / s.laneCount);
-        const long tiles = s.loopMode ? 1 : s.tileCount;
+        const long tiles = s.tileCount;
         for (long t = 0; t < tiles; ++t)
         {
             long rem = t;
@@ -689,21 +689,42 @@ auto Generator::EmitLoopBody(int k, std::vector<std::string> &lines) -> void
     }
     Body body;
     EmitBases(k, body);
-    lines.push_back("// " + s.text + "   (contraction as counted loops)");
+    lines.push_back("// " + s.text + (s.tile.empty() ? "   (contraction as counted loops)" : "   (contraction as counted loops around a register tile)"));
     for (const auto &l : body.bases) lines.push_back(l);
-    lines.push_back("double sum = 0.0;");
-    std::string indent;
-    for (size_t j = 0; j < s.contr.size(); ++j)
+    const long tc = s.tileCount;
+    auto sumName = [&](long t) { return tc == 1 ? std::string("sum") : "sum_" + str(t); };
+    for (long t = 0; t < tc; ++t) lines.push_back("double " + sumName(t) + " = 0.0;");
+    // Which operands depend on the tile; the contraction indices that none of those carries go innermost, so that
+    // what a tile entry reads is invariant in the inner loops and stays in (scalar) registers across them.
+    std::vector<char> onTile(s.in.size(), 0);
+    for (size_t v = 0; v < s.in.size(); ++v)
     {
-        const std::string c = IdxVar(s.contr[j]);
-        if (j + 1 == s.contr.size()) lines.push_back(indent + "#pragma unroll 4");
-        lines.push_back(indent + "for (int " + c + " = 0; " + c + " < " + str(extent[s.contr[j]]) + "; ++" + c + ")");
+        for (int id : s.in[v].idx) onTile[v] = onTile[v] || has(s.tile, id);
+    }
+    std::vector<int> order, inner;
+    for (int c : s.contr)
+    {
+        bool carried = false;
+        for (size_t v = 0; v < s.in.size(); ++v) carried = carried || (onTile[v] && has(s.in[v].idx, c));
+        (carried || s.tile.empty() ? order : inner).push_back(c);
+    }
+    order.insert(order.end(), inner.begin(), inner.end());
+    std::string indent;
+    for (size_t j = 0; j < order.size(); ++j)
+    {
+        const std::string c = IdxVar(order[j]);
+        // Around a register tile only the innermost loop is unrolled: with every loop unrolled the compiler requests
+        // all scalar operands of all terms at once and spills them.
+        if (j + 1 == order.size())
+            lines.push_back(indent + (tc > 1 && extent[order[j]] <= 8 ? "#pragma unroll" : "#pragma unroll 4"));
+        else if (tc > 1)
+            lines.push_back(indent + "#pragma unroll 1");
+        lines.push_back(indent + "for (int " + c + " = 0; " + c + " < " + str(extent[order[j]]) + "; ++" + c + ")");
         lines.push_back(indent + "{");
         indent += "    ";
     }
-    std::string prod;
-    for (size_t v = 0; v < s.in.size(); ++v)
-    {
+    std::vector<int> value(nidx, 0);
+    auto operand = [&](size_t v) {
         const VarRef &r = s.in[v];
         const Source src = SourceOf(k, static_cast<int>(v));
         const bool lds = (src == kFromLds);
@@ -715,31 +736,67 @@ auto Generator::EmitLoopBody(int k, std::vector<std::string> &lines) -> void
             const long st = lds ? LdsStride(r.uvar, d) : r.stride[d];
             off += (off.empty() ? "" : " + ") + IdxVar(id) + " * " + (lds ? str(st) : Lit(st));
         }
-        if (off.empty()) off = "0";
-        std::string opnd;
-        if (src == kFromConstant)
-            opnd = ConstPtrName(r.uvar) + "[" + ScalarBase(r) + Lit(uvars[r.uvar].viewOffset) + " + " + off + "]";
-        else if (lds)
-            opnd = "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
-        else
-            opnd = GlobalRead(r.uvar, "o_k" + str(k) + "v" + str(v) + " + " + off);
-        prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
+        const long fixed = LiteralOffset(r, s, lds, value);  // the tile entry's part (contraction values are zero)
+        if (fixed != 0 || off.empty()) off += (off.empty() ? "" : " + ") + (lds ? str(fixed) : Lit(fixed));
+        if (src == kFromConstant) return ConstPtrName(r.uvar) + "[" + ScalarBase(r) + Lit(uvars[r.uvar].viewOffset) + " + " + off + "]";
+        if (lds) return "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
+        return GlobalRead(r.uvar, "o_k" + str(k) + "v" + str(v) + " + " + off);
+    };
+    std::string common;
+    for (size_t v = 0; v < s.in.size(); ++v)
+    {
+        if (onTile[v]) continue;
+        const std::string opnd = operand(v);
+        common = common.empty() ? opnd : "(" + common + " * " + opnd + ")";
     }
-    lines.push_back(indent + "sum += " + prod + ";");
-    for (size_t j = 0; j < s.contr.size(); ++j)
+    if (tc > 1 && !common.empty())
+    {
+        lines.push_back(indent + "const double common = " + common + ";");
+        common = "common";
+    }
+    for (long t = 0; t < tc; ++t)
+    {
+        long rem = t;
+        for (int j = static_cast<int>(s.tile.size()) - 1; j >= 0; --j)
+        {
+            value[s.tile[j]] = static_cast<int>(rem % extent[s.tile[j]]);
+            rem /= extent[s.tile[j]];
+        }
+        std::string prod = common;
+        for (size_t v = 0; v < s.in.size(); ++v)
+        {
+            if (!onTile[v]) continue;
+            const std::string opnd = operand(v);
+            prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
+        }
+        lines.push_back(indent + sumName(t) + " += " + prod + ";");
+    }
+    for (size_t j = 0; j < order.size(); ++j)
     {
         indent.resize(indent.size() - 4);
         lines.push_back(indent + "}");
     }
-    const std::string gaddr = PtrName(s.out.uvar) + "[o_k" + str(k) + "g]";
-    const std::string laddr = "lds[o_k" + str(k) + "l]";
-    if (s.op == '=')
-        lines.push_back("const double r = sum;");
-    else
-        lines.push_back(std::string("const double r = ") + (OldValueInLds(k) ? laddr : gaddr) +
-                        (s.op == '+' ? " + sum;" : " - sum;"));
-    if (NeedsLdsCopy(k)) lines.push_back(laddr + " = r;");
-    if (StoresToGlobal(k) && !CopiesOutFromLds(k)) lines.push_back(GlobalStore(k, gaddr, "r"));
+    for (long t = 0; t < tc; ++t)
+    {
+        long rem = t;
+        for (int j = static_cast<int>(s.tile.size()) - 1; j >= 0; --j)
+        {
+            value[s.tile[j]] = static_cast<int>(rem % extent[s.tile[j]]);
+            rem /= extent[s.tile[j]];
+        }
+        const long goff = LiteralOffset(s.out, s, false, value);
+        const long loff = StoreOf(s.out.uvar).inLds ? LiteralOffset(s.out, s, true, value) : 0;
+        const std::string gaddr = PtrName(s.out.uvar) + "[o_k" + str(k) + "g" + (tc > 1 ? " + " + Lit(goff) : std::string()) + "]";
+        const std::string laddr = "lds[o_k" + str(k) + "l" + (tc > 1 ? " + " + str(loff) : std::string()) + "]";
+        const std::string name = tc == 1 ? std::string("r") : "r_" + str(t);
+        if (s.op == '=')
+            lines.push_back("const double " + name + " = " + sumName(t) + ";");
+        else
+            lines.push_back("const double " + name + " = " + (OldValueInLds(k) ? laddr : gaddr) +
+                            (s.op == '+' ? " + " : " - ") + sumName(t) + ";");
+        if (NeedsLdsCopy(k)) lines.push_back(laddr + " = " + name + ";");
+        if (StoresToGlobal(k) && !CopiesOutFromLds(k)) lines.push_back(GlobalStore(k, gaddr, name));
+    }
 }
 
 }  // namespace codegen

@@ -160,6 +160,98 @@ auto Generator::LinesPerInstruction(const Sub &s, const VarRef &r, const std::ve
     return counted > 0 ? total / static_cast<double>(counted) : 1.0;
 }
 
+// A kernel far above the machine balance (hundreds of multiply-adds per double that moves) is bound by instruction
+// issue, not by memory, and a long contraction written out term by term keeps every operand of every term in a
+// register of its own (3D stiffness assembly step: 270 loads + 25 results per work item, 256 registers, spills).
+// Such a kernel runs its contraction as counted loops around a register tile: per term the operands that do not
+// depend on the tile are loaded and multiplied once, and every tile entry takes one multiply-add, with its own
+// operands from scalar registers where they do not depend on the lanes.  The tile is the candidate with the fewest
+// instructions per output; among equals the one made of the output's slowest dimensions, so that the lanes keep
+// the fastest ones and stores stay contiguous.  (Stiffness step S = B1 B2 F1 with 225 terms and 15 625 outputs per
+// element: 3 832 us with one output per lane, 1 644 us unrolled with the tile (i1, j1), see the schedule comment
+// of the generated kernel for what it runs as now.)
+auto Generator::ChooseLoopTile(Sub &s, const std::vector<int> &mid) const -> bool
+{
+    if (envInt("ACRO_HIP_LOOP_TILE") < 0 || batch < 0 || !opt.noalias) return false;
+    if (s.matrixOp != 0 || s.out.repeated || s.flatItems || s.contrCount < 32 || mid.empty()) return false;
+    const long nin = static_cast<long>(s.in.size());
+    double moved = static_cast<double>(s.out.size) / static_cast<double>(E);
+    for (const auto &r : s.in)
+    {
+        if (r.repeated || r.uvar == s.out.uvar) return false;
+        if (has(r.idx, batch)) moved += static_cast<double>(r.size) / static_cast<double>(E);
+    }
+    const double outputs = static_cast<double>(product(mid, extent));
+    const double macs = outputs * static_cast<double>(s.contrCount) * static_cast<double>(std::max<long>(1, nin - 1));
+    if (macs < 64.0 * moved) return false;
+    // Where every operand carries few of the contraction indices ("M = B_q_i B_q_l B_r_j B_r_m B_s_k B_s_n W_q_r_s"),
+    // the unrolled body shares partial sums between the terms of one lane, which a loop cannot: that form stays.
+    long carried = 0;
+    for (const auto &r : s.in)
+    {
+        for (int c : s.contr) carried += has(r.idx, c) ? 1 : 0;
+    }
+    if (10 * carried < 7 * nin * static_cast<long>(s.contr.size())) return false;
+
+    auto perOutput = [&](const std::vector<int> &t) {
+        const long tc = product(t, extent);
+        long common = 0, commonLoads = 0, perEntry = 1;
+        for (const auto &r : s.in)
+        {
+            bool onTile = false;
+            for (int id : r.idx) onTile = onTile || has(t, id);
+            const bool uniform = IsUniform(s, r, t);
+            if (!onTile)
+            {
+                ++common;
+                if (!uniform) ++commonLoads;
+            }
+            else
+            {
+                perEntry += uniform ? 0 : 1;  // its load
+                ++perEntry;                    // its multiplication
+            }
+        }
+        if (common == 0) --perEntry;  // nothing to multiply the first tile operand with
+        const double perTerm = static_cast<double>(commonLoads + std::max<long>(0, common - 1)) + static_cast<double>(tc * perEntry);
+        return perTerm / static_cast<double>(tc);
+    };
+    const double flat = perOutput({});
+    std::vector<std::vector<int>> candidates;
+    for (size_t a = 0; a < mid.size(); ++a)
+    {
+        candidates.push_back({mid[a]});
+        for (size_t b = a + 1; b < mid.size(); ++b) candidates.push_back({mid[a], mid[b]});
+    }
+    double best = 0.5 * flat;  // worth it from half the instructions on
+    long bestPosition = 0;
+    std::vector<int> tile;
+    for (const auto &t : candidates)
+    {
+        const long tc = product(t, extent);
+        if (tc < 2 || tc > kMaxTile || product(mid, extent) / tc < 64) continue;
+        long position = 0;
+        for (int id : t)
+        {
+            for (size_t d = 0; d < s.out.idx.size(); ++d)
+            {
+                if (s.out.idx[d] == id) position += static_cast<long>(d);
+            }
+        }
+        const double cost = perOutput(t);
+        if (cost < best - 1e-9 || (std::fabs(cost - best) <= 1e-9 && !tile.empty() && position < bestPosition))
+        {
+            best = cost;
+            bestPosition = position;
+            tile = t;
+        }
+    }
+    if (tile.empty()) return false;
+    s.tile = tile;
+    s.loopMode = true;
+    return true;
+}
+
 auto Generator::ChooseTiles() -> void
 {
     for (auto &s : subs)
@@ -178,6 +270,10 @@ auto Generator::ChooseTiles() -> void
             s.loopMode = false;
             s.tile.clear();
             if (s.matrixOp == 1) s.tile.assign(s.out.idx.end() - 2, s.out.idx.end());
+        }
+        else if (ChooseLoopTile(s, mid))
+        {
+            // counted loops around a register tile
         }
         else if (s.contrCount > kMaxUnrolledContraction || s.contrCount * nin > kUnrollBudget)
         {
@@ -806,7 +902,7 @@ auto Generator::ChooseBatching() -> void
         // Larger workgroups leave fewer registers per lane (128 at 1 024 lanes, 256 at 512): size them by the
         // values a lane holds at once.
         long live = 0;
-        for (const auto &s : subs) live = std::max(live, s.loopMode ? 8 : LoadsPerItem(s, s.tile) + s.tileCount);
+        for (const auto &s : subs) live = std::max(live, s.loopMode ? 8 + s.tileCount : LoadsPerItem(s, s.tile) + s.tileCount);
         const long cap = live <= 48 ? 1024 : (live <= 100 ? 512 : 256);
         if (streaming && maxLane > 256) NT = static_cast<int>(std::min<long>(cap, (maxLane + 63) / 64 * 64));
     }

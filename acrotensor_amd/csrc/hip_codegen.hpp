@@ -73,6 +73,8 @@
 //                               partly filled passes stay behind a branch / a first phase of several passes keeps its item loop
 //   ACRO_HIP_LDS_BOTH_ENDS=-1   LDS tiles are always placed first-fit from the bottom (default: from both ends of the region
 //                               when that lets one more workgroup live on a compute unit)
+//   ACRO_HIP_LOOP_TILE=-1       kernels far above the machine balance keep their unrolled body or a plain counted loop (default:
+//                               counted loops around a register tile, see ChooseLoopTile)
 //   ACRO_HIP_STAGE=-1           small invariant operands with lane-dependent addresses stay in device memory (not staged in LDS)
 //   ACRO_HIP_SPLIT_LANES=-1     one lane per batch entry also for kernels with one output per entry (no lane exchanges)
 //   ACRO_HIP_WAVE_UNIFORM=-1    no readfirstlane on the batch entry of wavefronts that hold items of one entry only

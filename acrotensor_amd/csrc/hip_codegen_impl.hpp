@@ -247,6 +247,7 @@ class Generator
     static constexpr long kMaxLiveValues = 160;   // loaded operands + accumulators held by one lane
     static constexpr long kPrefetchDoubles = 48;  // per lane, held in registers from kernel entry to their phase
     void ChooseTiles();
+    bool ChooseLoopTile(Sub &s, const std::vector<int> &mid) const;
     void ForcedTile(int k, const std::vector<int> &mid, std::vector<int> &tile) const;
     void SetLanes(Sub &s);
     bool ForwardableFrom(const Sub &q, const VarRef &r, const std::vector<int> &lane) const;

@@ -351,6 +351,25 @@ def build_case(at, workloads, name):
         label = "Y[524288,27] = Bt (D o (B X)), B[64,27], D[524288,64]: dense element operator in one launch"
         abytes, flops = (E * (nd + nq + nd) + nq * nd) * 8, E * (4 * nq * nd + nq)
         units, unit_name = E * nd, "GDOF/s"
+    elif name == "stiffness":
+        # 3D stiffness matrix assembly, the 12-loop kernel of the reference's tests
+        # (unittest/kernel/test_TensorEngine.cpp:437-496) at 8 192 elements: 1 125 terms of 4 factors per output as
+        # written; `flops` counts the arithmetic of the two steps it is evaluated as (k3 first, then 225 terms per
+        # output: one product shared by a 5 x 5 tile of outputs and one multiply-add per output)
+        E = 8192
+        S, D = at.Tensor(E, 5, 5, 5, 5, 5, 5), at.Tensor(E, 5, 5, 5, 3, 3)
+        tables = [at.Tensor(5, 5, 5, 3, 3) for _ in range(3)]
+        for i, t in enumerate(tables):
+            t.data[...] = workloads.counter_uniform(0xAC2A, i, (5, 5, 5, 3, 3), -1.0, 1.0)
+        D.data[...] = workloads.counter_uniform(0xAC2A, 3, (E, 5, 5, 5, 3, 3), 0.5, 1.5)
+        for t in tables + [S, D]:
+            t.MoveToGPU()
+        k = "S_e_i1_i2_i3_j1_j2_j3 = B1_i1_j1_k1_m_n B2_i2_j2_k2_m_n B3_i3_j3_k3_m_n D_e_k1_k2_k3_m_n"
+        step = lambda: engine(k, S, tables[0], tables[1], tables[2], D)
+        label = "3D stiffness assembly S[8192,5,5,5,5,5,5] from three tables [5,5,5,3,3] and D[8192,5,5,5,3,3]"
+        abytes = (E * (15625 + 1125) + 3 * 1125) * 8
+        flops = E * (5625 * 5 * 2 + 625 * 225 * (1 + 2 * 25))
+        units, unit_name = E * 15625, "Gentries/s"
     elif name in ("scatter", "sumgather"):
         # node vector <-> element vector of the headline mesh size: 64^3 hex elements of degree 3
         import numpy as np
@@ -495,6 +514,10 @@ def other_workload(at, workloads, args):
         "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic", "config": {"workload": label},
         "gflops_as_written": flops / launch_s * 1e-9, "roofline": roofline,
     }
+    if name == "stiffness":
+        # this one is bound by arithmetic, not by memory: say so beside the HBM figures
+        result["gflops_as_evaluated"] = result.pop("gflops_as_written")
+        result["fp64_vector_peak_frac"] = flops / launch_s * 1e-9 / FP64_PEAK_GFLOPS
     if name in ("cfg1", "cfg2", "cfg3", "cfg5") and not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_for(name, workloads)
     return result
@@ -513,7 +536,7 @@ def main():
     ap.add_argument("--no-store-all", action="store_true")
     ap.add_argument("--no-all-configs", action="store_true",
                     help="leave out the block with the other four baseline configurations")
-    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "scatter_apply", "scatter_then_apply", "operator", "dense_apply", "shapes", "cfg1_sizes"],
+    ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "scatter_apply", "scatter_then_apply", "operator", "dense_apply", "stiffness", "shapes", "cfg1_sizes"],
                     help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
                          "remaining baseline configurations at their full sizes and for the node-vector <-> "
                          "element-vector steps either side of the operator apply")

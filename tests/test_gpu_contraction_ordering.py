@@ -173,3 +173,58 @@ def test_kernel_inside_a_multi_kernel_launch_is_reordered_too(at, engine, checke
     if not transient:
         M.MoveFromGPU()
         assert rel_err(M.data, expM) <= TOL
+
+
+# Kernels far above the machine balance (long contractions that every operand carries, many outputs): the contraction
+# runs as counted loops around a register tile, tile operands from scalar registers where they do not depend on lanes.
+LOOPED_TILE = [
+    ("A_e_i_j_p_q = I0_p_k I1_i_k I2_q_k I3_e_k I4_j_k", [(7, 50), (4, 50), (4, 50), (33, 50), (8, 50)]),
+    ("A_e_i_j_p_q = I0_k_l_m_j I1_p_k_l_m I2_e_k_l_m I3_k_l_m_q I4_i_k_l_m", [(4, 7, 6, 6), (6, 4, 7, 6), (18, 4, 7, 6), (4, 7, 6, 3), (5, 4, 7, 6)]),
+    ("A_i_e_j_p_q = I0_q_k_l I1_e_k_l I2_p_k_l I3_j_k I4_i_k_l", [(2, 8, 7), (8, 8, 7), (8, 8, 7), (3, 8), (4, 8, 7)]),
+    ("A_e_i_j_p_q = I0_j_k I1_i_k I2_e_k_q I3_p_k", [(3, 76), (6, 76), (16, 76, 6), (4, 76)]),
+    ("A_e_i_j_p_q = I0_e_k_l_q I1_q_k_l I2_k_l_i I3_k_l_j I4_p_k_l", [(26, 6, 6, 7), (7, 6, 6), (6, 6, 7), (6, 6, 8), (6, 6, 6)]),
+    ("A_e_i_j_p_q = I0_l_q I1_p_k_l I2_e_k_l_q I3_k_l_j I4_i_l", [(7, 8), (4, 6, 7), (7, 6, 7, 8), (6, 7, 4), (3, 7)]),
+]
+
+
+@pytest.mark.parametrize("op", ["=", "+=", "-="])
+@pytest.mark.parametrize("kernel,shapes", LOOPED_TILE)
+def test_compute_bound_kernel_loops_around_a_register_tile(at, engine, checker, kernel, shapes, op):
+    kernel = kernel.replace(" = ", " %s " % op)
+    rng = np.random.default_rng(len(kernel) * 11 + len(op))
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    init = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, init, *ins)
+    assert "around a register tile" in engine.GetLastImplementation()
+    if op == "-=":
+        expected = init - (expected - init)
+    assert rel_err(got, expected) <= TOL
+
+
+@pytest.mark.parametrize("transient", [False, True])
+def test_stiffness_assembly_step_loops_around_a_register_tile(at, engine, checker, transient):
+    # 3D stiffness assembly (reference unittest/kernel/test_TensorEngine.cpp:437-496): the k3 sum first, then 225 terms
+    # per output around a 5 x 5 tile of outputs with one table in scalar registers; followed here by a pointwise kernel
+    # that reads the result (from device memory: 15 625 outputs per element are no LDS tile)
+    k = "S_e_i1_i2_i3_j1_j2_j3 = B1_i1_j1_k1_m_n B2_i2_j2_k2_m_n B3_i3_j3_k3_m_n D_e_k1_k2_k3_m_n"
+    rng = np.random.default_rng(5)
+    E = 3
+    tables = [rng.integers(-2, 3, (5, 5, 5, 3, 3)).astype(np.float64) for _ in range(3)]
+    D = rng.integers(-2, 3, (E, 5, 5, 5, 3, 3)).astype(np.float64)
+    W = rng.integers(-2, 3, (E, 5, 5, 5, 5, 5, 5)).astype(np.float64)
+    tS, tZ = at.Tensor(E, 5, 5, 5, 5, 5, 5), at.Tensor(E, 5, 5, 5, 5, 5, 5)
+    tS.SetTransient(transient)
+    tin = [to_tensor(at, a) for a in tables + [D]]
+    tW = to_tensor(at, W)
+    engine.BeginMultiKernelLaunch()
+    engine(k, tS, *tin)
+    engine("Z_e_i1_i2_i3_j1_j2_j3 = S_e_i1_i2_i3_j1_j2_j3 W_e_i1_i2_i3_j1_j2_j3", tZ, tS, tW)
+    engine.EndMultiKernelLaunch()
+    assert "around a register tile" in engine.GetLastImplementation()
+    expected = np.zeros((E, 5, 5, 5, 5, 5, 5))
+    checker.contract(k, expected, *tables, D)
+    tZ.MoveFromGPU()
+    assert np.array_equal(tZ.data, expected * W)          # small integers: exact
+    if not transient:
+        tS.MoveFromGPU()
+        assert np.array_equal(tS.data, expected)
