@@ -328,10 +328,11 @@ auto Generator::StreamsOut(int k) const -> bool
 // How much of the 128-byte lines that one store instruction of kernel k touches does it fill, on average over
 // the instructions of the first wavefront?  A lane's stores to consecutive addresses are counted as one
 // instruction per pair of doubles (the compiler merges them into 16-byte stores).
-auto Generator::WaveStoreLineCoverage(int k) const -> double
+auto Generator::WaveStoreLineCoverage(int k, int entries) const -> double
 {
     const Sub &s = subs[k];
-    const long items = std::min<long>(64, static_cast<long>(NB) * s.laneCount);
+    // (entries > 0: for that many batch entries per workgroup instead of the number chosen, for use before it is)
+    const long items = std::min<long>(64, static_cast<long>(entries > 0 ? entries : NB) * s.laneCount);
     std::vector<std::vector<long>> perLane(items);
     for (long w = 0; w < items; ++w)
     {

@@ -695,16 +695,23 @@ auto Generator::ComputeLdsWishes() -> void
 // of the tensor, in whole lines.
 auto Generator::ChooseCopyOutTile() -> void
 {
-    if (subs.size() != 1 || envInt("ACRO_HIP_COPY_OUT_TILE") < 0 || envInt("ACRO_HIP_LDS_COPY_OUT") < 0 || envInt("ACRO_HIP_PERSIST") > 0) return;
-    const Sub &s = subs[0];
+    if (envInt("ACRO_HIP_COPY_OUT_TILE") < 0 || envInt("ACRO_HIP_LDS_COPY_OUT") < 0 || envInt("ACRO_HIP_PERSIST") > 0) return;
+    // the kernel that writes the group's last result (for a kernel evaluated in steps: its last step)
+    const int k = static_cast<int>(subs.size()) - 1;
+    const Sub &s = subs[k];
     if (s.loopMode || s.matrixOp != 0 || s.op != '=' || s.out.repeated || s.splitLanes != 0 || s.tile.empty()) return;
     const UVarInfo &u = uvars[s.out.uvar];
     Storage &st = stores[u.storage];
     if (!st.elementLocal || st.anyRepeated || st.members.size() != 1 || st.batchDim != 0 || !u.fixed.empty() || u.viewOffset != 0 || st.transient) return;
-    for (const auto &r : s.in)
+    for (int j = 0; j <= k; ++j)
     {
-        if (uvars[r.uvar].storage == u.storage) return;
+        if (j != k && uvars[subs[j].out.uvar].storage == u.storage) return;
+        for (const auto &r : subs[j].in)
+        {
+            if (uvars[r.uvar].storage == u.storage) return;
+        }
     }
+    if (st.tileSize > envInt("ACRO_HIP_COPY_OUT_MAX", 2048)) return;
     // the run of consecutive outputs of one work item: the trailing output dimensions that are tile indices
     long run = 1;
     for (size_t d = s.out.idx.size(); d-- > 0;)
@@ -712,12 +719,22 @@ auto Generator::ChooseCopyOutTile() -> void
         if (!has(s.tile, s.out.idx[d])) break;
         run *= s.out.ext[d];
     }
-    // and the lanes must not interleave at a finer grain (a lane index in the fastest dimension would)
-    if (run < 8 || st.tileSize > 2048) return;
+    // Long runs per lane, or (any group) store instructions that fill less than 30 % of the lines they touch because
+    // the register tile sits between the lanes' dimensions: 2D mass assembly "M_e_i1_i2_j1_j2 = B B B B D_e_k1_k2" with
+    // lanes (i2, j2) and tile (i1, j1) writes pieces of 32 bytes 128 bytes apart (52 % of the HBM peak; through the
+    // tile see the schedule comment).
+    bool scattered = false;
+    if (run < 8 && envInt("ACRO_HIP_COPY_OUT_TILE") < 2)
+    {
+        const int entries = static_cast<int>(std::max<long>(1, 64 / std::max<long>(1, s.laneCount)));
+        scattered = s.laneCount >= 2 && WaveStoreLineCoverage(k, entries) < 0.3;
+    }
+    if (subs.size() != 1 && !scattered) return;
+    if (run < 8 && !scattered) return;
     st.copyOutOnly = true;
     st.wantLds = true;
-    st.liveTo = 0;
-    st.phaseFrom = st.phaseTo = 0;
+    st.liveTo = k;
+    st.phaseFrom = st.phaseTo = PhaseOf(k);
 }
 
 auto Generator::ChooseStagedInputs() -> void

@@ -64,8 +64,10 @@
 //                               (default: twice the batch entries in workgroups of 512 lanes)
 //   ACRO_HIP_OPERATOR_COMPONENTS=-1  operators applied to vectors with trailing component indices ("A_e_i_k = B_i_j X_e_j_k")
 //                               run through the generic schedule, not on the matrix cores
-//   ACRO_HIP_COPY_OUT_TILE=-1   a kernel on its own whose lanes each write a long run of outputs stores them itself instead of
-//                               through an LDS tile that the workgroup writes out in whole lines
+//   ACRO_HIP_COPY_OUT_TILE=-1|2 -1: results are always stored by the lanes that computed them; 2: an LDS tile that the workgroup
+//                               writes out in whole lines only for a kernel on its own whose lanes each hold a long run of outputs
+//                               (default: also for the last kernel of any group whose store instructions would fill less than
+//                               30 % of the lines they touch).  ACRO_HIP_COPY_OUT_MAX=<doubles per batch entry> (default 2048)
 //   ACRO_HIP_ROW_SUMS=-1        an element matrix times an element vector with rows that are no multiple of four doubles runs as
 //                               written (lanes along the rows) instead of as products into LDS followed by row sums
 //   ACRO_HIP_PREFETCH_FIRST=-1 / ACRO_HIP_PREFETCH_CLAMP=-1 / ACRO_HIP_PREFETCH_PASSES=-1

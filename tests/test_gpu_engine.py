@@ -193,6 +193,22 @@ def test_3d_stiffness_twelve_loops(at, engine, checker):
     assert np.array_equal(got, expected)          # all terms are multiples of 0.5 below 2^53: exact
 
 
+@pytest.mark.parametrize("P,Q,E", [(2, 3, 1001), (4, 5, 203), (3, 4, 77), (8, 10, 5)])
+def test_2d_mass_assembly_results_leave_through_an_lds_tile(at, engine, checker, P, Q, E):
+    # unittest/kernel/test_TensorEngine.cpp:399-435 at other sizes.  With lanes (i2, j2) / (j1, j2) and a register tile
+    # in between, a store instruction would write pieces of a few doubles far apart: the results go to an LDS tile
+    # and the workgroup writes the tile out in whole lines (also for the kernel evaluated in two steps).
+    k = "M_e_i1_i2_j1_j2=B_k1_i1 B_k1_j1 B_k2_i2 B_k2_j2 D_e_k1_k2"
+    rng = np.random.default_rng(P * 100 + Q)
+    B = rng.integers(-2, 3, (Q, P)).astype(np.float64)
+    D = rng.integers(-3, 4, (E, Q, Q)).astype(np.float64)
+    got, expected = run_single(at, engine, checker, k, np.full((E, P, P, P, P), 7.0), B, B, B, B, D)
+    assert np.array_equal(got, expected)                      # small integers: exact whatever the order of the sums
+    assert np.array_equal(got, np.einsum("ai,aj,bk,bl,eab->eikjl", B, B, B, B, D))
+    if (P, Q) in ((2, 3), (4, 5)):
+        assert "M->lds+global" in engine.GetLastImplementation()
+
+
 @pytest.mark.parametrize("order", [1, 4])
 def test_d_tensor_construction(at, engine, checker, order):
     # unittest/kernel/test_TensorEngine.cpp:498-590
