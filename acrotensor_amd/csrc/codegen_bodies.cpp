@@ -602,6 +602,32 @@ auto Generator::EmitMatrixBody(int k, Body &body, ForwardMap &forwarded) -> void
 }
 
 // Counted-loop body (long contractions): one output per work item, no tile.
+// Lanes that share a contraction take its terms two at a time when the one contraction index is the fastest
+// dimension of every operand that carries it: one 16-byte load per operand and pair instead of two 8-byte loads (a
+// matrix of 2^20 rows of 64 times a shared vector: 59.8 % of the HBM peak with single terms; see the schedule comment
+// of the generated kernel for what it takes now).  ACRO_HIP_SPLIT_PAIRS=-1 switches that off.
+auto Generator::SplitLanesTakePairs(int k) const -> bool
+{
+    const Sub &s = subs[k];
+    if (s.splitLanes <= 0 || envInt("ACRO_HIP_SPLIT_PAIRS") < 0 || s.contr.size() != 1) return false;
+    if (s.contrCount % 2 != 0 || s.contrCount < 2L * s.splitLanes) return false;
+    // Long rows stream better term by term, eight 8-byte loads in flight per lane (rows of 1 024: 75.3 against 73.5 % of
+    // the HBM peak, four rows of 256: 76.6 against 74.7 %); the pairs pay where a lane has few terms (16 x 16 element
+    // matrix times vector 69.3 -> 76.4 %, 64 x 64 71.0 -> 72.0 %).
+    if (s.contrCount > 8L * s.splitLanes) return false;
+    bool any = false;
+    for (size_t v = 0; v < s.in.size(); ++v)
+    {
+        const VarRef &r = s.in[v];
+        if (!has(r.idx, s.contr[0])) continue;
+        const Source src = SourceOf(k, static_cast<int>(v));
+        if ((src != kFromGlobal && src != kFromConstant) || GatherSlot(r.uvar) >= 0 || r.repeated) return false;
+        if (r.idx.back() != s.contr[0] || r.stride.back() != 1) return false;
+        any = true;
+    }
+    return any;
+}
+
 // One output per batch entry, its contraction shared by s.splitLanes adjacent lanes.
 auto Generator::EmitSplitLanesBody(int k, std::vector<std::string> &lines) -> void
 {
@@ -613,9 +639,13 @@ auto Generator::EmitSplitLanesBody(int k, std::vector<std::string> &lines) -> vo
     for (const auto &l : body.bases) lines.push_back(l);
     lines.push_back("const int cl = w & " + str(L - 1) + ";");
     lines.push_back("double sum = 0.0;");
+    const bool pairs = SplitLanesTakePairs(k);
     // eight loads in flight per lane (row sums of 1 024 terms: 69 % of the HBM peak with 4, 75 % with 8, 73 % with 16)
-    lines.push_back("#pragma unroll 8");
-    lines.push_back("for (int c = cl; c < " + str(s.contrCount) + "; c += " + str(L) + ")");
+    lines.push_back(pairs ? "#pragma unroll 4" : "#pragma unroll 8");
+    if (pairs)
+        lines.push_back("for (int c = 2 * cl; c < " + str(s.contrCount) + "; c += " + str(2 * L) + ")");
+    else
+        lines.push_back("for (int c = cl; c < " + str(s.contrCount) + "; c += " + str(L) + ")");
     lines.push_back("{");
     long st = s.contrCount;
     for (size_t j = 0; j < s.contr.size(); ++j)
@@ -645,7 +675,16 @@ auto Generator::EmitSplitLanesBody(int k, std::vector<std::string> &lines) -> vo
         }
         if (off.empty()) off = "0";
         std::string opnd;
-        if (src == kFromConstant)
+        if (pairs && has(r.idx, s.contr[0]))
+        {
+            // both terms of the pair in one load (through the ordinary pointer also for operands that scalar loads
+            // would serve: the index differs from lane to lane here)
+            const std::string at = src == kFromConstant ? PtrName(r.uvar) + "[" + ScalarBase(r) + Lit(uvars[r.uvar].viewOffset) + " + " + off + "]"
+                                                        : PtrName(r.uvar) + "[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
+            lines.push_back("    const acro_pair p" + str(static_cast<long>(v)) + " = *reinterpret_cast<const acro_pair *>(&" + at + ");");
+            opnd = "p" + str(static_cast<long>(v)) + ".@";
+        }
+        else if (src == kFromConstant)
             opnd = ConstPtrName(r.uvar) + "[" + ScalarBase(r) + Lit(uvars[r.uvar].viewOffset) + " + " + off + "]";
         else if (lds)
             opnd = "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
@@ -653,7 +692,19 @@ auto Generator::EmitSplitLanesBody(int k, std::vector<std::string> &lines) -> vo
             opnd = GlobalRead(r.uvar, "o_k" + str(k) + "v" + str(v) + " + " + off);
         prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
     }
-    lines.push_back("    sum += " + prod + ";");
+    if (pairs)
+    {
+        for (const char *half : {"x", "y"})
+        {
+            std::string term = prod;
+            for (size_t at = term.find('@'); at != std::string::npos; at = term.find('@')) term.replace(at, 1, half);
+            lines.push_back("    sum += " + term + ";");
+        }
+    }
+    else
+    {
+        lines.push_back("    sum += " + prod + ";");
+    }
     lines.push_back("}");
     // The lanes of an output are adjacent and aligned, so every exchange partner works on the same output.  Lanes
     // 1 and 2 apart swap inside their quad; then every lane of a quad holds the same value and mirroring the

@@ -78,6 +78,7 @@
 //   ACRO_HIP_LOOP_TILE=-1       kernels far above the machine balance keep their unrolled body or a plain counted loop (default:
 //                               counted loops around a register tile, see ChooseLoopTile)
 //   ACRO_HIP_STAGE=-1           small invariant operands with lane-dependent addresses stay in device memory (not staged in LDS)
+//   ACRO_HIP_SPLIT_PAIRS=-1     lanes that share a contraction take its terms one at a time also where they have few of them
 //   ACRO_HIP_SPLIT_LANES=-1     one lane per batch entry also for kernels with one output per entry (no lane exchanges)
 //   ACRO_HIP_WAVE_UNIFORM=-1    no readfirstlane on the batch entry of wavefronts that hold items of one entry only
 //   ACRO_HIP_TRANSPOSE=-1       permutations with long fastest dimensions on both sides run as ordinary kernels (no LDS tiles)
