@@ -81,7 +81,8 @@
 //   ACRO_HIP_SPLIT_PAIRS=-1     lanes that share a contraction take its terms one at a time also where they have few of them
 //   ACRO_HIP_SPLIT_LANES=-1     one lane per batch entry also for kernels with one output per entry (no lane exchanges)
 //   ACRO_HIP_WAVE_UNIFORM=-1    no readfirstlane on the batch entry of wavefronts that hold items of one entry only
-//   ACRO_HIP_TRANSPOSE=-1       permutations with long fastest dimensions on both sides run as ordinary kernels (no LDS tiles)
+//   ACRO_HIP_TRANSPOSE=-1|2     -1: permutations with long fastest dimensions on both sides run as ordinary kernels (no LDS
+//                               tiles); 2: LDS tiles only where both dimensions have 32 entries or more (no rectangular tiles)
 //   ACRO_HIP_OPERATOR=-1        a dense operator applied to every batch entry runs through the generic schedule (operator staged
 //                               in LDS, one entry per lane) instead of the operator schedule
 //   ACRO_HIP_LIGHT=-1           streaming groups whose workgroups move less than 2.5 KB keep their batch size (no extra

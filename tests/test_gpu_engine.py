@@ -486,6 +486,10 @@ def test_split_contraction_of_few_long_rows(at, engine, checker, kernel, shapes,
     ("A_e_i_j = B_e_j_i", (5, 40, 50)),              # batched, matrices too large for one lane each
     ("A_j_k_i = B_i_k_j", (33, 2, 45)),
     ("A_k_j_i_l = B_l_i_k_j", (32, 37, 3, 41)),      # fastest dimensions l and j, two more in other places
+    ("A_i_j = B_j_i", (1000, 16)),                   # one side short: tiles of 16 x 64 entries
+    ("A_i_j -= B_j_i", (9, 2003)),                   # ... of 64 x 16, the short side ragged (9 of 16)
+    ("A_e_i_j = B_e_j_i", (3, 300, 8)),              # ... of 8 x 128, batched
+    ("A_i_e_j += B_j_e_i", (24, 2, 257)),            # 24 of 32 on one side
 ])
 def test_permutations_with_long_fastest_dimensions_go_through_lds_tiles(at, engine, checker, kernel, shape):
     rng = np.random.default_rng(sum(shape))
