@@ -349,7 +349,13 @@ auto Generator::ChooseTiles() -> void
                 // several outputs per entry a lane should have at least four terms of its own, or the exchanges
                 // outweigh the arithmetic (16 x 16 matrix-vector products with one term per lane: 47 % against
                 // 59 % unsplit).
-                const long atMost = mid.empty() ? s.contrCount : s.contrCount / 4;
+                // (one output per entry: one term per lane, or one pair of terms where the lanes can load pairs)
+                bool pairable = envInt("ACRO_HIP_SPLIT_PAIRS") >= 0 && s.contr.size() == 1 && s.contrCount % 2 == 0;
+                for (const auto &r : s.in)
+                {
+                    if (has(r.idx, s.contr[0]) && (r.repeated || r.idx.back() != s.contr[0] || r.stride.back() != 1)) pairable = false;
+                }
+                const long atMost = mid.empty() ? (pairable ? s.contrCount / 2 : s.contrCount) : s.contrCount / 4;
                 int lanes = 1;
                 while (lanes * 2 <= 16 && lanes * 2 <= atMost) lanes *= 2;
                 if (lanes >= (mid.empty() ? 2 : 4))
