@@ -113,6 +113,25 @@ struct SmallMatrix<3>
     }
 };
 
+// 1 x 1 "matrices" (ops/NativeCPUOps.hpp:38-44: the determinant is the entry, the inverse its reciprocal): a plain
+// stream, four entries per lane in workgroups of kLanes, so that the launch is bound by memory and not by the rate at
+// which 64-lane workgroups start (2^25 entries: 113 us either way with one workgroup per 64 entries).
+template <bool WANT_INV, bool WANT_DET>
+__global__ __launch_bounds__(kLanes) void batchScalarKernel(const double *__restrict__ A, double *__restrict__ Ainv,
+                                                            double *__restrict__ Adet, size_t n)
+{
+    const size_t first = (static_cast<size_t>(blockIdx.x) * kLanes) * 4 + threadIdx.x;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        const size_t i = first + static_cast<size_t>(j) * kLanes;
+        if (i >= n) break;
+        const double det = A[i];
+        if (WANT_DET) __builtin_nontemporal_store(det, &Adet[i]);
+        if (WANT_INV) __builtin_nontemporal_store(1.0 / det, &Ainv[i]);
+    }
+}
+
 // One workgroup = kMatLanes consecutive matrices.  WANT_INV / WANT_DET select the outputs.
 // The matrices of a workgroup are contiguous in memory, so the workgroup copies them to and from LDS as one
 // stream of 16-byte pieces (full-rate HBM access), and lane t works on matrix t out of LDS.  For 2x2 the lane
@@ -346,8 +365,13 @@ void launchBatchMatrix(int mdim, const double *A, double *Ainv, double *Adet, si
     switch (mdim)
     {
         case 1:
-            ACRO_LAUNCH_BATCH_MATRIX(1);
+        {
+            const size_t blocks = (num_mat + 4 * kLanes - 1) / (4 * kLanes);
+            ACROBATIC_ASSERT(blocks <= 0x7fffffffu, "Operand too large for a one-dimensional grid.");
+            hipLaunchKernelGGL((batchScalarKernel<WANT_INV, WANT_DET>), dim3(static_cast<unsigned>(blocks == 0 ? 1 : blocks)),
+                               dim3(kLanes), 0, stream(), A, Ainv, Adet, num_mat);
             break;
+        }
         case 2:
             ACRO_LAUNCH_BATCH_MATRIX(2);
             break;
