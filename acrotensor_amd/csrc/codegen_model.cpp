@@ -224,9 +224,88 @@ auto Generator::FactoriseKernels() -> void
     for (size_t ki = 0; ki < subs.size(); ++ki)
     {
         if (subs.size() == 1 && ProductThenRowSums(static_cast<int>(ki), subs[ki], expanded, counter)) continue;
-        if (!FactoriseKernel(static_cast<int>(ki), subs[ki], subs.size() == 1, expanded, counter)) expanded.push_back(subs[ki]);
+        if (FactoriseKernel(static_cast<int>(ki), subs[ki], subs.size() == 1, expanded, counter)) continue;
+        if (subs.size() == 1 && StageReusedOperands(static_cast<int>(ki), subs[ki], expanded, counter)) continue;
+        expanded.push_back(subs[ki]);
     }
     subs.swap(expanded);
+}
+
+// A kernel on its own whose per-entry operands are small and read many times over by the lanes of the entry (batched
+// matrix products "A_e_i_j = B_e_i_k C_e_k_j" with 16 x 16 matrices: every value 16 times, 32 loads per output
+// straight from device memory, lanes a row or a column apart: 28 % of the HBM peak) copies those operands to LDS tiles
+// first, with the lanes along the operand as it lies in memory, and computes from the tiles.  The copies are steps of
+// the generator's own ("_S1_e_i_k = B_e_i_k"), placed, fused and emitted like the steps of a reordered kernel.
+auto Generator::StageReusedOperands(int ki, const Sub &orig, std::vector<Sub> &result, int &counter) -> bool
+{
+    if (envInt("ACRO_HIP_STAGE_ENTRIES") < 0 || batch < 0 || !opt.noalias || orig.contr.empty() || orig.matrixOp != 0) return false;
+    if (orig.out.repeated || orig.in.size() < 2 || NumGatherSlots() > 0) return false;
+    const long outputs = product(orig.outIdx, extent) / extent[batch];
+    if (outputs < 64 || outputs > 1024) return false;
+    std::vector<char> staged(orig.in.size(), 0);
+    long total = 0;
+    int count = 0;
+    for (size_t v = 0; v < orig.in.size(); ++v)
+    {
+        const VarRef &r = orig.in[v];
+        if (r.repeated || r.uvar == orig.out.uvar || r.idx.empty() || r.idx[0] != batch) continue;
+        bool again = false;  // the same tensor twice: one tile would do, keep it simple
+        for (size_t w = 0; w < orig.in.size(); ++w) again = again || (w != v && orig.in[w].uvar == r.uvar);
+        if (again) continue;
+        const long perEntry = r.size / extent[batch];
+        // how often each value is read: work per entry (outputs x terms) over the operand's entries
+        const long reads = outputs * orig.contrCount / std::max<long>(1, perEntry);
+        if (perEntry < 16 || perEntry > 1024 || reads < 8) continue;
+        staged[v] = 1;
+        total += perEntry;
+        ++count;
+    }
+    // Two such operands: products of element matrices.  With one (an element vector under an element matrix, the
+    // vectors of a dense operator) the kernel has schedules of its own that read the big operand once and well.
+    if (count < 2 || total > 2048) return false;
+    DimensionedKernel *kernel = mk.Kernels[ki];
+    auto refText = [&](const std::string &name, const std::vector<int> &ids) {
+        std::string t = name;
+        for (int id : ids) t += "_" + idxName[id];
+        return t;
+    };
+    Sub fin = orig;
+    std::string finText = refText(kernel->GetVarName(-1), orig.out.idx) + " " + (orig.op == '=' ? "=" : std::string(1, orig.op) + "=");
+    for (size_t v = 0; v < orig.in.size(); ++v)
+    {
+        const VarRef &r = orig.in[v];
+        if (!staged[v])
+        {
+            finText += " " + refText(kernel->GetVarName(static_cast<int>(v)), r.idx);
+            continue;
+        }
+        UVarInfo info;
+        info.isVirtual = true;
+        info.isStagedCopy = true;
+        info.name = "_S" + str(static_cast<long>(++counter));
+        VarRef res;
+        res.uvar = static_cast<int>(uvars.size());
+        res.idx = r.idx;
+        res.ext = r.ext;
+        res.stride = r.stride;
+        res.size = r.size;
+        uvars.push_back(info);
+        Sub copy;
+        copy.op = '=';
+        copy.out = res;
+        copy.outIdx = res.idx;
+        copy.in.assign(1, r);
+        copy.contrCount = 1;
+        copy.flatItems = true;
+        copy.text = refText(info.name, res.idx) + " = " + refText(kernel->GetVarName(static_cast<int>(v)), r.idx);
+        result.push_back(copy);
+        fin.in[v] = res;
+        finText += " " + refText(info.name, res.idx);
+    }
+    fin.text = finText + "   (operands staged in LDS: " + orig.text + ")";
+    result.push_back(fin);
+    factorised = true;
+    return true;
 }
 
 // An element matrix applied to an element vector, "A_e_i = B_e_i_j C_e_j", whose rows are not a multiple of four

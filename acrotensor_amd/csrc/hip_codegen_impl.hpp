@@ -89,6 +89,7 @@ struct UVarInfo
     std::vector<int> fixed;       // leading indices of the storage that the view fixes
     bool plainView = true;        // the view is "leading indices fixed, all trailing dimensions kept"
     bool isVirtual = false;       // intermediate of a factorised kernel: lives in LDS only, no kernel parameter
+    bool isStagedCopy = false;    // ... that is a plain copy of an operand (StageReusedOperands)
 };
 
 // A tensor's memory: what kernel parameters point to, what LDS tiles mirror and what stores are elided for.
@@ -227,6 +228,7 @@ class Generator
     void FactoriseSearch(const Sub &orig, std::vector<int> &live, std::vector<std::vector<int>> &idxOf, std::vector<int> &remaining, double cost, std::vector<FactorStep> &steps, double &best, long &bestSlowest, std::vector<FactorStep> &bestSteps, long &visits) const;
     void FactoriseKernels();
     bool ProductThenRowSums(int ki, const Sub &orig, std::vector<Sub> &result, int &counter);
+    bool StageReusedOperands(int ki, const Sub &orig, std::vector<Sub> &result, int &counter);
     bool FactoriseKernel(int ki, const Sub &orig, bool alone, std::vector<Sub> &result, int &counter);
     void BuildStorages();
     bool Covered(const Storage &st, const std::vector<int> &fixed, const std::vector<std::vector<int>> &written) const;

@@ -193,6 +193,23 @@ def test_3d_stiffness_twelve_loops(at, engine, checker):
     assert np.array_equal(got, expected)          # all terms are multiples of 0.5 below 2^53: exact
 
 
+@pytest.mark.parametrize("kernel,shapes", [
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(37, 16, 16), (37, 16, 16)]),          # the reference's I_b_i_k = TI_b_i_j T_b_j_k, larger
+    ("A_e_i_j += B_e_i_k C_e_j_k", [(21, 16, 12), (21, 20, 12)]),         # second factor transposed, rectangular
+    ("A_e_j_i -= B_e_k_i C_e_k_j W_e", [(40, 7, 32), (40, 7, 24), (40,)]),   # both transposed, output transposed, a factor per entry
+    ("A_e_i_j = C_e_k_j B_e_i_k D_e_i_j", [(14, 9, 11), (14, 13, 9), (14, 13, 11)]),   # pointwise factor on the result
+])
+def test_products_of_element_matrices_stage_their_operands_in_lds(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(len(kernel))
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "operands staged in LDS" in engine.GetLastImplementation()
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
+
+
 @pytest.mark.parametrize("P,Q,E", [(2, 3, 1001), (4, 5, 203), (3, 4, 77), (8, 10, 5)])
 def test_2d_mass_assembly_results_leave_through_an_lds_tile(at, engine, checker, P, Q, E):
     # unittest/kernel/test_TensorEngine.cpp:399-435 at other sizes.  With lanes (i2, j2) / (j1, j2) and a register tile
