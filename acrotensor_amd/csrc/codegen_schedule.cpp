@@ -1149,7 +1149,13 @@ auto Generator::ChooseBatching() -> void
         }
         st.elide = ok && anyRead;
     }
-    if (envInt("ACRO_HIP_LDS_PAD") > 0) PadLdsTiles(budgetDoubles);  // opt-in: see PadLdsTiles
+    // Padding of every tile is opt-in (see PadLdsTiles); the copies of operands that StageReusedOperands makes are
+    // padded always: their lanes read them along any dimension (32 x 32 matrices with the second factor transposed:
+    // a 32-way bank conflict on every read, 10.5 % of the HBM peak unpadded).
+    if (envInt("ACRO_HIP_LDS_PAD") > 0)
+        PadLdsTiles(budgetDoubles, false);
+    else
+        PadLdsTiles(budgetDoubles, true);
 
     // A launch that writes several times what it reads streams better with fewer workgroups resident per CU
     // (fewer write streams interleave at the memory controllers): workgroups of 128 lanes become 256 lanes with
@@ -1309,7 +1315,7 @@ auto Generator::SetLdsStrides(Storage &st, const std::vector<int> &pad, int padE
     st.tileSize = static_cast<int>(run + padEntry);
 }
 
-auto Generator::PadLdsTiles(int budgetDoubles) -> void
+auto Generator::PadLdsTiles(int budgetDoubles, bool stagedCopiesOnly) -> void
 {
     // Padding must not cost a resident workgroup: a CU has 160 KB of LDS, handed out in granules of 1 280 bytes
     // (the p=7 diffusion chain at 53 440 bytes fits three times, at 54 080 bytes only twice).
@@ -1322,6 +1328,7 @@ auto Generator::PadLdsTiles(int budgetDoubles) -> void
     {
         Storage &st = stores[si];
         if (!st.inLds || st.staged) continue;
+        if (stagedCopiesOnly && !(st.members.size() == 1 && uvars[st.members[0]].isStagedCopy)) continue;
         const int ndim = static_cast<int>(st.dims.size()) - 1;
         std::vector<int> pad(ndim, 0), bestPad(ndim, 0);
         int bestEntry = 0;

@@ -284,7 +284,7 @@ class Generator
     std::vector<long> LaneAddresses(const Sub &s, const VarRef &r, int nb) const;
     long LdsCostOfStorage(int si, int nb) const;
     void SetLdsStrides(Storage &st, const std::vector<int> &pad, int padEntry) const;
-    void PadLdsTiles(int budgetDoubles);
+    void PadLdsTiles(int budgetDoubles, bool stagedCopiesOnly);
 
     // --------------------------------------------------------------------------------------- emission
     std::ostringstream out;
