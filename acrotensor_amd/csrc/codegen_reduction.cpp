@@ -11,7 +11,7 @@ auto Generator::UseReductionSchedule() const -> bool
     if (subs.size() != 1 || NumGatherSlots() > 0) return false;
     const Sub &s = subs[0];
     if (s.out.repeated) return false;
-    return s.contrCount >= kReductionMinContraction && product(s.outIdx, extent) <= kReductionMaxOutputs;
+    return s.contrCount >= kReductionMinContraction && product(s.outIdx, extent) <= envInt("ACRO_HIP_RED_MAX_OUTPUTS", kReductionMaxOutputs);
 }
 
 // Expression for the element offset of an occurrence given variables named i_<index> for every loop index.
@@ -82,7 +82,21 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     // its slice of A as 16-byte pieces and the slice's entry of B once, i.e. 6 load instructions per 80 bytes;
     // with one lane per (slice, output entry) every lane loads B again and the same bytes take 18 load
     // instructions (A alone streamed at 6.1 TB/s that way, A and B together at 5.0 - 5.5 TB/s).
-    const bool pencil = outputsFastest && O <= 16 && envInt("ACRO_HIP_RED_PENCIL") >= 0;
+    // The same for up to 64 outputs that are products of few loads ("A_i_j = B_e_i C_e_j" with 8 x 8 outputs: 16
+    // loads and 64 accumulators per slice; one lane per (slice, output) reads every value eight times: 21.7 % of the
+    // HBM peak).
+    long loadsPerSlice = 0;
+    for (const auto &r : s.in)
+    {
+        long n = 1;
+        std::set<int> seen;
+        for (int id : r.idx)
+        {
+            if (has(s.outIdx, id) && seen.insert(id).second) n *= extent[id];
+        }
+        loadsPerSlice += n;
+    }
+    const bool pencil = outputsFastest && (O <= 16 || (O <= 64 && 2 * loadsPerSlice <= O)) && envInt("ACRO_HIP_RED_PENCIL") >= 0;
     const int NTr = kReductionLanes;
     // Contraction index fastest and more than four outputs ("S_i = A_i_n" with 64 rows): with all outputs in every
     // workgroup only NTr / O lanes would walk along a row (32-byte pieces of 64 different rows per load

@@ -853,3 +853,22 @@ def test_element_matrix_times_vector_with_odd_rows(at, engine, checker, kernel, 
     if "-=" in kernel:
         expected = 2.0 * out0 - expected
     assert rel_err(got, expected) <= TOL
+
+
+@pytest.mark.parametrize("n,m,op", [(5000, 8, "="), (3001, 4, "+="), (2500, 7, "-="), (2100, 11, "=")])
+def test_small_gram_matrix_over_the_batch(at, engine, checker, n, m, op):
+    # "A_i_j = B_e_i C_e_j": a contraction over the long index with m x m outputs that are products of two short loads;
+    # up to 8 x 8 a lane owns whole slices (m + m loads, m x m accumulators), beyond that one lane per (slice, output)
+    kernel = "A_i_j %s B_e_i C_e_j" % op
+    rng = np.random.default_rng(n + m)
+    B, C = rng.uniform(-1, 1, (n, m)), rng.uniform(-1, 1, (n, m))
+    out0 = rng.uniform(-1, 1, (m, m))
+    got, expected = run_single(at, engine, checker, kernel, out0, B, C)
+    src = engine.GetLastImplementation()
+    assert "reduction schedule" in src
+    assert ("a lane owns whole slices" in src) == (m <= 8)
+    if op == "-=":
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
+    again, _ = run_single(at, engine, checker, kernel, out0, B, C)
+    assert np.array_equal(got, again)                   # fixed order of additions: reproducible
