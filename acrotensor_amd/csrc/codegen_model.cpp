@@ -236,12 +236,19 @@ auto Generator::FactoriseKernels() -> void
 // straight from device memory, lanes a row or a column apart: 28 % of the HBM peak) copies those operands to LDS tiles
 // first, with the lanes along the operand as it lies in memory, and computes from the tiles.  The copies are steps of
 // the generator's own ("_S1_e_i_k = B_e_i_k"), placed, fused and emitted like the steps of a reordered kernel.
-auto Generator::StageReusedOperands(int ki, const Sub &orig, std::vector<Sub> &result, int &counter) -> bool
+auto Generator::StageReusedOperands(int ki, const Sub &asWritten, std::vector<Sub> &result, int &counter) -> bool
 {
-    if (envInt("ACRO_HIP_STAGE_ENTRIES") < 0 || batch < 0 || !opt.noalias || orig.contr.empty() || orig.matrixOp != 0) return false;
+    if (envInt("ACRO_HIP_STAGE_ENTRIES") < 0 || batch < 0 || !opt.noalias || asWritten.contr.empty() || asWritten.matrixOp != 0) return false;
+    Sub orig = asWritten;
     if (orig.out.repeated || orig.in.size() < 2 || NumGatherSlots() > 0) return false;
     const long outputs = product(orig.outIdx, extent) / extent[batch];
-    if (outputs < 64 || outputs > 1024) return false;
+    if (outputs < 4 || outputs > 1024) return false;
+    // Tiny matrices (fewer than 64 outputs) are staged as well unless every operand's entry is a power of two of
+    // doubles: those lie in whole lines and the lanes read them well from device memory (4 x 4 products with one
+    // output per lane: 90 % of the HBM peak, 51 % staged), the others do not (3 x 3: 64 -> 82 %, 5 x 5: 46 -> 77 %,
+    // 6 x 6: 48 -> 80 %, 7 x 7: 46 -> 77 %, with some 500 outputs per workgroup of 256 lanes).
+    const bool tiny = outputs < 64;
+    bool wholeLines = true;
     std::vector<char> staged(orig.in.size(), 0);
     long total = 0;
     int count = 0;
@@ -253,16 +260,116 @@ auto Generator::StageReusedOperands(int ki, const Sub &orig, std::vector<Sub> &r
         for (size_t w = 0; w < orig.in.size(); ++w) again = again || (w != v && orig.in[w].uvar == r.uvar);
         if (again) continue;
         const long perEntry = r.size / extent[batch];
-        // how often each value is read: work per entry (outputs x terms) over the operand's entries
-        const long reads = outputs * orig.contrCount / std::max<long>(1, perEntry);
-        if (perEntry < 16 || perEntry > 1024 || reads < 8) continue;
+        // how many outputs each value goes into: the output indices that the operand does not carry
+        long reads = 1;
+        for (int id : orig.outIdx) reads *= (id == batch || has(r.idx, id)) ? 1 : extent[id];
+        wholeLines = wholeLines && (perEntry & (perEntry - 1)) == 0;
+        // (tiny ones: matrices only, an output index and a contraction index each; vectors under a shared operator
+        // belong to the operator schedule)
+        bool carriesOutput = false, carriesContraction = false;
+        for (int id : r.idx)
+        {
+            carriesOutput = carriesOutput || (id != batch && has(orig.outIdx, id));
+            carriesContraction = carriesContraction || has(orig.contr, id);
+        }
+        if (tiny && !(carriesOutput && carriesContraction)) continue;
+        if (perEntry < (tiny ? 4 : 16) || perEntry > 1024 || reads < (tiny ? 2 : 8)) continue;
         staged[v] = 1;
         total += perEntry;
         ++count;
     }
     // Two such operands: products of element matrices.  With one (an element vector under an element matrix, the
     // vectors of a dense operator) the kernel has schedules of its own that read the big operand once and well.
-    if (count < 2 || total > 2048) return false;
+    if (count < 2 || total > 2048 || (tiny && wholeLines)) return false;
+    // With one output per lane every multiply-add reads both of its factors from LDS, and LDS bounds the kernel
+    // (24 x 24 products: 48 % of the HBM peak, 30 x 30: 35 %).  A lane that owns a 2 x 2 block of outputs reads half
+    // as much.  Register tiles are whole indices, so an output index of even extent is split in two, "i = 2 i' + i''"
+    // (extent divisible by three only: in three), in every operand, which describes the same memory with one
+    // dimension more, and the halves i'' become the tile (24 x 24: 83 %, 30 x 30: 80 %, 12 x 12: 72 -> 89 %).
+    std::vector<int> blockIdx;
+    bool splittable = !tiny && envInt("ACRO_HIP_STAGE_ENTRIES") < 2;
+    for (size_t v = 0; v < orig.in.size(); ++v)
+    {
+        const int u = orig.in[v].uvar;
+        for (size_t w = 0; w < orig.in.size(); ++w) splittable = splittable && (w == v || orig.in[w].uvar != u);
+        splittable = splittable && u != orig.out.uvar;
+    }
+    // (every operand must be a whole tensor of its own: its storage is then described by the split dimensions)
+    auto wholeTensor = [&](const VarRef &r) {
+        if (static_cast<size_t>(r.uvar) >= opt.views.size()) return true;
+        const HipOperandView &view = opt.views[r.uvar];
+        long entries = 1;
+        for (int d : view.root_dims) entries *= d;
+        bool shared = false;
+        for (size_t u = 0; u < opt.views.size(); ++u)
+            shared = shared || (static_cast<int>(u) != r.uvar && opt.views[u].storage >= 0 && opt.views[u].storage == view.storage);
+        return view.storage < 0 || (!shared && view.offset == 0 && (view.root_dims.empty() || entries == r.size));
+    };
+    splittable = splittable && wholeTensor(orig.out);
+    for (const auto &r : orig.in) splittable = splittable && wholeTensor(r);
+    if (splittable)
+    {
+        const std::vector<int> outputIds = orig.outIdx;
+        for (int id : outputIds)
+        {
+            if (id == batch || extent[id] < 4) continue;
+            const int t = extent[id] % 2 == 0 ? 2 : (extent[id] % 3 == 0 ? 3 : 1);
+            if (t == 1) continue;
+            // two new loop indices, named after the old one
+            auto fresh = [&](std::string name) {
+                while (std::find(idxName.begin(), idxName.end(), name) != idxName.end()) name += "x";
+                return name;
+            };
+            const int hi = nidx, lo = nidx + 1;
+            nidx += 2;
+            idxName.push_back(fresh(idxName[id] + "hi"));
+            extent.push_back(extent[id] / t);
+            idxName.push_back(fresh(idxName[id] + "lo"));
+            extent.push_back(t);
+            auto splitRef = [&](VarRef &r) {
+                VarRef n = r;
+                n.idx.clear();
+                n.ext.clear();
+                n.stride.clear();
+                for (size_t d = 0; d < r.idx.size(); ++d)
+                {
+                    if (r.idx[d] != id)
+                    {
+                        n.idx.push_back(r.idx[d]);
+                        n.ext.push_back(r.ext[d]);
+                        n.stride.push_back(r.stride[d]);
+                        continue;
+                    }
+                    n.idx.push_back(hi);
+                    n.ext.push_back(r.ext[d] / t);
+                    n.stride.push_back(r.stride[d] * t);
+                    n.idx.push_back(lo);
+                    n.ext.push_back(t);
+                    n.stride.push_back(r.stride[d]);
+                }
+                r = n;
+            };
+            splitRef(orig.out);
+            for (auto &r : orig.in) splitRef(r);
+            std::vector<int> ids;
+            for (int o : orig.outIdx)
+            {
+                if (o != id) ids.push_back(o);
+                else
+                {
+                    ids.push_back(hi);
+                    ids.push_back(lo);
+                }
+            }
+            orig.outIdx = ids;
+            blockIdx.push_back(lo);
+        }
+        if (!blockIdx.empty())
+        {
+            reshaped.insert(orig.out.uvar);
+            for (const auto &r : orig.in) reshaped.insert(r.uvar);
+        }
+    }
     DimensionedKernel *kernel = mk.Kernels[ki];
     auto refText = [&](const std::string &name, const std::vector<int> &ids) {
         std::string t = name;
@@ -303,6 +410,7 @@ auto Generator::StageReusedOperands(int ki, const Sub &orig, std::vector<Sub> &r
         finText += " " + refText(info.name, res.idx);
     }
     fin.text = finText + "   (operands staged in LDS: " + orig.text + ")";
+    fin.wantedTile = blockIdx;
     result.push_back(fin);
     factorised = true;
     return true;
@@ -508,7 +616,7 @@ auto Generator::BuildStorages() -> void
     {
         UVarInfo &op = uvars[u];
         Storage &st = stores[op.storage];
-        const bool hasView = static_cast<size_t>(u) < opt.views.size() && !opt.views[u].root_dims.empty();
+        const bool hasView = static_cast<size_t>(u) < opt.views.size() && !opt.views[u].root_dims.empty() && reshaped.count(u) == 0;
         if (st.dims.empty())
         {
             st.dims = hasView ? opt.views[u].root_dims : op.dims;

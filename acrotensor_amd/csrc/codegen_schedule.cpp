@@ -324,6 +324,14 @@ auto Generator::ChooseTiles() -> void
                 streamingOnly = streamingOnly && (has(r.idx, batch) || (smallInvariantToo && r.size <= 1024)) && !r.repeated;
             const long outputs = product(mid, extent), loadsPerOutput = s.contrCount * nin;
             if (streamingOnly && ((outputs <= 32 && loadsPerOutput <= 16) || (outputs <= 64 && loadsPerOutput <= 4))) best.clear();
+            // The same for a tiny product whose operands were copied to LDS tiles first: one output per lane keeps the
+            // stores of a wavefront contiguous.
+            bool fromStagedCopies = (outputs < 64 || (outputs < 200 && s.wantedTile.empty())) && !s.in.empty();
+            for (const auto &r : s.in) fromStagedCopies = fromStagedCopies && (uvars[r.uvar].isStagedCopy || !has(r.idx, batch));
+            bool anyStagedCopy = false;
+            for (const auto &r : s.in) anyStagedCopy = anyStagedCopy || uvars[r.uvar].isStagedCopy;
+            if (fromStagedCopies && anyStagedCopy) best.clear();
+            if (!s.wantedTile.empty() && product(s.wantedTile, extent) * s.contrCount * nin <= kUnrollBudget) best = s.wantedTile;
             ForcedTile(static_cast<int>(&s - subs.data()), mid, best);
             if (s.flatItems) best.clear();
             s.tile = best;
@@ -1077,6 +1085,27 @@ auto Generator::ChooseBatching() -> void
         }
     }
 
+    // Products of tiny element matrices whose operands are copied to LDS first (3 x 3 to 7 x 7): some 500 outputs per
+    // workgroup of 256 lanes, two passes of its lanes (3 x 3: 75 % of the HBM peak with 14 or 28 entries per workgroup,
+    // 82 % with 56; 5 x 5: 72 / 77 / 72 % with 5, 20 and 40; 7 x 7: 69 / 77 / 72 % with 5, 10 and 20).
+    if (opt.force_nb <= 0 && opt.force_nt <= 0 && envInt("ACRO_HIP_NB") <= 0 && envInt("ACRO_HIP_NT") <= 0 && batch >= 0)
+    {
+        const Sub &last = subs.back();
+        bool anyStagedCopy = false;
+        for (const auto &r : last.in) anyStagedCopy = anyStagedCopy || uvars[r.uvar].isStagedCopy;
+        if (anyStagedCopy && last.tile.empty() && last.laneCount < 64 && !last.loopMode)
+        {
+            NB = static_cast<int>(std::min<long>(E, std::max<long>(NB, 512 / last.laneCount)));
+            NT = 256;
+        }
+        // (matrices of 11 x 11 and 13 x 13, whose indices cannot be split into blocks: four passes, 69 -> 85 and 81 %)
+        else if (anyStagedCopy && last.tile.empty() && last.laneCount < 200 && !last.loopMode)
+        {
+            NB = static_cast<int>(std::min<long>(E, std::max<long>(NB, 1024 / last.laneCount)));
+            NT = 256;
+        }
+    }
+
     // Everything that wants LDS gets it while the workgroup stays within the 64 KB a workgroup may declare
     // statically; otherwise shrink the batch, and finally leave the largest tiles in device memory.
     const int budgetDoubles = 64 * 1024 / 8;
@@ -1330,7 +1359,13 @@ auto Generator::PadLdsTiles(int budgetDoubles, bool stagedCopiesOnly) -> void
         if (!st.inLds || st.staged) continue;
         if (stagedCopiesOnly && !(st.members.size() == 1 && uvars[st.members[0]].isStagedCopy)) continue;
         const int ndim = static_cast<int>(st.dims.size()) - 1;
-        std::vector<int> pad(ndim, 0), bestPad(ndim, 0);
+        // Rows of odd length in the copy of an operand get one double more, whatever the count below says: pairs of
+        // values along a row are then 16 bytes aligned and read with one instruction (25 x 25 matrix products
+        // 42 -> 50 % of the HBM peak, 27 x 27: 40 -> 57 %).
+        std::vector<int> natural(ndim, 0);
+        if (ndim >= 2 && st.dims.back() % 2 == 1 && st.dims.back() >= 17 && st.members.size() == 1 && uvars[st.members[0]].isStagedCopy)
+            natural[0] = 1;
+        std::vector<int> pad = natural, bestPad = natural;
         int bestEntry = 0;
         SetLdsStrides(st, pad, 0);
         long best = LdsCostOfStorage(static_cast<int>(si), NB);
@@ -1343,6 +1378,7 @@ auto Generator::PadLdsTiles(int budgetDoubles, bool stagedCopiesOnly) -> void
                 const int limit = p == ndim ? 16 : 8;
                 for (int cand = 0; cand <= limit; ++cand)
                 {
+                    if (p == 0 && natural[0] == 1 && cand % 2 == 0) continue;  // rows stay even
                     std::vector<int> trial = bestPad;
                     int trialEntry = bestEntry;
                     if (p == ndim)
@@ -1364,7 +1400,8 @@ auto Generator::PadLdsTiles(int budgetDoubles, bool stagedCopiesOnly) -> void
         const int total = PlaceLds(NB);
         if (total > budgetDoubles || best >= unpadded || (envInt("ACRO_HIP_LDS_PAD") < 2 && resident(total) < residentBefore))
         {
-            SetLdsStrides(st, std::vector<int>(ndim, 0), 0);  // no room or no gain: natural layout
+            SetLdsStrides(st, natural, 0);  // no room or no gain: natural layout
+            if (PlaceLds(NB) > budgetDoubles) SetLdsStrides(st, std::vector<int>(ndim, 0), 0);
         }
     }
     ldsDoubles = PlaceLds(NB);

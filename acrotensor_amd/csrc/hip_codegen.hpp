@@ -78,6 +78,7 @@
 //   ACRO_HIP_LOOP_TILE=-1       kernels far above the machine balance keep their unrolled body or a plain counted loop (default:
 //                               counted loops around a register tile, see ChooseLoopTile)
 //   ACRO_HIP_STAGE_ENTRIES=-1   products of element matrices read their operands from device memory (no copies to LDS tiles first)
+//   ACRO_HIP_STAGE_ENTRIES=2    ... are staged, but their output indices are not split into blocks (one output or one row per lane)
 //   ACRO_HIP_STAGE=-1           small invariant operands with lane-dependent addresses stay in device memory (not staged in LDS)
 //   ACRO_HIP_SPLIT_PAIRS=-1     lanes that share a contraction take its terms one at a time also where they have few of them
 //   ACRO_HIP_SPLIT_LANES=-1     one lane per batch entry also for kernels with one output per entry (no lane exchanges)

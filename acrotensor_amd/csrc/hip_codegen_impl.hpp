@@ -56,6 +56,7 @@ struct Sub
     // schedule
     std::vector<int> lane;    // loop ids enumerated by the work items (last one fastest)
     std::vector<int> tile;    // loop ids kept in registers by one work item
+    std::vector<int> wantedTile;  // the register tile asked for by the step that built this kernel (empty: the cost model's)
     bool loopMode = false;    // contraction as counted loops instead of unrolled code
     bool fusedWithPrev = false;
     std::vector<char> forwardedIn;  // per input occurrence: served from the registers of an earlier kernel of the chain
@@ -178,6 +179,7 @@ class Generator
     std::vector<int> extent;
     std::vector<Sub> subs;
     std::vector<UVarInfo> uvars;
+    std::set<int> reshaped;  // whole tensors whose dimensions were split by StageReusedOperands: their storage has the split extents
     std::vector<Storage> stores;
     // Per kernel and input occurrence: every entry it reads has been written to the storage's tile by an earlier
     // kernel of the group (so it can be served from LDS); per kernel: the same for the old value of a += output.

@@ -240,9 +240,18 @@ def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE):
     # one lane per entry would read 512-byte rows 512 bytes apart and overflow the vector cache: one lane per row
     src = TE.GetImplementation("A_e_i = B_e_i_j C_e_j", at.Tensor(4096, 8), at.Tensor(4096, 8, 8), at.Tensor(4096, 8))
     assert "lanes(i)=8 tile()=1" in src
-    # 8 x 8 products keep a row of outputs per lane
+    # 8 x 8 products: operands copied to LDS first, a 2 x 2 block of outputs per lane (the output indices split in two)
     src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 8, 8), at.Tensor(4096, 8, 8), at.Tensor(4096, 8, 8))
-    assert "tile(k)=8" in src or "tile(i)=8" in src
+    assert "operands staged in LDS" in src and "lanes(ihi,khi)=16 tile(ilo,klo)=4" in src
+    # 11 x 11: no blocks, one output per lane and some thousand outputs per workgroup; 3 x 3 likewise with some 500
+    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 11, 11), at.Tensor(4096, 11, 11), at.Tensor(4096, 11, 11))
+    assert "8 per workgroup of 256 lanes" in src and "lanes(i,k)=121 tile()=1" in src
+    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 3, 3), at.Tensor(4096, 3, 3), at.Tensor(4096, 3, 3))
+    assert "56 per workgroup of 256 lanes" in src and "operands staged in LDS" in src and "lanes(i,k)=9 tile()=1" in src
+    # slices are not whole tensors: their indices stay as they are
+    big = at.Tensor(2, 4096, 8, 8)
+    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 8, 8), at.SliceTensor(big, 1), at.Tensor(4096, 8, 8))
+    assert "operands staged in LDS" in src and "ihi" not in src
 
 
 def scatter_then_mass_apply_source(TE, transient_x):

@@ -210,6 +210,46 @@ def test_products_of_element_matrices_stage_their_operands_in_lds(at, engine, ch
     assert rel_err(got, expected) <= TOL
 
 
+@pytest.mark.parametrize("kernel,shapes,expect", [
+    # 3 x 3 (the reference's unittest/kernel/test_TensorEngine.cpp:292-331 is 2 x 2): one output per lane, 56 entries per workgroup
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(1001, 3, 3), (1001, 3, 3)], "56 per workgroup of 256 lanes"),
+    ("A_e_i_j -= B_e_k_i C_e_j_k", [(333, 5, 7), (333, 6, 5)], "lanes(i,j)=42 tile()=1"),
+    ("A_e_i_j += B_e_i_k C_e_k_l D_e_l_j", [(77, 3, 3), (77, 3, 3), (77, 3, 3)], "operands staged in LDS"),
+    # even extents: both output indices split in two, a 2 x 2 block of outputs per lane
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(203, 12, 12), (203, 12, 12)], "lanes(ihi,jhi)=36 tile(ilo,jlo)=4"),
+    ("A_e_j_i += B_e_k_i C_e_j_k W_e", [(57, 9, 24), (57, 30, 9), (57,)], "tile(jlo,ilo)=4"),
+    # divisible by three only: 3 x 3 blocks; one index split, the other prime
+    ("A_e_i_j -= B_e_i_k C_e_j_k", [(45, 9, 10), (45, 15, 10)], "tile(ilo,jlo)=9"),
+    ("A_e_i_j = B_e_i_k C_e_k_j D_e_i_j", [(31, 24, 8), (31, 8, 25), (31, 24, 25)], "tile(ilo)=2"),
+    # no blocks: one output per lane, several entries per workgroup; rows of odd length are padded in LDS
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(203, 11, 11), (203, 11, 11)], "8 per workgroup of 256 lanes"),
+    ("A_e_i_j += B_e_i_k C_e_k_j", [(29, 25, 25), (29, 25, 25)], "LDS 10400 bytes"),
+])
+def test_products_of_small_element_matrices(at, engine, checker, kernel, shapes, expect):
+    rng = np.random.default_rng(len(kernel) + shapes[0][0])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    src = engine.GetLastImplementation()
+    assert "operands staged in LDS" in src and expect in src
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
+
+
+def test_product_of_slices_keeps_its_indices(at, engine, checker):
+    # operands that are views into larger tensors are not described by split dimensions
+    rng = np.random.default_rng(12)
+    big = rng.uniform(-1, 1, (2, 50, 12, 12))
+    C = rng.uniform(-1, 1, (50, 12, 12))
+    tbig, tC, tA = to_tensor(at, big), to_tensor(at, C), at.Tensor(50, 12, 12)
+    engine("A_e_i_j = B_e_i_k C_e_k_j", tA, at.SliceTensor(tbig, 1), tC)
+    tA.MoveFromGPU()
+    src = engine.GetLastImplementation()
+    assert "operands staged in LDS" in src and "ihi" not in src
+    assert rel_err(tA.data, np.einsum("eik,ekj->eij", big[1], C)) <= TOL
+
+
 @pytest.mark.parametrize("P,Q,E", [(2, 3, 1001), (4, 5, 203), (3, 4, 77), (8, 10, 5)])
 def test_2d_mass_assembly_results_leave_through_an_lds_tile(at, engine, checker, P, Q, E):
     # unittest/kernel/test_TensorEngine.cpp:399-435 at other sizes.  With lanes (i2, j2) / (j1, j2) and a register tile
