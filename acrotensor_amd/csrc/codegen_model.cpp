@@ -264,15 +264,6 @@ auto Generator::StageReusedOperands(int ki, const Sub &asWritten, std::vector<Su
         long reads = 1;
         for (int id : orig.outIdx) reads *= (id == batch || has(r.idx, id)) ? 1 : extent[id];
         wholeLines = wholeLines && (perEntry & (perEntry - 1)) == 0;
-        // (tiny ones: matrices only, an output index and a contraction index each; vectors under a shared operator
-        // belong to the operator schedule)
-        bool carriesOutput = false, carriesContraction = false;
-        for (int id : r.idx)
-        {
-            carriesOutput = carriesOutput || (id != batch && has(orig.outIdx, id));
-            carriesContraction = carriesContraction || has(orig.contr, id);
-        }
-        if (tiny && !(carriesOutput && carriesContraction)) continue;
         if (perEntry < (tiny ? 4 : 16) || perEntry > 1024 || reads < (tiny ? 2 : 8)) continue;
         staged[v] = 1;
         total += perEntry;
@@ -281,6 +272,23 @@ auto Generator::StageReusedOperands(int ki, const Sub &asWritten, std::vector<Su
     // Two such operands: products of element matrices.  With one (an element vector under an element matrix, the
     // vectors of a dense operator) the kernel has schedules of its own that read the big operand once and well.
     if (count < 2 || total > 2048 || (tiny && wholeLines)) return false;
+    // (tiny entries under one shared operator, "A_e_i = B_i_j X_e_j W_e D_e_j", belong to the operator schedule)
+    int operators = 0;
+    for (const auto &r : orig.in)
+    {
+        bool contracted = false, free = false;
+        for (int id : r.idx) (has(orig.contr, id) ? contracted : free) = true;
+        operators += (!has(r.idx, batch) && contracted && free) ? 1 : 0;
+    }
+    if (tiny && operators == 1) return false;
+    // (the same for vectors of any length with pointwise factors of their shape, "A_e_i = B_i_j X_e_j D_e_j")
+    bool vectorsOnly = true;
+    for (size_t v = 0; v < orig.in.size(); ++v)
+    {
+        if (!staged[v]) continue;
+        for (int id : orig.in[v].idx) vectorsOnly = vectorsOnly && (id == batch || !has(orig.outIdx, id));
+    }
+    if (operators == 1 && vectorsOnly) return false;
     // With one output per lane every multiply-add reads both of its factors from LDS, and LDS bounds the kernel
     // (24 x 24 products: 48 % of the HBM peak, 30 x 30: 35 %).  A lane that owns a 2 x 2 block of outputs reads half
     // as much.  Register tiles are whole indices, so an output index of even extent is split in two, "i = 2 i' + i''"

@@ -138,7 +138,18 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
     o.rows = product(rows, extent);
     o.cols = product(cols, extent);
     o.entries = product(lead, extent) * o.comp;
-    if (o.rows > 1024 || o.rows * o.cols > 4096) return false;
+    if (o.rows > 1024 || o.rows * o.cols > 4096)
+    {
+        // Too large for LDS as a whole (the gradient at every point of an element, 192 x 64; 375 x 125): blocks of
+        // rows that fit, each applied by a launch of its own to all entries, on the matrix cores.  The vectors are
+        // read once per block, from the last-level cache where they fit (generic schedule, a row per lane with the
+        // operator read from device memory by every workgroup: 2.4 % of the HBM peak).
+        const long paddedCols = (o.cols + 7) / 8 * 8;
+        o.blockRows = 8192 / paddedCols / 16 * 16;
+        if (!alone || o.cols > 256 || o.rows > 8192 || o.blockRows < 16 || o.trailing || o.comp > 1 || envInt("ACRO_HIP_OPERATOR_BLOCKS") < 0 ||
+            envInt("ACRO_HIP_OPERATOR_MFMA") < 0)
+            return false;
+    }
     // With components: vectors in 8-byte loads, no pointwise factors, and only where the generic schedule (an
     // entry and a row per lane) runs out of scalar registers for the operator or of coalescing for its stores
     // (64 x 64 with three components: 7 % of the HBM peak).
@@ -173,6 +184,7 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
     if (!o.cores) return o.rows >= 16 && o.cols >= 16 && !o.transposed && !o.trailing && s.in.size() == 2 && o.comp == 1;  // (its lanes walk the operator's rows)
     // A lane holds cols / 4 vector elements and rows / 4 results; the padded operator must fit the 64 KB of LDS
     // that a workgroup may declare.
+    if (o.blockRows > 0) return true;
     if (o.rows > 256 || o.cols > 256 || ((o.rows + 15) / 16 * 16) * ((o.cols + 7) / 8 * 8) > 8192) return false;
     if (o.trailing)
     {
@@ -206,7 +218,7 @@ auto Generator::UseOperatorSequence() const -> bool
     for (int k = 0; k < NumOpKernels(); ++k)
     {
         OperatorShape o;
-        if (!OperatorPattern(o, k, false) || !o.cores || o.rows * o.cols < 512) return false;
+        if (!OperatorPattern(o, k, false) || !o.cores || o.rows * o.cols < 512 || o.blockRows > 0) return false;
     }
     return true;
 }
@@ -218,6 +230,7 @@ auto Generator::OperatorPair(OperatorShape &first, OperatorShape &second) const 
     if (NumOpKernels() != 2 || envInt("ACRO_HIP_OPERATOR_PAIR") < 0) return false;
     if (!OperatorPattern(first, 0, false) || !OperatorPattern(second, 1, false)) return false;
     if (!first.cores || !second.cores || first.trailing || second.trailing || first.comp > 1 || second.comp > 1) return false;
+    if (first.blockRows > 0 || second.blockRows > 0) return false;
     const Sub &k0 = OpKernel(0), &k1 = OpKernel(1);
     if (k0.op != '=' || second.x->uvar != k0.out.uvar || second.x->idx != k0.out.idx) return false;
     if (uvars[k1.out.uvar].storage == uvars[k0.out.uvar].storage) return false;
@@ -277,6 +290,26 @@ auto Generator::EmitOperator(HipKernelPlan &plan) -> void
     const Sub &s = OpKernel(0);
     OperatorShape shape;
     OperatorPattern(shape);
+    if (shape.blockRows > 0)
+    {
+        std::string schedule;
+        int lds = 0;
+        for (long r0 = 0; r0 < shape.rows; r0 += shape.blockRows, ++opBlock)
+        {
+            OperatorShape block = shape;
+            block.allRows = shape.rows;
+            block.rowOffset = r0;
+            block.rows = std::min(shape.blockRows, shape.rows - r0);
+            EmitOperatorMatrixCores(plan, block);
+            schedule += plan.schedule;
+            lds = std::max(lds, plan.lds_bytes);
+        }
+        opBlock = 0;
+        plan.schedule = schedule;
+        plan.lds_bytes = lds;
+        plan.module_name = plan.launches.front().function_name;
+        return;
+    }
     const VarRef *opr = shape.op, *x = shape.x;
     const long nJ = shape.cols, nI = shape.rows;
     const long E = shape.entries;        // entries of this schedule: all leading indices together
@@ -388,6 +421,9 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     const Sub &s = OpKernel(opSub);
     const VarRef &opr = *shape.op, &x = *shape.x;
     const long nI = shape.rows, nJ = shape.cols, E = shape.entries;
+    // (a block of rows of a larger operator: rows row0 .. row0 + nI of nAll)
+    const long nAll = shape.allRows > 0 ? shape.allRows : nI, row0 = shape.rowOffset;
+    const bool first = opSub == 0 && opBlock == 0;
     // Sizes that the instruction's 16 x 4 blocks do not divide: the operator's copy in LDS is padded with zero
     // rows and columns, the entries' vectors read as zero past their end, outputs past the last row are not
     // stored.  Pairs of doubles (16-byte loads) need an even row length and an even first element.
@@ -397,6 +433,20 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     // 33 x 33 63 -> 41 %, 9 x 9 59 -> 39 %; only 27 x 27 gained, 66 -> 70 %.)
     const long nIp = (nI + 15) / 16 * 16, nJp = pairs ? (nJ + 7) / 8 * 8 : (nJ + 3) / 4 * 4;
     const long tilesN = nIp / 16, steps = nJp / 4;
+    // Rows that the instruction's 16-row blocks do not divide: a lane's stores would be single doubles in runs of 128
+    // bytes that start anywhere in a line (81 x 8: 31 % of the HBM peak, 80 x 8: 73 %).  The 16 entries of a trip lie
+    // next to each other in memory, so the wavefront collects their results in LDS in memory order and writes them
+    // out as one contiguous range.
+    // (all 16 entries at once where LDS allows, else 8 or 4 at a time)
+    int stageRounds = 0;
+    if (!next && shape.allRows == 0 && shape.comp == 1 && nI % 16 != 0 && envInt("ACRO_HIP_OPERATOR_STAGE_OUT") >= 0)
+    {
+        for (int rounds : {1, 2, 4})
+        {
+            if (stageRounds == 0 && (nIp * nJp + 64 / rounds * nI) * 8 <= 64 * 1024) stageRounds = rounds;
+        }
+    }
+    const bool viaStage = stageRounds > 0;
     const long steps2 = (nI + 3) / 4;                 // the second operator contracts over this one's rows
     const long midStride = nI % 2 == 0 ? nI + 1 : nI; // odd: the lanes' rows of the hand-over buffer start in different banks
     const long tiles = (E + 15) / 16;
@@ -405,7 +455,9 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     // With one or two loads per lane and trip a wavefront has little in flight, and twice the wavefronts help
     // once the tensors exceed the 256 MB of last-level cache (8 x 8 on 2^23 entries: 227 us with 512
     // workgroups, 185 us with 1 024, 216 us with 2 048; 64 x 64 on 2^18: 47 / 54 / 62 us).
-    const long most = pairs && nJp <= 16 ? 1024 : 512;
+    // (An operator above 32 KB: one workgroup per CU, since every workgroup reads all of it.  192 x 64 on 2^15 entries:
+    // 34.6 -> 26.9 us; 375 x 125 on 2^17: 410 -> 320 us; 1 024 workgroups: 558 us.)
+    const long most = nIp * nJp > 4096 ? 256 : (pairs && nJp <= 16 ? 1024 : 512);
     const long blocks = std::max<long>(1, std::min<long>(most, (tiles + 3) / 4));
     for (const auto &st : stores)
     {
@@ -416,13 +468,16 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     const std::string dimName = mk.GetDimensionedNameString();
     char hex[32];
     std::snprintf(hex, sizeof(hex), "%016llx",
-                  static_cast<unsigned long long>(hashString(dimName + "/operator-mfma/" + str(opSub) + "/" + (Positional() ? "p" : "u") + (pairs ? "2" : "1") + (next ? "+" : "") + (shape.comp > 1 ? "c" + str(shape.comp) : ""))));
+                  static_cast<unsigned long long>(hashString(dimName + "/operator-mfma/" + str(opSub) + (shape.allRows > 0 ? "@" + str(row0) : std::string()) + "/" + (Positional() ? "p" : "u") + (pairs ? "2" : "1") + (next ? "+" : "") + (shape.comp > 1 ? "c" + str(shape.comp) : ""))));
     plan.module_name = std::string("acro_op_") + hex;
     std::ostringstream sched;
-    sched << "operator schedule on the FP64 matrix cores: " << nI << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator")
-          << " in LDS in operand order";
+    sched << "operator schedule on the FP64 matrix cores: ";
+    if (shape.allRows > 0) sched << "rows " << row0 << " - " << row0 + nI - 1 << " of the " << nAll << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator");
+    else sched << nI << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator");
+    sched << " in LDS in operand order";
     if (nIp != nI || nJp != nJ) sched << " (padded to " << nIp << " x " << nJp << ")";
     if (shape.comp > 1) sched << ", " << shape.comp << " components per vector element";
+    if (viaStage) sched << ", results written out through LDS";
     sched << ", " << E << " entries, 16 per wavefront and trip, "
           << tilesN * steps << " v_mfma_f64_16x16x4 per trip, " << blocks << " workgroups of 256 lanes\n  [" << opSub << "] " << s.text << "\n";
     if (next)
@@ -430,7 +485,7 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
               << " applied to the first result on chip (handed over through " << 16 * midStride * 8 << " bytes of LDS per wavefront)\n";
     plan.schedule = sched.str();
 
-    if (opSub == 0) out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
+    if (first) out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
     {
         std::istringstream lines(plan.schedule);
         std::string l;
@@ -440,7 +495,7 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     const bool stream = s.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0;
     // term group g (lane / 16) of step s stands for this j
     const std::string termOf = pairs ? "8 * (step >> 1) + 2 * (l >> 4) + (step & 1)" : "4 * step + (l >> 4)";
-    out << (opSub == 0 ? "" : "\n") << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
+    out << (first ? "" : "\n") << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
     // Two doubles moved by one 16-byte instruction.  The type only promises the 8-byte alignment that every
     // operand has (a caller's device buffer, a slice at an odd offset of it); the hardware takes such
     // addresses for accesses to device memory.
@@ -450,11 +505,13 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     out << "    for (int f = threadIdx.x; f < " << nIp * nJp << "; f += 256)\n    {\n";
     out << "        const int l = f & 63, step = (f >> 6) % " << steps << ", t = (f >> 6) / " << steps << ";\n";
     out << "        const int row = 16 * t + (l & 15), j = " << termOf << ";\n";
-    const std::string element = B + "[" + Lit(uvars[opr.uvar].viewOffset) + (shape.transposed ? " + j * " + str(nI) + " + row]" : " + row * " + str(nJ) + " + j]");
+    const std::string rowHere = row0 > 0 ? "(row + " + str(row0) + ")" : std::string("row");
+    const std::string element = B + "[" + Lit(uvars[opr.uvar].viewOffset) + (shape.transposed ? " + j * " + str(nAll) + " + " + rowHere + "]" : " + " + rowHere + " * " + str(nJ) + " + j]");
     if (nIp != nI || nJp != nJ)
         out << "        frag[f] = row < " << nI << " && j < " << nJ << " ? " << element << " : 0.0;\n    }\n";
     else
         out << "        frag[f] = " << element << ";\n    }\n";
+    if (viaStage) out << "    __shared__ double stage[" << 64 / stageRounds * nI << "];\n";
     if (next)
     {
         // the second operator: its columns are the first one's rows, terms in natural order
@@ -547,8 +604,57 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
         const long rowsP = (rows + 15) / 16 * 16;
         const bool streams = ks.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0;
         const long C = sh.comp;
+        // (a block of rows: the entries' results lie `stride` apart and start at row `off`)
+        const long stride = sh.allRows > 0 ? sh.allRows : rows, off = sh.rowOffset;
+        if (viaStage)
+        {
+            const int perRound = 4 / stageRounds;   // result registers (entries g + 4 r) per round
+            out << "        double *mid = stage + (threadIdx.x >> 6) * " << 4 * perRound * rows << ";\n";
+            for (int h = 0; h < stageRounds; ++h)
+            {
+                out << "#pragma unroll\n";
+                out << "        for (int r = " << h * perRound << "; r < " << (h + 1) * perRound << "; ++r)\n        {\n";
+                std::string staged = accName + "[t][r]";
+                const bool scaledHere = !sh.perEntry.empty() || !sh.perOutput.empty() || !sh.perRow.empty();
+                if (scaledHere)
+                    out << "            const long en = " << (ragged ? "tile * 16 + g + 4 * r < " + str(E) + " ? tile * 16 + g + 4 * r : " + str(E - 1) : std::string("tile * 16 + g + 4 * r")) << ";\n";
+                if (!sh.perEntry.empty())
+                {
+                    out << "            const double se = ";
+                    for (size_t i = 0; i < sh.perEntry.size(); ++i)
+                        out << (i ? " * " : "") << PtrName(sh.perEntry[i]->uvar) << "[" << Lit(uvars[sh.perEntry[i]->uvar].viewOffset) << " + en]";
+                    out << ";\n";
+                    staged += " * se";
+                }
+                for (const VarRef *w : sh.perOutput)
+                    staged += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + " + en * " + str(rows) + " + 16 * t + c]";
+                for (const VarRef *w : sh.perRow)
+                    staged += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + " + 16 * t + c]";
+                out << "#pragma unroll\n";
+                out << "            for (int t = 0; t < " << rowsP / 16 << "; ++t)\n";
+                out << "                if (16 * t + c < " << rows << ") mid[(4 * " << (h ? "(r - " + str(static_cast<long>(h * perRound)) + ")" : std::string("r")) << " + g) * " << rows << " + 16 * t + c] = " << staged << ";\n";
+                out << "        }\n";
+                out << "        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");\n        __builtin_amdgcn_wave_barrier();\n";
+                out << "        {\n";
+                const long firstEntry = 4L * h * perRound, entries = 4L * perRound;
+                out << "            double *a = " << PtrName(ks.out.uvar) << " + " << Lit(uvars[ks.out.uvar].viewOffset) << " + (tile * 16 + " << firstEntry << ") * " << rows << ";\n";
+                if (ragged)
+                    out << "            const long left = " << E << " - tile * 16 - " << firstEntry << ";\n"
+                        << "            const int count = (int)(left < 0 ? 0 : (left < " << entries << " ? left : " << entries << ")) * " << rows << ";\n";
+                else
+                    out << "            const int count = " << entries * rows << ";\n";
+                out << "            for (int i = lane; i < count; i += 64)\n";
+                if (streams)
+                    out << "                __builtin_nontemporal_store(mid[i], a + i);\n";
+                else
+                    out << "                a[i]" << (ks.op == '=' ? " = " : (ks.op == '+' ? " += " : " -= ")) << "mid[i];\n";
+                out << "        }\n";
+                out << "        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");\n        __builtin_amdgcn_wave_barrier();\n";
+            }
+            return;
+        }
         if (!toLds && C == 1)
-            out << "        double *a = " << PtrName(ks.out.uvar) << " + " << Lit(uvars[ks.out.uvar].viewOffset) << " + (tile * 16 + g) * " << rows << " + c;\n";
+            out << "        double *a = " << PtrName(ks.out.uvar) << " + " << Lit(uvars[ks.out.uvar].viewOffset) << " + (tile * 16 + g) * " << stride << (off ? " + " + str(off) : std::string()) << " + c;\n";
         out << "#pragma unroll\n";
         out << "        for (int r = 0; r < 4; ++r)\n        {\n";
         if (ragged) out << "            if (tile * 16 + g + 4 * r >= " << E << ") continue;\n";
@@ -572,9 +678,9 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
             value += " * se";
         }
         for (const VarRef *w : sh.perOutput)
-            value += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + " + en * " + str(rows) + " + 16 * t + c]";
+            value += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + " + en * " + str(stride) + (off ? " + " + str(off) : std::string()) + " + 16 * t + c]";
         for (const VarRef *w : sh.perRow)
-            value += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + " + 16 * t + c]";
+            value += " * " + PtrName(w->uvar) + "[" + Lit(uvars[w->uvar].viewOffset) + (off ? " + " + str(off) : std::string()) + " + 16 * t + c]";
         out << "#pragma unroll\n";
         out << "            for (int t = 0; t < " << rowsP / 16 << "; ++t)\n";
         std::string guard = rowsP != rows ? "if (16 * t + c < " + str(rows) + ") " : "";
@@ -583,9 +689,9 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
         else if (C > 1)
             out << "                " << guard << "a[" << 16 * C << " * t]" << (ks.op == '=' ? " = " : (ks.op == '+' ? " += " : " -= ")) << value << ";\n";
         else if (streams)
-            out << "                " << guard << "__builtin_nontemporal_store(" << value << ", a + 4 * r * " << rows << " + 16 * t);\n";
+            out << "                " << guard << "__builtin_nontemporal_store(" << value << ", a + 4 * r * " << stride << " + 16 * t);\n";
         else
-            out << "                " << guard << "a[4 * r * " << rows << " + 16 * t]" << (ks.op == '=' ? " = " : (ks.op == '+' ? " += " : " -= ")) << value << ";\n";
+            out << "                " << guard << "a[4 * r * " << stride << " + 16 * t]" << (ks.op == '=' ? " = " : (ks.op == '+' ? " += " : " -= ")) << value << ";\n";
         out << "        }\n";
     };
     (void)A;
@@ -636,7 +742,7 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
 
     plan.source = out.str();
     plan.nb = 64;
-    plan.lds_bytes = static_cast<int>((nIp * nJp + (next ? (next->rows + 15) / 16 * 16 * steps2 * 4 + 64 * midStride : 0)) * 8);
+    plan.lds_bytes = static_cast<int>((nIp * nJp + (next ? (next->rows + 15) / 16 * 16 * steps2 * 4 + 64 * midStride : 0) + (viaStage ? 64 / stageRounds * nI : 0)) * 8);
     FillParams(plan, false);
     HipLaunch launch;
     launch.function_name = plan.module_name;

@@ -294,6 +294,11 @@ auto Generator::ChooseTiles() -> void
             {
                 const long tc = product(t, extent);
                 if (tc > kMaxTile || tc * s.contrCount * nin > kUnrollBudget) continue;
+                // (the copies of staged operands are made by many lanes per entry: the kernel that reads them keeps at
+                // least four, or its workgroups would be mostly idle there)
+                bool readsStagedCopy = false;
+                for (const auto &r : s.in) readsStagedCopy = readsStagedCopy || uvars[r.uvar].isStagedCopy;
+                if (readsStagedCopy && !t.empty() && product(mid, extent) / tc < 4) continue;
                 const long loads = LoadsPerItem(s, t);
                 // (operands staged in LDS tiles are cheap to read again: the compiler need not keep them all, and a
                 // row of outputs per lane halves the reads: 16 x 16 matrix products 77 -> 84 % of the HBM peak)
@@ -327,7 +332,16 @@ auto Generator::ChooseTiles() -> void
             // The same for a tiny product whose operands were copied to LDS tiles first: one output per lane keeps the
             // stores of a wavefront contiguous.
             bool fromStagedCopies = (outputs < 64 || (outputs < 200 && s.wantedTile.empty())) && !s.in.empty();
-            for (const auto &r : s.in) fromStagedCopies = fromStagedCopies && (uvars[r.uvar].isStagedCopy || !has(r.idx, batch));
+            for (const auto &r : s.in)
+            {
+                fromStagedCopies = fromStagedCopies && (uvars[r.uvar].isStagedCopy || !has(r.idx, batch));
+                // (matrices: every copy carries an output index; copies that all outputs of an entry share leave the
+                // tile to the cost model, "Y_e_i_j = B_q_i B_r_j D_e_q_r U_e_q_r": 60 % with one output per lane,
+                // 77 % with a row)
+                bool carriesOutput = false;
+                for (int id : r.idx) carriesOutput = carriesOutput || has(mid, id);
+                if (uvars[r.uvar].isStagedCopy && !carriesOutput) fromStagedCopies = false;
+            }
             bool anyStagedCopy = false;
             for (const auto &r : s.in) anyStagedCopy = anyStagedCopy || uvars[r.uvar].isStagedCopy;
             if (fromStagedCopies && anyStagedCopy) best.clear();
@@ -354,7 +368,11 @@ auto Generator::ChooseTiles() -> void
             {
                 if (perEntry(r) > perEntry(*most)) most = &r;
             }
-            const bool streams = has(most->idx, batch) && most->idx.back() == s.contr.back();
+            bool streams = has(most->idx, batch) && most->idx.back() == s.contr.back();
+            // ... and a row of its own for every output: where the outputs of an entry all read the same few values
+            // ("Y_e_i_j = B_q_i B_r_j D_e_q_r U_e_q_r") the lanes of an entry would only repeat each other's loads
+            // (8.7 % of the HBM peak against 55 % with a row of outputs per lane)
+            for (int id : mid) streams = streams && has(most->idx, id);
             if (streams)
             {
                 // At most a row of 16 lanes: the exchanges inside a row are register moves, not LDS traffic.  With

@@ -89,6 +89,8 @@
 //                               in LDS, one entry per lane) instead of the operator schedule
 //   ACRO_HIP_LIGHT=-1           streaming groups whose workgroups move less than 2.5 KB keep their batch size (no extra
 //                               passes to bring a workgroup to 8 KB)
+//   ACRO_HIP_OPERATOR_BLOCKS=-1 operators of more than 4 096 entries are not applied in blocks of rows (generic schedule instead)
+//   ACRO_HIP_OPERATOR_STAGE_OUT=-1  results of operators whose rows 16 does not divide are stored by the lanes that hold them
 //   ACRO_HIP_OPERATOR_FOLD=-1   a pointwise kernel that rescales an operator kernel's transient result is not folded into it
 //   ACRO_HIP_OPERATOR_PAIR=-1   two operator-shaped kernels with a transient intermediate are not joined into one matrix-core kernel
 //   ACRO_HIP_OPERATOR_SEQUENCE=-1  groups of several large operator-shaped kernels run as one fused chain kernel instead of one

@@ -396,6 +396,9 @@ class Generator
     {
         const VarRef *op = nullptr, *x = nullptr;
         long rows = 0, cols = 0, entries = 0;
+        // An operator too large for LDS is applied in blocks of rows, one launch per block: `blockRows` rows at a
+        // time (0: whole).  The emitter then sees `rows` rows starting at `rowOffset` of `allRows`.
+        long blockRows = 0, rowOffset = 0, allRows = 0;
         bool transposed = false;   // the operator is stored with the contracted indices first: "B_j_i"
         bool cores = false;        // sizes and alignment suit the FP64 matrix cores
         bool pairs = false;        // the entries' vectors (and weights of their shape) come in 16-byte loads
@@ -415,6 +418,7 @@ class Generator
 
 
     int opSub = 0;            // the kernel that the operator emitters work on
+    int opBlock = 0;          // ... and the block of rows, for an operator applied in blocks
     bool opSequence = false;  // ... as one of several launches
     void EmitOperator(HipKernelPlan &plan);
     void EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape &shape, const OperatorShape *next = nullptr, int nextSub = -1);

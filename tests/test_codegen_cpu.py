@@ -199,14 +199,16 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     src = TE.GetImplementation("A_e_i1_i2 -= X_e_j1_j2 B_i1_i2_j1_j2", at.Tensor(77, 5, 6), at.Tensor(77, 4, 7), at.Tensor(5, 6, 4, 7))
     assert "30 x 28 operator in LDS in operand order (padded to 32 x 32)" in src
     assert "frag[f] = row < 30 && j < 28 ? T2[0 + row * 28 + j] : 0.0;" in src
-    assert "8 * q + 2 * g >= 28 ? double2{0.0, 0.0} :" in src and "if (16 * t + c < 30) a[4 * r * 30 + 16 * t] -= acc[t][r];" in src
+    assert "8 * q + 2 * g >= 28 ? double2{0.0, 0.0} :" in src and "if (16 * t + c < 30) mid[(4 * r + g) * 30 + 16 * t + c] = acc[t][r];" in src and "a[i] -= mid[i];" in src
     src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 30), at.Tensor(30, 27), at.Tensor(1000, 27))
     assert "(padded to 32 x 28)" in src and "j = 4 * step + (l >> 4);" in src and "xv[q] = 4 * q + g >= 27 ? 0.0 : x[4 * q];" in src
     # pointwise factors: per entry, per output and per row on the result, per element and per column on the vectors
     src = TE.GetImplementation("A_e_i -= B_i_j X_e_j W_e D_e_j R_i F_e_i C_j", at.Tensor(1000, 10), at.Tensor(10, 12), at.Tensor(1000, 12),
                                at.Tensor(1000), at.Tensor(1000, 12), at.Tensor(10), at.Tensor(1000, 10), at.Tensor(12))
     assert "operator schedule on the FP64 matrix cores: 10 x 12 operator" in src and "const double se = T3[0 + en];" in src
-    assert "-= acc[t][r] * se * T6[0 + en * 10 + 16 * t + c] * T5[0 + 16 * t + c];" in src
+    # (10 rows: the results of a trip's 16 entries are collected in LDS in memory order and leave as one contiguous range)
+    assert "mid[(4 * r + g) * 10 + 16 * t + c] = acc[t][r] * se * T6[0 + en * 10 + 16 * t + c] * T5[0 + 16 * t + c];" in src
+    assert "results written out through LDS" in src and "for (int i = lane; i < count; i += 64)" in src and "a[i] -= mid[i];" in src
     assert "const acro_pair f = *reinterpret_cast<const acro_pair *>(T4 + 0 + ex * 12 + 2 * g + 8 * q);" in src and "const double *f = T7 + 0 + 2 * g + 8 * q;" in src
     # the entries as the fastest dimension: the operator becomes the instruction's first operand
     src = TE.GetImplementation("A_i_e -= B_i_j X_j_e W_e", at.Tensor(30, 1002), at.Tensor(30, 27), at.Tensor(27, 1002), at.Tensor(1002))
@@ -215,6 +217,10 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     src = TE.GetImplementation("A_i_e = B_i_j X_j_e", at.Tensor(64, 1001), at.Tensor(64, 64), at.Tensor(64, 1001))
     assert "1001 entries, 16 per wavefront and trip" in src and "__builtin_nontemporal_store(v, a);" in src and "acc1" not in src
     assert "operator schedule" not in TE.GetImplementation("A_i_e = B_i_j X_j_e", at.Tensor(16, 3000), at.Tensor(16, 16), at.Tensor(16, 3000))
+    # an operator too large for LDS: blocks of rows, a launch each
+    src = TE.GetImplementation("G_e_d_q = D_d_q_i X_e_i", at.Tensor(1000, 3, 64), at.Tensor(3, 64, 64), at.Tensor(1000, 64))
+    assert "rows 0 - 127 of the 192 x 64 operator" in src and "rows 128 - 191 of the 192 x 64 operator" in src and src.count("__global__") == 2
+    assert "frag[f] = T1[0 + (row + 128) * 64 + j];" in src and "double *a = T0 + 0 + (tile * 16 + g) * 192 + 128 + c;" in src
     # very long vectors or very many rows would not fit a lane's registers: not this schedule
     assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 5), at.Tensor(5, 818), at.Tensor(900, 818))
     assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 300), at.Tensor(300, 12), at.Tensor(900, 12))

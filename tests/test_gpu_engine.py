@@ -612,6 +612,29 @@ def test_dense_operator_applied_to_every_entry(at, engine, checker, kernel, shap
     assert rel_err(got, expected) <= TOL
 
 
+@pytest.mark.parametrize("kernel,shapes,expect", [
+    # rows that 16 does not divide: the 16 entries of a trip leave through LDS as one contiguous range
+    ("A_e_i = B_i_j X_e_j", [(81, 8), (1003, 8)], "results written out through LDS"),
+    ("A_e_i -= B_i_j X_e_j W_e R_e_i", [(27, 12), (999, 12), (999,), (999, 27)], "results written out through LDS"),
+    ("A_e_i += B_j_i X_e_j", [(8, 125), (2001, 8)], "__shared__ double stage[4000]"),      # 8 entries at a time
+    ("A_e_i = B_i_j X_e_j", [(250, 16), (517, 16)], "left < 4 ? left : 4"),                 # 4 at a time
+    # too large for LDS: blocks of rows, one launch each (the gradient at the 64 points of an element)
+    ("G_e_d_q = D_d_q_i X_e_i", [(3, 64, 64), (1001, 64)], "rows 128 - 191 of the 192 x 64 operator"),
+    ("A_e_i -= B_j_i X_e_j W_e R_i", [(125, 375), (403, 125), (403,), (375,)], "rows 320 - 374 of the 375 x 125 operator (stored transposed)"),
+    ("A_e_i += X_e_j B_i_j D_e_j", [(1500, 30), (1000, 30), (1500, 30)], "rows 768 - 999 of the 1000 x 30 operator"),
+])
+def test_dense_operators_with_odd_rows_or_too_large_for_lds(at, engine, checker, kernel, shapes, expect):
+    rng = np.random.default_rng(shapes[0][0] + len(kernel))
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    src = engine.GetLastImplementation()
+    assert "operator schedule on the FP64 matrix cores" in src and expect in src
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
+
+
 @pytest.mark.parametrize("kernel,shapes", [
     ("A_e_i = B_i_j X_e_j W_e", [(64, 64), (1000, 64), (1000,)]),                    # one factor per entry
     ("A_e_i += B_i_j X_e_j W_e", [(40, 24), (43, 24), (43,)]),                       # three trips, the last with 11 entries
