@@ -343,6 +343,7 @@ class Generator
     bool StoresToGlobal(int k) const { return !StoreOf(subs[k].out.uvar).elide && !StoreIsDead(k); }
     bool StreamsOut(int k) const;
     double WaveStoreLineCoverage(int k, int entries = 0) const;
+    bool WritesDominate() const;
     bool SplitLanesTakePairs(int k) const;
     std::string GlobalStore(int k, const std::string &gaddr, const std::string &value) const;
     bool NeedsLdsCopy(int k) const;
