@@ -92,12 +92,14 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
     // and X share, the batch index first, number the entries
     if (s.out.idx.empty()) return false;
     std::vector<int> lead, rows, cols;
-    if (s.out.idx[0] == batch && o.x->idx[0] == batch)
+    size_t sharedLeading = 0;
+    while (sharedLeading < s.out.idx.size() && sharedLeading < o.x->idx.size() && s.out.idx[sharedLeading] == o.x->idx[sharedLeading] &&
+           !has(o.op->idx, s.out.idx[sharedLeading]))
+        ++sharedLeading;
+    // (the batch index anywhere among them: "A_i_e_j = B_i_e_k C_k_j" has the entries (i, e))
+    if (has(std::vector<int>(s.out.idx.begin(), s.out.idx.begin() + sharedLeading), batch))
     {
-        size_t shared = 0;
-        while (shared < s.out.idx.size() && shared < o.x->idx.size() && s.out.idx[shared] == o.x->idx[shared] &&
-               !has(o.op->idx, s.out.idx[shared]))
-            ++shared;
+        const size_t shared = sharedLeading;
         lead.assign(s.out.idx.begin(), s.out.idx.begin() + shared);
         rows.assign(s.out.idx.begin() + shared, s.out.idx.end());
         cols.assign(o.x->idx.begin() + shared, o.x->idx.end());

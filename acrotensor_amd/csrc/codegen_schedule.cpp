@@ -328,7 +328,11 @@ auto Generator::ChooseTiles() -> void
             for (const auto &r : s.in)
                 streamingOnly = streamingOnly && (has(r.idx, batch) || (smallInvariantToo && r.size <= 1024)) && !r.repeated;
             const long outputs = product(mid, extent), loadsPerOutput = s.contrCount * nin;
-            if (streamingOnly && ((outputs <= 32 && loadsPerOutput <= 16) || (outputs <= 64 && loadsPerOutput <= 4))) best.clear();
+            // (without a contraction, products of the entries' own values "A_e_i_j_k_l = B_e_i_j C_e_k_l", up to 256
+            // outputs: 62 -> 84 % of the HBM peak, 16 x 16 outer product 81 -> 87 %; with 512 outputs and more a
+            // register tile wins, 73 against 55 %)
+            const long flatUpTo = s.contr.empty() ? 256 : 64;
+            if (streamingOnly && ((outputs <= 32 && loadsPerOutput <= 16) || (outputs <= flatUpTo && loadsPerOutput <= 4))) best.clear();
             // The same for a tiny product whose operands were copied to LDS tiles first: one output per lane keeps the
             // stores of a wavefront contiguous.
             bool fromStagedCopies = (outputs < 64 || (outputs < 200 && s.wantedTile.empty())) && !s.in.empty();

@@ -622,6 +622,8 @@ def test_dense_operator_applied_to_every_entry(at, engine, checker, kernel, shap
     ("G_e_d_q = D_d_q_i X_e_i", [(3, 64, 64), (1001, 64)], "rows 128 - 191 of the 192 x 64 operator"),
     ("A_e_i -= B_j_i X_e_j W_e R_i", [(125, 375), (403, 125), (403,), (375,)], "rows 320 - 374 of the 375 x 125 operator (stored transposed)"),
     ("A_e_i += X_e_j B_i_j D_e_j", [(1500, 30), (1000, 30), (1500, 30)], "rows 768 - 999 of the 1000 x 30 operator"),
+    # the batch index second among the indices that number the entries
+    ("A_i_e_j -= B_i_e_k C_k_j W_i_e", [(8, 501, 16), (16, 12), (8, 501)], "4008 entries"),
 ])
 def test_dense_operators_with_odd_rows_or_too_large_for_lds(at, engine, checker, kernel, shapes, expect):
     rng = np.random.default_rng(shapes[0][0] + len(kernel))
