@@ -21,6 +21,11 @@ auto Generator::Run() -> HipKernelPlan
         return plan;
     }
     plan.fusable = true;
+    if (UseGramSchedule())
+    {
+        EmitGram(plan);
+        return plan;
+    }
     if (UseReductionSchedule())
     {
         EmitReduction(plan);

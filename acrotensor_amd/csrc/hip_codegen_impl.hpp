@@ -370,6 +370,17 @@ class Generator
     std::string ParamList() const;
     void EmitReduction(HipKernelPlan &plan);
     bool UseTransposeSchedule() const;
+
+    // "A_I_J = B_N_I C_N_J [W_N]": the I x J matrix of sums over a long leading range N
+    struct GramShape
+    {
+        const VarRef *b = nullptr, *c = nullptr, *w = nullptr;
+        long rows = 0, cols = 0, range = 0;
+        bool swapped = false;   // the result is stored as J x I
+    };
+    bool GramPattern(GramShape &g) const;
+    bool UseGramSchedule() const;
+    void EmitGram(HipKernelPlan &plan);
     void EmitTranspose(HipKernelPlan &plan);
 
     // ------------------------------------------------------------------------------ operator schedule

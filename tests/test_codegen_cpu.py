@@ -119,6 +119,21 @@ def test_split_contraction_with_few_outputs_gives_a_lane_whole_slices(TE, monkey
     assert src.count("__global__") == 1 and "__hip_atomic_fetch_add" in src
 
 
+def test_many_outputs_summed_over_the_batch_take_the_gram_schedule(TE):
+    src = TE.GetImplementation("A_i_j = B_e_i C_e_j", at.Tensor(64, 64), at.Tensor(100000, 64), at.Tensor(100000, 64))
+    assert "Gram schedule on the FP64 matrix cores: 64 x 64 outputs, sums over 100000 rows" in src and src.count("__global__") == 2
+    assert "acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(bv[u][ti], cv[u][tj], acc[ti][tj], 0, 0, 0);" in src and "atomic" not in src
+    # rows of the range past its end and outputs past the last read as zero; the result stored as J x I; a weight per row
+    src = TE.GetImplementation("A_j_i -= B_e_q_i C_e_q_j W_e_q", at.Tensor(50, 40), at.Tensor(1001, 3, 40), at.Tensor(1001, 3, 50), at.Tensor(1001, 3))
+    assert "40 x 50 outputs (stored transposed), sums over 3003 rows" in src and "(inRange && 16 * ti + r < 40) ? b[16 * ti] : 0.0;" in src
+    assert "sums[j * 40 + i]" in src and "bq[u][ti] *= w;" in src and "result[0 + o] - t;" in src
+    # up to 128 outputs: the reduction schedule; more than 16 blocks of 16 x 16: neither
+    assert "reduction schedule" in TE.GetImplementation("A_i_j = B_e_i C_e_j", at.Tensor(8, 8), at.Tensor(100000, 8), at.Tensor(100000, 8))
+    assert "Gram schedule" not in TE.GetImplementation("A_i_j = B_e_i C_e_j", at.Tensor(80, 80), at.Tensor(100000, 80), at.Tensor(100000, 80))
+    # the range must lead both operands
+    assert "Gram schedule" not in TE.GetImplementation("A_i_j = B_i_e C_e_j", at.Tensor(64, 64), at.Tensor(64, 100000), at.Tensor(100000, 64))
+
+
 def test_long_contraction_uses_counted_loops(TE):
     wl = workloads.config1(n=4096)
     tensors = workloads.bind_to_engine(wl, at)
@@ -358,6 +373,11 @@ def generated_sources(TE):
     for transient in (True, False):
         yield "geometric factors from the Jacobians", geometric_factor_source(TE, 7, 4, 3, transient)
     yield "geometric factors, 2 x 2", geometric_factor_source(TE, 7, 3, 2, True)
+    yield "Gram matrix over the batch", TE.GetImplementation("A_j_i -= B_e_q_i C_e_q_j W_e_q", at.Tensor(50, 40), at.Tensor(1001, 3, 40), at.Tensor(1001, 3, 50), at.Tensor(1001, 3))
+    yield "products of element matrices in 2 x 2 blocks", TE.GetImplementation("A_e_i_j += B_e_i_k C_e_j_k", at.Tensor(100, 12, 10), at.Tensor(100, 12, 9), at.Tensor(100, 10, 9))
+    yield "products of tiny element matrices", TE.GetImplementation("A_e_i_j = B_e_i_k C_e_k_j", at.Tensor(1001, 3, 3), at.Tensor(1001, 3, 3), at.Tensor(1001, 3, 3))
+    yield "operator schedule, blocks of rows", TE.GetImplementation("G_e_d_q -= D_d_q_i X_e_i W_e", at.Tensor(1001, 3, 65), at.Tensor(3, 65, 64), at.Tensor(1001, 64), at.Tensor(1001))
+    yield "operator schedule, results through LDS", TE.GetImplementation("A_e_i += B_j_i X_e_j", at.Tensor(2001, 125), at.Tensor(8, 125), at.Tensor(2001, 8))
 
 
 GEOMETRIC_FACTORS = {

@@ -923,17 +923,37 @@ def test_element_matrix_times_vector_with_odd_rows(at, engine, checker, kernel, 
 @pytest.mark.parametrize("n,m,op", [(5000, 8, "="), (3001, 4, "+="), (2500, 7, "-="), (2100, 11, "=")])
 def test_small_gram_matrix_over_the_batch(at, engine, checker, n, m, op):
     # "A_i_j = B_e_i C_e_j": a contraction over the long index with m x m outputs that are products of two short loads;
-    # up to 8 x 8 a lane owns whole slices (m + m loads, m x m accumulators), beyond that one lane per (slice, output)
+    # up to 8 x 8 a lane owns whole slices (m + m loads, m x m accumulators), beyond that the matrix cores take over
     kernel = "A_i_j %s B_e_i C_e_j" % op
     rng = np.random.default_rng(n + m)
     B, C = rng.uniform(-1, 1, (n, m)), rng.uniform(-1, 1, (n, m))
     out0 = rng.uniform(-1, 1, (m, m))
     got, expected = run_single(at, engine, checker, kernel, out0, B, C)
     src = engine.GetLastImplementation()
-    assert "reduction schedule" in src
-    assert ("a lane owns whole slices" in src) == (m <= 8)
+    assert ("reduction schedule" in src and "a lane owns whole slices" in src) if m <= 8 else ("Gram schedule" in src)
     if op == "-=":
         expected = 2.0 * out0 - expected
     assert rel_err(got, expected) <= TOL
     again, _ = run_single(at, engine, checker, kernel, out0, B, C)
     assert np.array_equal(got, again)                   # fixed order of additions: reproducible
+
+
+@pytest.mark.parametrize("kernel,shapes", [
+    ("A_i_j = B_e_i C_e_j", [(40000, 64), (40000, 64)]),                              # 16 blocks per wavefront
+    ("A_j_i -= B_e_q_i C_e_q_j W_e_q", [(1001, 3, 40), (1001, 3, 50), (1001, 3)]),      # ragged everywhere, transposed, weighted
+    ("A_i_j_k += C_n_j_k B_n_i", [(2300, 5, 7), (2300, 12)]),                           # operands the other way round: 35 x 12
+    ("A_i_j = B_e_i C_e_j", [(2049, 16), (2049, 16)]),                                 # one more row than a multiple of four
+])
+def test_many_outputs_summed_over_the_batch(at, engine, checker, kernel, shapes):
+    # more outputs than the reduction schedule takes: 16 x 16 blocks on the FP64 matrix cores, four rows of the range per
+    # instruction, partial sums of the workgroups added by a second kernel in a fixed order
+    rng = np.random.default_rng(shapes[0][0])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "Gram schedule on the FP64 matrix cores" in engine.GetLastImplementation()
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= 4 * TOL            # sums of 10^3 - 10^5 terms in another order than the oracle's
+    again, _ = run_single(at, engine, checker, kernel, out0, *ins)
+    assert np.array_equal(got, again)                   # reproducible
