@@ -349,6 +349,26 @@ auto Generator::ChooseTiles() -> void
             bool anyStagedCopy = false;
             for (const auto &r : s.in) anyStagedCopy = anyStagedCopy || uvars[r.uvar].isStagedCopy;
             if (fromStagedCopies && anyStagedCopy) best.clear();
+            // Entries as the fastest dimension of every tensor: whatever the tile, a wavefront reads 64 consecutive
+            // entries per load, so the tile with the fewest loads per output wins (3 x 3 products of such layouts: a
+            // lane per entry with all nine outputs, 18 loads, instead of nine lanes with six loads each).
+            if (EntriesAreFastest())
+            {
+                double fewest = 1e300;
+                for (const auto &t : candidates)
+                {
+                    const long tc = product(t, extent);
+                    if (tc > kMaxTile || tc * s.contrCount * nin > kUnrollBudget) continue;
+                    const long loads = LoadsPerItem(s, t);
+                    if (loads + tc > kMaxLiveValues && !t.empty()) continue;
+                    const double perOutput = static_cast<double>(loads) / tc;
+                    if (perOutput < fewest * (1.0 - 1e-9))
+                    {
+                        fewest = perOutput;
+                        best = t;
+                    }
+                }
+            }
             if (!s.wantedTile.empty() && product(s.wantedTile, extent) * s.contrCount * nin <= kUnrollBudget) best = s.wantedTile;
             ForcedTile(static_cast<int>(&s - subs.data()), mid, best);
             if (s.flatItems) best.clear();
@@ -1275,6 +1295,37 @@ auto Generator::ChooseBatching() -> void
         else
             for (size_t si = 0; si < stores.size(); ++si) stores[si].ldsOffset = before[si];
     }
+}
+
+// A kernel on its own whose tensors all have the batch index as their fastest dimension ("A_i_e = B_i_e C_i_e",
+// structure-of-arrays layouts): with the work items numbered entry by entry, neighbouring lanes are a whole row of the
+// batch apart (24 % of the HBM peak for that product).  The items are numbered with the entry fastest instead, 64 or
+// more entries per workgroup, so that a wavefront reads and writes 64 consecutive entries of one row.
+auto Generator::EntriesAreFastest() const -> bool
+{
+    if (envInt("ACRO_HIP_ENTRIES_FASTEST") < 0 || subs.size() != 1 || batch < 0 || E < 4096) return false;
+    if (opt.force_nb > 0 || opt.force_nt > 0 || envInt("ACRO_HIP_NB") > 0 || envInt("ACRO_HIP_NT") > 0) return false;
+    const Sub &s = subs[0];
+    if (s.matrixOp != 0) return false;
+    auto entryLast = [&](const VarRef &r) { return !r.repeated && !r.idx.empty() && r.idx.back() == batch; };
+    if (!entryLast(s.out)) return false;
+    for (const auto &r : s.in)
+    {
+        if (has(r.idx, batch) && !entryLast(r)) return false;
+    }
+    return true;
+}
+
+auto Generator::ChooseEntriesFastest() -> void
+{
+    entriesFastest = false;
+    if (!EntriesAreFastest() || ldsDoubles > 0) return;
+    const Sub &s = subs[0];
+    if (s.splitLanes != 0 || s.loopMode || s.laneCount > 1024) return;
+    NB = s.laneCount >= 4 ? 64 : (s.laneCount >= 2 ? 128 : 256);
+    NT = 256;
+    batchUniform = false;
+    entriesFastest = true;
 }
 
 // ----------------------------------------------------------------------------- LDS bank conflicts

@@ -93,6 +93,7 @@ auto Generator::Run() -> HipKernelPlan
             return plan;
         }
     }
+    ChooseEntriesFastest();
     Emit(plan);
     return plan;
 }

@@ -193,6 +193,7 @@ class Generator
     bool batchUniform = false;  // one batch entry per workgroup: the batch index is a scalar
     double busyLanes = 1.0;     // share of busy lanes in the wavefronts that the chosen batching issues
     bool lightWorkgroups = false;  // the batch was raised because a workgroup would have moved too few bytes
+    bool entriesFastest = false;   // the work items of a workgroup are numbered with the batch entry fastest
     bool wide = false;          // 64-bit device-memory offsets
 
     // Literal of a device-memory stride or offset, and the type such offsets are computed in.
@@ -282,6 +283,8 @@ class Generator
     int PlaceLds(int nb);
     int PlaceLdsFromBothEnds(int nb);
     void ChooseBatching();
+    bool EntriesAreFastest() const;
+    void ChooseEntriesFastest();
     static long ConflictCycles(const std::vector<long> &addr);
     std::vector<long> LaneAddresses(const Sub &s, const VarRef &r, int nb) const;
     long LdsCostOfStorage(int si, int nb) const;

@@ -134,6 +134,14 @@ def test_many_outputs_summed_over_the_batch_take_the_gram_schedule(TE):
     assert "Gram schedule" not in TE.GetImplementation("A_i_j = B_i_e C_e_j", at.Tensor(64, 64), at.Tensor(64, 100000), at.Tensor(100000, 64))
 
 
+def test_entry_last_layouts_number_the_items_with_the_entry_fastest(TE):
+    src = TE.GetImplementation("A_i_e = B_i_e C_i_e", at.Tensor(16, 100000), at.Tensor(16, 100000), at.Tensor(16, 100000))
+    assert "64 per workgroup of 256 lanes, numbered with the entry fastest" in src and "const int b = w & 63;" in src and "const int r_ = w / 64;" in src
+    # one tensor with the entry first, or a small batch: the usual numbering
+    assert "entry fastest" not in TE.GetImplementation("A_i_e = B_e_i C_i_e", at.Tensor(16, 100000), at.Tensor(100000, 16), at.Tensor(16, 100000))
+    assert "entry fastest" not in TE.GetImplementation("A_i_e = B_i_e C_i_e", at.Tensor(16, 1000), at.Tensor(16, 1000), at.Tensor(16, 1000))
+
+
 def test_long_contraction_uses_counted_loops(TE):
     wl = workloads.config1(n=4096)
     tensors = workloads.bind_to_engine(wl, at)
@@ -373,6 +381,7 @@ def generated_sources(TE):
     for transient in (True, False):
         yield "geometric factors from the Jacobians", geometric_factor_source(TE, 7, 4, 3, transient)
     yield "geometric factors, 2 x 2", geometric_factor_source(TE, 7, 3, 2, True)
+    yield "entries fastest", TE.GetImplementation("A_i_j_e -= B_i_k_e C_k_j_e", at.Tensor(3, 3, 4099), at.Tensor(3, 3, 4099), at.Tensor(3, 3, 4099))
     yield "Gram matrix over the batch", TE.GetImplementation("A_j_i -= B_e_q_i C_e_q_j W_e_q", at.Tensor(50, 40), at.Tensor(1001, 3, 40), at.Tensor(1001, 3, 50), at.Tensor(1001, 3))
     yield "products of element matrices in 2 x 2 blocks", TE.GetImplementation("A_e_i_j += B_e_i_k C_e_j_k", at.Tensor(100, 12, 10), at.Tensor(100, 12, 9), at.Tensor(100, 10, 9))
     yield "products of tiny element matrices", TE.GetImplementation("A_e_i_j = B_e_i_k C_e_k_j", at.Tensor(1001, 3, 3), at.Tensor(1001, 3, 3), at.Tensor(1001, 3, 3))

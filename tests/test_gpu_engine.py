@@ -957,3 +957,23 @@ def test_many_outputs_summed_over_the_batch(at, engine, checker, kernel, shapes)
     assert rel_err(got, expected) <= 4 * TOL            # sums of 10^3 - 10^5 terms in another order than the oracle's
     again, _ = run_single(at, engine, checker, kernel, out0, *ins)
     assert np.array_equal(got, again)                   # reproducible
+
+
+@pytest.mark.parametrize("kernel,shapes,expect", [
+    ("A_i_e = B_i_e C_i_e", [(16, 5000), (16, 5000)], "lanes(i)=16"),
+    ("A_i_j_e -= B_i_k_e C_k_j_e", [(3, 3, 4099), (3, 3, 4099)], "lanes()=1 tile(i,j)=9"),          # ragged last workgroup
+    ("A_i_e += B_i_k C_k_e W_e", [(5, 7), (7, 6001), (6001,)], "entry fastest"),
+    ("A_e = B_e C_e", [(70001,), (70001,)], "256 per workgroup of 256 lanes, numbered with the entry fastest"),
+])
+def test_tensors_with_the_batch_index_last(at, engine, checker, kernel, shapes, expect):
+    # structure-of-arrays layouts: the work items are numbered with the entry fastest, so that the lanes of a wavefront
+    # read consecutive entries
+    rng = np.random.default_rng(len(kernel))
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    src = engine.GetLastImplementation()
+    assert "numbered with the entry fastest" in src and expect in src
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
