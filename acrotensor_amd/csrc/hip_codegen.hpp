@@ -35,6 +35,15 @@
 //    and padded with zeros to whole 16 x 4 blocks; pointwise factors per entry, output, row, vector element or
 //    column stay in the same launch; a second operator applied to a transient result runs in the same kernel, the
 //    intermediate passing from the result layout to the operand layout through a per-wavefront piece of LDS.
+//    A larger operator is applied in blocks of rows that fit LDS, one launch per block; results of operators whose
+//    rows 16 does not divide leave through LDS as one contiguous range per trip.
+//  * Products of element matrices ("A_e_i_j = B_e_i_k C_e_k_j") copy their per-entry operands to LDS tiles with the
+//    lanes along memory and compute from the tiles; output indices of even extent are split in two so that a lane owns
+//    a 2 x 2 block of outputs.
+//  * "A_i_j = B_n_i C_n_j" with more than 64 outputs runs the "Gram schedule": four rows of the range per
+//    v_mfma_f64_16x16x4, up to 16 blocks of 16 x 16 sums per wavefront, partial matrices added by a second kernel.
+//  * A kernel whose tensors all have the batch index as their fastest dimension numbers its work items with the entry
+//    fastest, so that a wavefront reads consecutive entries.
 //  * A streaming group whose workgroups would move less than 2.5 KB takes more batch entries per workgroup.
 //  * Contractions too long to unroll fall back to counted loops with the same lane mapping.
 //
