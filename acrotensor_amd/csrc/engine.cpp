@@ -488,26 +488,47 @@ TensorKernel *TensorEngine::GetAddTensorKernel(const std::string &kernel_str, co
 DimensionedKernel *TensorEngine::GetAddDimensionedKernel(TensorKernel *kernel, Tensor *output,
                                                          std::vector<Tensor *> &inputs)
 {
+    // The same ranks and extents as in the previous call with this kernel string: the same dimensioned kernel (they
+    // passed the checks below then).
+    DimsOfThisCall.clear();
+    auto note = [&](const Tensor *t) {
+        DimsOfThisCall.push_back(t->GetRank());
+        for (int d = 0; d < t->GetRank(); ++d) DimsOfThisCall.push_back(t->GetDim(d));
+    };
+    note(output);
+    for (const Tensor *t : inputs) note(t);
+    DimensionedMemo &memo = LastDimensioned[kernel];
+    if (memo.kernel != nullptr && memo.dims == DimsOfThisCall) return memo.kernel;
     // Rank and extent checks happen inside GetLoopIdxSizes, before anything is cached.
     std::string key = kernel->GetDimensionedNameString(output, inputs);
     auto it = DimensionedKernelMap.find(key);
-    if (it != DimensionedKernelMap.end()) return it->second;
-    DimensionedKernel *dk = new DimensionedKernel(kernel, output, inputs);
-    DimensionedKernelMap[key] = dk;
+    DimensionedKernel *dk = it != DimensionedKernelMap.end() ? it->second : nullptr;
+    if (dk == nullptr)
+    {
+        dk = new DimensionedKernel(kernel, output, inputs);
+        DimensionedKernelMap[key] = dk;
+    }
+    memo.dims = DimsOfThisCall;
+    memo.kernel = dk;
     return dk;
 }
 
 KernelExecutor *TensorEngine::GetAddKernelExecutor()
 {
+    if (LastCaptureExecutor != nullptr && LastCapture == MKLKernels) return LastCaptureExecutor;
     std::string key;
     for (DimensionedKernel *k : MKLKernels) key += k->GetDimensionedNameString() + ";";
     auto it = ExecutorMap.find(key);
-    if (it != ExecutorMap.end()) return it->second;
-
-    DimensionedMultiKernel *mk = new DimensionedMultiKernel(MKLKernels);
-    OwnedMultiKernels.push_back(mk);
-    KernelExecutor *executor = KernelExecutor::Create(ExecutorType, mk);
-    ExecutorMap[key] = executor;
+    KernelExecutor *executor = it != ExecutorMap.end() ? it->second : nullptr;
+    if (executor == nullptr)
+    {
+        DimensionedMultiKernel *mk = new DimensionedMultiKernel(MKLKernels);
+        OwnedMultiKernels.push_back(mk);
+        executor = KernelExecutor::Create(ExecutorType, mk);
+        ExecutorMap[key] = executor;
+    }
+    LastCapture = MKLKernels;
+    LastCaptureExecutor = executor;
     return executor;
 }
 
@@ -634,6 +655,9 @@ void TensorEngine::Clear()
     delete Ops;
     Ops = nullptr;
     LastExecutor = nullptr;
+    LastDimensioned.clear();
+    LastCapture.clear();
+    LastCaptureExecutor = nullptr;
     ResetCapture();
 }
 

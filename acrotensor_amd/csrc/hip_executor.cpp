@@ -249,22 +249,51 @@ class HipExecutor : public KernelExecutor
         for (const auto &g : gathered) g.operand->SwitchToGPU();
         for (int ki = 0; ki < K; ++ki) MoveTensorsToGPU(outputs[ki], inputs[ki]);
 
-        HipCodegenOptions options;
-        bool fallback = false;
-        Bind(outputs, inputs, gathered, options, fallback);
-        if (fallback)
+        // The same tensors in the same places as in the previous call, with the same buffers and marks: the same
+        // binding, and the variant it led to (the usual case inside a solver's loop; the analysis below costs several
+        // microseconds of host time for a group of kernels, more than a small batch takes on the device).
+        ThisCall.clear();
+        auto note = [&](const Tensor *t) {
+            Seen s;
+            s.tensor = t;
+            s.host = t->GetData();
+            s.device = t->GetDeviceData();
+            s.size = static_cast<size_t>(t->GetSize());
+            s.transient = t->IsTransient();
+            ThisCall.push_back(s);
+        };
+        for (int ki = 0; ki < K; ++ki)
         {
-            MaterialiseGathered(gathered, nullptr);
-            KernelExecutor::ExecuteMulti(outputs, inputs);
-            return;
+            note(outputs[ki]);
+            for (const Tensor *t : inputs[ki]) note(t);
         }
-        Variant &v = GetVariant(options);
+        const bool repeated = gathered.empty() && LastCallVariant != nullptr && ThisCall == LastCall;
+        HipCodegenOptions options;
+        if (!repeated)
+        {
+            LastCallVariant = nullptr;
+            bool fallback = false;
+            Bind(outputs, inputs, gathered, options, fallback);
+            if (fallback)
+            {
+                MaterialiseGathered(gathered, nullptr);
+                KernelExecutor::ExecuteMulti(outputs, inputs);
+                return;
+            }
+        }
+        Variant &v = repeated ? *LastCallVariant : GetVariant(options);
+        LastVariant = &v;
         if (!v.plan.fusable)
         {
             ACROBATIC_ASSERT(K > 1, "Internal error: a single kernel must always be executable.");
             MaterialiseGathered(gathered, nullptr);
             KernelExecutor::ExecuteMulti(outputs, inputs);
             return;
+        }
+        if (gathered.empty())
+        {
+            LastCall.swap(ThisCall);
+            LastCallVariant = &v;
         }
         MaterialiseGathered(gathered, v.plan.gathers_applied ? &options.gathered : nullptr);
         std::vector<const int *> gatherMap(gathered.size(), nullptr);
@@ -330,6 +359,20 @@ class HipExecutor : public KernelExecutor
 
     std::map<std::string, std::unique_ptr<Variant>> Variants;
     Variant *LastVariant = nullptr;
+    // one entry per tensor of a call, in call order
+    struct Seen
+    {
+        const Tensor *tensor;
+        const double *host, *device;
+        size_t size;
+        bool transient;
+        bool operator==(const Seen &o) const
+        {
+            return tensor == o.tensor && host == o.host && device == o.device && size == o.size && transient == o.transient;
+        }
+    };
+    std::vector<Seen> ThisCall, LastCall;
+    Variant *LastCallVariant = nullptr;
 };
 
 KernelExecutor *CreateHipExecutor(DimensionedMultiKernel *multi_kernel)

@@ -109,6 +109,17 @@ class TensorEngine
     std::unordered_map<std::string, DimensionedKernel *> DimensionedKernelMap;
     std::unordered_map<std::string, KernelExecutor *> ExecutorMap;
     std::vector<DimensionedMultiKernel *> OwnedMultiKernels;
+    // What the previous call with the same kernel string / the previous capture resolved to: a repeated call with the
+    // same extents (the usual case inside a solver's loop) skips building and hashing the name strings.
+    struct DimensionedMemo
+    {
+        std::vector<int> dims;  // rank and extents of the output and of every input
+        DimensionedKernel *kernel = nullptr;
+    };
+    std::unordered_map<const TensorKernel *, DimensionedMemo> LastDimensioned;
+    std::vector<int> DimsOfThisCall;
+    std::vector<DimensionedKernel *> LastCapture;
+    KernelExecutor *LastCaptureExecutor = nullptr;
     std::string ComputeLocation;
     NonContractionOps *Ops;
 

@@ -977,3 +977,46 @@ def test_tensors_with_the_batch_index_last(at, engine, checker, kernel, shapes, 
     if "-=" in kernel:
         expected = 2.0 * out0 - expected
     assert rel_err(got, expected) <= TOL
+
+
+def test_repeated_captures_follow_changes_of_tensors_and_marks(at, engine, checker):
+    # a repeated call with the same tensors reuses the previous binding; any change of a tensor, a buffer or a mark
+    # must be seen: other tensors of the same shapes, a transient mark set and cleared, a slice of another parent
+    rng = np.random.default_rng(77)
+    E = 300
+    B = rng.uniform(-1, 1, (5, 4))
+    X1, X2 = rng.uniform(-1, 1, (E, 4)), rng.uniform(-1, 1, (E, 4))
+    tB, tX1, tX2 = to_tensor(at, B), to_tensor(at, X1), to_tensor(at, X2)
+    tU, tY1, tY2 = at.Tensor(E, 5), at.Tensor(E, 4), at.Tensor(E, 4)
+
+    def run(tX, tY):
+        engine.BeginMultiKernelLaunch()
+        engine("U_e_q = B_q_i X_e_i", tU, tB, tX)
+        engine("Y_e_i = B_q_i U_e_q", tY, tB, tU)
+        engine.EndMultiKernelLaunch()
+        tY.MoveFromGPU()
+        return tY.data.copy()
+
+    ref1, ref2 = (X1 @ B.T) @ B, (X2 @ B.T) @ B
+    for _ in range(3):
+        assert rel_err(run(tX1, tY1), ref1) <= TOL
+    assert rel_err(run(tX2, tY1), ref2) <= TOL                 # another input
+    assert rel_err(run(tX2, tY2), ref2) <= TOL                 # another output
+    tU.SetTransient(True)                                      # U need not reach device memory any more
+    tU.MoveToGPU()
+    assert rel_err(run(tX1, tY1), ref1) <= TOL
+    tU.SetTransient(False)
+    assert rel_err(run(tX1, tY2), ref1) <= TOL
+    tU.MoveFromGPU()
+    assert rel_err(tU.data, X1 @ B.T) <= TOL                   # stored again
+    # slices of two parents at the same place in the call
+    P1, P2 = rng.uniform(-1, 1, (2, E, 4)), rng.uniform(-1, 1, (2, E, 4))
+    tP1, tP2 = to_tensor(at, P1), to_tensor(at, P2)
+    for parent, values in ((tP1, P1), (tP2, P2), (tP1, P1)):
+        for k in (0, 1):
+            assert rel_err(run(at.SliceTensor(parent, k), tY1), (values[k] @ B.T) @ B) <= TOL
+    # single kernels: the same string on other tensors, then with the output as "+="
+    for tX, X in ((tX1, X1), (tX2, X2), (tX1, X1)):
+        engine("U_e_q = B_q_i X_e_i", tU, tB, tX)
+        tU.MoveFromGPU()
+        assert rel_err(tU.data, X @ B.T) <= TOL
