@@ -1020,3 +1020,17 @@ def test_repeated_captures_follow_changes_of_tensors_and_marks(at, engine, check
         engine("U_e_q = B_q_i X_e_i", tU, tB, tX)
         tU.MoveFromGPU()
         assert rel_err(tU.data, X @ B.T) <= TOL
+
+
+def test_gram_matrix_of_one_tensor_and_of_slices(at, engine, checker):
+    rng = np.random.default_rng(5)
+    B = rng.uniform(-1, 1, (7001, 20))
+    tB, tA = to_tensor(at, B), at.Tensor(20, 20)
+    engine("A_i_j = B_e_i B_e_j", tA, tB, tB)                  # the same tensor on both sides
+    tA.MoveFromGPU()
+    assert "Gram schedule" in engine.GetLastImplementation() and rel_err(tA.data, B.T @ B) <= 4 * TOL
+    big = rng.uniform(-1, 1, (2, 7001, 20))
+    tbig = to_tensor(at, big)
+    engine("A_i_j += B_e_i C_e_j", tA, at.SliceTensor(tbig, 1), at.SliceTensor(tbig, 0))   # views at an offset
+    tA.MoveFromGPU()
+    assert "Gram schedule" in engine.GetLastImplementation() and rel_err(tA.data, B.T @ B + big[1].T @ big[0]) <= 4 * TOL
