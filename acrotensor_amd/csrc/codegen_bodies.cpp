@@ -635,8 +635,11 @@ auto Generator::EmitMatrixBody(int k, Body &body, ForwardMap &forwarded) -> void
 auto Generator::SplitLanesTakePairs(int k) const -> bool
 {
     const Sub &s = subs[k];
-    if (s.splitLanes <= 0 || envInt("ACRO_HIP_SPLIT_PAIRS") < 0 || s.contr.size() != 1) return false;
-    if (s.contrCount % 2 != 0 || s.contrCount < 2L * s.splitLanes) return false;
+    if (s.splitLanes <= 0 || envInt("ACRO_HIP_SPLIT_PAIRS") < 0 || s.contr.empty()) return false;
+    // (several contraction indices: the pairs run along the last one, which the flattened range walks fastest; its
+    // extent is even, so the two terms of a pair share all the other indices.  "A_e = B_e_i_j C_i D_j": 56 -> 66 %.)
+    const int fastest = s.contr.back();
+    if (extent[fastest] % 2 != 0 || s.contrCount < 2L * s.splitLanes) return false;
     // Long rows stream better term by term, eight 8-byte loads in flight per lane (rows of 1 024: 75.3 against 73.5 % of
     // the HBM peak, four rows of 256: 76.6 against 74.7 %); the pairs pay where a lane has few terms (16 x 16 element
     // matrix times vector 69.3 -> 76.4 %, 64 x 64 71.0 -> 72.0 %).
@@ -645,10 +648,10 @@ auto Generator::SplitLanesTakePairs(int k) const -> bool
     for (size_t v = 0; v < s.in.size(); ++v)
     {
         const VarRef &r = s.in[v];
-        if (!has(r.idx, s.contr[0])) continue;
+        if (!has(r.idx, fastest)) continue;
         const Source src = SourceOf(k, static_cast<int>(v));
         if ((src != kFromGlobal && src != kFromConstant) || GatherSlot(r.uvar) >= 0 || r.repeated) return false;
-        if (r.idx.back() != s.contr[0] || r.stride.back() != 1) return false;
+        if (r.idx.back() != fastest || r.stride.back() != 1) return false;
         any = true;
     }
     return any;
@@ -701,7 +704,7 @@ auto Generator::EmitSplitLanesBody(int k, std::vector<std::string> &lines) -> vo
         }
         if (off.empty()) off = "0";
         std::string opnd;
-        if (pairs && has(r.idx, s.contr[0]))
+        if (pairs && has(r.idx, s.contr.back()))
         {
             // both terms of the pair in one load (through the ordinary pointer also for operands that scalar loads
             // would serve: the index differs from lane to lane here)
