@@ -192,6 +192,14 @@ KERNEL_SHAPES = [
     ("S_i = A_n_i", [(1 << 20, 64)], (64,)),
     ("S_i = A_i_n", [(64, 1 << 20)], (64,)),
     ("A_i_j = B_j_i", [(8192, 8192)], (8192, 8192)),
+    ("A_i_j = B_e_i C_e_j", [(1 << 21, 32), (1 << 21, 32)], (32, 32)),
+    ("A_i_j = B_e_i C_e_j", [(1 << 20, 64), (1 << 20, 64)], (64, 64)),
+    ("A_e = B_e_i_j C_i D_j", [(1 << 20, 8, 8), (8,), (8,)], (1 << 20,)),
+    ("A_i_e = B_i_e C_i_e", [(16, 1 << 22), (16, 1 << 22)], (16, 1 << 22)),
+    ("G_e_d_q = D_d_q_i X_e_i", [(3, 64, 64), (1 << 18, 64)], (1 << 18, 3, 64)),
+    ("A_e_i = B_i_j X_e_j", [(81, 8), (1 << 20, 8)], (1 << 20, 81)),
+    ("Y_e_i_j = B_q_i B_r_j D_e_q_r U_e_q_r", [(5, 4), (5, 4), (1 << 20, 5, 5), (1 << 20, 5, 5)], (1 << 20, 4, 4)),
+    ("U_e_q_r_s = B_q_i B_r_j B_s_k X_e_i_j_k", [(5, 4), (5, 4), (5, 4), (1 << 18, 4, 4, 4)], (1 << 18, 5, 5, 5)),
 ]
 
 
