@@ -148,9 +148,16 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
         // operator read from device memory by every workgroup: 2.4 % of the HBM peak).
         const long paddedCols = (o.cols + 7) / 8 * 8;
         o.blockRows = 8192 / paddedCols / 16 * 16;
-        if (!alone || o.cols > 256 || o.rows > 8192 || o.blockRows < 16 || o.trailing || o.comp > 1 || envInt("ACRO_HIP_OPERATOR_BLOCKS") < 0 ||
+        if (!alone || o.cols > 256 || o.rows > 8192 || o.blockRows < 16 || o.trailing || envInt("ACRO_HIP_OPERATOR_BLOCKS") < 0 ||
             envInt("ACRO_HIP_OPERATOR_MFMA") < 0)
             return false;
+    }
+    // With components a lane holds rows / 4 results for each of them: at most 16 blocks of 16 rows in all, more rows
+    // in blocks of rows as above.
+    if (o.comp > 1 && !o.trailing && alone && envInt("ACRO_HIP_OPERATOR_BLOCKS") >= 0 && envInt("ACRO_HIP_OPERATOR_MFMA") >= 0 && o.comp <= 16)
+    {
+        const long most = 16 * (16 / o.comp);
+        if (ComponentsTogether(o) && (o.blockRows > most || (o.blockRows == 0 && o.rows > most))) o.blockRows = most;
     }
     // With components: vectors in 8-byte loads, no pointwise factors, and only where the generic schedule (an
     // entry and a row per lane) runs out of scalar registers for the operator or of coalescing for its stores
@@ -302,7 +309,10 @@ auto Generator::EmitOperator(HipKernelPlan &plan) -> void
             block.allRows = shape.rows;
             block.rowOffset = r0;
             block.rows = std::min(shape.blockRows, shape.rows - r0);
-            EmitOperatorMatrixCores(plan, block);
+            if (shape.comp > 1 && ComponentsTogether(shape))
+                EmitOperatorComponents(plan, block);
+            else
+                EmitOperatorMatrixCores(plan, block);
             schedule += plan.schedule;
             lds = std::max(lds, plan.lds_bytes);
         }
@@ -319,6 +329,8 @@ auto Generator::EmitOperator(HipKernelPlan &plan) -> void
     {
         if (shape.trailing)
             EmitOperatorEntriesFastest(plan, shape);
+        else if (shape.comp > 1 && ComponentsTogether(shape))
+            EmitOperatorComponents(plan, shape);
         else
             EmitOperatorMatrixCores(plan, shape);
         return;
@@ -665,7 +677,7 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
             // entry (e, k): its outputs lie C doubles apart
             out << "            const long en_ = tile * 16 + g + 4 * r;\n";
             out << "            double *a = " << PtrName(ks.out.uvar) << " + " << Lit(uvars[ks.out.uvar].viewOffset) << " + (en_ / " << C << ") * "
-                << rows * C << " + en_ % " << C << " + c * " << C << ";\n";
+                << stride * C << (off ? " + " + str(off * C) : std::string()) << " + en_ % " << C << " + c * " << C << ";\n";
         }
         // the result's pointwise factors
         std::string value = accName + "[t][r]";
@@ -745,6 +757,165 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     plan.source = out.str();
     plan.nb = 64;
     plan.lds_bytes = static_cast<int>((nIp * nJp + (next ? (next->rows + 15) / 16 * 16 * steps2 * 4 + 64 * midStride : 0) + (viaStage ? 64 / stageRounds * nI : 0)) * 8);
+    FillParams(plan, false);
+    HipLaunch launch;
+    launch.function_name = plan.module_name;
+    launch.grid = static_cast<unsigned>(blocks);
+    launch.block = 256;
+    for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
+    plan.launches.push_back(launch);
+}
+
+// Vectors and results with component indices behind the operator's ("V_e_q_c = B_q_i X_e_i_c", a vector field
+// interpolated component by component).  A wavefront takes 16 entries (all their components) per trip: a lane loads the
+// C components of its vector elements, which lie next to each other, every block of the operator read from LDS serves C
+// instructions, and the results of a trip, 16 entries x rows x C doubles that lie next to each other in memory, are
+// collected in LDS in memory order and written out as one range (all 16 entries at once where LDS allows, else 8 or 4
+// at a time, else by the lanes that hold them).  Treating (entry, component) pairs as the entries instead, as this
+// schedule first did, reads and writes single doubles C apart: 27 x 27 x 3 62 %, 64 x 27 x 3 55 % of the HBM peak.
+// Measured against the entries (entry, component): 16 x 16 x 3 68 -> 72 %, 27 x 27 x 3 62 -> 68 %, 125 x 64 x 3 (two blocks
+// of rows) 23 -> 34 %; 64 x 64 x 3 61 -> 59 % and 216 x 125 x 3 21 -> 15 %, which keep the entries (entry, component).
+auto Generator::ComponentsTogether(const OperatorShape &o) const -> bool
+{
+    if (o.comp <= 1 || o.comp > 16 || o.trailing || envInt("ACRO_HIP_OPERATOR_COMPONENTS") >= 2) return false;
+    const long padded = ((o.rows + 15) / 16 * 16) * ((o.cols + 3) / 4 * 4);
+    return padded <= 1024 || (o.rows * o.cols > 4096 && o.cols <= 64);
+}
+
+auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape &shape) -> void
+{
+    const Sub &s = OpKernel(opSub);
+    const VarRef &opr = *shape.op, &x = *shape.x;
+    const long nI = shape.rows, nJ = shape.cols, C = shape.comp, NE = shape.entries / shape.comp;
+    const long nAll = shape.allRows > 0 ? shape.allRows : nI, row0 = shape.rowOffset;
+    const bool first = opSub == 0 && opBlock == 0;
+    const long nIp = (nI + 15) / 16 * 16, nJp = (nJ + 3) / 4 * 4;
+    const long tilesN = nIp / 16, steps = nJp / 4;
+    const long tiles = (NE + 15) / 16;
+    const bool ragged = NE % 16 != 0;
+    int stageRounds = 0;
+    if (shape.allRows == 0 && envInt("ACRO_HIP_OPERATOR_STAGE_OUT") >= 0)
+    {
+        for (int rounds : {1, 2, 4})
+        {
+            if (stageRounds == 0 && (nIp * nJp + 64 / rounds * nI * C) * 8 <= 64 * 1024) stageRounds = rounds;
+        }
+    }
+    const long most = nIp * nJp > 4096 ? 256 : 512;
+    const long blocks = std::max<long>(1, std::min<long>(most, (tiles + 3) / 4));
+    for (const auto &st : stores)
+    {
+        long entries = 1;
+        for (int d : st.dims) entries *= d;
+        if (entries >= (1L << 31) - 1) wide = true;
+    }
+    const std::string dimName = mk.GetDimensionedNameString();
+    char hex[32];
+    std::snprintf(hex, sizeof(hex), "%016llx",
+                  static_cast<unsigned long long>(hashString(dimName + "/operator-mfma-components/" + str(opSub) + (shape.allRows > 0 ? "@" + str(row0) : std::string()) + "/" +
+                                                             (Positional() ? "p" : "u") + "c" + str(C))));
+    plan.module_name = std::string("acro_op_") + hex;
+    std::ostringstream sched;
+    sched << "operator schedule on the FP64 matrix cores: ";
+    if (shape.allRows > 0) sched << "rows " << row0 << " - " << row0 + nI - 1 << " of the " << nAll << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator");
+    else sched << nI << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator");
+    sched << " in LDS in operand order";
+    if (nIp != nI || nJp != nJ) sched << " (padded to " << nIp << " x " << nJp << ")";
+    sched << ", " << C << " components per vector element";
+    if (stageRounds > 0) sched << ", results written out through LDS";
+    sched << ", " << NE << " entries, 16 per wavefront and trip, " << tilesN * steps * C << " v_mfma_f64_16x16x4 per trip, " << blocks
+          << " workgroups of 256 lanes\n  [" << opSub << "] " << s.text << "\n";
+    plan.schedule = sched.str();
+    if (first) out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
+    {
+        std::istringstream lines(plan.schedule);
+        std::string l;
+        while (std::getline(lines, l)) out << "// " << l << "\n";
+    }
+    const std::string B = PtrName(opr.uvar), X = PtrName(x.uvar), A = PtrName(s.out.uvar);
+    const bool streams = s.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0;
+    out << (first ? "" : "\n") << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
+    out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << plan.module_name << "(" << ParamList() << ")\n{\n";
+    out << "    __shared__ double frag[" << nIp * nJp << "];\n";
+    out << "    for (int f = threadIdx.x; f < " << nIp * nJp << "; f += 256)\n    {\n";
+    out << "        const int l = f & 63, step = (f >> 6) % " << steps << ", t = (f >> 6) / " << steps << ";\n";
+    out << "        const int row = 16 * t + (l & 15), j = 4 * step + (l >> 4);\n";
+    const std::string rowHere = row0 > 0 ? "(row + " + str(row0) + ")" : std::string("row");
+    const std::string element = B + "[" + Lit(uvars[opr.uvar].viewOffset) + (shape.transposed ? " + j * " + str(nAll) + " + " + rowHere + "]" : " + " + rowHere + " * " + str(nJ) + " + j]");
+    if (nIp != nI || nJp != nJ)
+        out << "        frag[f] = row < " << nI << " && j < " << nJ << " ? " << element << " : 0.0;\n    }\n";
+    else
+        out << "        frag[f] = " << element << ";\n    }\n";
+    const int perRound = stageRounds > 0 ? 4 / stageRounds : 0;   // result registers (entries g + 4 r) per round
+    if (stageRounds > 0) out << "    __shared__ double stage[" << 4 * 4 * perRound * nI * C << "];\n";
+    out << "    __syncthreads();\n";
+    out << "    const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;\n";
+    out << "    const long waves = (long)gridDim.x * 4;\n";
+    out << "    for (long tile = (long)blockIdx.x * 4 + (threadIdx.x >> 6); tile < " << tiles << "; tile += waves)\n    {\n";
+    if (ragged)
+        out << "        const long ex = tile * 16 + c < " << NE << " ? tile * 16 + c : " << NE - 1 << ";  // past the end: any valid entry, never stored\n";
+    else
+        out << "        const long ex = tile * 16 + c;\n";
+    out << "        const double *x = " << X << " + " << Lit(uvars[x.uvar].viewOffset) << " + ex * " << nJ * C << " + g * " << C << ";\n";
+    out << "        double xv[" << C << "][" << steps << "];\n";
+    out << "#pragma unroll\n        for (int q = 0; q < " << steps << "; ++q)\n";
+    out << "#pragma unroll\n            for (int k = 0; k < " << C << "; ++k) xv[k][q] = ";
+    if (nJp != nJ) out << "4 * q + g >= " << nJ << " ? 0.0 : ";
+    out << "x[" << 4 * C << " * q + k];\n";
+    out << "        acro_double4 acc[" << C << "][" << tilesN << "];\n";
+    out << "#pragma unroll\n        for (int k = 0; k < " << C << "; ++k)\n";
+    out << "#pragma unroll\n            for (int t = 0; t < " << tilesN << "; ++t) acc[k][t] = acro_double4{0.0, 0.0, 0.0, 0.0};\n";
+    out << "#pragma unroll\n        for (int step = 0; step < " << steps << "; ++step)\n";
+    out << "#pragma unroll\n            for (int t = 0; t < " << tilesN << "; ++t)\n            {\n";
+    out << "                const double b = frag[(t * " << steps << " + step) * 64 + lane];\n";
+    out << "#pragma unroll\n                for (int k = 0; k < " << C << "; ++k) acc[k][t] = __builtin_amdgcn_mfma_f64_16x16x4f64(xv[k][step], b, acc[k][t], 0, 0, 0);\n";
+    out << "            }\n";
+    // register r of a lane holds entry 4 r + g of the trip and row 16 t + c
+    const long rowsC = nI * C, strideC = nAll * C;
+    const std::string rowGuard = nIp != nI ? "if (16 * t + c < " + str(nI) + ") " : std::string();
+    if (stageRounds > 0)
+    {
+        out << "        double *mid = stage + (threadIdx.x >> 6) * " << 4 * perRound * rowsC << ";\n";
+        for (int h = 0; h < stageRounds; ++h)
+        {
+            out << "#pragma unroll\n        for (int r = " << h * perRound << "; r < " << (h + 1) * perRound << "; ++r)\n";
+            out << "#pragma unroll\n            for (int t = 0; t < " << tilesN << "; ++t)\n";
+            out << "#pragma unroll\n                for (int k = 0; k < " << C << "; ++k)\n";
+            out << "                    " << rowGuard << "mid[(4 * " << (h ? "(r - " + str(static_cast<long>(h * perRound)) + ")" : std::string("r")) << " + g) * " << rowsC
+                << " + (16 * t + c) * " << C << " + k] = acc[k][t][r];\n";
+            out << "        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");\n        __builtin_amdgcn_wave_barrier();\n";
+            out << "        {\n";
+            const long firstEntry = 4L * h * perRound, entries = 4L * perRound;
+            out << "            double *a = " << A << " + " << Lit(uvars[s.out.uvar].viewOffset) << " + (tile * 16 + " << firstEntry << ") * " << rowsC << ";\n";
+            if (ragged)
+                out << "            const long left = " << NE << " - tile * 16 - " << firstEntry << ";\n"
+                    << "            const int count = (int)(left < 0 ? 0 : (left < " << entries << " ? left : " << entries << ")) * " << rowsC << ";\n";
+            else
+                out << "            const int count = " << entries * rowsC << ";\n";
+            out << "            for (int i = lane; i < count; i += 64)\n";
+            if (streams)
+                out << "                __builtin_nontemporal_store(mid[i], a + i);\n";
+            else
+                out << "                a[i]" << (s.op == '=' ? " = " : (s.op == '+' ? " += " : " -= ")) << "mid[i];\n";
+            out << "        }\n";
+            out << "        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");\n        __builtin_amdgcn_wave_barrier();\n";
+        }
+    }
+    else
+    {
+        out << "#pragma unroll\n        for (int r = 0; r < 4; ++r)\n        {\n";
+        if (ragged) out << "            if (tile * 16 + g + 4 * r >= " << NE << ") continue;\n";
+        out << "            double *a = " << A << " + " << Lit(uvars[s.out.uvar].viewOffset) << " + (tile * 16 + g + 4 * r) * " << strideC << " + " << row0 * C << " + c * " << C << ";\n";
+        out << "#pragma unroll\n            for (int t = 0; t < " << tilesN << "; ++t)\n";
+        out << "#pragma unroll\n                for (int k = 0; k < " << C << "; ++k)\n";
+        out << "                    " << rowGuard << "a[" << 16 * C << " * t + k]" << (s.op == '=' ? " = " : (s.op == '+' ? " += " : " -= ")) << "acc[k][t][r];\n";
+        out << "        }\n";
+    }
+    out << "    }\n}\n";
+
+    plan.source = out.str();
+    plan.nb = 64;
+    plan.lds_bytes = static_cast<int>((nIp * nJp + (stageRounds > 0 ? 4 * 4 * perRound * rowsC : 0)) * 8);
     FillParams(plan, false);
     HipLaunch launch;
     launch.function_name = plan.module_name;

@@ -438,6 +438,8 @@ class Generator
     void EmitOperator(HipKernelPlan &plan);
     void EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape &shape, const OperatorShape *next = nullptr, int nextSub = -1);
     void EmitOperatorEntriesFastest(HipKernelPlan &plan, const OperatorShape &shape);
+    void EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape &shape);
+    bool ComponentsTogether(const OperatorShape &o) const;
     void Emit(HipKernelPlan &plan);
 };
 

@@ -867,6 +867,10 @@ def test_operator_kernels_on_buffers_that_are_only_8_byte_aligned(at, engine, ch
     ("A_e_i_k -= B_j_i X_e_j_k", [(33, 20), (77, 33, 2)], True),            # operator stored transposed, padded to 32 x 36
     ("A_e_q_i_k = B_i_j X_e_q_j_k", [(30, 17), (50, 4, 17, 5)], True),      # two leading indices, five components
     ("A_e_i_k_l = B_i_j X_e_j_k_l", [(24, 24), (101, 24, 2, 3)], True),     # two component indices
+    ("V_e_q_c = B_q_i X_e_i_c", [(27, 27), (1001, 27, 3)], True),           # the components of an entry together, results through LDS
+    ("V_e_q_c -= B_i_q X_e_i_c", [(16, 20), (517, 16, 2)], True),           # operator stored transposed, two components
+    ("V_e_q_c = B_q_i X_e_i_c", [(125, 64), (203, 64, 3)], True),           # too large for LDS: two blocks of rows, components together
+    ("V_e_q_c += B_q_i X_e_i_c", [(216, 125), (301, 125, 2)], True),        # blocks of rows, entries (entry, component)
     ("A_e_i_k = B_i_j X_e_j_k", [(8, 8), (1000, 8, 3)], False),             # small operator: the generic schedule
     ("A_e_i_k = B_i_j X_e_j_k W_e", [(32, 32), (100, 32, 3), (100,)], False),  # with a factor: the generic schedule
 ])
