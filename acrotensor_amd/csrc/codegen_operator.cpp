@@ -130,8 +130,35 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
     std::vector<int> plain = rows, swapped = cols;
     plain.insert(plain.end(), cols.begin(), cols.end());
     swapped.insert(swapped.end(), rows.begin(), rows.end());
-    if (o.op->idx != plain && o.op->idx != swapped) return false;
-    o.transposed = o.op->idx != plain;
+    if (o.op->idx != plain && o.op->idx != swapped)
+    {
+        // Any other order of the same indices ("J_e_q_n_m = G_q_i_n X_e_i_m": row indices q, n around the column
+        // index i): the operator's copy in LDS is filled through the strides of its dimensions.  Matrix cores only.
+        std::vector<int> sorted = o.op->idx, all = plain;
+        std::sort(sorted.begin(), sorted.end());
+        std::sort(all.begin(), all.end());
+        if (sorted != all || o.op->repeated || envInt("ACRO_HIP_OPERATOR_ANY_ORDER") < 0) return false;
+        o.mixed = true;
+        long rowDiv = 1;
+        for (size_t d = rows.size(); d-- > 0;)
+        {
+            for (size_t q = 0; q < o.op->idx.size(); ++q)
+            {
+                if (o.op->idx[q] == rows[d]) o.rowTerms.push_back({rowDiv, static_cast<long>(extent[rows[d]]), o.op->stride[q]});
+            }
+            rowDiv *= extent[rows[d]];
+        }
+        long colDiv = 1;
+        for (size_t d = cols.size(); d-- > 0;)
+        {
+            for (size_t q = 0; q < o.op->idx.size(); ++q)
+            {
+                if (o.op->idx[q] == cols[d]) o.colTerms.push_back({colDiv, static_cast<long>(extent[cols[d]]), o.op->stride[q]});
+            }
+            colDiv *= extent[cols[d]];
+        }
+    }
+    o.transposed = !o.mixed && o.op->idx != plain;
     for (int id : cols)
     {
         if (!has(s.contr, id)) return false;
@@ -190,7 +217,7 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
         }
         else return false;
     }
-    if (!o.cores) return o.rows >= 16 && o.cols >= 16 && !o.transposed && !o.trailing && s.in.size() == 2 && o.comp == 1;  // (its lanes walk the operator's rows)
+    if (!o.cores) return o.rows >= 16 && o.cols >= 16 && !o.transposed && !o.mixed && !o.trailing && s.in.size() == 2 && o.comp == 1;  // (its lanes walk the operator's rows)
     // A lane holds cols / 4 vector elements and rows / 4 results; the padded operator must fit the 64 KB of LDS
     // that a workgroup may declare.
     if (o.blockRows > 0) return true;
@@ -255,6 +282,24 @@ auto Generator::OperatorPair(OperatorShape &first, OperatorShape &second) const 
     const long n1 = ((first.rows + 15) / 16 * 16) * (first.pairs ? (first.cols + 7) / 8 * 8 : (first.cols + 3) / 4 * 4);
     const long n2 = ((second.rows + 15) / 16 * 16) * ((second.cols + 3) / 4 * 4);
     return (n1 + n2 + 64 * (first.rows + 1)) * 8 <= 64 * 1024;
+}
+
+// Index of the operator's entry (row, j) in its own memory: rows by columns, columns by rows, or any order of its
+// dimensions (then `row` and `j` are taken apart into the indices they number).
+auto Generator::OperatorEntry(const OperatorShape &shape, const std::string &row, const std::string &j, long allRows) const -> std::string
+{
+    if (!shape.mixed) return shape.transposed ? j + " * " + str(allRows) + " + " + row : row + " * " + str(shape.cols) + " + " + j;
+    std::string expr;
+    auto add = [&](const std::string &flat, const std::vector<OperatorShape::Term> &terms) {
+        for (const auto &t : terms)
+        {
+            std::string v = t.div == 1 ? flat : "(" + flat + " / " + str(t.div) + ")";
+            expr += (expr.empty() ? "" : " + ") + ("(" + v + " % " + str(t.ext) + ")") + " * " + str(t.stride);
+        }
+    };
+    add(row, shape.rowTerms);
+    add(j, shape.colTerms);
+    return expr;
 }
 
 auto Generator::UseOperatorSchedule() const -> bool
@@ -486,8 +531,8 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     plan.module_name = std::string("acro_op_") + hex;
     std::ostringstream sched;
     sched << "operator schedule on the FP64 matrix cores: ";
-    if (shape.allRows > 0) sched << "rows " << row0 << " - " << row0 + nI - 1 << " of the " << nAll << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator");
-    else sched << nI << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator");
+    if (shape.allRows > 0) sched << "rows " << row0 << " - " << row0 + nI - 1 << " of the " << nAll << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : (shape.mixed ? " operator (dimensions in another order)" : " operator"));
+    else sched << nI << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : (shape.mixed ? " operator (dimensions in another order)" : " operator"));
     sched << " in LDS in operand order";
     if (nIp != nI || nJp != nJ) sched << " (padded to " << nIp << " x " << nJp << ")";
     if (shape.comp > 1) sched << ", " << shape.comp << " components per vector element";
@@ -520,7 +565,7 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     out << "        const int l = f & 63, step = (f >> 6) % " << steps << ", t = (f >> 6) / " << steps << ";\n";
     out << "        const int row = 16 * t + (l & 15), j = " << termOf << ";\n";
     const std::string rowHere = row0 > 0 ? "(row + " + str(row0) + ")" : std::string("row");
-    const std::string element = B + "[" + Lit(uvars[opr.uvar].viewOffset) + (shape.transposed ? " + j * " + str(nAll) + " + " + rowHere + "]" : " + " + rowHere + " * " + str(nJ) + " + j]");
+    const std::string element = B + "[" + Lit(uvars[opr.uvar].viewOffset) + " + " + OperatorEntry(shape, rowHere, "j", nAll) + "]";
     if (nIp != nI || nJp != nJ)
         out << "        frag[f] = row < " << nI << " && j < " << nJ << " ? " << element << " : 0.0;\n    }\n";
     else
@@ -817,8 +862,8 @@ auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape 
     plan.module_name = std::string("acro_op_") + hex;
     std::ostringstream sched;
     sched << "operator schedule on the FP64 matrix cores: ";
-    if (shape.allRows > 0) sched << "rows " << row0 << " - " << row0 + nI - 1 << " of the " << nAll << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator");
-    else sched << nI << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : " operator");
+    if (shape.allRows > 0) sched << "rows " << row0 << " - " << row0 + nI - 1 << " of the " << nAll << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : (shape.mixed ? " operator (dimensions in another order)" : " operator"));
+    else sched << nI << " x " << nJ << (shape.transposed ? " operator (stored transposed)" : (shape.mixed ? " operator (dimensions in another order)" : " operator"));
     sched << " in LDS in operand order";
     if (nIp != nI || nJp != nJ) sched << " (padded to " << nIp << " x " << nJp << ")";
     sched << ", " << C << " components per vector element";
@@ -841,7 +886,7 @@ auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape 
     out << "        const int l = f & 63, step = (f >> 6) % " << steps << ", t = (f >> 6) / " << steps << ";\n";
     out << "        const int row = 16 * t + (l & 15), j = 4 * step + (l >> 4);\n";
     const std::string rowHere = row0 > 0 ? "(row + " + str(row0) + ")" : std::string("row");
-    const std::string element = B + "[" + Lit(uvars[opr.uvar].viewOffset) + (shape.transposed ? " + j * " + str(nAll) + " + " + rowHere + "]" : " + " + rowHere + " * " + str(nJ) + " + j]");
+    const std::string element = B + "[" + Lit(uvars[opr.uvar].viewOffset) + " + " + OperatorEntry(shape, rowHere, "j", nAll) + "]";
     if (nIp != nI || nJp != nJ)
         out << "        frag[f] = row < " << nI << " && j < " << nJ << " ? " << element << " : 0.0;\n    }\n";
     else
@@ -956,7 +1001,7 @@ auto Generator::EmitOperatorEntriesFastest(HipKernelPlan &plan, const OperatorSh
     plan.module_name = std::string("acro_op_") + hex;
     std::ostringstream sched;
     sched << "operator schedule on the FP64 matrix cores, entries fastest: " << nI << " x " << nJ
-          << (shape.transposed ? " operator (stored transposed)" : " operator") << " in LDS in operand order";
+          << (shape.transposed ? " operator (stored transposed)" : (shape.mixed ? " operator (dimensions in another order)" : " operator")) << " in LDS in operand order";
     if (nIp != nI || nJp != nJ) sched << " (padded to " << nIp << " x " << nJp << ")";
     sched << ", " << E << " entries, " << per << " per wavefront and trip, " << tilesM * steps * (pairs ? 2 : 1)
           << " v_mfma_f64_16x16x4 per trip, " << blocks << " workgroups of 256 lanes\n  [" << opSub << "] " << s.text << "\n";
@@ -980,7 +1025,7 @@ auto Generator::EmitOperatorEntriesFastest(HipKernelPlan &plan, const OperatorSh
     out << "    for (int f = threadIdx.x; f < " << nIp * nJp << "; f += 256)\n    {\n";
     out << "        const int l = f & 63, step = (f >> 6) % " << steps << ", t = (f >> 6) / " << steps << ";\n";
     out << "        const int row = 16 * t + (l & 15), j = 4 * step + (l >> 4);\n";
-    const std::string element = B + "[" + offsetOf(opr) + (shape.transposed ? " + j * " + str(nI) + " + row]" : " + row * " + str(nJ) + " + j]");
+    const std::string element = B + "[" + offsetOf(opr) + " + " + OperatorEntry(shape, "row", "j", nI) + "]";
     if (nIp != nI || nJp != nJ)
         out << "        frag[f] = row < " << nI << " && j < " << nJ << " ? " << element << " : 0.0;\n    }\n";
     else

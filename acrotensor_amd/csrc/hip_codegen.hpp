@@ -100,6 +100,8 @@
 //                               passes to bring a workgroup to 8 KB)
 //   ACRO_HIP_ENTRIES_FASTEST=-1 tensors with the batch index last: work items numbered entry by entry all the same
 //   ACRO_HIP_GRAM=-1            "A_i_j = B_n_i C_n_j" with more than 64 outputs does not take the Gram schedule (matrix cores, two launches)
+//   ACRO_HIP_OPERATOR_ANY_ORDER=-1  operators whose dimensions are neither rows by columns nor columns by rows: generic schedule
+//   ACRO_HIP_OPERATOR_COMPONENTS=2  vectors with components: always entries (entry, component), never the components of an entry together
 //   ACRO_HIP_OPERATOR_BLOCKS=-1 operators of more than 4 096 entries are not applied in blocks of rows (generic schedule instead)
 //   ACRO_HIP_OPERATOR_STAGE_OUT=-1  results of operators whose rows 16 does not divide are stored by the lanes that hold them
 //   ACRO_HIP_OPERATOR_FOLD=-1   a pointwise kernel that rescales an operator kernel's transient result is not folded into it

@@ -415,6 +415,14 @@ class Generator
         // time (0: whole).  The emitter then sees `rows` rows starting at `rowOffset` of `allRows`.
         long blockRows = 0, rowOffset = 0, allRows = 0;
         bool transposed = false;   // the operator is stored with the contracted indices first: "B_j_i"
+        // the operator's dimensions in any other order: per row index and per column index (fastest first) what to
+        // divide the row / column number by, its extent and its stride in the operator
+        bool mixed = false;
+        struct Term
+        {
+            long div, ext, stride;
+        };
+        std::vector<Term> rowTerms, colTerms;
         bool cores = false;        // sizes and alignment suit the FP64 matrix cores
         bool pairs = false;        // the entries' vectors (and weights of their shape) come in 16-byte loads
         bool trailing = false;     // the entries are the fastest dimension: "A_i_e = B_i_j X_j_e"
@@ -440,6 +448,7 @@ class Generator
     void EmitOperatorEntriesFastest(HipKernelPlan &plan, const OperatorShape &shape);
     void EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape &shape);
     bool ComponentsTogether(const OperatorShape &o) const;
+    std::string OperatorEntry(const OperatorShape &shape, const std::string &row, const std::string &j, long allRows) const;
     void Emit(HipKernelPlan &plan);
 };
 

@@ -244,6 +244,10 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     src = TE.GetImplementation("G_e_d_q = D_d_q_i X_e_i", at.Tensor(1000, 3, 64), at.Tensor(3, 64, 64), at.Tensor(1000, 64))
     assert "rows 0 - 127 of the 192 x 64 operator" in src and "rows 128 - 191 of the 192 x 64 operator" in src and src.count("__global__") == 2
     assert "frag[f] = T1[0 + (row + 128) * 64 + j];" in src and "double *a = T0 + 0 + (tile * 16 + g) * 192 + 128 + c;" in src
+    # the operator's dimensions in any order: its copy in LDS is filled through their strides
+    src = TE.GetImplementation("J_e_q_n_m = G_q_i_n X_e_i_m", at.Tensor(501, 27, 3, 3), at.Tensor(27, 27, 3), at.Tensor(501, 27, 3))
+    assert "81 x 27 operator (dimensions in another order)" in src and "3 components per vector element" in src
+    assert "T1[0 + (row % 3) * 1 + ((row / 3) % 27) * 81 + (j % 27) * 3]" in src
     # very long vectors or very many rows would not fit a lane's registers: not this schedule
     assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 5), at.Tensor(5, 818), at.Tensor(900, 818))
     assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 300), at.Tensor(300, 12), at.Tensor(900, 12))

@@ -1041,3 +1041,21 @@ def test_gram_matrix_of_one_tensor_and_of_slices(at, engine, checker):
     engine("A_i_j += B_e_i C_e_j", tA, at.SliceTensor(tbig, 1), at.SliceTensor(tbig, 0))   # views at an offset
     tA.MoveFromGPU()
     assert "Gram schedule" in engine.GetLastImplementation() and rel_err(tA.data, B.T @ B + big[1].T @ big[0]) <= 4 * TOL
+
+
+@pytest.mark.parametrize("kernel,shapes", [
+    ("J_e_q_n_m = G_q_i_n X_e_i_m", [(27, 27, 3), (501, 27, 3)]),                  # Jacobians: row indices q, n around the column index
+    ("A_e_i1_i2 += B_i1_j1_i2_j2 X_e_j1_j2", [(6, 4, 5, 7), (1003, 4, 7)]),       # rows and columns interleaved
+    ("A_e_i1_i2 -= B_j2_i2_j1_i1 X_e_j1_j2 W_e", [(7, 5, 4, 6), (777, 4, 7), (777,)]),   # every dimension the other way round
+    ("G_e_d_q = D_q_i_d X_e_i", [(70, 64, 3), (1001, 64)]),                        # too large for LDS as well: blocks of rows
+])
+def test_dense_operator_with_dimensions_in_any_order(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(len(kernel))
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    src = engine.GetLastImplementation()
+    assert "operator schedule on the FP64 matrix cores" in src and "dimensions in another order" in src
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
