@@ -111,6 +111,52 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
             rows.pop_back();
             cols.pop_back();
         }
+        // Component indices between the result's row indices ("J_e_q_m_n = X_e_i_m G_q_i_n": Jacobians with the
+        // component m in front of the derivative index n): the vectors carry them last as before, and the results of
+        // a trip are put into memory order as they are collected in LDS.
+        std::vector<int> between;
+        for (int id : rows)
+        {
+            if (!has(o.op->idx, id)) between.push_back(id);
+        }
+        if (!between.empty())
+        {
+            if (o.comp > 1 || !alone || between.size() >= cols.size() || envInt("ACRO_HIP_OPERATOR_ANY_ORDER") < 0) return false;
+            if (!std::equal(between.begin(), between.end(), cols.end() - between.size())) return false;
+            for (int id : between)
+            {
+                if (has(s.contr, id) || std::count(rows.begin(), rows.end(), id) != 1) return false;
+            }
+            // per output dimension behind the entries' (fastest first): does it number rows or components, what to
+            // divide that number by, its extent and its stride in the result
+            long rowDiv = 1, compDiv = 1;
+            for (size_t d = rows.size(); d-- > 0;)
+            {
+                const bool isComp = has(between, rows[d]);
+                OperatorShape::Term t;
+                t.div = isComp ? compDiv : rowDiv;
+                t.ext = extent[rows[d]];
+                t.stride = s.out.stride[shared + d];
+                (isComp ? o.outCompTerms : o.outRowTerms).push_back(t);
+                (isComp ? compDiv : rowDiv) *= extent[rows[d]];
+            }
+            // (the components in the vectors' order: the same as in the result, or the numbering would differ)
+            std::vector<int> inResultOrder;
+            for (int id : rows)
+            {
+                if (has(between, id)) inResultOrder.push_back(id);
+            }
+            if (inResultOrder != between) return false;
+            o.outMixed = true;
+            o.comp = compDiv;
+            std::vector<int> only;
+            for (int id : rows)
+            {
+                if (!has(between, id)) only.push_back(id);
+            }
+            rows = only;
+            cols.resize(cols.size() - between.size());
+        }
     }
     else
     {
@@ -179,12 +225,19 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
             envInt("ACRO_HIP_OPERATOR_MFMA") < 0)
             return false;
     }
+    if (o.outMixed)
+    {
+        const long rowsP = (o.rows + 15) / 16 * 16, colsP = (o.cols + 3) / 4 * 4;
+        if (o.blockRows > 0 || o.comp > 16 || o.comp * (rowsP / 16) > 24 || s.in.size() != 2 || envInt("ACRO_HIP_OPERATOR_STAGE_OUT") < 0 ||
+            envInt("ACRO_HIP_OPERATOR_MFMA") < 0 || envInt("ACRO_HIP_OPERATOR_COMPONENTS") != 0 || (rowsP * colsP + 16 * o.rows * o.comp) * 8 > 64 * 1024)
+            return false;
+    }
     // With components a lane holds rows / 4 results for each of them: at most 16 blocks of 16 rows in all, more rows
     // in blocks of rows as above.
     if (o.comp > 1 && !o.trailing && alone && envInt("ACRO_HIP_OPERATOR_BLOCKS") >= 0 && envInt("ACRO_HIP_OPERATOR_MFMA") >= 0 && o.comp <= 16)
     {
         const long most = 16 * (16 / o.comp);
-        if (ComponentsTogether(o) && (o.blockRows > most || (o.blockRows == 0 && o.rows > most))) o.blockRows = most;
+        if (!o.outMixed && ComponentsTogether(o) && (o.blockRows > most || (o.blockRows == 0 && o.rows > most))) o.blockRows = most;
     }
     // With components: vectors in 8-byte loads, no pointwise factors, and only where the generic schedule (an
     // entry and a row per lane) runs out of scalar registers for the operator or of coalescing for its stores
@@ -823,6 +876,7 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
 auto Generator::ComponentsTogether(const OperatorShape &o) const -> bool
 {
     if (o.comp <= 1 || o.comp > 16 || o.trailing || envInt("ACRO_HIP_OPERATOR_COMPONENTS") >= 2) return false;
+    if (o.outMixed) return true;
     const long padded = ((o.rows + 15) / 16 * 16) * ((o.cols + 3) / 4 * 4);
     return padded <= 1024 || (o.rows * o.cols > 4096 && o.cols <= 64);
 }
@@ -846,6 +900,7 @@ auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape 
             if (stageRounds == 0 && (nIp * nJp + 64 / rounds * nI * C) * 8 <= 64 * 1024) stageRounds = rounds;
         }
     }
+    ACROBATIC_ASSERT(!shape.outMixed || stageRounds > 0, "HIP generator: components between the row indices need the LDS stage");
     const long most = nIp * nJp > 4096 ? 256 : 512;
     const long blocks = std::max<long>(1, std::min<long>(most, (tiles + 3) / 4));
     for (const auto &st : stores)
@@ -926,8 +981,22 @@ auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape 
             out << "#pragma unroll\n        for (int r = " << h * perRound << "; r < " << (h + 1) * perRound << "; ++r)\n";
             out << "#pragma unroll\n            for (int t = 0; t < " << tilesN << "; ++t)\n";
             out << "#pragma unroll\n                for (int k = 0; k < " << C << "; ++k)\n";
+            std::string inEntry = "(16 * t + c) * " + str(C) + " + k";
+            if (shape.outMixed)
+            {
+                inEntry.clear();
+                auto add = [&](const std::string &flat, const std::vector<OperatorShape::Term> &terms) {
+                    for (const auto &term : terms)
+                    {
+                        const std::string v = term.div == 1 ? flat : "(" + flat + " / " + str(term.div) + ")";
+                        inEntry += (inEntry.empty() ? "" : " + ") + ("(" + v + " % " + str(term.ext) + ")") + " * " + str(term.stride);
+                    }
+                };
+                add("(16 * t + c)", shape.outRowTerms);
+                add("k", shape.outCompTerms);
+            }
             out << "                    " << rowGuard << "mid[(4 * " << (h ? "(r - " + str(static_cast<long>(h * perRound)) + ")" : std::string("r")) << " + g) * " << rowsC
-                << " + (16 * t + c) * " << C << " + k] = acc[k][t][r];\n";
+                << " + " << inEntry << "] = acc[k][t][r];\n";
             out << "        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");\n        __builtin_amdgcn_wave_barrier();\n";
             out << "        {\n";
             const long firstEntry = 4L * h * perRound, entries = 4L * perRound;

@@ -423,6 +423,9 @@ class Generator
             long div, ext, stride;
         };
         std::vector<Term> rowTerms, colTerms;
+        // component indices between the result's row indices: where row number and component number go in an entry
+        bool outMixed = false;
+        std::vector<Term> outRowTerms, outCompTerms;
         bool cores = false;        // sizes and alignment suit the FP64 matrix cores
         bool pairs = false;        // the entries' vectors (and weights of their shape) come in 16-byte loads
         bool trailing = false;     // the entries are the fastest dimension: "A_i_e = B_i_j X_j_e"

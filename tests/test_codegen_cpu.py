@@ -248,6 +248,12 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     src = TE.GetImplementation("J_e_q_n_m = G_q_i_n X_e_i_m", at.Tensor(501, 27, 3, 3), at.Tensor(27, 27, 3), at.Tensor(501, 27, 3))
     assert "81 x 27 operator (dimensions in another order)" in src and "3 components per vector element" in src
     assert "T1[0 + (row % 3) * 1 + ((row / 3) % 27) * 81 + (j % 27) * 3]" in src
+    # components between the result's row indices: put into memory order while a trip's results are collected in LDS
+    src = TE.GetImplementation("J_e_q_m_n = X_e_i_m G_q_i_n", at.Tensor(501, 27, 3, 3), at.Tensor(501, 27, 3), at.Tensor(27, 27, 3))
+    assert "81 x 27 operator (dimensions in another order)" in src and "3 components per vector element, results written out through LDS" in src
+    assert "mid[(4 * r + g) * 243 + ((16 * t + c) % 3) * 1 + (((16 * t + c) / 3) % 27) * 9 + (k % 3) * 3] = acc[k][t][r];" in src
+    # (not for operators applied in blocks of rows)
+    assert "operator schedule" not in TE.GetImplementation("J_e_q_m_n = X_e_i_m G_q_i_n", at.Tensor(501, 64, 3, 3), at.Tensor(501, 64, 3), at.Tensor(64, 64, 3))
     # very long vectors or very many rows would not fit a lane's registers: not this schedule
     assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 5), at.Tensor(5, 818), at.Tensor(900, 818))
     assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 300), at.Tensor(300, 12), at.Tensor(900, 12))
