@@ -227,17 +227,17 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
     }
     if (o.outMixed)
     {
-        const long rowsP = (o.rows + 15) / 16 * 16, colsP = (o.cols + 3) / 4 * 4;
-        if (o.blockRows > 0 || o.comp > 16 || o.comp * (rowsP / 16) > 24 || s.in.size() != 2 || envInt("ACRO_HIP_OPERATOR_STAGE_OUT") < 0 ||
-            envInt("ACRO_HIP_OPERATOR_MFMA") < 0 || envInt("ACRO_HIP_OPERATOR_COMPONENTS") != 0 || (rowsP * colsP + 16 * o.rows * o.comp) * 8 > 64 * 1024)
+        if (o.comp > 16 || s.in.size() != 2 || envInt("ACRO_HIP_OPERATOR_BLOCKS") < 0 || envInt("ACRO_HIP_OPERATOR_MFMA") < 0 ||
+            envInt("ACRO_HIP_OPERATOR_COMPONENTS") != 0)
             return false;
     }
     // With components a lane holds rows / 4 results for each of them: at most 16 blocks of 16 rows in all, more rows
     // in blocks of rows as above.
     if (o.comp > 1 && !o.trailing && alone && envInt("ACRO_HIP_OPERATOR_BLOCKS") >= 0 && envInt("ACRO_HIP_OPERATOR_MFMA") >= 0 && o.comp <= 16)
     {
-        const long most = 16 * (16 / o.comp);
-        if (!o.outMixed && ComponentsTogether(o) && (o.blockRows > most || (o.blockRows == 0 && o.rows > most))) o.blockRows = most;
+        // (components between the row indices have no other schedule to fall back on: half as many registers again)
+        const long most = 16 * ((o.outMixed ? 24 : 16) / o.comp);
+        if (ComponentsTogether(o) && (o.blockRows > most || (o.blockRows == 0 && o.rows > most))) o.blockRows = most;
     }
     // With components: vectors in 8-byte loads, no pointwise factors, and only where the generic schedule (an
     // entry and a row per lane) runs out of scalar registers for the operator or of coalescing for its stores
@@ -641,6 +641,9 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     // (A contiguous range of trips per workgroup instead of this stride: the same or up to 8 % slower.)
     out << "    const long waves = (long)gridDim.x * 4;\n";
     out << "    for (long tile = (long)blockIdx.x * 4 + (threadIdx.x >> 6); tile < " << tiles << "; tile += waves)\n    {\n";
+    // (a kernel that the compiler can only fit into the registers with spills is compiled again with this macro:
+    // the operator's values are then read from LDS on every trip instead of being kept in registers across trips)
+    out << "#ifdef ACRO_KEEP_OPERATOR_IN_LDS\n        __asm__ volatile(\"\" ::: \"memory\");\n#endif\n";
     if (ragged)
         out << "        const long ex = tile * 16 + c < " << E << " ? tile * 16 + c : " << E - 1 << ";  // past the end: any valid entry, never stored\n";
     else
@@ -900,7 +903,6 @@ auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape 
             if (stageRounds == 0 && (nIp * nJp + 64 / rounds * nI * C) * 8 <= 64 * 1024) stageRounds = rounds;
         }
     }
-    ACROBATIC_ASSERT(!shape.outMixed || stageRounds > 0, "HIP generator: components between the row indices need the LDS stage");
     const long most = nIp * nJp > 4096 ? 256 : 512;
     const long blocks = std::max<long>(1, std::min<long>(most, (tiles + 3) / 4));
     for (const auto &st : stores)
@@ -952,6 +954,9 @@ auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape 
     out << "    const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;\n";
     out << "    const long waves = (long)gridDim.x * 4;\n";
     out << "    for (long tile = (long)blockIdx.x * 4 + (threadIdx.x >> 6); tile < " << tiles << "; tile += waves)\n    {\n";
+    // (a kernel that the compiler can only fit into the registers with spills is compiled again with this macro:
+    // the operator's values are then read from LDS on every trip instead of being kept in registers across trips)
+    out << "#ifdef ACRO_KEEP_OPERATOR_IN_LDS\n        __asm__ volatile(\"\" ::: \"memory\");\n#endif\n";
     if (ragged)
         out << "        const long ex = tile * 16 + c < " << NE << " ? tile * 16 + c : " << NE - 1 << ";  // past the end: any valid entry, never stored\n";
     else
@@ -973,6 +978,20 @@ auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape 
     // register r of a lane holds entry 4 r + g of the trip and row 16 t + c
     const long rowsC = nI * C, strideC = nAll * C;
     const std::string rowGuard = nIp != nI ? "if (16 * t + c < " + str(nI) + ") " : std::string();
+    // components between the result's row indices: where row `row` and component k of an entry lie
+    auto mixedOffset = [&](const std::string &row) {
+        std::string at;
+        auto add = [&](const std::string &flat, const std::vector<OperatorShape::Term> &terms) {
+            for (const auto &term : terms)
+            {
+                const std::string v = term.div == 1 ? flat : "(" + flat + " / " + str(term.div) + ")";
+                at += (at.empty() ? "" : " + ") + ("(" + v + " % " + str(term.ext) + ")") + " * " + str(term.stride);
+            }
+        };
+        add(row, shape.outRowTerms);
+        add("k", shape.outCompTerms);
+        return at;
+    };
     if (stageRounds > 0)
     {
         out << "        double *mid = stage + (threadIdx.x >> 6) * " << 4 * perRound * rowsC << ";\n";
@@ -981,20 +1000,7 @@ auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape 
             out << "#pragma unroll\n        for (int r = " << h * perRound << "; r < " << (h + 1) * perRound << "; ++r)\n";
             out << "#pragma unroll\n            for (int t = 0; t < " << tilesN << "; ++t)\n";
             out << "#pragma unroll\n                for (int k = 0; k < " << C << "; ++k)\n";
-            std::string inEntry = "(16 * t + c) * " + str(C) + " + k";
-            if (shape.outMixed)
-            {
-                inEntry.clear();
-                auto add = [&](const std::string &flat, const std::vector<OperatorShape::Term> &terms) {
-                    for (const auto &term : terms)
-                    {
-                        const std::string v = term.div == 1 ? flat : "(" + flat + " / " + str(term.div) + ")";
-                        inEntry += (inEntry.empty() ? "" : " + ") + ("(" + v + " % " + str(term.ext) + ")") + " * " + str(term.stride);
-                    }
-                };
-                add("(16 * t + c)", shape.outRowTerms);
-                add("k", shape.outCompTerms);
-            }
+            const std::string inEntry = shape.outMixed ? mixedOffset("(16 * t + c)") : "(16 * t + c) * " + str(C) + " + k";
             out << "                    " << rowGuard << "mid[(4 * " << (h ? "(r - " + str(static_cast<long>(h * perRound)) + ")" : std::string("r")) << " + g) * " << rowsC
                 << " + " << inEntry << "] = acc[k][t][r];\n";
             out << "        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");\n        __builtin_amdgcn_wave_barrier();\n";
@@ -1019,10 +1025,13 @@ auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape 
     {
         out << "#pragma unroll\n        for (int r = 0; r < 4; ++r)\n        {\n";
         if (ragged) out << "            if (tile * 16 + g + 4 * r >= " << NE << ") continue;\n";
-        out << "            double *a = " << A << " + " << Lit(uvars[s.out.uvar].viewOffset) << " + (tile * 16 + g + 4 * r) * " << strideC << " + " << row0 * C << " + c * " << C << ";\n";
+        out << "            double *a = " << A << " + " << Lit(uvars[s.out.uvar].viewOffset) << " + (tile * 16 + g + 4 * r) * " << strideC;
+        if (!shape.outMixed) out << " + " << row0 * C << " + c * " << C;
+        out << ";\n";
         out << "#pragma unroll\n            for (int t = 0; t < " << tilesN << "; ++t)\n";
         out << "#pragma unroll\n                for (int k = 0; k < " << C << "; ++k)\n";
-        out << "                    " << rowGuard << "a[" << 16 * C << " * t + k]" << (s.op == '=' ? " = " : (s.op == '+' ? " += " : " -= ")) << "acc[k][t][r];\n";
+        const std::string where = shape.outMixed ? mixedOffset("(16 * t + c" + (row0 > 0 ? " + " + str(row0) : std::string()) + ")") : str(16 * C) + " * t + k";
+        out << "                    " << rowGuard << "a[" << where << "]" << (s.op == '=' ? " = " : (s.op == '+' ? " += " : " -= ")) << "acc[k][t][r];\n";
         out << "        }\n";
     }
     out << "    }\n}\n";
@@ -1103,6 +1112,9 @@ auto Generator::EmitOperatorEntriesFastest(HipKernelPlan &plan, const OperatorSh
     out << "    const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;\n";
     out << "    const long waves = (long)gridDim.x * 4;\n";
     out << "    for (long trip = (long)blockIdx.x * 4 + (threadIdx.x >> 6); trip < " << trips << "; trip += waves)\n    {\n";
+    // (a kernel that the compiler can only fit into the registers with spills is compiled again with this macro:
+    // the operator's values are then read from LDS on every trip instead of being kept in registers across trips)
+    out << "#ifdef ACRO_KEEP_OPERATOR_IN_LDS\n        __asm__ volatile(\"\" ::: \"memory\");\n#endif\n";
     out << "        const long e = trip * " << per << " + " << (pairs ? "2 * c" : "c") << ";\n";
     if (ragged)
         out << "        const long ex = e < " << E << " ? e : " << E - (pairs ? 2 : 1) << ";  // past the end: any valid entry, never stored\n";

@@ -206,6 +206,34 @@ void HipKernel::EnsureLoaded()
         err = hipModuleLoadData(&module, CodeObject.data());
     }
     ACRO_HIP_CHECK(err);
+    // Kernels that keep no arrays in private memory by design (the matrix-core schedules) carry a switch that trades
+    // registers for LDS reads.  When the compiler has fit one of them into the registers only with spills, compile
+    // the module again with the switch on: spill code around the matrix-core accumulators is slow, and the compiler
+    // has been seen to lose half of a spilled 64-bit value there (a result off in its low 32 bits).
+    static const char *const kSwitch = "ACRO_KEEP_OPERATOR_IN_LDS";
+    if (Source.find(std::string("#ifdef ") + kSwitch) != std::string::npos && Source.compare(0, 8, "#define ") != 0)
+    {
+        bool spills = false;
+        for (size_t at = Source.find("__global__"); at != std::string::npos && !spills; at = Source.find("__global__", at + 1))
+        {
+            const size_t name = Source.find("void ", at), paren = Source.find('(', name);
+            if (name == std::string::npos || paren == std::string::npos) break;
+            hipFunction_t function;
+            int privateBytes = 0;
+            ACRO_HIP_CHECK(hipModuleGetFunction(&function, module, Source.substr(name + 5, paren - name - 5).c_str()));
+            ACRO_HIP_CHECK(hipFuncGetAttribute(&privateBytes, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, function));
+            spills = privateBytes > 0;
+        }
+        if (spills)
+        {
+            ACRO_HIP_CHECK(hipModuleUnload(module));
+            Source = std::string("#define ") + kSwitch + " 1\n" + Source;
+            CacheHit = false;
+            CodeObject.clear();
+            Compile();
+            ACRO_HIP_CHECK(hipModuleLoadData(&module, CodeObject.data()));
+        }
+    }
     Module = module;
 }
 

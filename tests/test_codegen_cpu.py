@@ -252,8 +252,12 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     src = TE.GetImplementation("J_e_q_m_n = X_e_i_m G_q_i_n", at.Tensor(501, 27, 3, 3), at.Tensor(501, 27, 3), at.Tensor(27, 27, 3))
     assert "81 x 27 operator (dimensions in another order)" in src and "3 components per vector element, results written out through LDS" in src
     assert "mid[(4 * r + g) * 243 + ((16 * t + c) % 3) * 1 + (((16 * t + c) / 3) % 27) * 9 + (k % 3) * 3] = acc[k][t][r];" in src
-    # (not for operators applied in blocks of rows)
-    assert "operator schedule" not in TE.GetImplementation("J_e_q_m_n = X_e_i_m G_q_i_n", at.Tensor(501, 64, 3, 3), at.Tensor(501, 64, 3), at.Tensor(64, 64, 3))
+    # (operators applied in blocks of rows store from the registers)
+    src = TE.GetImplementation("J_e_q_m_n = X_e_i_m G_q_i_n", at.Tensor(501, 64, 3, 3), at.Tensor(501, 64, 3), at.Tensor(64, 64, 3))
+    assert "rows 128 - 191 of the 192 x 64 operator (dimensions in another order)" in src and src.count("__global__") == 2
+    assert "a[((16 * t + c + 128) % 3) * 1 + (((16 * t + c + 128) / 3) % 64) * 9 + (k % 3) * 3] = acc[k][t][r];" in src
+    # the switch for a kernel that the compiler can only fit into the registers with spills
+    assert src.count('#ifdef ACRO_KEEP_OPERATOR_IN_LDS\n        __asm__ volatile("" ::: "memory");\n#endif\n') == 2
     # very long vectors or very many rows would not fit a lane's registers: not this schedule
     assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 5), at.Tensor(5, 818), at.Tensor(900, 818))
     assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 300), at.Tensor(300, 12), at.Tensor(900, 12))

@@ -1050,6 +1050,9 @@ def test_gram_matrix_of_one_tensor_and_of_slices(at, engine, checker):
     ("G_e_d_q = D_q_i_d X_e_i", [(70, 64, 3), (1001, 64)]),                        # too large for LDS as well: blocks of rows
     ("J_e_q_m_n = X_e_i_m G_q_i_n", [(501, 27, 3), (27, 27, 3)]),                  # the component m between the row indices
     ("J_e_m_q_n += G_q_n_i X_e_i_m", [(13, 2, 10), (333, 10, 3)]),                 # ... in front of them, few rows
+    ("J_e_q_m_n = X_e_i_m G_q_i_n", [(301, 64, 3), (64, 64, 3)]),                  # ... of an operator applied in blocks of rows
+    # (its blocks of 128 rows do not fit the registers when the operator's values are kept across trips: compiled again without)
+    ("O_e_i0_m0_i1_i2 += I0_e_j0_j1_m0 I1_j1_i0_i2_j0_i1", [(1368, 26, 2, 2), (2, 37, 3, 26, 10)]),
     ("J_e_q_m_k_n -= G_n_q_i X_e_i_m_k", [(3, 9, 10), (205, 10, 2, 2)]),           # two components, both between
 ])
 def test_dense_operator_with_dimensions_in_any_order(at, engine, checker, kernel, shapes):
