@@ -363,13 +363,15 @@ auto Generator::WaveStoreLineCoverage(int k, int entries) const -> double
     for (long w = 0; w < items; ++w)
     {
         std::vector<int> value(nidx, 0);
-        long rest = w % s.laneCount;
+        // (numbered with the entry fastest: neighbouring lanes take neighbouring entries of one lane item)
+        const long perGroup = entries > 0 ? entries : NB;
+        long rest = entriesFastest ? (w / perGroup) % s.laneCount : w % s.laneCount;
         for (int j = static_cast<int>(s.lane.size()) - 1; j >= 0; --j)
         {
             value[s.lane[j]] = static_cast<int>(rest % extent[s.lane[j]]);
             rest /= extent[s.lane[j]];
         }
-        if (batch >= 0) value[batch] = static_cast<int>(w / s.laneCount);
+        if (batch >= 0) value[batch] = static_cast<int>(entriesFastest ? w % perGroup : w / s.laneCount);
         const long tiles = s.tileCount;
         for (long t = 0; t < tiles; ++t)
         {
