@@ -242,7 +242,8 @@ auto Generator::StageReusedOperands(int ki, const Sub &asWritten, std::vector<Su
     Sub orig = asWritten;
     if (orig.out.repeated || orig.in.size() < 2 || NumGatherSlots() > 0) return false;
     const long outputs = product(orig.outIdx, extent) / extent[batch];
-    if (outputs < 4 || outputs > 1024) return false;
+    const long stageMost = envInt("ACRO_HIP_STAGE_MOST", 8000);
+    if (outputs < 4 || outputs > stageMost / 2) return false;
     // Tiny matrices (fewer than 64 outputs) are staged as well unless every operand's entry is a power of two of
     // doubles: those lie in whole lines and the lanes read them well from device memory (4 x 4 products with one
     // output per lane: 90 % of the HBM peak, 51 % staged), the others do not (3 x 3: 64 -> 82 %, 5 x 5: 46 -> 77 %,
@@ -264,14 +265,28 @@ auto Generator::StageReusedOperands(int ki, const Sub &asWritten, std::vector<Su
         long reads = 1;
         for (int id : orig.outIdx) reads *= (id == batch || has(r.idx, id)) ? 1 : extent[id];
         wholeLines = wholeLines && (perEntry & (perEntry - 1)) == 0;
-        if (perEntry < (tiny ? 4 : 16) || perEntry > 1024 || reads < (tiny ? 2 : 8)) continue;
+        if (perEntry < (tiny ? 4 : 16) || perEntry > stageMost / 2 || reads < (tiny ? 2 : 8)) continue;
         staged[v] = 1;
         total += perEntry;
         ++count;
     }
     // Two such operands: products of element matrices.  With one (an element vector under an element matrix, the
     // vectors of a dense operator) the kernel has schedules of its own that read the big operand once and well.
-    if (count < 2 || total > 2048 || (tiny && wholeLines)) return false;
+    if (count < 2 || total > stageMost || (tiny && wholeLines)) return false;
+    // More than 1 024 outputs or 2 048 staged values per entry (products of 33 x 33 to 62 x 62 matrices, which the lanes
+    // read straight from device memory at 9 - 12 % of the HBM peak: staged 49 - 66 %): only the two factors of a
+    // product, each of which carries a contracted index
+    if (outputs > 1024 || total > 2048)
+    {
+        bool factors = count == 2;
+        for (size_t v = 0; v < orig.in.size(); ++v)
+        {
+            bool contracted = false;
+            for (int id : orig.in[v].idx) contracted = contracted || has(orig.contr, id);
+            factors = factors && (!staged[v] || contracted);
+        }
+        if (!factors) return false;
+    }
     // (tiny entries under one shared operator, "A_e_i = B_i_j X_e_j W_e D_e_j", belong to the operator schedule)
     int operators = 0;
     for (const auto &r : orig.in)
@@ -321,7 +336,15 @@ auto Generator::StageReusedOperands(int ki, const Sub &asWritten, std::vector<Su
         for (int id : outputIds)
         {
             if (id == batch || extent[id] < 4) continue;
-            const int t = extent[id] % 2 == 0 ? 2 : (extent[id] % 3 == 0 ? 3 : 1);
+            int t = extent[id] % 2 == 0 ? 2 : (extent[id] % 3 == 0 ? 3 : (extent[id] % 5 == 0 && envInt("ACRO_HIP_SPLIT_FIVE") >= 0 ? 5 : 1));
+            if (t == 5)
+            {
+                // blocks of five only while a hundred lane items are left per entry (25 x 25 in 5 x 5 blocks: 25 items,
+                // two waves in eight busy, 49 % of the HBM peak)
+                long items = 1;
+                for (int other : orig.outIdx) items *= (other == batch || has(blockIdx, other)) ? 1 : extent[other];
+                if (items / 5 < envInt("ACRO_HIP_SPLIT_FIVE_ITEMS", 100)) t = 1;
+            }
             if (t == 1) continue;
             // two new loop indices, named after the old one
             auto fresh = [&](std::string name) {

@@ -186,6 +186,7 @@ KERNEL_SHAPES = [
     ("A_e_i_j = B_e_i_k C_e_k_j", [(29127, 24, 24), (29127, 24, 24)], (29127, 24, 24)),
     ("A_e_i_j = B_e_i_k C_e_k_j", [(138654, 11, 11), (138654, 11, 11)], (138654, 11, 11)),
     ("A_e_i_j = B_e_i_k C_e_k_j", [(26843, 25, 25), (26843, 25, 25)], (26843, 25, 25)),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(10485, 40, 40), (10485, 40, 40)], (10485, 40, 40)),
     ("A_i = C_i_j B_j", [(1 << 20, 64), (64,)], (1 << 20,)),
     ("M_e_i1_i2_j1_j2 = B_k1_i1 B_k1_j1 B_k2_i2 B_k2_j2 D_e_k1_k2", [(5, 4)] * 4 + [(1 << 19, 5, 5)], (1 << 19, 4, 4, 4, 4)),
     ("A_i_j = B_j_i", [(1 << 22, 16)], (16, 1 << 22)),

@@ -291,6 +291,16 @@ def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE):
     assert "8 per workgroup of 256 lanes" in src and "lanes(i,k)=121 tile()=1" in src
     src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 3, 3), at.Tensor(4096, 3, 3), at.Tensor(4096, 3, 3))
     assert "56 per workgroup of 256 lanes" in src and "operands staged in LDS" in src and "lanes(i,k)=9 tile()=1" in src
+    # 25 x 25: blocks of five along one index only (125 lane items per entry; both would leave 25); 35 x 35 and 62 x 62:
+    # an entry's operands fill most of a workgroup's LDS; 64 x 64 does not fit
+    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 25, 25), at.Tensor(4096, 25, 25), at.Tensor(4096, 25, 25))
+    assert "operands staged in LDS" in src and "lanes(ihi,k)=125 tile(ilo)=5" in src
+    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 35, 35), at.Tensor(4096, 35, 35), at.Tensor(4096, 35, 35))
+    assert "operands staged in LDS" in src and "lanes(ihi,k)=245 tile(ilo)=5" in src and "1 per workgroup of 256 lanes" in src
+    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 62, 62), at.Tensor(4096, 62, 62), at.Tensor(4096, 62, 62))
+    assert "operands staged in LDS" in src and "LDS 61504 bytes" in src
+    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 64, 64), at.Tensor(4096, 64, 64), at.Tensor(4096, 64, 64))
+    assert "operands staged in LDS" not in src
     # slices are not whole tensors: their indices stay as they are
     big = at.Tensor(2, 4096, 8, 8)
     src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 8, 8), at.SliceTensor(big, 1), at.Tensor(4096, 8, 8))

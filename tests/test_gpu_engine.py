@@ -223,7 +223,14 @@ def test_products_of_element_matrices_stage_their_operands_in_lds(at, engine, ch
     ("A_e_i_j = B_e_i_k C_e_k_j D_e_i_j", [(31, 24, 8), (31, 8, 25), (31, 24, 25)], "tile(ilo)=2"),
     # no blocks: one output per lane, several entries per workgroup; rows of odd length are padded in LDS
     ("A_e_i_j = B_e_i_k C_e_k_j", [(203, 11, 11), (203, 11, 11)], "8 per workgroup of 256 lanes"),
-    ("A_e_i_j += B_e_i_k C_e_k_j", [(29, 25, 25), (29, 25, 25)], "LDS 10400 bytes"),
+    ("A_e_i_j += B_e_i_k C_e_k_j", [(29, 23, 23), (29, 23, 23)], "LDS 8832 bytes"),
+    # divisible by five only: blocks of five along one index while a hundred lane items are left per entry
+    ("A_e_i_j += B_e_i_k C_e_k_j", [(29, 25, 25), (29, 25, 25)], "lanes(ihi,j)=125 tile(ilo)=5"),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(41, 25, 15), (41, 15, 20)], "lanes(ihi,jhi)=50 tile(ilo,jlo)=10"),
+    # larger than 32 x 32: an entry's operands fill most of a workgroup's LDS
+    ("A_e_i_j -= B_e_i_k C_e_k_j", [(39, 35, 35), (39, 35, 35)], "lanes(ihi,j)=245 tile(ilo)=5"),
+    ("A_e_i_j = B_e_k_i C_e_j_k", [(51, 47, 45), (51, 40, 47)], "1 per workgroup of 256 lanes"),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(67, 62, 62), (67, 62, 62)], "LDS 61504 bytes"),
 ])
 def test_products_of_small_element_matrices(at, engine, checker, kernel, shapes, expect):
     rng = np.random.default_rng(len(kernel) + shapes[0][0])
