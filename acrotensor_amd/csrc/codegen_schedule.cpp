@@ -381,9 +381,11 @@ auto Generator::ChooseTiles() -> void
         // flattened contraction, so that the lanes of a wavefront read consecutive addresses, and the partial sums
         // are added in a butterfly of lane exchanges (a fixed order: results are reproducible).  The same for a
         // kernel with few outputs per entry and a contraction along the fastest dimension of a streaming operand
-        // ("A_e_i = B_e_i_n", "Y_e_i = M_e_i_j X_e_j" with an element matrix of 27 x 27).
+        // ("A_e_i = B_e_i_n", "Y_e_i = M_e_i_j X_e_j" with an element matrix of 27 x 27).  Up to 64 rows, or any number
+        // of rows of 32 terms and more (65 x 65 62 -> 83 % of the HBM peak, 100 x 100 59 -> 85 %, 200 x 64 72 -> 84 %;
+        // 256 x 16 90 -> 88 %, hence not for short rows).
         if (subs.size() == 1 && batch >= 0 && s.matrixOp == 0 && !s.out.repeated && envInt("ACRO_HIP_SPLIT_LANES") >= 0 &&
-            !s.contr.empty() && (mid.empty() ? s.contrCount >= 8 : (s.contrCount >= 16 && product(mid, extent) <= 64)))
+            !s.contr.empty() && (mid.empty() ? s.contrCount >= 8 : (s.contrCount >= 16 && product(mid, extent) <= (s.contrCount >= 32 ? envInt("ACRO_HIP_SPLIT_LANES_ROWS", 1024) : 64))))
         {
             // the operand that an entry reads most of carries the batch index and the fastest contraction index last
             const VarRef *most = &s.in[0];

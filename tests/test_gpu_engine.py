@@ -511,6 +511,8 @@ def test_kernels_whose_schedule_follows_the_memory_access_pattern(at, engine, ch
     ("A_e_i = B_e_i_j C_e_j", [(203, 16, 16), (203, 16)]),       # element matrix times element vector: 4 lanes per row
     ("A_e_i += B_e_i_j C_e_j", [(35, 20, 20), (35, 20)]),        # 20 terms over 4 lanes (rows of odd length: two steps through LDS)
     ("A_e_i = B_e_i_j C_e_j", [(9, 64, 64), (9, 64)]),           # 16 lanes per row, four passes per entry
+    ("A_e_i -= B_e_i_j C_e_j D_e_i", [(130, 100, 100), (130, 100), (130, 100)]),   # more than 64 rows of 32 terms and more: 16 lanes per row
+    ("A_e_i = B_e_i_j C_j", [(1030, 300, 33), (33,)]),           # ... rows of odd length
     ("A_e_i_k = B_e_i_k_n", [(21, 3, 5, 100)]),                  # two lane indices next to the shared contraction
     ("A_e -= B_e_i_j C_i D_j", [(1001, 8, 8), (8,), (8,)]),      # bilinear form: pairs of terms along j, C_i once per pair
     ("A_e_i = B_e_i_j_k C_e_j D_e_k", [(203, 8, 8, 8), (203, 8), (203, 8)]),
