@@ -21,7 +21,21 @@ auto Generator::UseTransposeSchedule() const -> bool
     if (s.in[0].uvar == s.out.uvar || s.in[0].idx.size() != s.out.idx.size() || s.out.idx.size() < 2) return false;
     const int a = s.in[0].idx.back(), b = s.out.idx.back();
     if (a == b) return false;
-    if (extent[a] >= 32 && extent[b] >= 32) return true;
+    if (extent[a] >= 32 && extent[b] >= 32)
+    {
+        // Small matrices per entry ("A_e_i_j = B_e_j_i", 40 x 40 to 100 x 100): a lane per element writes along the rows
+        // of the result and reads down the columns of an operand that the caches hold for the whole entry, which beats
+        // tiles of 32 x 32 that such extents fill badly (40 x 40: 37 -> 90 % of the HBM peak, 45 x 45 31 -> 89 %,
+        // 64 x 64 78 -> 87 %, 64 x 100 59 -> 85 %, 100 x 100 44 -> 60 %; 32 x 32 stays, 80 against 70 %, and so does
+        // 200 x 200, 64 against 37 %).
+        const long na = extent[a], nb = extent[b];
+        const double filled = static_cast<double>(na * nb) / static_cast<double>(((na + 31) / 32 * 32) * ((nb + 31) / 32 * 32));
+        const size_t n = s.out.idx.size();
+        bool perEntry = n > 2 && envInt("ACRO_HIP_TRANSPOSE") < 3 && s.out.idx[n - 2] == a && s.in[0].idx[n - 2] == b;
+        for (size_t d = 0; perEntry && d + 2 < n; ++d) perEntry = s.out.idx[d] == s.in[0].idx[d];
+        if (perEntry && na * nb > 1024 && (na * nb <= 4096 || (na * nb <= 10000 && filled < 0.8))) return false;
+        return true;
+    }
     // One side short (a matrix of 2^22 x 16): tiles of 16 x 64 (8 x 128) entries, see EmitTranspose.
     const int shorter = std::min(extent[a], extent[b]), longer = std::max(extent[a], extent[b]);
     return envInt("ACRO_HIP_TRANSPOSE") < 2 && shorter >= 8 && longer >= 256;

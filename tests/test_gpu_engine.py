@@ -552,7 +552,8 @@ def test_split_contraction_of_few_long_rows(at, engine, checker, kernel, shapes,
     ("A_i_j = B_j_i", (70, 100)),                    # ragged tiles on both sides
     ("A_i_j += B_j_i", (64, 32)),
     ("A_i_e_j -= B_j_e_i", (70, 3, 100)),            # a dimension in between
-    ("A_e_i_j = B_e_j_i", (5, 40, 50)),              # batched, matrices too large for one lane each
+    ("A_e_i_j = B_e_j_i", (5, 128, 160)),            # batched, matrices larger than the caches hold per entry
+    ("A_e_i_j -= B_e_j_i", (11, 32, 32)),            # ... and small ones that fill the tiles
     ("A_j_k_i = B_i_k_j", (33, 2, 45)),
     ("A_k_j_i_l = B_l_i_k_j", (32, 37, 3, 41)),      # fastest dimensions l and j, two more in other places
     ("A_i_j = B_j_i", (1000, 16)),                   # one side short: tiles of 16 x 64 entries
@@ -569,6 +570,22 @@ def test_permutations_with_long_fastest_dimensions_go_through_lds_tiles(at, engi
     if "-=" in kernel:
         expected = 2.0 * out0 - expected
     assert np.array_equal(got, expected)             # moves (and one addition): bit for bit
+
+
+@pytest.mark.parametrize("kernel,shape", [
+    ("A_e_i_j = B_e_j_i", (5, 40, 50)),              # tiles of 32 x 32 would be filled badly
+    ("A_e_i_j += B_e_j_i", (7, 64, 64)),
+    ("A_e_f_i_j -= B_e_f_j_i", (3, 2, 100, 100)),
+])
+def test_small_matrices_per_entry_are_transposed_by_a_lane_per_element(at, engine, checker, kernel, shape):
+    rng = np.random.default_rng(sum(shape))
+    B = rng.uniform(-1, 1, shape)
+    out0 = rng.uniform(-1, 1, output_shape(kernel, [shape]))
+    got, expected = run_single(at, engine, checker, kernel, out0, B)
+    assert "transpose schedule" not in engine.GetLastImplementation()
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert np.array_equal(got, expected)
 
 
 @pytest.mark.parametrize("kernel,shapes", [
