@@ -525,8 +525,7 @@ auto Generator::FactoriseKernel(int ki, const Sub &orig, bool alone, std::vector
 {
     const int nin = static_cast<int>(orig.in.size());
     if (batch < 0 || nin < 3 || orig.contr.empty() || !opt.noalias || orig.out.repeated) return false;
-    if (alone && orig.contrCount >= kReductionMinContraction && product(orig.outIdx, extent) <= envInt("ACRO_HIP_RED_MAX_OUTPUTS", kReductionMaxOutputs))
-        return false;  // the reduction schedule serves it
+    if (alone && ReductionServes(orig)) return false;  // the reduction schedule serves it
     for (const auto &r : orig.in)
     {
         if (r.repeated || r.uvar == orig.out.uvar) return false;

@@ -6,12 +6,31 @@ namespace acro
 namespace codegen
 {
 
+// Few outputs and a long contraction; or many outputs summed over a long contraction ("S_i_j = A_e_i_j" with 32 x 32
+// outputs, "S_i = A_e_i B_e" with 5 000): as written such a kernel has one lane per output walk the whole contraction
+// (0.2 - 6 % of the HBM peak).  With the outputs as the fastest dimension of the big operand any number of them is
+// served (a lane per output, see EmitReduction), the other way round the finishing kernel holds up to 1 024.
+auto Generator::ReductionServes(const Sub &s) const -> bool
+{
+    if (s.contrCount < kReductionMinContraction) return false;
+    const long outputs = product(s.outIdx, extent);
+    if (outputs <= envInt("ACRO_HIP_RED_MAX_OUTPUTS", kReductionMaxOutputs)) return true;
+    if (envInt("ACRO_HIP_RED_WIDE") < 0 || s.in.empty()) return false;
+    const VarRef *big = &s.in[0];
+    for (const auto &r : s.in)
+    {
+        if (r.size > big->size) big = &r;
+    }
+    if (big->idx.empty()) return false;
+    return has(s.outIdx, big->idx.back()) ? outputs <= 65536 : outputs <= 1024;
+}
+
 auto Generator::UseReductionSchedule() const -> bool
 {
     if (subs.size() != 1 || NumGatherSlots() > 0) return false;
     const Sub &s = subs[0];
     if (s.out.repeated) return false;
-    return s.contrCount >= kReductionMinContraction && product(s.outIdx, extent) <= envInt("ACRO_HIP_RED_MAX_OUTPUTS", kReductionMaxOutputs);
+    return ReductionServes(s);
 }
 
 // Expression for the element offset of an occurrence given variables named i_<index> for every loop index.
@@ -102,18 +121,23 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     // workgroup only NTr / O lanes would walk along a row (32-byte pieces of 64 different rows per load
     // instruction).  Instead a workgroup takes four outputs, 64 adjacent lanes each, and the workgroups are dealt
     // out over groups of outputs as well as over the contraction range.
-    const bool byRows = !pencil && !outputsFastest && O > 4 && NTr / O < 64 && envInt("ACRO_HIP_ONE_PASS") <= 0 &&
+    const bool byRows = !pencil && !outputsFastest && O > 4 && NTr / O < 64 && (envInt("ACRO_HIP_ONE_PASS") <= 0 || O > NTr) &&
                         envInt("ACRO_HIP_RED_ROWS") >= 0;
-    const long Sn = pencil ? NTr : (byRows ? 64 : NTr / O);  // contraction slices per workgroup and step
-    const long Ow = NTr / Sn, Go = byRows ? (O + Ow - 1) / Ow : 1;  // outputs per workgroup, groups of outputs
+    // More than 256 outputs that are the fastest dimension of the big operand ("S_i_j = A_e_i_j" with 16 x 16 outputs
+    // and more): a workgroup takes 256 neighbouring outputs, a lane each, and a share of the contraction range; the
+    // lanes of a wavefront read 512 consecutive bytes per term.  The finishing kernel has a workgroup per 256 outputs.
+    const bool wide = !pencil && !byRows && O > NTr;   // (up to 256 outputs: a lane per output in every workgroup, below)
+    ACROBATIC_ASSERT(!wide || outputsFastest || O <= NTr, "HIP generator: too many outputs for the reduction schedule.");
+    const long Sn = pencil ? NTr : (byRows ? 64 : (wide ? 1 : NTr / O));  // contraction slices per workgroup and step
+    const long Ow = NTr / Sn, Go = (byRows || wide) ? (O + Ow - 1) / Ow : 1;  // outputs per workgroup, groups of outputs
     // First-stage workgroups.  Pencil: one per CU (256 on this device) without unrolling, i.e. about 20 KB of
     // loads in flight per CU and one 4.7 MB window moving through the operands; more workgroups or deeper
     // unrolling measured slower at every n (n = 2^24: 206 us with 256 workgroups, 216 with 512, 252 with 2 048;
     // 214 / 263 us with the loop unrolled 2 / 4 times).  One lane per (slice, output entry): 8 bytes per lane
     // and load, so up to 512 workgroups and four loads in flight per lane (also swept: 256 - 8 192 workgroups,
     // unroll 1 - 8).
-    const long G = byRows ? std::min<long>(std::max<long>(1, 1024 / Go), std::max<long>(1, Nc / (Sn * 16)))
-                          : std::min<long>(pencil ? 256 : 512, std::max<long>(1, Nc / (Sn * (pencil ? 4 : 16))));
+    const long G = (byRows || (wide && Go > 1)) ? std::min<long>(std::max<long>(1, 1024 / Go), std::max<long>(1, Nc / (Sn * 16)))
+                                                : std::min<long>(pencil ? 256 : 512, std::max<long>(1, Nc / (Sn * (pencil ? 4 : 16))));
     // G counts the shares of the contraction range (rows of partials in the scratch buffer); the grid has one
     // workgroup per share and group of outputs.
     const long gridG = G * Go;
@@ -122,20 +146,21 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     // measured 16.8 instead of 17.2 us for the pair of launches at n = 2^20), at most 1024.  The one-pass
     // variant finishes with the lanes of the partial kernel.
     int NTf = NTr;
-    if (envInt("ACRO_HIP_ONE_PASS") <= 0)
+    const bool twoKernels = envInt("ACRO_HIP_ONE_PASS") <= 0 || wide || O > NTr;
+    if (twoKernels && !wide)
     {
         NTf = kReductionLanes;
-        while (NTf < 1024 && G * O > NTf * 4) NTf *= 2;
+        while (NTf < 1024 && (G * O > NTf * 4 || NTf < O)) NTf *= 2;
     }
-    const long S2 = NTf / O;
+    const long S2 = wide ? 1 : NTf / O;
 
     const std::string dimName = mk.GetDimensionedNameString();
     char hex[32];
     std::snprintf(hex, sizeof(hex), "%016llx",
                   static_cast<unsigned long long>(hashString(dimName + "/reduction/" + (opt.noalias ? "n" : "a") +
                                                              (Positional() ? "p" : "u") +
-                                                             (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "2" : (envInt("ACRO_HIP_ONE_PASS") >= 2 ? "1l" : "1")) + "/" + str(envInt("ACRO_HIP_RED_PENCIL")) +
-                                                             (byRows ? "/rows" : ""))));
+                                                             (twoKernels ? "2" : (envInt("ACRO_HIP_ONE_PASS") >= 2 ? "1l" : "1")) + "/" + str(envInt("ACRO_HIP_RED_PENCIL")) +
+                                                             (byRows ? "/rows" : (wide ? "/wide" : "")))));
     plan.module_name = std::string("acro_red_") + hex;
     const std::string fPartial = plan.module_name + "_partial", fFinal = plan.module_name + "_final";
 
@@ -144,9 +169,10 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
           << " workgroups x " << Sn << " slices ("
           << (pencil ? "a lane owns whole slices"
                      : (byRows ? "four outputs per workgroup, 64 adjacent lanes along each"
-                               : (outputsFastest ? "output entries on adjacent lanes" : "slices on adjacent lanes")))
+                               : (wide ? "256 outputs per workgroup, a lane each"
+                                       : (outputsFastest ? "output entries on adjacent lanes" : "slices on adjacent lanes"))))
           << "), partials added in a fixed order by "
-          << (envInt("ACRO_HIP_ONE_PASS") <= 0 ? "a second kernel" : "the workgroup that finishes last") << "\n  [0] " << s.text << "\n";
+          << (twoKernels ? "a second kernel" : "the workgroup that finishes last") << "\n  [0] " << s.text << "\n";
     plan.schedule = sched.str();
 
     out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
@@ -169,7 +195,6 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         }
     };
 
-    const bool twoKernels = envInt("ACRO_HIP_ONE_PASS") <= 0;
     const std::string counter = "(unsigned int *)(scratch + " + str(G * O) + ")";
 
     // ---- stage 1: per-workgroup partial sums
@@ -273,6 +298,25 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         out << "        for (int k = 0; k < 16; ++k) t += red[" << NTr << " + lane * 16 + k];\n";
         out << "        scratch[(long)gc * " << O << " + og * " << Ow << " + lane] = t;\n    }\n}\n";
     }
+    else if (wide)
+    {
+        out << "    const int og = blockIdx.x % " << Go << ", gc = blockIdx.x / " << Go << ";\n";
+        out << "    const int o = og * " << Ow << " + lane;\n";
+        out << "    if (o < " << O << ")\n    {\n";
+        out << "        double sum = 0.0;\n";
+        decompose(s.outIdx, "o", "        ");
+        out << "#pragma unroll 8\n";
+        out << "        for (long c = gc; c < " << Nc << "; c += " << G << ")\n        {\n";
+        decompose(s.contr, "c", "            ");
+        std::string prod;
+        for (const auto &r : s.in)
+        {
+            const std::string opnd = PtrName(r.uvar) + "[" + FullOffset(r) + "]";
+            prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
+        }
+        out << "            sum += " << prod << ";\n        }\n";
+        out << "        scratch[(long)gc * " << O << " + o] = sum;\n    }\n}\n";
+    }
     else
     {
         if (outputsFastest)
@@ -298,7 +342,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         out << "        for (int k = 0; k < " << Sn << "; ++k) t += red["
             << (outputsFastest ? "k * " + str(O) + " + lane" : "lane * " + str(Sn) + " + k") << "];\n";
     }
-    if (byRows)
+    if (byRows || wide)
     {
         // written above
     }
@@ -333,7 +377,24 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
             out << "        " << dst << " = " << dst << (s.op == '+' ? " + t;\n" : " - t;\n");
         out << "    }\n";
     };
-    if (twoKernels)
+    if (wide)
+    {
+        // a lane per output adds its partials in order
+        out << "\nextern \"C\" __global__ __launch_bounds__(" << NTf << ") void " << fFinal << "(double *"
+            << (opt.noalias ? "__restrict__ " : "") << "result, const double *__restrict__ scratch)\n{\n";
+        out << "    const int o = blockIdx.x * " << NTf << " + threadIdx.x;\n";
+        out << "    if (o < " << O << ")\n    {\n        double t = 0.0;\n";
+        out << "#pragma unroll 8\n";
+        out << "        for (long g = 0; g < " << G << "; ++g) t += scratch[g * " << O << " + o];\n";
+        decompose(s.outIdx, "o", "        ");
+        const std::string dst = "result[" + FullOffset(s.out) + "]";
+        if (s.op == '=')
+            out << "        " << dst << " = t;\n";
+        else
+            out << "        " << dst << " = " << dst << (s.op == '+' ? " + t;\n" : " - t;\n");
+        out << "    }\n}\n";
+    }
+    else if (twoKernels)
     {
         out << "\nextern \"C\" __global__ __launch_bounds__(" << NTf << ") void " << fFinal << "(double *"
             << (opt.noalias ? "__restrict__ " : "") << "result, const double *__restrict__ scratch)\n{\n";
@@ -381,7 +442,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     {
         HipLaunch fin;
         fin.function_name = fFinal;
-        fin.grid = 1;
+        fin.grid = wide ? static_cast<unsigned>((O + NTf - 1) / NTf) : 1;
         fin.block = NTf;
         fin.params.push_back(uvars[s.out.uvar].storage);
         fin.params.push_back(-1);

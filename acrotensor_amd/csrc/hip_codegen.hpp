@@ -113,6 +113,7 @@
 //   ACRO_HIP_OPERATOR_MFMA=-1   the operator schedule never uses the FP64 matrix cores (a lane keeps its row for four entries,
 //                               whose vectors come through scalar loads, whatever the operator's sizes)
 //   ACRO_HIP_RED_PENCIL=-1      split contractions: one lane per (slice, output entry) also when there are few outputs
+//   ACRO_HIP_RED_WIDE=-1        sums over a long index with more than 128 outputs keep the generic schedule
 //   ACRO_HIP_RED_ROWS=-1        split contractions of few long rows: all outputs in every workgroup, NT / outputs lanes along a row
 //   ACRO_HIP_ONE_PASS=1         split contractions: the workgroup that finishes last adds the per-workgroup partials
 //                               instead of a second kernel (measured 18.4 against 16.3 us: the device-scope release

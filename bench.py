@@ -192,6 +192,7 @@ KERNEL_SHAPES = [
     ("A_i_j = B_j_i", [(1 << 22, 16)], (16, 1 << 22)),
     ("S_i = A_n_i", [(1 << 20, 64)], (64,)),
     ("S_i = A_i_n", [(64, 1 << 20)], (64,)),
+    ("S_i_j = A_e_i_j", [(1 << 17, 32, 32)], (32, 32)),
     ("A_i_j = B_j_i", [(8192, 8192)], (8192, 8192)),
     ("A_i_j = B_e_i C_e_j", [(1 << 21, 32), (1 << 21, 32)], (32, 32)),
     ("A_i_j = B_e_i C_e_j", [(1 << 20, 64), (1 << 20, 64)], (64, 64)),

@@ -307,6 +307,19 @@ def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE):
     assert "operands staged in LDS" in src and "ihi" not in src
 
 
+def test_sums_over_a_long_index_take_the_reduction_schedule_whatever_the_number_of_outputs(TE):
+    # a lane per output and workgroup, the summed range dealt out over the workgroups; a finishing workgroup per 256 outputs
+    src = TE.GetImplementation("S_i_j = A_e_i_j", at.Tensor(32, 32), at.Tensor(32768, 32, 32))
+    assert "reduction schedule: 1024 output entries, contraction of 32768 terms split over 256 workgroups x 1 slices (256 outputs per workgroup, a lane each)" in src
+    assert "for (long c = gc; c < 32768; c += 256)" in src and "const int o = blockIdx.x * 256 + threadIdx.x;" in src
+    # up to 256 outputs every workgroup has them all; with the summed index fastest a workgroup takes four rows (up to 1 024)
+    assert "output entries on adjacent lanes" in TE.GetImplementation("S_i = A_e_i", at.Tensor(200), at.Tensor(50000, 200))
+    assert "four outputs per workgroup" in TE.GetImplementation("S_i = A_i_e", at.Tensor(1000), at.Tensor(1000, 50000))
+    assert "reduction schedule" not in TE.GetImplementation("S_i = A_i_e", at.Tensor(1025), at.Tensor(1025, 50000))
+    # short sums are not reductions
+    assert "reduction schedule" not in TE.GetImplementation("S_i = A_e_i", at.Tensor(5000), at.Tensor(2000, 5000))
+
+
 def scatter_then_mass_apply_source(TE, transient_x):
     wl = workloads.config4(E=27)
     tensors = workloads.bind_to_engine(wl, at, transient=True)

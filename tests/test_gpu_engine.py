@@ -993,6 +993,27 @@ def test_many_outputs_summed_over_the_batch(at, engine, checker, kernel, shapes)
 
 
 @pytest.mark.parametrize("kernel,shapes,expect", [
+    ("S_i_j = A_e_i_j", [(3001, 32, 32)], "256 outputs per workgroup, a lane each"),            # the sum of element matrices
+    ("S_i -= A_e_i B_e", [(2500, 5000), (2500,)], "256 outputs per workgroup, a lane each"),
+    ("S_j_i += A_e_f_i_j B_e_f", [(700, 3, 9, 33), (700, 3)], "256 outputs per workgroup, a lane each"),   # 297 outputs, transposed, two summed indices
+    ("S_i_j = A_e_i_j", [(4001, 12, 12)], "output entries on adjacent lanes"),                  # up to 256: every workgroup has them all
+    ("S_i += A_i_e B_e", [(300, 5003), (5003,)], "four outputs per workgroup"),                  # summed index fastest: by rows
+])
+def test_sums_over_a_long_index_with_many_outputs(at, engine, checker, kernel, shapes, expect):
+    rng = np.random.default_rng(shapes[0][0])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    src = engine.GetLastImplementation()
+    assert "reduction schedule" in src and expect in src
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= 4 * TOL            # sums of thousands of terms in another order than the oracle's
+    again, _ = run_single(at, engine, checker, kernel, out0, *ins)
+    assert np.array_equal(got, again)                   # fixed order of additions: reproducible
+
+
+@pytest.mark.parametrize("kernel,shapes,expect", [
     ("A_i_e = B_i_e C_i_e", [(16, 5000), (16, 5000)], "lanes(i)=16"),
     ("A_i_j_e -= B_i_k_e C_k_j_e", [(3, 3, 4099), (3, 3, 4099)], "lanes()=1 tile(i,j)=9"),          # ragged last workgroup
     ("A_i_e += B_i_k C_k_e W_e", [(5, 7), (7, 6001), (6001,)], "entry fastest"),
