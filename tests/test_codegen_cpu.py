@@ -195,8 +195,9 @@ def test_streaming_kernels_with_light_workgroups_take_more_entries(TE, monkeypat
     outer = lambda: TE.GetImplementation("A_e_i_j = B_e_i C_e_j", at.Tensor(E, 8, 8), at.Tensor(E, 8), at.Tensor(E, 8))
     assert "16 per workgroup of 256 lanes" in outer() and "w0 < 1024; w0 += 256" in outer()
     assert "32 per workgroup of 256 lanes" in TE.GetImplementation("A_e_i = B_e_i", at.Tensor(E, 16), at.Tensor(E, 16))
-    # 3 KB per workgroup and more stay as they are (the old value of += counts)
+    # 3 KB per workgroup and more stay as they are (the old value of += counts), unless an item has four factors or more
     assert "8 per workgroup of 128 lanes" in TE.GetImplementation("A_e_i += B_e_i", at.Tensor(E, 16), at.Tensor(E, 16))
+    assert "16 per workgroup of 256 lanes" in TE.GetImplementation("A_e_i = B_e_i C_e_i D_i F_e", at.Tensor(E, 32), at.Tensor(E, 32), at.Tensor(E, 32), at.Tensor(32), at.Tensor(E))
     assert "8 per workgroup of 128 lanes" in TE.GetImplementation("A_e_i = B_e_i C_e_i D_e_i", *[at.Tensor(E, 16)] * 4)
     # few entries: never more than there are
     assert "batch index e extent 9, 8 per workgroup" in TE.GetImplementation("A_e_i_j = B_e_i C_e_j", at.Tensor(9, 8, 8), at.Tensor(9, 8), at.Tensor(9, 8))
