@@ -2,6 +2,7 @@
 // Semantics follow the reference's kernel/TensorKernel.cpp:26-403, kernel/DimensionedKernel.cpp:12-265 and
 // kernel/DimensionedMultiKernel.cpp:25-390; the implementation is a cursor-based scanner plus small index-set
 // helpers.
+#include <limits>
 #include <algorithm>
 #include <cctype>
 #include <set>
@@ -78,8 +79,11 @@ std::string scanEqOperator(Cursor &cur)
 
 std::vector<int> rowMajorStrides(const std::vector<int> &dims)
 {
+    // (the interface has them as int, like the reference's: in a loop space of 2^31 points and more the outer strides
+    // saturate instead of overflowing; the generator works with 64-bit strides of its own)
     std::vector<int> strides(dims.size(), 1);
-    for (int d = static_cast<int>(dims.size()) - 2; d >= 0; --d) strides[d] = strides[d + 1] * dims[d + 1];
+    for (int d = static_cast<int>(dims.size()) - 2; d >= 0; --d)
+        strides[d] = static_cast<int>(std::min<long>(std::numeric_limits<int>::max(), static_cast<long>(strides[d + 1]) * dims[d + 1]));
     return strides;
 }
 
