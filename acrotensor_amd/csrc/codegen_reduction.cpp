@@ -22,6 +22,9 @@ auto Generator::ReductionServes(const Sub &s) const -> bool
         if (r.size > big->size) big = &r;
     }
     if (big->idx.empty()) return false;
+    // a sum that streams the big operand, every value of which goes into one or two terms; a nest of contractions over
+    // small operands ("Y_e_i = A_e_i_j_k B_j_l C_l_m D_m_i") is for the reordering to take apart instead
+    if (static_cast<double>(outputs) * static_cast<double>(s.contrCount) > 2.0 * static_cast<double>(big->size)) return false;
     return has(s.outIdx, big->idx.back()) ? outputs <= 65536 : outputs <= 1024;
 }
 
