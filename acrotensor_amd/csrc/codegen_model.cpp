@@ -427,11 +427,37 @@ auto Generator::StageReusedOperands(int ki, const Sub &asWritten, std::vector<Su
         res.ext = r.ext;
         res.stride = r.stride;
         res.size = r.size;
+        // The factor that carries the last output index with a contracted index as its fastest dimension ("A_e_i_j =
+        // B_e_i_k C_e_j_k": C): neighbouring lanes would read its copy a row apart.  The copy is laid out with the
+        // contracted indices in front instead, so that they read neighbouring values as they do for "C_e_k_j"
+        // (12 x 12: 82 -> 87 % of the HBM peak, 24 x 24 72 -> 82 %, 40 x 40 46 -> 58 %); the lanes of the copying step still follow the operand in memory.
+        if (envInt("ACRO_HIP_STAGE_TRANSPOSED") >= 0 && !orig.outIdx.empty() && has(r.idx, orig.outIdx.back()) && has(orig.contr, r.idx.back()) &&
+            r.idx[0] == batch)
+        {
+            std::vector<size_t> order(1, 0);
+            for (size_t d = 1; d < r.idx.size(); ++d)
+            {
+                if (has(orig.contr, r.idx[d])) order.push_back(d);
+            }
+            for (size_t d = 1; d < r.idx.size(); ++d)
+            {
+                if (!has(orig.contr, r.idx[d])) order.push_back(d);
+            }
+            res.idx.clear();
+            res.ext.clear();
+            for (size_t d : order)
+            {
+                res.idx.push_back(r.idx[d]);
+                res.ext.push_back(r.ext[d]);
+            }
+            res.stride.assign(order.size(), 1);
+            for (size_t d = order.size() - 1; d-- > 0;) res.stride[d] = res.stride[d + 1] * res.ext[d + 1];
+        }
         uvars.push_back(info);
         Sub copy;
         copy.op = '=';
         copy.out = res;
-        copy.outIdx = res.idx;
+        copy.outIdx = r.idx;
         copy.in.assign(1, r);
         copy.contrCount = 1;
         copy.flatItems = true;

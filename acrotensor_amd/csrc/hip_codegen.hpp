@@ -88,6 +88,7 @@
 //                               counted loops around a register tile, see ChooseLoopTile)
 //   ACRO_HIP_STAGE_ENTRIES=-1   products of element matrices read their operands from device memory (no copies to LDS tiles first)
 //   ACRO_HIP_STAGE_ENTRIES=2    ... are staged, but their output indices are not split into blocks (one output or one row per lane)
+//   ACRO_HIP_STAGE_TRANSPOSED=-1 ... and the copy of a factor whose fastest dimension is contracted keeps the operand's layout
 //   ACRO_HIP_SPLIT_FIVE=-1      ... and extents divisible by five only are not split in five
 //   ACRO_HIP_STAGE_MOST=<n>     ... at most n staged values per entry (default 8000; 2048: matrices up to 32 x 32 only)
 //   ACRO_HIP_STAGE=-1           small invariant operands with lane-dependent addresses stay in device memory (not staged in LDS)

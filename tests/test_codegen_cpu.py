@@ -302,6 +302,9 @@ def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE):
     assert "operands staged in LDS" in src and "LDS 61504 bytes" in src
     src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 64, 64), at.Tensor(4096, 64, 64), at.Tensor(4096, 64, 64))
     assert "operands staged in LDS" not in src
+    # second factor transposed: its copy in LDS has the contracted index in front, the copying lanes follow the operand
+    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_k_j", at.Tensor(4096, 24, 24), at.Tensor(4096, 24, 24), at.Tensor(4096, 24, 24))
+    assert "_S2_e_j_khi_klo = C_e_khi_klo_j : lanes(khi,klo,j)=576" in src
     # slices are not whole tensors: their indices stay as they are
     big = at.Tensor(2, 4096, 8, 8)
     src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 8, 8), at.SliceTensor(big, 1), at.Tensor(4096, 8, 8))
