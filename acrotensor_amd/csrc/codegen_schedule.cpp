@@ -1131,6 +1131,15 @@ auto Generator::ChooseBatching() -> void
                 lightWorkgroups = true;
             }
         }
+        // One entry of 129 - 256 items per workgroup, an item per lane ("A_e_i_j = B_e_i_j C_i_j" with 16 x 16, rows of
+        // 256): two entries in two passes (copy 71 -> 79 % of the HBM peak, with a shared factor 62 -> 74 %, product of
+        // two 66 -> 77 %; four entries 77 / 70 %).
+        else if (streaming && !shared && perEntry > 0.0 && perEntry < 8192.0 && NB == 1 && E >= 2 && maxLane > 128 && maxLane <= NT &&
+                 envInt("ACRO_HIP_LIGHT") < 2)
+        {
+            NB = 2;
+            lightWorkgroups = true;
+        }
     }
 
     // Products of tiny element matrices whose operands are copied to LDS first (3 x 3 to 7 x 7): some 500 outputs per
