@@ -201,6 +201,8 @@ def test_streaming_kernels_with_light_workgroups_take_more_entries(TE, monkeypat
     assert "8 per workgroup of 128 lanes" in TE.GetImplementation("A_e_i = B_e_i C_e_i D_e_i", *[at.Tensor(E, 16)] * 4)
     # one entry of 256 items per workgroup, an item per lane: two entries in two passes
     assert "2 per workgroup of 256 lanes" in TE.GetImplementation("A_e_i_j = B_e_i_j C_i_j", at.Tensor(E, 16, 16), at.Tensor(E, 16, 16), at.Tensor(16, 16))
+    # 512 pointwise items per entry: two passes of 256 lanes
+    assert "1 per workgroup of 256 lanes" in TE.GetImplementation("A_e_i_j = B_e_i_j C_i_j", at.Tensor(E, 16, 32), at.Tensor(E, 16, 32), at.Tensor(16, 32))
     # few entries: never more than there are
     assert "batch index e extent 9, 8 per workgroup" in TE.GetImplementation("A_e_i_j = B_e_i C_e_j", at.Tensor(9, 8, 8), at.Tensor(9, 8), at.Tensor(9, 8))
     monkeypatch.setenv("ACRO_HIP_LIGHT", "-1")     # (other sizes: the engine keeps what it generated for the sizes above)
