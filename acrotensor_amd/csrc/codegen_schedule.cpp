@@ -789,7 +789,7 @@ auto Generator::ChooseCopyOutTile() -> void
     if (run < 8 && envInt("ACRO_HIP_COPY_OUT_TILE") < 2)
     {
         const int entries = static_cast<int>(std::max<long>(1, 64 / std::max<long>(1, s.laneCount)));
-        scattered = s.laneCount >= 2 && WaveStoreLineCoverage(k, entries) < 0.3;
+        scattered = s.laneCount >= 2 && WaveStoreLineCoverage(k, entries) < 0.01 * envInt("ACRO_HIP_COPY_OUT_COVERAGE", 30);
     }
     if (subs.size() != 1 && !scattered) return;
     if (run < 8 && !scattered) return;

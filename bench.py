@@ -87,6 +87,21 @@ def time_steps(at, workloads, wl, engine, tensors, steps, warmup):
     return wall, ev.ms * 1e-3
 
 
+def time_steps_rotating(at, workloads, wl, engine, sets, steps, warmup):
+    """`steps` launches issued round-robin over the buffer sets."""
+    n = len(sets)
+    for i in range(max(n, warmup)):
+        workloads.launch(wl, engine, sets[i % n])
+    at.synchronize()
+    t0 = time.perf_counter()
+    with at.hip_event_timer() as ev:
+        for i in range(steps):
+            workloads.launch(wl, engine, sets[i % n])
+    at.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, ev.ms * 1e-3
+
+
 def host_checker():
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle  # tests/oracle.py - checker access, used here only for the reported CPU baselines
@@ -151,6 +166,28 @@ def cpu_baseline_for(name, workloads):
 
 FP64_PEAK_GFLOPS = 78600.0
 
+_MEMO = {}
+
+
+def memo(fn, *args):
+    """Host arrays and workloads are generated once and shared by the buffer sets of a rotated measurement (they are
+    only ever copied from)."""
+    key = (fn.__name__,) + args
+    if key not in _MEMO:
+        _MEMO[key] = fn(*args)
+    return _MEMO[key]
+
+
+def sets_beyond_the_last_level_cache(abytes, requested=0):
+    """Number of buffer sets to rotate over so that a set's data cannot survive in the 256 MB memory-side cache
+    between two launches on it: together the sets exceed 1 GiB; a launch that moves 2 GiB or more needs no second
+    set.  `requested` > 0 overrides."""
+    if requested > 0:
+        return requested
+    if abytes >= (2 << 30):
+        return 1
+    return min(32, (1 << 30) // abytes + 1)
+
 
 # Single kernels a user of the reference's API writes, at large batch sizes: (kernel, input shapes, output shape).
 KERNEL_SHAPES = [
@@ -207,18 +244,25 @@ KERNEL_SHAPES = [
 
 def kernel_shapes(at, args):
     """One line for the whole list: per kernel the launch time by HIP events and algorithmic bytes / time against the
-    HBM peak; `value` is the geometric mean of those fractions."""
+    HBM peak, re-launched on one set of tensors (`frac`) and round-robin over enough sets to exceed 1 GiB
+    (`frac_cold`); `value` is the geometric mean of the cold fractions."""
     import math
     import numpy as np
+    t_start = time.perf_counter()
     engine = at.TensorEngine("HIP")
     steps = min(args.steps, 20)
     results = []
     for kernel, in_shapes, out_shape in KERNEL_SHAPES:
-        tensors = [at.Tensor(*s) for s in in_shapes] + [at.Tensor(*out_shape)]
-        for t in tensors:
-            t.SwitchToGPU()
-            t.Set(0.5)
-        step = lambda: engine(kernel, tensors[-1], *tensors[:-1])
+        abytes = sum(int(np.prod(s)) * 8 for s in in_shapes) + int(np.prod(out_shape)) * 8 * (2 if "+=" in kernel else 1)
+        n_sets = sets_beyond_the_last_level_cache(abytes, args.rotate)
+        sets = []
+        for _ in range(n_sets):
+            tensors = [at.Tensor(*s) for s in in_shapes] + [at.Tensor(*out_shape)]
+            for t in tensors:
+                t.SwitchToGPU()
+                t.Set(0.5)
+            sets.append(tensors)
+        step = lambda i=0: engine(kernel, sets[i][-1], *sets[i][:-1])
         for _ in range(5):
             step()
         at.synchronize()
@@ -226,28 +270,101 @@ def kernel_shapes(at, args):
             for _ in range(steps):
                 step()
         launch_s = ev.ms * 1e-3 / steps
-        abytes = sum(int(np.prod(s)) * 8 for s in in_shapes) + int(np.prod(out_shape)) * 8 * (2 if "+=" in kernel else 1)
+        rounds = max(2, -(-steps // n_sets))
+        for i in range(n_sets):
+            step(i)
+        at.synchronize()
+        with at.hip_event_timer() as ev:
+            for _ in range(rounds):
+                for i in range(n_sets):
+                    step(i)
+        cold_s = ev.ms * 1e-3 / (rounds * n_sets)
         results.append({"kernel": kernel, "inputs": [list(s) for s in in_shapes], "launch_us": launch_s * 1e6,
                         "algorithmic_bytes": abytes, "frac": abytes / launch_s * 1e-9 / HBM_PEAK_GBS,
+                        "buffer_sets": n_sets, "launch_us_cold": cold_s * 1e6,
+                        "frac_cold": abytes / cold_s * 1e-9 / HBM_PEAK_GBS,
                         "schedule": engine.GetLastImplementation().splitlines()[1][3:]})
-        del tensors
+        del sets, tensors
     mean = math.exp(sum(math.log(r["frac"]) for r in results) / len(results))
-    total_s = sum(r["launch_us"] for r in results) * 1e-6
+    mean_cold = math.exp(sum(math.log(r["frac_cold"]) for r in results) / len(results))
+    total_s = sum(r["launch_us_cold"] for r in results) * 1e-6
     return {
-        "metric": "fraction of the HBM peak, geometric mean over %d single-kernel shapes (1 GPU)" % len(results),
-        "value": mean, "unit": "fraction of 8 TB/s", "n_gpus": 1, "steps": steps, "warmup": 5,
+        "metric": "fraction of the HBM peak, geometric mean over %d single-kernel shapes, buffers rotated (1 GPU)" % len(results),
+        "value": mean_cold, "value_warm": mean, "unit": "fraction of 8 TB/s", "n_gpus": 1, "steps": steps, "warmup": 5,
         "ms_per_step": total_s * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
-        "data": "synthetic", "config": {"workload": "kernel shapes, one launch each per step"}, "kernels": results,
+        "data": "synthetic", "config": {"workload": "kernel shapes, one launch each per step"},
+        "seconds": time.perf_counter() - t_start, "kernels": results,
     }
 
 
-def build_case(at, workloads, name):
+def next_rows(at, workloads, args):
+    """The steps either side of the operator apply at the size of the headline mesh: node vector <-> element vector,
+    geometric-factor setup from the Jacobians, and scatter + apply in one launch; each with its launch time by HIP
+    events on one buffer set and rotated, the kernel it ran, and the compiled reference on one host core."""
+    import numpy as np
+    block = {}
+    for name in ("scatter", "sumgather", "jdsetup", "scatter_apply"):
+        engine, steps_list, label, units, unit_name, abytes, flops = build_sets(at, workloads, name, args.rotate)
+        wall, launch_s, roofline = measure_case(at, engine, steps_list, abytes, flops, 100, 10, args.settle_seconds,
+                                                PRECOMPILED.get(name))
+        block[name] = {
+            "workload": label, "launch_us": launch_s * 1e6, "algorithmic_bytes": abytes, "frac": roofline["frac"],
+            "buffer_sets": roofline["buffer_sets"], "launch_us_cold": roofline["launch_us_cold"],
+            "frac_cold": roofline["frac_cold"], "value_cold": units / (roofline["launch_us_cold"] * 1e-6) * 1e-9,
+            "unit": unit_name, "kernel": roofline["kernel"], "kernel_source_sha1_16": roofline["kernel_source_sha1_16"],
+        }
+        del engine, steps_list
+        if args.no_cpu_baseline:
+            continue
+        checker, kind = host_checker()
+        dofs, nodes = memo(workloads.hex_mesh_dof_map, 64, 64, 64, 3)
+        if name in ("scatter", "sumgather"):
+            L = memo(workloads.counter_uniform, 0xAC26, 0, (nodes,), -1.0, 1.0)
+            Ev = memo(workloads.counter_uniform, 0xAC26, 1, (dofs.size,), -1.0, 1.0)
+            flat = dofs.ravel()
+            passes = 3
+            t0 = time.perf_counter()
+            for _ in range(passes):
+                if name == "scatter":
+                    checker.scatter(L, flat)
+                else:
+                    checker.sum_gather(Ev, flat, nodes)
+            dt = (time.perf_counter() - t0) / passes
+            value, sample = dofs.size / dt * 1e-9, "whole mesh, mean of %d passes of %.3f s" % (passes, dt)
+        elif name == "jdsetup":
+            n, Q = 2048, 10
+            J = 0.1 * memo(workloads.counter_uniform, 0xAC28, 2, (n, Q, Q, Q, 3, 3), -1.0, 1.0) + np.eye(3)
+            W = memo(workloads.counter_uniform, 0xAC28, 0, (Q, Q, Q), 0.1, 1.0)
+            C = memo(workloads.counter_uniform, 0xAC28, 1, (n, Q, Q, Q), 0.5, 1.5)
+            D = np.zeros((n, 3, 3, Q, Q, Q))
+            t0 = time.perf_counter()
+            Jinv, Jdet = checker.batch_matrix_inv_det(J)
+            checker.contract("D_e_m_n_k1_k2_k3 = W_k1_k2_k3 C_e_k1_k2_k3 Jdet_e_k1_k2_k3 Jinv_e_k1_k2_k3_n_j Jinv_e_k1_k2_k3_m_j",
+                             D, W, C, Jdet, Jinv, Jinv)
+            dt = time.perf_counter() - t0
+            value, sample = n * Q ** 3 / dt * 1e-9, "%d of 16384 elements, inverse + determinant + contraction, one pass, %.1f s" % (n, dt)
+        else:
+            n = 65536
+            wl = workloads.config4(E=n)
+            L = memo(workloads.counter_uniform, 0xAC29, 0, (nodes,), -1.0, 1.0)
+            t0 = time.perf_counter()
+            wl.arrays["X"] = checker.scatter(L, dofs[:n].ravel()).reshape(n, 4, 4, 4)
+            workloads.run_on_checker(wl, checker)
+            dt = time.perf_counter() - t0
+            value, sample = wl.dof / dt * 1e-9, "%d of 262144 elements, scatter + 7-kernel chain, one pass, %.1f s" % (n, dt)
+        block[name]["cpu_baseline"] = {"value": value, "unit": unit_name, "cores": 1, "kind": kind, "sample": sample}
+    return block
+
+
+def build_case(at, workloads, name, engine=None):
     """Tensors on the device and a step function for one workload: cfg1 / cfg2 / cfg3 / cfg5 at the sizes of the
     baseline configurations, FlatIndexedScatter / FlatIndexedSumGather on the headline mesh, and the other pipelines.
+    Every call allocates a buffer set of its own (same values); calls that pass the same engine share its kernels.
     Returns (engine, step, label, units per step, unit name, algorithmic bytes, flops as written)."""
-    engine = at.TensorEngine("HIP")
+    if engine is None:
+        engine = at.TensorEngine("HIP")
     if name == "cfg2":
-        J = workloads.config2_inputs()
+        J = memo(workloads.config2_inputs)
         E, Q = J.shape[:2]
         tJ, Jinv, Jdet = at.Tensor(*J.shape), at.Tensor(*J.shape), at.Tensor(E, Q)
         tJ.data[...] = J
@@ -263,10 +380,10 @@ def build_case(at, workloads, name):
         E, Q = 16384, 10
         W, C, Jdet = at.Tensor(Q, Q, Q), at.Tensor(E, Q, Q, Q), at.Tensor(E, Q, Q, Q)
         Jinv, D = at.Tensor(E, Q, Q, Q, 3, 3), at.Tensor(E, 3, 3, Q, Q, Q)
-        W.data[...] = workloads.counter_uniform(0xAC27, 0, (Q, Q, Q), 0.1, 1.0)
-        C.data[...] = workloads.counter_uniform(0xAC27, 1, (E, Q, Q, Q), 0.5, 1.5)
-        Jdet.data[...] = workloads.counter_uniform(0xAC27, 2, (E, Q, Q, Q), 0.5, 1.5)
-        Jinv.data[...] = workloads.counter_uniform(0xAC27, 3, (E, Q, Q, Q, 3, 3), -1.0, 1.0)
+        W.data[...] = memo(workloads.counter_uniform, 0xAC27, 0, (Q, Q, Q), 0.1, 1.0)
+        C.data[...] = memo(workloads.counter_uniform, 0xAC27, 1, (E, Q, Q, Q), 0.5, 1.5)
+        Jdet.data[...] = memo(workloads.counter_uniform, 0xAC27, 2, (E, Q, Q, Q), 0.5, 1.5)
+        Jinv.data[...] = memo(workloads.counter_uniform, 0xAC27, 3, (E, Q, Q, Q, 3, 3), -1.0, 1.0)
         for t in (W, C, Jdet, Jinv, D):
             t.MoveToGPU()
         k = "D_e_m_n_k1_k2_k3 = W_k1_k2_k3 C_e_k1_k2_k3 Jdet_e_k1_k2_k3 Jinv_e_k1_k2_k3_n_j Jinv_e_k1_k2_k3_m_j"
@@ -281,9 +398,9 @@ def build_case(at, workloads, name):
         E, Q = 16384, 10
         W, C, J = at.Tensor(Q, Q, Q), at.Tensor(E, Q, Q, Q), at.Tensor(E, Q, Q, Q, 3, 3)
         Jinv, Jdet, D = at.Tensor(E, Q, Q, Q, 3, 3), at.Tensor(E, Q, Q, Q), at.Tensor(E, 3, 3, Q, Q, Q)
-        W.data[...] = workloads.counter_uniform(0xAC28, 0, (Q, Q, Q), 0.1, 1.0)
-        C.data[...] = workloads.counter_uniform(0xAC28, 1, (E, Q, Q, Q), 0.5, 1.5)
-        J.data[...] = workloads.counter_uniform(0xAC28, 2, (E, Q, Q, Q, 3, 3), -0.1, 0.1)
+        W.data[...] = memo(workloads.counter_uniform, 0xAC28, 0, (Q, Q, Q), 0.1, 1.0)
+        C.data[...] = memo(workloads.counter_uniform, 0xAC28, 1, (E, Q, Q, Q), 0.5, 1.5)
+        J.data[...] = memo(workloads.counter_uniform, 0xAC28, 2, (E, Q, Q, Q, 3, 3), -0.1, 0.1)
         J.data[...] += [[1.0, 0.0, 0.0], [0.0, 1.0, 0.0], [0.0, 0.0, 1.0]]
         for t in (Jinv, Jdet):
             t.SetTransient(True)
@@ -306,13 +423,13 @@ def build_case(at, workloads, name):
         # through the element-to-node map and the element vector never exists; scatter_then_apply runs the two steps
         # one after the other.
         import numpy as np
-        wl = workloads.config4(E=262144)
+        wl = memo(workloads.config4, 262144)
         tensors = workloads.bind_to_engine(wl, at, transient=True)
-        dofs, nodes = workloads.hex_mesh_dof_map(64, 64, 64, 3)
+        dofs, nodes = memo(workloads.hex_mesh_dof_map, 64, 64, 64, 3)
         M = at.IndexMapping(nodes, dofs.size)
         M.map[:] = dofs.ravel()
         L = at.Tensor(nodes)
-        L.data[...] = workloads.counter_uniform(0xAC29, 0, (nodes,), -1.0, 1.0)
+        L.data[...] = memo(workloads.counter_uniform, 0xAC29, 0, (nodes,), -1.0, 1.0)
         tensors["X"].SetTransient(name == "scatter_apply")
         for t in list(tensors.values()) + [L]:
             t.MoveToGPU()
@@ -341,8 +458,8 @@ def build_case(at, workloads, name):
         # one dense 64 x 64 operator applied to 2^18 vectors: the one GEMM-shaped kernel of this engine (FP64 matrix cores)
         E, n = 1 << 18, 64
         B, X, A = at.Tensor(n, n), at.Tensor(E, n), at.Tensor(E, n)
-        B.data[...] = workloads.counter_uniform(0xAC28, 0, (n, n), -1.0, 1.0)
-        X.data[...] = workloads.counter_uniform(0xAC28, 1, (E, n), -1.0, 1.0)
+        B.data[...] = memo(workloads.counter_uniform, 0xAC28, 0, (n, n), -1.0, 1.0)
+        X.data[...] = memo(workloads.counter_uniform, 0xAC28, 1, (E, n), -1.0, 1.0)
         for t in (B, X, A):
             t.MoveToGPU()
         step = lambda: engine("A_e_i = B_i_j X_e_j", A, B, X)
@@ -354,9 +471,9 @@ def build_case(at, workloads, name):
         # 64 points, both products in one matrix-core kernel, the intermediate transient
         E, nd, nq = 1 << 19, 27, 64
         B, X, D, U, Y = at.Tensor(nq, nd), at.Tensor(E, nd), at.Tensor(E, nq), at.Tensor(E, nq), at.Tensor(E, nd)
-        B.data[...] = workloads.counter_uniform(0xAC29, 0, (nq, nd), -1.0, 1.0)
-        X.data[...] = workloads.counter_uniform(0xAC29, 1, (E, nd), -1.0, 1.0)
-        D.data[...] = workloads.counter_uniform(0xAC29, 2, (E, nq), 0.5, 1.5)
+        B.data[...] = memo(workloads.counter_uniform, 0xAC29, 0, (nq, nd), -1.0, 1.0)
+        X.data[...] = memo(workloads.counter_uniform, 0xAC29, 1, (E, nd), -1.0, 1.0)
+        D.data[...] = memo(workloads.counter_uniform, 0xAC29, 2, (E, nq), 0.5, 1.5)
         U.SetTransient(True)
         for t in (B, X, D, U, Y):
             t.MoveToGPU()
@@ -378,8 +495,8 @@ def build_case(at, workloads, name):
         S, D = at.Tensor(E, 5, 5, 5, 5, 5, 5), at.Tensor(E, 5, 5, 5, 3, 3)
         tables = [at.Tensor(5, 5, 5, 3, 3) for _ in range(3)]
         for i, t in enumerate(tables):
-            t.data[...] = workloads.counter_uniform(0xAC2A, i, (5, 5, 5, 3, 3), -1.0, 1.0)
-        D.data[...] = workloads.counter_uniform(0xAC2A, 3, (E, 5, 5, 5, 3, 3), 0.5, 1.5)
+            t.data[...] = memo(workloads.counter_uniform, 0xAC2A, i, (5, 5, 5, 3, 3), -1.0, 1.0)
+        D.data[...] = memo(workloads.counter_uniform, 0xAC2A, 3, (E, 5, 5, 5, 3, 3), 0.5, 1.5)
         for t in tables + [S, D]:
             t.MoveToGPU()
         k = "S_e_i1_i2_i3_j1_j2_j3 = B1_i1_j1_k1_m_n B2_i2_j2_k2_m_n B3_i3_j3_k3_m_n D_e_k1_k2_k3_m_n"
@@ -391,12 +508,12 @@ def build_case(at, workloads, name):
     elif name in ("scatter", "sumgather"):
         # node vector <-> element vector of the headline mesh size: 64^3 hex elements of degree 3
         import numpy as np
-        dofs, nodes = workloads.hex_mesh_dof_map(64, 64, 64, 3)
+        dofs, nodes = memo(workloads.hex_mesh_dof_map, 64, 64, 64, 3)
         M = at.IndexMapping(nodes, dofs.size)
         M.map[:] = dofs.ravel()
         L, Ev = at.Tensor(nodes), at.Tensor(dofs.size)
-        L.data[...] = workloads.counter_uniform(0xAC26, 0, (nodes,), -1.0, 1.0)
-        Ev.data[...] = workloads.counter_uniform(0xAC26, 1, (dofs.size,), -1.0, 1.0)
+        L.data[...] = memo(workloads.counter_uniform, 0xAC26, 0, (nodes,), -1.0, 1.0)
+        Ev.data[...] = memo(workloads.counter_uniform, 0xAC26, 1, (dofs.size,), -1.0, 1.0)
         for t in (L, Ev):
             t.MoveToGPU()
         if name == "scatter":
@@ -412,7 +529,7 @@ def build_case(at, workloads, name):
         # inputs for 2048 elements, repeated 32 times along the element index on the device (generating and
         # uploading all 4.7 GB of geometric factors from the host takes minutes; no timing depends on the values)
         period, times = 2048, 32
-        small = workloads.config5(E=period)
+        small = memo(workloads.config5, period)
         tensors = workloads.bind_to_engine_repeated(small, at, engine, times, transient=True)
         wl = small
         step = lambda: workloads.launch(wl, engine, tensors)
@@ -421,7 +538,7 @@ def build_case(at, workloads, name):
         abytes, flops = small.algorithmic_bytes * times, small.flops * times
         units, unit_name = small.dof * times, "GDOF/s"
     else:
-        wl = {"cfg1": workloads.config1, "cfg3": workloads.config3}[name]()
+        wl = memo({"cfg1": workloads.config1, "cfg3": workloads.config3}[name])
         tensors = workloads.bind_to_engine(wl, at, transient=True, inputs_only=True)
         for t in tensors.values():
             t.MoveToGPU()
@@ -435,10 +552,29 @@ def build_case(at, workloads, name):
 PRECOMPILED = {"cfg2": "batchMatrixKernel<3,inv,det>", "scatter": "scatterKernel2", "sumgather": "sumGatherKernel"}
 
 
-def measure_case(at, engine, step, abytes, flops, steps, warmup, settle_seconds, precompiled=None):
+def build_sets(at, workloads, name, rotate=0):
+    """One buffer set to time re-launches on (the first) plus as many more as it takes to push a set out of the
+    memory-side cache between two launches on it.  Returns (engine, [step per set], label, units, unit name,
+    algorithmic bytes, flops)."""
+    engine, step, label, units, unit_name, abytes, flops = build_case(at, workloads, name)
+    steps = [step]
+    for _ in range(sets_beyond_the_last_level_cache(abytes, rotate) - 1):
+        steps.append(build_case(at, workloads, name, engine)[1])
+    return engine, steps, label, units, unit_name, abytes, flops
+
+
+def measure_case(at, engine, steps_list, abytes, flops, steps, warmup, settle_seconds, precompiled=None):
+    """Times one workload twice with HIP events: re-launched on one buffer set (`launch_us`, `frac`: whatever of the
+    set fits the 256 MB memory-side cache is served from there), and launched round-robin over all the sets
+    (`launch_us_cold`, `frac_cold`: every byte comes from and goes to HBM).  With one set the two are the same
+    measurement."""
+    if callable(steps_list):
+        steps_list = [steps_list]
+    step = steps_list[0]
     # sustained load before anything is timed (see settle_clocks): bursts of launches, not one launch per
     # synchronisation, or the device drops back to idle clocks between them
-    step()
+    for s in steps_list:
+        s()
     at.synchronize()
     t0 = time.perf_counter()
     step()
@@ -464,6 +600,22 @@ def measure_case(at, engine, step, abytes, flops, steps, warmup, settle_seconds,
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(engine, precompiled), "algorithmic_bytes": abytes,
                 "launch_us": launch_s * 1e6, "kernel": names[0] if names else None, "kernel_source_sha1_16": digest}
+    cold_s = launch_s
+    n = len(steps_list)
+    if n > 1:
+        rounds = max(2, -(-steps // n))
+        for _ in range(max(1, warmup // n)):
+            for s in steps_list:
+                s()
+        at.synchronize()
+        with at.hip_event_timer() as ev:
+            for _ in range(rounds):
+                for s in steps_list:
+                    s()
+        at.synchronize()
+        cold_s = ev.ms * 1e-3 / (rounds * n)
+    roofline.update({"buffer_sets": n, "launch_us_cold": cold_s * 1e6, "achieved_cold": abytes / cold_s * 1e-9,
+                     "frac_cold": abytes / cold_s * 1e-9 / HBM_PEAK_GBS})
     return wall, launch_s, roofline
 
 
@@ -472,20 +624,40 @@ def all_configs(at, workloads, args):
     baseline beside each."""
     block = {}
     for name in ("cfg1", "cfg2", "cfg3", "cfg5"):
-        engine, step, label, units, unit_name, abytes, flops = build_case(at, workloads, name)
+        engine, steps_list, label, units, unit_name, abytes, flops = build_sets(at, workloads, name, args.rotate)
         steps = 50 if name == "cfg5" else 200
-        wall, launch_s, roofline = measure_case(at, engine, step, abytes, flops, steps, 10, args.settle_seconds,
+        wall, launch_s, roofline = measure_case(at, engine, steps_list, abytes, flops, steps, 10, args.settle_seconds,
                                                 PRECOMPILED.get(name))
         block[name] = {
             "workload": label, "launch_us": launch_s * 1e6, "steps": steps, "algorithmic_bytes": abytes,
             "GBps": roofline["achieved"], "frac": roofline["frac"], "gflops_as_written": flops / launch_s * 1e-9,
-            "value": units / launch_s * 1e-9, "unit": unit_name, "traffic": roofline["traffic"],
+            "value": units / launch_s * 1e-9, "unit": unit_name, "buffer_sets": roofline["buffer_sets"],
+            "launch_us_cold": roofline["launch_us_cold"], "GBps_cold": roofline["achieved_cold"],
+            "frac_cold": roofline["frac_cold"], "traffic": roofline["traffic"],
             "kernel": roofline["kernel"], "kernel_source_sha1_16": roofline["kernel_source_sha1_16"],
         }
-        del engine, step
+        if name == "cfg1":
+            block[name]["graph_replay_us"] = graph_replay_us(at, steps_list[0], 500)
+        del engine, steps_list
         if not args.no_cpu_baseline:
             block[name]["cpu_baseline"] = cpu_baseline_for(name, workloads)
     return block
+
+
+def graph_replay_us(at, step, replays):
+    """The step recorded once as a launch sequence (hipGraph) and replayed: time per replay by HIP events."""
+    step()
+    at.synchronize()
+    with at.recorded_launches() as seq:
+        step()
+    for _ in range(50):
+        seq.launch()
+    at.synchronize()
+    with at.hip_event_timer() as ev:
+        for _ in range(replays):
+            seq.launch()
+    at.synchronize()
+    return ev.ms * 1e3 / replays
 
 
 def cfg1_sizes(at, args):
@@ -522,9 +694,9 @@ def cfg1_sizes(at, args):
 
 def other_workload(at, workloads, args):
     name = args.workload
-    engine, step, label, units, unit_name, abytes, flops = build_case(at, workloads, name)
+    engine, steps_list, label, units, unit_name, abytes, flops = build_sets(at, workloads, name, args.rotate)
     steps, warmup = min(args.steps, 200), min(args.warmup, 20)
-    wall, launch_s, roofline = measure_case(at, engine, step, abytes, flops, steps, warmup, args.settle_seconds,
+    wall, launch_s, roofline = measure_case(at, engine, steps_list, abytes, flops, steps, warmup, args.settle_seconds,
                                             PRECOMPILED.get(name))
     result = {
         "metric": "%s throughput (1 GPU)" % name, "value": units * steps / wall * 1e-9, "unit": unit_name, "n_gpus": 1,
@@ -548,12 +720,18 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--settle-seconds", type=float, default=0.25,
                     help="untimed launches before the warm-up, until clocks have settled under sustained load")
+    ap.add_argument("--rotate", type=int, default=0,
+                    help="buffer sets that the cold figures rotate over: 0 (default) as many as it takes to exceed 1 GiB "
+                         "together, 1 none (cold figures then repeat the ordinary ones), N that many")
     ap.add_argument("--elements", type=int, default=262144)
     ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store-all", action="store_true")
     ap.add_argument("--no-all-configs", action="store_true",
                     help="leave out the block with the other four baseline configurations")
+    ap.add_argument("--no-next-rows", action="store_true",
+                    help="leave out the block with scatter, sum-gather, geometric-factor setup and scatter + apply")
+    ap.add_argument("--no-shapes", action="store_true", help="leave out the summary of the single-kernel shapes")
     ap.add_argument("--workload", default="cfg4", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "scatter", "sumgather", "dsetup", "jdsetup", "scatter_apply", "scatter_then_apply", "operator", "dense_apply", "stiffness", "shapes", "cfg1_sizes"],
                     help="cfg4 (default) is the headline metric; the others print the same kind of line for the "
                          "remaining baseline configurations at their full sizes and for the node-vector <-> "
@@ -584,9 +762,17 @@ def main():
 
     wl = workloads.config4(E=args.elements)
     engine = at.TensorEngine("HIP")
-    tensors = workloads.bind_to_engine(wl, at, transient=True)
-    for t in tensors.values():
-        t.MoveToGPU()
+    n_sets = sets_beyond_the_last_level_cache(wl.algorithmic_bytes, args.rotate)
+    sets = []
+    for _ in range(n_sets):
+        bound = workloads.bind_to_engine(wl, at, transient=True, inputs_only=True)
+        for name, t in bound.items():
+            if name in wl.inputs:
+                t.MoveToGPU()
+            else:
+                t.SwitchToGPU()                              # written before it is read: device memory only
+        sets.append(bound)
+    tensors = sets[0]
 
     if args.calibration_copy:
         tensors["X"].Mult(1.0)
@@ -597,6 +783,11 @@ def main():
     ms_per_step = wall / args.steps * 1e3
     launch_s = dev / args.steps
     achieved = wl.algorithmic_bytes / launch_s * 1e-9
+    # the same steps round-robin over the buffer sets: no byte of a set survives in the memory-side cache until
+    # the set's next launch
+    wall_cold, dev_cold = time_steps_rotating(at, workloads, wl, engine, sets, args.steps, args.warmup)
+    cold_s = dev_cold / args.steps
+    achieved_cold = wl.algorithmic_bytes / cold_s * 1e-9
 
     result = {
         "metric": METRIC,
@@ -620,6 +811,8 @@ def main():
         },
         "pct_hbm_peak": 100.0 * achieved / HBM_PEAK_GBS,
         "kernel_gdof_per_s": wl.dof / launch_s * 1e-9,
+        "value_cold": wl.dof * args.steps / wall_cold * 1e-9,
+        "pct_hbm_peak_cold": 100.0 * achieved_cold / HBM_PEAK_GBS,
         "roofline": {
             "bound": "hbm",
             "achieved": achieved,
@@ -629,22 +822,32 @@ def main():
             "traffic": measured_traffic(engine),
             "algorithmic_bytes": wl.algorithmic_bytes,
             "launch_us": launch_s * 1e6,
+            "buffer_sets": n_sets,
+            "launch_us_cold": cold_s * 1e6,
+            "achieved_cold": achieved_cold,
+            "frac_cold": achieved_cold / HBM_PEAK_GBS,
+            "cold": "the same %d steps issued round-robin over %d sets of X, D and Y (distinct allocations, same "
+                    "values, %.2f GB together): nothing a launch touches is left in the 256 MB memory-side cache "
+                    "from the set's previous launch" % (args.steps, n_sets, n_sets * wl.algorithmic_bytes * 1e-9),
             "kernel": kernel_identity(engine)[0][0],
             "kernel_source_sha1_16": kernel_identity(engine)[1],
         },
     }
 
     if not args.no_store_all:
-        for name in wl.transient:
-            tensors[name].SetTransient(False)
+        for bound in sets:
+            for name in wl.transient:
+                bound[name].SetTransient(False)
         n2 = max(10, args.steps // 4)
         # The first launch compiles the other kernel while the device idles: settle again before timing.
         workloads.launch(wl, engine, tensors)
         at.synchronize()
         settle_clocks(at, workloads, wl, engine, tensors, args.settle_seconds)
         wall2, dev2 = time_steps(at, workloads, wl, engine, tensors, n2, max(5, args.warmup // 4))
+        wall2c, dev2c = time_steps_rotating(at, workloads, wl, engine, sets, n2, max(5, args.warmup // 4))
         stored_bytes = args.elements * (64 + 125 + 64 + 610) * 8
         moved = stored_bytes / (dev2 / n2) * 1e-9
+        moved_cold = stored_bytes / (dev2c / n2) * 1e-9
         result["store_all"] = {
             "what": "the same launch with T1..V2 as ordinary tensors: every intermediate is also written to HBM, "
                     "as with the reference (what a caller gets who only changes the policy string)",
@@ -654,19 +857,32 @@ def main():
             "hbm_bytes_moved": stored_bytes,
             "achieved_GBs_incl_intermediates": moved,
             "frac_of_hbm_peak_on_bytes_moved": moved / HBM_PEAK_GBS,
+            "launch_us_cold": dev2c / n2 * 1e6,
+            "frac_of_hbm_peak_on_bytes_moved_cold": moved_cold / HBM_PEAK_GBS,
             "traffic": measured_traffic(engine),
             "kernel": kernel_identity(engine)[0][0],
             "kernel_source_sha1_16": kernel_identity(engine)[1],
         }
-        for name in wl.transient:
-            tensors[name].SetTransient(True)
+        for bound in sets:
+            for name in wl.transient:
+                bound[name].SetTransient(True)
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(workloads, min(args.cpu_sample_elems, args.elements))
 
+    del tensors, sets, bound
     if not args.no_all_configs:
-        del tensors
         result["all_configs"] = all_configs(at, workloads, args)
+    if not args.no_next_rows:
+        result["next_rows"] = next_rows(at, workloads, args)
+    if not args.no_shapes:
+        full = kernel_shapes(at, args)
+        worst = min(full["kernels"], key=lambda r: r["frac_cold"])
+        result["shapes_summary"] = {
+            "what": "single kernels of other shapes (bench.py --workload shapes lists them): fraction of the HBM peak "
+                    "by HIP events, buffers rotated", "n": len(full["kernels"]), "geomean": full["value_warm"],
+            "geomean_cold": full["value"], "min_cold": worst["frac_cold"], "min_cold_kernel": worst["kernel"],
+            "min_cold_inputs": worst["inputs"], "seconds": full["seconds"]}
 
     print(json.dumps(result))
 
