@@ -310,7 +310,7 @@ auto Generator::StoreIsDead(int k) const -> bool
 auto Generator::StreamsOut(int k) const -> bool
 {
     if (envInt("ACRO_HIP_NT_STORE") < 0) return false;
-    if (static_cast<long>(ldsDoubles) * 8 > 20 * 1024) return false;
+    if (static_cast<long>(ldsDoubles) * 8 > 20 * 1024 && envInt("ACRO_HIP_NT_STORE") < 2) return false;
     const double coverage = WaveStoreLineCoverage(k);
     if (coverage < 0.45) return false;
     // Lines filled in part and a launch that writes more to device memory than it reads: ordinary stores (single-kernel

@@ -140,7 +140,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     // and load, so up to 512 workgroups and four loads in flight per lane (also swept: 256 - 8 192 workgroups,
     // unroll 1 - 8).
     const long G = (byRows || (wide && Go > 1)) ? std::min<long>(std::max<long>(1, 1024 / Go), std::max<long>(1, Nc / (Sn * 16)))
-                                                : std::min<long>(pencil ? 256 : 512, std::max<long>(1, Nc / (Sn * (pencil ? 4 : 16))));
+                                                : std::min<long>(pencil ? envInt("ACRO_HIP_RED_GROUPS", 256) : 512, std::max<long>(1, Nc / (Sn * (pencil ? 4 : 16))));
     // G counts the shares of the contraction range (rows of partials in the scratch buffer); the grid has one
     // workgroup per share and group of outputs.
     const long gridG = G * Go;
@@ -215,7 +215,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     {
         for (long o = 0; o < O; ++o) out << "    double acc" << o << " = 0.0;\n";
         out << "    {\n        const long g = " << gExpr << ";\n";
-        out << "#pragma unroll 1\n";
+        out << "#pragma unroll " << envInt("ACRO_HIP_RED_UNROLL", 1) << "\n";
         out << "        for (long c = g * " << Sn << " + lane; c < " << Nc << "; c += " << G * Sn << ")\n        {\n";
         decompose(s.contr, "c", "            ");
         // operand bases (contraction part of the address) and memoised loads (output part is a literal)

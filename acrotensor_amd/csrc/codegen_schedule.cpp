@@ -789,7 +789,9 @@ auto Generator::ChooseCopyOutTile() -> void
     if (run < 8 && envInt("ACRO_HIP_COPY_OUT_TILE") < 2)
     {
         const int entries = static_cast<int>(std::max<long>(1, 64 / std::max<long>(1, s.laneCount)));
-        scattered = s.laneCount >= 2 && WaveStoreLineCoverage(k, entries) < 0.01 * envInt("ACRO_HIP_COPY_OUT_COVERAGE", 30);
+        const double coverage = WaveStoreLineCoverage(k, entries);
+        scattered = s.laneCount >= 2 && (coverage < 0.01 * envInt("ACRO_HIP_COPY_OUT_COVERAGE", 30) ||
+                                         (coverage < 0.95 && envInt("ACRO_HIP_COPY_OUT_WRITERS") >= 0 && WritesDominate()));
     }
     if (subs.size() != 1 && !scattered) return;
     if (run < 8 && !scattered) return;
@@ -1294,7 +1296,7 @@ auto Generator::ChooseBatching() -> void
             // in 256 lanes -> 8 in 512: 336 -> 311 us; 8 in 256 lanes 332 us, 16 in 1 024 lanes 331 us).
             bool throughLds = false;
             for (int k = 0; k < K; ++k) throughLds = throughLds || CopiesOutFromLds(k);
-            if (throughLds && NB >= 2 && opt.force_nb <= 0 && envInt("ACRO_HIP_NB") <= 0 && 2L * NB <= E && envInt("ACRO_HIP_WRITE_BATCH") >= 0)
+            if (throughLds && NB >= envInt("ACRO_HIP_WRITE_BATCH_FROM", 1) && opt.force_nb <= 0 && envInt("ACRO_HIP_NB") <= 0 && 2L * NB <= E && envInt("ACRO_HIP_WRITE_BATCH") >= 0)
             {
                 const int wider = PlaceLds(2 * NB);
                 if (wider <= budgetDoubles / 2)

@@ -57,8 +57,11 @@ def test_mass_assembly_is_evaluated_as_a_chain_of_small_contractions(TE):
     src = TE.GetImplementation(k, tensors[out], *[tensors[n] for n in ins])
     # one index is summed per step; the two partial results are tensors of the generator's own that live in LDS
     assert src.count("contraction=4 unrolled") == 3 and "contraction=64" not in src
-    assert "_F1->lds\n" in src and "_F2->lds\n" in src and "_F2<-lds" in src and "M->global" in src
-    assert src.count("__syncthreads()") == 2
+    assert "_F1->lds\n" in src and "_F2->lds\n" in src and "_F2<-lds" in src
+    # a launch that writes far more than it reads and whose lanes would store pieces of 72 bytes: the result leaves
+    # through an LDS tile, whole lines per store instruction
+    assert "M->lds+global" in src and "// M: LDS tiles -> device memory" in src
+    assert src.count("__syncthreads()") == 3
     # kernel parameters are the user's tensors only: M, B, W
     signature = [l for l in src.splitlines() if "__global__" in l][0]
     assert signature.count("double *") == 3
