@@ -78,6 +78,7 @@ SIGNATURES = {
     "acro_engine_flat_indexed_scatter": (ctypes.c_int, [handle, handle, handle, handle]),
     "acro_engine_flat_indexed_sum_gather": (ctypes.c_int, [handle, handle, handle, handle]),
     "acro_hip_compile": (ctypes.c_int, [ctypes.c_char_p, ctypes.c_char_p, c_size_t_p]),
+    "acro_hip_compile_private_bytes": (ctypes.c_int, [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_char_p, ctypes.POINTER(ctypes.c_int)]),
     "acro_describe_kernels": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(ctypes.c_char_p), c_int_p, c_int_p,
                                              ctypes.c_char_p, ctypes.c_size_t, c_size_t_p]),
 }

@@ -58,6 +58,13 @@ void require(bool cond, const char *msg)
     if (!cond) throw_error(msg);
 }
 
+}  // namespace
+
+static void resolveNoAllocScratch();  // defined with the scratch array below
+
+namespace
+{
+
 void copyOut(const std::string &s, char *buf, size_t buflen, size_t *needed)
 {
     if (needed != nullptr) *needed = s.size() + 1;
@@ -394,6 +401,9 @@ int acro_engine_contract(acro_engine *e, const char *kernel, acro_tensor *out, a
         require(e != nullptr && kernel != nullptr && out != nullptr, "null argument");
         std::vector<Tensor *> in = unwrap(inputs, num_inputs);
         e->te(std::string(kernel), out->t, in);
+        // The call that must not allocate requires this one to have run first on the device; the address of its
+        // scratch array is looked up here, where loading code and allocating is allowed.
+        if (!e->te.InMultiKernelLaunch()) resolveNoAllocScratch();
     });
 }
 
@@ -409,26 +419,35 @@ static __device__ __align__(256) double scratch[ACRO_NO_ALLOC_SCRATCH_DOUBLES];
 
 namespace
 {
-// Device address of `scratch` on the current device, looked up once per device.  The array's name means nothing as
-// a pointer in host code; only this address is ever handed to kernels and fills.
+std::mutex scratchLock;
+std::map<int, double *> scratchByDevice;
+
+// Device address of `scratch` on the current device; null until resolveNoAllocScratch() has run there.  The array's
+// name means nothing as a pointer in host code; only this address is ever handed to kernels and fills.
 double *scratchOnCurrentDevice()
 {
-    static std::mutex lock;
-    static std::map<int, double *> known;
     int device = 0;
     ACRO_HIP_CHECK(hipGetDevice(&device));
-    std::lock_guard<std::mutex> guard(lock);
-    auto it = known.find(device);
-    if (it == known.end())
-    {
-        void *address = nullptr;
-        ACRO_HIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
-        require(address != nullptr, "the scratch array has no address on this device");
-        it = known.emplace(device, static_cast<double *>(address)).first;
-    }
-    return it->second;
+    std::lock_guard<std::mutex> guard(scratchLock);
+    auto it = scratchByDevice.find(device);
+    return it == scratchByDevice.end() ? nullptr : it->second;
 }
 }  // namespace
+
+// Looks the address up once per device.  The first look-up on a device may load this library's code object there
+// and allocate device memory for it and for the array, so it is done by the ordinary entry point, never by the
+// one that promises not to allocate.
+static void resolveNoAllocScratch()
+{
+    int device = 0;
+    ACRO_HIP_CHECK(hipGetDevice(&device));
+    std::lock_guard<std::mutex> guard(scratchLock);
+    if (scratchByDevice.count(device) != 0) return;
+    void *address = nullptr;
+    ACRO_HIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+    require(address != nullptr, "the scratch array has no address on this device");
+    scratchByDevice.emplace(device, static_cast<double *>(address));
+}
 
 extern "C" {
 
@@ -442,6 +461,8 @@ int acro_engine_contract_no_alloc(acro_engine *e, const char *kernel, acro_tenso
                 "acro_engine_contract_no_alloc cannot be used between BeginMultiKernelLaunch and EndMultiKernelLaunch");
         std::vector<Tensor *> in = unwrap(inputs, num_inputs);
         double *ptr = scratchOnCurrentDevice();
+        require(ptr != nullptr, "acro_engine_contract_no_alloc: nothing has run through acro_engine_contract on this device yet; "
+                                "run the same operation once through the ordinary entry point before");
         hip::NoAllocation scope(ptr, ACRO_NO_ALLOC_SCRATCH_DOUBLES);
         e->te(std::string(kernel), out->t, in);
     });
@@ -545,6 +566,16 @@ int acro_hip_compile(const char *module_name, const char *source, size_t *code_s
         require(module_name != nullptr && source != nullptr, "null argument");
         HipKernel kernel(module_name, source);
         if (code_size != nullptr) *code_size = kernel.GetCodeObjectSize();
+    });
+}
+
+int acro_hip_compile_private_bytes(const char *module_name, const char *source, const char *function, int *bytes)
+{
+    return guarded([&] {
+        require(module_name != nullptr && source != nullptr && function != nullptr && bytes != nullptr, "null argument");
+        HipKernel kernel(module_name, source);
+        *bytes = kernel.PrivateSegmentBytes(function);
+        require(*bytes >= 0, (std::string("the code object holds no kernel called ") + function).c_str());
     });
 }
 

@@ -64,7 +64,7 @@ auto Generator::OpKernel(int k) const -> const Sub &
 // `k`: the kernel of the group; `alone`: it is the whole group (inputs are then never written in the launch).
 auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bool
 {
-    if ((alone && NumOpKernels() != 1) || batch < 0 || !opt.noalias || NumGatherSlots() > 0 || envInt("ACRO_HIP_OPERATOR") < 0) return false;
+    if ((alone && NumOpKernels() != 1) || batch < 0 || !opt.noalias || NumGatherSlots() > 0 || envInt("ACRO_HIP_OPERATOR") < 0 || opt.no_matrix_cores) return false;
     const Sub &s = OpKernel(k);
     if (s.matrixOp != 0 || s.in.size() < 2 || s.contr.empty() || s.out.repeated) return false;
     // the operator: the one operand without the batch index that carries contracted and free indices;

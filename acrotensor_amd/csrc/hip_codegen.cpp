@@ -105,6 +105,26 @@ auto Generator::FirstOccurrence(int u) const -> std::pair<int, int>
 
 }  // namespace codegen
 
+namespace
+{
+
+// Every launch of a module that contains a matrix-core instruction is named for the spill check at compile time.
+HipKernelPlan withSpillGuard(HipKernelPlan plan)
+{
+    if (!plan.fusable || plan.source.find("__builtin_amdgcn_mfma") == std::string::npos) return plan;
+    for (const HipLaunch &launch : plan.launches)
+    {
+        bool known = false;
+        for (const std::string &name : plan.matrix_core_functions) known = known || name == launch.function_name;
+        if (!known) plan.matrix_core_functions.push_back(launch.function_name);
+    }
+    if (plan.source.find("#ifdef ACRO_KEEP_OPERATOR_IN_LDS") != std::string::npos)
+        plan.register_relief_macro = "ACRO_KEEP_OPERATOR_IN_LDS";
+    return plan;
+}
+
+}  // namespace
+
 HipKernelPlan GenerateHipKernel(const DimensionedMultiKernel &mk, const HipCodegenOptions &options)
 {
     // Partial results of a reordered kernel may take up to 48 KB of LDS per batch entry; when the tiles that are
@@ -114,10 +134,10 @@ HipKernelPlan GenerateHipKernel(const DimensionedMultiKernel &mk, const HipCodeg
     {
         codegen::Generator g(mk, options, maxTile);
         HipKernelPlan plan = g.Run();
-        if (!g.factorisationAbandoned) return plan;
+        if (!g.factorisationAbandoned) return withSpillGuard(std::move(plan));
     }
     codegen::Generator g(mk, options, 0);
-    return g.Run();
+    return withSpillGuard(g.Run());
 }
 
 }  // namespace acro

@@ -160,6 +160,10 @@ struct HipCodegenOptions
     // value numbers the (map, source) pair among the extra kernel parameters.  Only for operands that are read, never
     // written, by the group, and not in positional mode.
     std::vector<int> gathered;
+    // True: no schedule that uses the FP64 matrix cores (the operator and Gram schedules) is chosen.  The executor asks
+    // for this after a matrix-core kernel has come out of the compiler with private memory (register spills) that the
+    // schedule's register-relief switch did not remove: such a kernel is never launched.
+    bool no_matrix_cores = false;
 };
 
 // One kernel launch of a plan.  params: >= 0 is an index into HipKernelPlan::param_occurrence (a storage's device
@@ -203,6 +207,12 @@ struct HipKernelPlan
     int lds_bytes = 0;
     int nb = 0;
     bool gathers_applied = false;  // the source reads gathered operands through their maps (HipCodegenOptions::gathered)
+    // Kernels of `source` that hold matrix-core accumulators: they keep nothing in private memory by design, and a
+    // code object that reports private memory for one of them has register spills, which the compiler has been seen to
+    // get wrong around those accumulators.  register_relief_macro, when not empty, names a preprocessor switch of
+    // the source that trades registers for LDS reads.
+    std::vector<std::string> matrix_core_functions;
+    std::string register_relief_macro;
     std::string schedule;          // human readable schedule summary (also a comment in the source)
 };
 

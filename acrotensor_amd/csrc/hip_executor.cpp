@@ -100,7 +100,35 @@ class HipExecutor : public KernelExecutor
         {
             std::unique_ptr<Variant> v(new Variant);
             v->plan = GenerateHipKernel(*MultiKernel, options);
-            if (v->plan.fusable) v->kernel.reset(new HipKernel(v->plan.module_name, v->plan.source));
+            if (v->plan.fusable)
+            {
+                v->kernel.reset(new HipKernel(v->plan.module_name, v->plan.source, v->plan.matrix_core_functions,
+                                              v->plan.register_relief_macro));
+                if (!v->kernel->PrivateMemoryRemains().empty())
+                {
+                    // A matrix-core kernel that the compiler could only fit with register spills, also with the
+                    // schedule's register-relief switch (or the schedule has none): never launched.  The same group
+                    // through the schedules that do without the matrix cores.
+                    const std::string refused = v->kernel->PrivateMemoryRemains();
+                    HipCodegenOptions plain = options;
+                    plain.no_matrix_cores = true;
+                    v->plan = GenerateHipKernel(*MultiKernel, plain);
+                    v->kernel.reset();
+                    if (v->plan.fusable)
+                    {
+                        const size_t firstLine = v->plan.source.find('\n') + 1;
+                        v->plan.source.insert(firstLine, "// (matrix-core kernel " + refused + " needed private memory, i.e. register spills, "
+                                                         "and was refused: this is the schedule without the matrix cores)\n");
+                        v->kernel.reset(new HipKernel(v->plan.module_name, v->plan.source, v->plan.matrix_core_functions,
+                                                      v->plan.register_relief_macro));
+                        ACROBATIC_ASSERT(v->kernel->PrivateMemoryRemains().empty(), "Internal error: matrix-core kernel in a plan without matrix cores.");
+                    }
+                }
+                else if (v->kernel->ReliefApplied())
+                {
+                    v->plan.source = v->kernel->GetSource();  // what was compiled: the relief macro defined in front
+                }
+            }
             it = Variants.emplace(key, std::move(v)).first;
         }
         LastVariant = it->second.get();
@@ -260,6 +288,18 @@ class HipExecutor : public KernelExecutor
             s.device = t->GetDeviceData();
             s.size = static_cast<size_t>(t->GetSize());
             s.transient = t->IsTransient();
+            // what Bind derives from a slice's parents: the tensor it is a view of, where, and that tensor's shape
+            const Tensor *root = t;
+            s.offset = 0;
+            while (const SliceTensor *sl = dynamic_cast<const SliceTensor *>(root))
+            {
+                s.offset += sl->GetOffset();
+                root = sl->GetParent();
+            }
+            s.root = root;
+            s.root_device = root->GetDeviceData();
+            s.root_shape = 1469598103934665603ull;
+            for (int d = 0; d < root->GetRank(); ++d) s.root_shape = (s.root_shape ^ static_cast<unsigned>(root->GetDim(d))) * 1099511628211ull;
             ThisCall.push_back(s);
         };
         for (int ki = 0; ki < K; ++ki)
@@ -362,13 +402,15 @@ class HipExecutor : public KernelExecutor
     // one entry per tensor of a call, in call order
     struct Seen
     {
-        const Tensor *tensor;
-        const double *host, *device;
-        size_t size;
+        const Tensor *tensor, *root;
+        const double *host, *device, *root_device;
+        size_t size, offset;
+        unsigned long long root_shape;
         bool transient;
         bool operator==(const Seen &o) const
         {
-            return tensor == o.tensor && host == o.host && device == o.device && size == o.size && transient == o.transient;
+            return tensor == o.tensor && host == o.host && device == o.device && size == o.size && transient == o.transient &&
+                   root == o.root && root_device == o.root_device && offset == o.offset && root_shape == o.root_shape;
         }
     };
     std::vector<Seen> ThisCall, LastCall;

@@ -28,12 +28,20 @@ const char *const kCompileOptions[] = {
 };
 constexpr int kNumCompileOptions = sizeof(kCompileOptions) / sizeof(kCompileOptions[0]);
 
+// The two experiment hooks below replace what the library compiles, so they are only honoured when
+// ACRO_HIP_DEBUG_HOOKS=1 says that this is wanted.
+bool debugHooks()
+{
+    const char *env = std::getenv("ACRO_HIP_DEBUG_HOOKS");
+    return env != nullptr && std::string(env) == "1";
+}
+
 // Experiment hook: further options for the run-time compiler, separated by blanks (ACRO_HIP_COMPILE_OPTIONS="-mllvm
 // -amdgpu-..."); they are part of the key of the on-disk cache.
 std::vector<std::string> extraCompileOptions()
 {
     std::vector<std::string> extra;
-    const char *env = std::getenv("ACRO_HIP_COMPILE_OPTIONS");
+    const char *env = debugHooks() ? std::getenv("ACRO_HIP_COMPILE_OPTIONS") : nullptr;
     if (env == nullptr) return extra;
     std::istringstream words(env);
     std::string word;
@@ -103,12 +111,91 @@ void rtcCheck(hiprtcResult r, const char *what)
 
 }  // namespace
 
-HipKernel::HipKernel(const std::string &module_name, const std::string &source)
-    : FunctionName(module_name), Source(source), CacheHit(false), Module(nullptr)
+// The code object is an ELF file (64-bit, little endian) in which every kernel has a 64-byte descriptor under the
+// symbol "<name>.kd"; bytes 4 - 7 of the descriptor are private_segment_fixed_size.  hipRTC may wrap the ELF file in
+// a bundle ("__CLANG_OFFLOAD_BUNDLE__"): the first ELF file inside it is taken (there is one target).
+int HipKernel::PrivateSegmentBytes(const std::vector<char> &code_object, const std::string &function)
+{
+    const unsigned char *base = reinterpret_cast<const unsigned char *>(code_object.data());
+    size_t size = code_object.size();
+    auto rd = [&](size_t at, int bytes) -> uint64_t {
+        uint64_t v = 0;
+        if (at + bytes > size) return 0;
+        for (int i = bytes - 1; i >= 0; --i) v = (v << 8) | base[at + i];
+        return v;
+    };
+    if (size >= 24 && std::string(code_object.data(), 24) == "__CLANG_OFFLOAD_BUNDLE__")
+    {
+        const uint64_t entries = rd(24, 8);
+        size_t at = 32;
+        for (uint64_t e = 0; e < entries; ++e)
+        {
+            const uint64_t offset = rd(at, 8), length = rd(at + 8, 8), triple = rd(at + 16, 8);
+            at += 24 + triple;
+            if (offset + length <= size && length >= 4 && std::string(code_object.data() + offset, 4) == "\x7f" "ELF")
+            {
+                base += offset;
+                size = length;
+                break;
+            }
+        }
+    }
+    if (size < 64 || std::string(reinterpret_cast<const char *>(base), 4) != "\x7f" "ELF" || base[4] != 2 || base[5] != 1) return -1;
+    const uint64_t shoff = rd(0x28, 8), shentsize = rd(0x3A, 2), shnum = rd(0x3C, 2);
+    const std::string wanted = function + ".kd";
+    for (uint64_t i = 0; i < shnum; ++i)
+    {
+        const size_t sh = shoff + i * shentsize;
+        const uint64_t type = rd(sh + 4, 4);
+        if (type != 2 && type != 11) continue;  // SHT_SYMTAB, SHT_DYNSYM
+        const uint64_t symoff = rd(sh + 0x18, 8), symsize = rd(sh + 0x20, 8), link = rd(sh + 0x28, 4), entsize = rd(sh + 0x38, 8);
+        if (entsize == 0 || link >= shnum) continue;
+        const size_t strsh = shoff + link * shentsize;
+        const uint64_t stroff = rd(strsh + 0x18, 8), strsize = rd(strsh + 0x20, 8);
+        for (uint64_t s = 0; s + entsize <= symsize; s += entsize)
+        {
+            const size_t sym = symoff + s;
+            const uint64_t name = rd(sym, 4), shndx = rd(sym + 6, 2), value = rd(sym + 8, 8);
+            if (name >= strsize || stroff + name + wanted.size() + 1 > size) continue;
+            if (std::string(reinterpret_cast<const char *>(base) + stroff + name) != wanted) continue;
+            if (shndx == 0 || shndx >= shnum) continue;
+            const size_t sec = shoff + shndx * shentsize;
+            const uint64_t addr = rd(sec + 0x10, 8), offset = rd(sec + 0x18, 8);
+            const size_t descriptor = offset + (value - addr);
+            if (descriptor + 64 > size) return -1;
+            return static_cast<int>(rd(descriptor + 4, 4));
+        }
+    }
+    return -1;
+}
+
+std::string HipKernel::FirstKernelWithPrivateMemory() const
+{
+    // Test hook: ACRO_HIP_TEST_PRIVATE_BYTES="first,second" stands for what the code object says on the first and on
+    // the second (relief) compilation, so that both branches can be exercised with a kernel that does not spill.
+    if (const char *env = std::getenv("ACRO_HIP_TEST_PRIVATE_BYTES"))
+    {
+        const std::string text(env);
+        const size_t comma = text.find(',');
+        const std::string mine = Relieved ? (comma == std::string::npos ? text : text.substr(comma + 1)) : text.substr(0, comma);
+        return std::atoi(mine.c_str()) > 0 && !Guarded.empty() ? Guarded[0] : std::string();
+    }
+    for (const std::string &name : Guarded)
+    {
+        const int bytes = PrivateSegmentBytes(CodeObject, name);
+        ACROBATIC_ASSERT(bytes >= 0, "Kernel " + name + " is not in the code object of " + FunctionName + ".");
+        if (bytes > 0) return name;
+    }
+    return std::string();
+}
+
+HipKernel::HipKernel(const std::string &module_name, const std::string &source,
+                     const std::vector<std::string> &no_private_memory, const std::string &relief_macro)
+    : FunctionName(module_name), Source(source), CacheHit(false), Guarded(no_private_memory), Module(nullptr)
 {
     // Experiment hook: $ACRO_HIP_KERNEL_OVERRIDE_DIR/<module name>.hip, when it exists, is compiled in place of the
     // generated source (same function names and parameters), e.g. a hand-edited copy of what GetImplementation printed.
-    if (const char *dir = std::getenv("ACRO_HIP_KERNEL_OVERRIDE_DIR"))
+    if (const char *dir = debugHooks() ? std::getenv("ACRO_HIP_KERNEL_OVERRIDE_DIR") : nullptr)
     {
         std::ifstream in(std::string(dir) + "/" + module_name + ".hip");
         if (in)
@@ -120,6 +207,16 @@ HipKernel::HipKernel(const std::string &module_name, const std::string &source)
         }
     }
     Compile();
+    Spilling = FirstKernelWithPrivateMemory();
+    if (!Spilling.empty() && !relief_macro.empty())
+    {
+        Source = "#define " + relief_macro + " 1\n" + Source;
+        CacheHit = false;
+        CodeObject.clear();
+        Relieved = true;
+        Compile();
+        Spilling = FirstKernelWithPrivateMemory();
+    }
 }
 
 HipKernel::~HipKernel()
@@ -206,32 +303,18 @@ void HipKernel::EnsureLoaded()
         err = hipModuleLoadData(&module, CodeObject.data());
     }
     ACRO_HIP_CHECK(err);
-    // Kernels that keep no arrays in private memory by design (the matrix-core schedules) carry a switch that trades
-    // registers for LDS reads.  When the compiler has fit one of them into the registers only with spills, compile
-    // the module again with the switch on: spill code around the matrix-core accumulators is slow, and the compiler
-    // has been seen to lose half of a spilled 64-bit value there (a result off in its low 32 bits).
-    static const char *const kSwitch = "ACRO_KEEP_OPERATOR_IN_LDS";
-    if (Source.find(std::string("#ifdef ") + kSwitch) != std::string::npos && Source.compare(0, 8, "#define ") != 0)
+    // What the compile-time check read from the kernel descriptors, confirmed by the loaded module.
+    for (const std::string &name : Guarded)
     {
-        bool spills = false;
-        for (size_t at = Source.find("__global__"); at != std::string::npos && !spills; at = Source.find("__global__", at + 1))
+        hipFunction_t function;
+        int privateBytes = 0;
+        ACRO_HIP_CHECK(hipModuleGetFunction(&function, module, name.c_str()));
+        ACRO_HIP_CHECK(hipFuncGetAttribute(&privateBytes, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, function));
+        if (privateBytes > 0)
         {
-            const size_t name = Source.find("void ", at), paren = Source.find('(', name);
-            if (name == std::string::npos || paren == std::string::npos) break;
-            hipFunction_t function;
-            int privateBytes = 0;
-            ACRO_HIP_CHECK(hipModuleGetFunction(&function, module, Source.substr(name + 5, paren - name - 5).c_str()));
-            ACRO_HIP_CHECK(hipFuncGetAttribute(&privateBytes, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, function));
-            spills = privateBytes > 0;
-        }
-        if (spills)
-        {
-            ACRO_HIP_CHECK(hipModuleUnload(module));
-            Source = std::string("#define ") + kSwitch + " 1\n" + Source;
-            CacheHit = false;
-            CodeObject.clear();
-            Compile();
-            ACRO_HIP_CHECK(hipModuleLoadData(&module, CodeObject.data()));
+            (void)hipModuleUnload(module);
+            throw_error("Matrix-core kernel " + name + " was loaded with " + std::to_string(privateBytes) +
+                        " bytes of private memory per work item (register spills): it is not launched.");
         }
     }
     Module = module;
@@ -239,6 +322,7 @@ void HipKernel::EnsureLoaded()
 
 void HipKernel::Launch(const std::string &function_name, unsigned grid, unsigned grid_y, unsigned block, void **args)
 {
+    ACROBATIC_ASSERT(Spilling.empty(), "Matrix-core kernel " + Spilling + " has private memory (register spills): it is not launched.");
     EnsureLoaded();
     auto it = Functions.find(function_name);
     if (it == Functions.end())

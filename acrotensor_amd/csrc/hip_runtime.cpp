@@ -101,7 +101,17 @@ void SetStream(void *hip_stream)
         hipError_t err = hipEventRecord(handover, outgoing);
         if (err == hipSuccess) err = hipStreamWaitEvent(incoming, handover, 0);
         (void)hipEventDestroy(handover);  // released by the runtime once the event has completed
-        ACRO_HIP_CHECK(err);
+        if (err != hipSuccess)
+        {
+            // The hand-over failed (an adopted stream that its owner has destroyed already, say).  The switch is made
+            // all the same, so that the library does not stay bound to a stream it cannot use, and the failure is
+            // reported: work queued before the switch is then NOT ordered before what follows.
+            (void)hipGetLastError();
+            std::lock_guard<std::mutex> guard(g_lock);
+            g_adopted_stream = (incoming == g_own_stream) ? nullptr : incoming;
+            throw_error(std::string("Changing the stream: the outgoing stream could not be ordered before the incoming one (") +
+                        hipGetErrorString(err) + "); the switch has been made without that ordering.");
+        }
     }
     std::lock_guard<std::mutex> guard(g_lock);
     g_adopted_stream = (incoming == g_own_stream) ? nullptr : incoming;

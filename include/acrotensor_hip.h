@@ -32,7 +32,10 @@ int acro_hip_is_ready(void);
 /* Block until all work issued by the library has finished. */
 int acro_hip_synchronize(void);
 /* Adopt an externally created hipStream_t (NULL: back to the library's own stream).  Stands in for the
- * reference's setCudaContext(), util/CudaUtil.hpp:93-98. */
+ * reference's setCudaContext(), util/CudaUtil.hpp:93-98.  Work queued before the switch is ordered ahead of work
+ * queued after it (an event on the outgoing stream that the incoming one waits for; the host does not wait).  An
+ * adopted stream must stay alive until the library has been switched away from it: if the hand-over fails because
+ * it is gone, the switch is still made and the call reports the failure (no ordering across that switch). */
 int acro_hip_set_stream(void *hip_stream);
 void *acro_hip_get_stream(void);
 
@@ -108,8 +111,9 @@ int acro_engine_contract(acro_engine *e, const char *kernel, acro_tensor *out, a
  * serving loops, harnesses that forbid hipMalloc); no counterpart in the reference, whose launches never allocate
  * because its kernels have no scratch memory (exec/CudaExecutor.cpp:70-101).  This call allocates no device or
  * page-locked memory and loads no code object: every tensor must already be resident on the device, and the same
- * kernel string on tensors of the same extents must have run once through acro_engine_contract (which compiles and
- * loads the kernel); otherwise the call fails with a message saying so.  Kernels that need scratch memory beyond
+ * kernel string on tensors of the same extents must have run once through acro_engine_contract on that device (which
+ * compiles and loads the kernel, and looks up the device address of the scratch array below: the first look-up on a
+ * device may load code and allocate, so it is never done here); otherwise the call fails with a message saying so.  Kernels that need scratch memory beyond
  * their operands (split contractions such as "S_i_j = A_n_i_j B_n": per-workgroup partial sums) take it from one
  * array of ACRO_NO_ALLOC_SCRATCH_BYTES that the library holds on every device it runs on until the process ends; a
  * kernel that needs more is refused with a message.  All calls on a device share that array, which keeps the last
@@ -150,6 +154,12 @@ int acro_engine_flat_indexed_sum_gather(acro_engine *e, acro_tensor *Aout, acro_
 /* Compiles HIP C++ source for gfx950 with the options the library uses for generated kernels; needs no device.
  * Returns 0 and the code-object size in *code_size, or non-zero with the compiler log in acro_last_error(). */
 int acro_hip_compile(const char *module_name, const char *source, size_t *code_size);
+/* Compiles the same way and reports the private (scratch) memory per work item, in bytes, that the code object
+ * declares for the kernel `function`: non-zero means register spills or arrays in private memory.  This is the figure
+ * the library checks for every generated matrix-core kernel before it will launch it (such a kernel is compiled again
+ * with its register-relief switch, and replaced by a schedule without the matrix cores if that does not help).
+ * Diagnostics; the reference has no counterpart (NVRTC output is launched as it comes, util/CudaUtil.cpp:43-84). */
+int acro_hip_compile_private_bytes(const char *module_name, const char *source, const char *function, int *bytes);
 
 /* ---- kernel IR introspection, host only (kernel/TensorKernel.hpp, DimensionedKernel.hpp,
  *      DimensionedMultiKernel.hpp) ---- */
