@@ -241,6 +241,10 @@ auto Generator::StageReusedOperands(int ki, const Sub &asWritten, std::vector<Su
     if (envInt("ACRO_HIP_STAGE_ENTRIES") < 0 || batch < 0 || !opt.noalias || asWritten.contr.empty() || asWritten.matrixOp != 0) return false;
     Sub orig = asWritten;
     if (orig.out.repeated || orig.in.size() < 2 || NumGatherSlots() > 0) return false;
+    {
+        ProductShape onMatrixCores;  // products of larger element matrices have a schedule of their own
+        if (ProductPattern(asWritten, onMatrixCores)) return false;
+    }
     const long outputs = product(orig.outIdx, extent) / extent[batch];
     const long stageMost = envInt("ACRO_HIP_STAGE_MOST", 8000);
     if (outputs < 4 || outputs > stageMost / 2) return false;

@@ -1,0 +1,357 @@
+// Kernel code generator, the product schedule: products of element matrices on the FP64 matrix cores,
+// "A_e_i_j = B_e_i_k C_e_k_j" with either factor stored either way round.
+#include "hip_codegen_impl.hpp"
+
+namespace acro
+{
+namespace codegen
+{
+
+// "A_e_r_c (=|+=|-=) R_e_{r,k} C_e_{k,c}": every batch entry holds an M x K and a K x N matrix (each stored with the
+// contracted index last or first) and receives their M x N product, all three contiguous per entry.  The reference
+// maps a thread to an output and loops over k (exec/CudaExecutor.cpp:193-263); the staged vector-ALU schedule of this
+// generator does the same out of LDS tiles, where every multiply-add reads one or both of its factors from LDS: from
+// 33 x 33 on it is bound by LDS (55 x 55: 22 % of the HBM peak, 63 x 63: 32 %), and these sizes carry as much
+// arithmetic as traffic.  v_mfma_f64_16x16x4 multiplies a 16 x 4 block by a 4 x 16 block per instruction with one
+// operand value per lane each.
+//
+// A wavefront owns a strip of 16 rows of one entry's result.  It loads its strip of the row factor straight from
+// device memory in the layout the instruction wants (lane = row + 16 * term group), 16 bytes per lane where the
+// contracted index is the fastest dimension (the two doubles go to two successive steps: the terms of a step are
+// permuted, k = 8 [s / 2] + 2 g + s mod 2, which a sum does not mind).  The column factor is needed by every strip:
+// the wavefronts of an entry load it once, each a share of its 16-column blocks, also in instruction layout, and
+// leave it in LDS fragment by fragment, so that the reads in the multiply loop are 64 consecutive doubles (no bank
+// conflicts).  Rows and columns past the end read the last valid one (their results are not stored), terms past
+// the end read as zero.  The accumulators (register q of a lane: row 4 q + lane / 16, column lane % 16 of the block)
+// go to a tile in LDS in the result's memory order, and the workgroup writes the tiles of its entries, one contiguous
+// range of the result, in whole lines with non-temporal stores.
+auto Generator::ProductPattern(const Sub &s, ProductShape &p) const -> bool
+{
+    if (envInt("ACRO_HIP_PRODUCT") < 0 || opt.no_matrix_cores || batch < 0 || !opt.noalias || NumGatherSlots() > 0) return false;
+    if (mk.GetNumKernels() != 1 || s.matrixOp != 0 || s.out.repeated || s.in.size() != 2 || s.contr.size() != 1) return false;
+    if (s.out.idx.size() != 3 || s.out.idx[0] != batch) return false;
+    const int k = s.contr[0], r = s.out.idx[1], c = s.out.idx[2];
+    for (const auto &v : s.in)
+    {
+        if (v.repeated || v.idx.size() != 3 || v.idx[0] != batch) return false;
+        // (the pattern is also asked for while the model is being built, before storages are known)
+        if (v.uvar == s.out.uvar || (uvars[v.uvar].storage >= 0 && uvars[v.uvar].storage == uvars[s.out.uvar].storage)) return false;
+        const bool kLast = v.idx[2] == k, kFirst = v.idx[1] == k;
+        if (!kLast && !kFirst) return false;
+        const int other = kLast ? v.idx[1] : v.idx[2];
+        if (other == r && !p.row)
+        {
+            p.row = &v;
+            p.rowKFast = kLast;
+        }
+        else if (other == c && !p.col)
+        {
+            p.col = &v;
+            p.colKFast = kLast;
+        }
+        else
+            return false;
+    }
+    if (!p.row || !p.col) return false;
+    p.M = extent[r];
+    p.N = extent[c];
+    p.K = extent[k];
+    p.E = extent[batch];
+    // From 17 rows or columns on (up to 16 x 16 the staged schedule has a lane per output and is bound by memory);
+    // a wavefront holds one strip of at most eight column blocks, an entry at most eight strips.
+    const long lo = envInt("ACRO_HIP_PRODUCT_FROM", 17), hi = envInt("ACRO_HIP_PRODUCT_TO", 128);
+    if (std::max(p.M, p.N) < lo || p.M > hi || p.N > hi || p.K > 128 || p.K < 8 || p.M < 8 || p.N < 8) return false;
+    // Up to 36 x 36 the staged vector-ALU schedule is as fast or a little faster where it can give a lane a block of
+    // outputs, i.e. where both extents have a divisor 2, 3 or 5 (rotated buffers, % of the HBM peak, staged / here:
+    // 20 x 20 75 / 71, 24 x 24 75 / 72, 25 x 25 74 / 71, 28 x 28 74 / 73, 33 x 33 67 / 64, 36 x 36 71 / 70; without such
+    // a divisor 17 x 17 59 / 67, 31 x 31 42 / 71, 37 x 37 37 / 70; larger: 40 x 40 69 / 69, 45 x 45 67 / 69, 48 x 48 69 / 70,
+    // 53 x 53 28 / 68, 55 x 55 23 / 68, 56 x 56 58 / 69, 63 x 63 32 / 67, 64 x 64 15 / 70).
+    auto blocks = [](long n) { return n % 2 == 0 || n % 3 == 0 || n % 5 == 0; };
+    if (std::max(p.M, p.N) <= 36 && blocks(p.M) && blocks(p.N) && envInt("ACRO_HIP_PRODUCT") < 2) return false;
+    p.TI = (p.M + 15) / 16;
+    p.TJ = (p.N + 15) / 16;
+    if (p.TI > 8 || p.TJ > 8) return false;
+    // The row factor goes into registers strip by strip, each wavefront its own 16 rows.  Straight from device memory
+    // where a wavefront's loads fall on whole lines: rows of a multiple of 128 bytes read along the contracted index in
+    // pairs (mode 0), or blocks of 16 rows read across it, 128 contiguous bytes per term (mode 1).  Otherwise (mode 2)
+    // the strip, one contiguous range of device memory, is read front to back and passes through a piece of LDS of the
+    // wavefront's own, which the column factor's fragments take over afterwards.
+    // (View offsets are known only once the model is complete, and whether the schedule applies must not depend on
+    // them: the size test takes the larger footprint.)
+    p.rowMode = !p.rowKFast ? 1 : (p.K % 16 == 0 && uvars[p.row->uvar].viewOffset % 2 == 0 && envInt("ACRO_HIP_PRODUCT_DIRECT") >= 0 ? 0 : 2);
+    p.pairMap = p.rowMode == 0;
+    p.steps = p.pairMap ? 2 * ((p.K + 7) / 8) : (p.K + 3) / 4;
+    const long stepsMost = 2 * ((p.K + 7) / 8);
+    if (std::max<long>(std::max(p.TI, p.TJ) * stepsMost * 64, p.M * p.N) * 8 > 64 * 1024) return false;
+    const long perEntry = std::max<long>(std::max<long>(p.rowMode == 2 ? p.TI : 0, p.TJ) * p.steps * 64, p.M * p.N);
+    // entries per workgroup: up to four wavefronts, 64 KB of LDS (fragments of the factors, then the result tiles)
+    p.NBE = std::max<long>(1, std::min<long>(4 / p.TI, (64 * 1024 / 8) / perEntry));
+    if (envInt("ACRO_HIP_PRODUCT_ENTRIES") > 0) p.NBE = std::min<long>(envInt("ACRO_HIP_PRODUCT_ENTRIES"), (64 * 1024 / 8) / perEntry);
+    p.NBE = std::min(p.NBE, p.E);
+    p.ldsPerEntry = perEntry;
+    return true;
+}
+
+auto Generator::UseProductSchedule() const -> bool
+{
+    ProductShape p;
+    return subs.size() == 1 && ProductPattern(subs[0], p);
+}
+
+auto Generator::EmitProduct(HipKernelPlan &plan) -> void
+{
+    const Sub &s = subs[0];
+    ProductShape p;
+    ProductPattern(s, p);
+    const long M = p.M, N = p.N, K = p.K, E = p.E, TI = p.TI, TJ = p.TJ, steps = p.steps, NBE = p.NBE;
+    const long NW = NBE * TI, NT = NW * 64, MN = M * N, LT = TI * 64;   // LT: lanes that share an entry
+    const long groups = (E + NBE - 1) / NBE;
+    const long ldsDoublesHere = NBE * p.ldsPerEntry;
+    const std::string dimName = mk.GetDimensionedNameString();
+    char hex[32];
+    std::snprintf(hex, sizeof(hex), "%016llx",
+                  static_cast<unsigned long long>(hashString(dimName + "/product/" + (Positional() ? "p" : "u") + str(NBE) +
+                                                             str(p.rowMode))));
+    plan.module_name = std::string("acro_prod_") + hex;
+
+    std::ostringstream sched;
+    sched << "product schedule on the FP64 matrix cores: " << M << " x " << K << " by " << K << " x " << N << " per entry (row factor "
+          << (p.rowKFast ? "with the contracted index last" : "with the contracted index first")
+          << (p.rowMode == 2 ? ", strips through LDS" : ", read straight into registers") << "; column factor "
+          << (p.colKFast ? "with the contracted index last" : "with the contracted index first") << ", through LDS), " << TI
+          << " strips of 16 rows x " << TJ << " blocks of 16 columns, " << steps << " steps of four terms" << (p.pairMap ? " (terms in pairs)" : "")
+          << ", " << NBE << (NBE == 1 ? " entry" : " entries") << " per workgroup of " << NT << " lanes, LDS " << ldsDoublesHere * 8
+          << " bytes, results written out through LDS\n  [0] " << s.text << "\n";
+    plan.schedule = sched.str();
+    out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
+    {
+        std::istringstream lines(plan.schedule);
+        std::string l;
+        while (std::getline(lines, l)) out << "// " << l << "\n";
+    }
+    const std::string R = PtrName(p.row->uvar), C = PtrName(p.col->uvar), A = PtrName(s.out.uvar);
+    const long rOff = uvars[p.row->uvar].viewOffset, cOff = uvars[p.col->uvar].viewOffset, aOff = uvars[s.out.uvar].viewOffset;
+
+    // term of step s for term group g, and step / group of term k
+    auto termOf = [&](const std::string &step) {
+        return p.pairMap ? "(8 * ((" + step + ") / 2) + 2 * g + (" + step + ") % 2)" : "(4 * (" + step + ") + g)";
+    };
+    const std::string stepOfK = p.pairMap ? "(2 * (k / 8) + k % 2)" : "(k / 4)";
+    const std::string groupOfK = p.pairMap ? "((k % 8) / 2)" : "(k % 4)";
+
+    // A factor's matrix of one entry is one contiguous range of device memory: the lanes of the entry read it front to
+    // back from the line boundary at or before its first double, 16 bytes each, and put every value where the matrix
+    // instruction will want it: fragment (block of 16 rows or columns, step), term group, and within the group of 16
+    // the place (row + term) mod 16, which spreads the values that a wavefront writes at once, a run along either
+    // dimension of the matrix, over the banks (the readers undo the rotation).
+    struct Staged
+    {
+        std::string ptr, name;
+        long offset, rows, kFast, base, blocks;
+    };
+    std::vector<Staged> staged;
+    staged.push_back({C, "c", cOff, N, p.colKFast ? 1 : 0, 0, TJ});
+    // the strip of the row factor (mode 2): 16 rows of K doubles, read by the one wavefront that owns it
+    long stripIts = 0;
+    if (p.rowMode == 2)
+    {
+        long lead = 0;
+        for (long en = 0; en < 16; ++en)
+            for (long st = 0; st < TI; ++st) lead = std::max(lead, (rOff + (en * M + 16 * st) * K) % 16);
+        stripIts = ((16 * K + lead + 1) / 2 + 63) / 64;
+    }
+    // 16-byte pieces per lane: the matrix and the most doubles that can lie between a line boundary and its first one
+    auto itsOf = [&](const Staged &f) {
+        long lead = 0;
+        for (long en = 0; en < 16; ++en) lead = std::max(lead, (f.offset + en * f.rows * K) % 16);
+        return ((f.rows * K + lead + 1) / 2 + LT - 1) / LT;
+    };
+
+    // loads of the factors of the workgroup's entries into registers (no branches around the single loads: all of them
+    // are in flight together.  A pair that would reach past the end of the tensor is replaced by the last whole pair,
+    // whose values are then not used; the last double of a tensor of odd length is read on its own.)
+    auto emitLoads = [&](const std::string &eg, const std::string &ind) {
+        out << ind << "{\n";
+        out << ind << "    const long en = (" << eg << ") * " << NBE << " + slot < " << E << " ? (" << eg << ") * " << NBE << " + slot : " << E - 1 << ";\n";
+        for (const Staged &f : staged)
+        {
+            const long size = f.rows * K, tensorEnd = f.offset + E * size, lastPair = (tensorEnd - 2) & ~1L;
+            out << ind << "    const long " << f.name << "First = (" << f.offset << "L + en * " << size << "L) & ~15L;\n";
+            out << "#pragma unroll\n" << ind << "    for (int it = 0; it < " << itsOf(f) << "; ++it)\n" << ind << "    {\n";
+            out << ind << "        const long at = " << f.name << "First + 2 * (it * " << LT << " + lt);\n";
+            out << ind << "        " << f.name << "v[it] = *reinterpret_cast<const acro_pair *>(" << f.ptr << " + (at < " << lastPair << "L ? at : " << lastPair << "L));\n";
+            if (tensorEnd % 2 != 0)
+                out << ind << "        if (it == " << itsOf(f) - 1 << " && at == " << tensorEnd - 1 << "L) " << f.name << "v[it].x = " << f.ptr << "[" << tensorEnd - 1 << "L];\n";
+            out << ind << "    }\n";
+        }
+        if (p.rowMode == 2)
+        {
+            const long tensorEnd = rOff + E * M * K, lastPair = (tensorEnd - 2) & ~1L;
+            out << ind << "    const long rFirst = (" << rOff << "L + (en * " << M << " + 16 * strip) * " << K << "L) & ~15L;\n";
+            out << "#pragma unroll\n" << ind << "    for (int it = 0; it < " << stripIts << "; ++it)\n" << ind << "    {\n";
+            out << ind << "        const long at = rFirst + 2 * (it * 64 + lane);\n";
+            out << ind << "        rv[it] = *reinterpret_cast<const acro_pair *>(" << R << " + (at < " << lastPair << "L ? at : " << lastPair << "L));\n";
+            if (tensorEnd % 2 != 0)
+                out << ind << "        if (at == " << tensorEnd - 1 << "L) rv[it].x = " << R << "[" << tensorEnd - 1 << "L];\n";
+            out << ind << "    }\n";
+        }
+        else
+        {
+            out << ind << "    const double *rm = " << R << " + " << rOff << "L + en * " << M * K << "L;\n";
+            out << ind << "    const int m = 16 * strip + c < " << M << " ? 16 * strip + c : " << M - 1 << ";\n";
+            if (p.rowKFast)
+            {
+                out << "#pragma unroll\n" << ind << "    for (int u = 0; u < " << steps / 2 << "; ++u)\n" << ind << "    {\n";
+                out << ind << "        const int k = 8 * u + 2 * g;\n";
+                out << ind << "        acro_pair v = {0.0, 0.0};\n";
+                out << ind << "        if (k < " << K << ") v = *reinterpret_cast<const acro_pair *>(rm + m * " << K << " + k);\n";
+                out << ind << "        a[2 * u] = v.x;\n" << ind << "        a[2 * u + 1] = v.y;\n" << ind << "    }\n";
+            }
+            else
+            {
+                out << "#pragma unroll\n" << ind << "    for (int s = 0; s < " << steps << "; ++s)\n" << ind << "    {\n";
+                out << ind << "        const int k = " << termOf("s") << ";\n";
+                out << ind << "        a[s] = k < " << K << " ? rm[k * " << M << " + m] : 0.0;\n" << ind << "    }\n";
+            }
+        }
+        out << ind << "}\n";
+    };
+
+    out << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
+    out << "typedef double acro_pair __attribute__((ext_vector_type(2)));\n";
+    out << "\nextern \"C\" __global__ __launch_bounds__(" << NT << ") void " << plan.module_name << "(" << ParamList() << ")\n{\n";
+    out << "    __shared__ double lds[" << ldsDoublesHere << "];\n";
+    out << "    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;\n";
+    out << "    const int slot = wave / " << TI << ", strip = wave % " << TI << ", lt = strip * 64 + lane;   // lt: lane among those of the entry\n";
+    out << "    double *frag = lds + slot * " << p.ldsPerEntry << ";\n";
+    for (const Staged &f : staged) out << "    acro_pair " << f.name << "v[" << itsOf(f) << "];\n";
+    if (p.rowMode == 2) out << "    acro_pair rv[" << stripIts << "];\n";
+    out << "    double a[" << steps << "];\n";
+    emitLoads("(long)blockIdx.x", "    ");
+    out << "    {\n";
+    out << "        const long e0 = (long)blockIdx.x * " << NBE << ";\n";
+    out << "        const long e = e0 + slot < " << E << " ? e0 + slot : " << E - 1 << ";   // (a slot past the last entry repeats it; nothing of it is stored)\n";
+    // terms past the end read as zero: the places of the last step(s) whose term does not exist
+    long np = 0;
+    std::string sOfW, gOfW;
+    if (p.pairMap && K % 8 != 0)
+    {
+        np = 2 * (4 - (K % 8) / 2);
+        sOfW = str(steps - 2) + " + w % 2";
+        gOfW = str((K % 8) / 2) + " + w / 2";
+    }
+    else if (!p.pairMap && K % 4 != 0)
+    {
+        np = 4 - K % 4;
+        sOfW = str(steps - 1);
+        gOfW = str(K % 4) + " + w";
+    }
+    if (p.rowMode == 2)
+    {
+        // ---- the strip: to the fragments of this wavefront's block of rows, and from there into its registers
+        out << "        {\n            double *fr = frag + strip * " << steps * 64 << ";\n";
+        out << "            const long base = " << rOff << "L + (e * " << M << " + 16 * strip) * " << K << "L;\n";
+        out << "            const int lead = (int)(base - (base & ~15L));   // doubles between the line boundary and the strip\n";
+        out << "            const int size = (" << M << " - 16 * strip < 16 ? " << M << " - 16 * strip : 16) * " << K << ";\n";
+        out << "#pragma unroll\n            for (int it = 0; it < " << stripIts << "; ++it)\n            {\n";
+        out << "#pragma unroll\n                for (int h = 0; h < 2; ++h)\n                {\n";
+        out << "                    const int j = 2 * (it * 64 + lane) + h - lead;\n";
+        out << "                    if (j < 0 || j >= size) continue;\n";
+        out << "                    const int x = j / " << K << ", k = j % " << K << ";\n";
+        out << "                    fr[" << stepOfK << " * 64 + " << groupOfK << " * 16 + ((x + k) & 15)] = h == 0 ? rv[it].x : rv[it].y;\n";
+        out << "                }\n            }\n";
+        if (np > 0)
+        {
+            out << "            for (int z = lane; z < " << np * 16 << "; z += 64)\n            {\n";
+            out << "                const int w = z / 16;\n";
+            out << "                fr[(" << sOfW << ") * 64 + (" << gOfW << ") * 16 + (z & 15)] = 0.0;\n            }\n";
+        }
+        // (a wavefront's LDS accesses complete in program order: no workgroup barrier between its writes and its reads)
+        out << "            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");\n            __builtin_amdgcn_wave_barrier();\n";
+        out << "#pragma unroll\n            for (int s = 0; s < " << steps << "; ++s) a[s] = fr[s * 64 + g * 16 + ((c + " << termOf("s") << ") & 15)];\n";
+        out << "        }\n";
+        out << "        __syncthreads();   // every strip is in registers: the column factor's fragments take the place\n";
+    }
+    // ---- staged values to their fragments
+    for (const Staged &f : staged)
+    {
+        const long size = f.rows * K;
+        out << "        {\n            double *fr = frag + " << f.base << ";\n";
+        out << "            const long base = " << f.offset << "L + e * " << size << "L;\n";
+        out << "            const int lead = (int)(base - (base & ~15L));   // doubles between the line boundary and the matrix\n";
+        out << "#pragma unroll\n            for (int it = 0; it < " << itsOf(f) << "; ++it)\n            {\n";
+        out << "#pragma unroll\n                for (int h = 0; h < 2; ++h)\n                {\n";
+        out << "                    const int j = 2 * (it * " << LT << " + lt) + h - lead;\n";
+        out << "                    if (j < 0 || j >= " << size << ") continue;\n";
+        if (f.kFast)
+            out << "                    const int x = j / " << K << ", k = j % " << K << ";\n";
+        else
+            out << "                    const int k = j / " << f.rows << ", x = j % " << f.rows << ";\n";
+        out << "                    fr[((x / 16) * " << steps << " + " << stepOfK << ") * 64 + " << groupOfK << " * 16 + ((x + k) & 15)] = h == 0 ? "
+            << f.name << "v[it].x : " << f.name << "v[it].y;\n";
+        out << "                }\n            }\n";
+        if (np > 0)
+        {
+            out << "            for (int z = lt; z < " << f.blocks * np * 16 << "; z += " << LT << ")\n            {\n";
+            out << "                const int blk = z / " << np * 16 << ", w = (z / 16) % " << np << ";\n";
+            out << "                fr[(blk * " << steps << " + " << sOfW << ") * 64 + (" << gOfW << ") * 16 + (z & 15)] = 0.0;\n            }\n";
+        }
+        out << "        }\n";
+    }
+    out << "        acro_double4 acc[" << TJ << "];\n";
+    out << "#pragma unroll\n        for (int J = 0; J < " << TJ << "; ++J) acc[J] = acro_double4{0.0, 0.0, 0.0, 0.0};\n";
+    out << "        __syncthreads();\n";
+    out << "#pragma unroll\n        for (int s = 0; s < " << steps << "; ++s)\n        {\n";
+    out << "            const int q = g * 16 + ((c + " << termOf("s") << ") & 15);   // this lane's place in a fragment of step s\n";
+    out << "#pragma unroll\n            for (int J = 0; J < " << TJ << "; ++J)\n";
+    out << "                acc[J] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[s], frag[(J * " << steps << " + s) * 64 + q], acc[J], 0, 0, 0);\n";
+    out << "        }\n";
+    out << "        __syncthreads();   // every fragment has been read: the tiles of the results take their place\n";
+    out << "        {\n";
+    out << "            double *tile = lds + slot * " << MN << ";\n";
+    out << "#pragma unroll\n            for (int J = 0; J < " << TJ << "; ++J)\n";
+    out << "#pragma unroll\n                for (int q = 0; q < 4; ++q)\n                {\n";
+    out << "                    const int m = 16 * strip + 4 * q + g, n = 16 * J + c;\n";
+    out << "                    if (m < " << M << " && n < " << N << ") tile[m * " << N << " + n] = acc[J][q];\n";
+    out << "                }\n        }\n";
+    out << "        __syncthreads();\n";
+    out << "        {   // LDS tiles -> device memory: the entries of the workgroup are one contiguous range; 16 bytes per lane, whole lines per instruction\n";
+    out << "            const int count = (int)(" << E << " - e0 < " << NBE << " ? " << E << " - e0 : " << NBE << ") * " << MN << ";\n";
+    out << "            const long base = " << aOff << "L + e0 * " << MN << "L, first = base & ~15L;\n";
+    const bool streams = s.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0;
+    const std::string combine = s.op == '=' ? "" : (s.op == '+' ? "+" : "-");
+    out << "            for (int i = threadIdx.x; 2 * i < count + 15; i += " << NT << ")\n            {\n";
+    out << "                const long at = first + 2 * i;\n";
+    out << "                const int j = (int)(at - base);\n";
+    out << "                if (j >= 0 && j + 1 < count)\n                {\n";
+    out << "                    acro_pair v = {lds[j], lds[j + 1]};\n";
+    out << "                    acro_pair *d = reinterpret_cast<acro_pair *>(" << A << " + at);\n";
+    if (s.op == '=')
+        out << "                    " << (streams ? "__builtin_nontemporal_store(v, d);" : "*d = v;") << "\n";
+    else
+        out << "                    *d = *d " << combine << " v;\n";
+    out << "                }\n                else\n                {\n";
+    for (int h = 0; h < 2; ++h)
+    {
+        const std::string jj = h == 0 ? "j" : "j + 1", aa = h == 0 ? "at" : "at + 1";
+        out << "                    if (" << jj << " >= 0 && " << jj << " < count) " << A << "[" << aa << "] = "
+            << (s.op == '=' ? "" : A + "[" + aa + "] " + combine + " ") << "lds[" << jj << "];\n";
+    }
+    out << "                }\n            }\n";
+    out << "        }\n";
+    out << "    }\n}\n";
+
+    plan.source = out.str();
+    plan.nb = static_cast<int>(NBE);
+    plan.lds_bytes = static_cast<int>(ldsDoublesHere * 8);
+    FillParams(plan, false);
+    HipLaunch launch;
+    launch.function_name = plan.module_name;
+    launch.grid = static_cast<unsigned>(groups);
+    launch.block = static_cast<unsigned>(NT);
+    for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
+    plan.launches.push_back(launch);
+}
+
+}  // namespace codegen
+}  // namespace acro

@@ -36,6 +36,11 @@ auto Generator::Run() -> HipKernelPlan
         EmitTranspose(plan);
         return plan;
     }
+    if (UseProductSchedule())
+    {
+        EmitProduct(plan);
+        return plan;
+    }
     if (UseOperatorSchedule())
     {
         EmitOperator(plan);

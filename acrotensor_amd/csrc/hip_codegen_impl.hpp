@@ -10,6 +10,7 @@
 //   codegen_reduction.cpp  the reduction schedule (few outputs, long contraction) and the kernel-parameter helpers
 //   codegen_transpose.cpp  the transpose schedule (32 x 32 tiles through LDS)
 //   codegen_operator.cpp   the operator schedules (a dense operator applied to every entry, on the FP64 matrix cores)
+//   codegen_product.cpp    the product schedule (products of element matrices on the FP64 matrix cores)
 //   codegen_chain.cpp      emission of the fused chain kernel: phases, prefetch, item loops, LDS copy-out
 #ifndef ACRO_HIP_CODEGEN_IMPL_HPP
 #define ACRO_HIP_CODEGEN_IMPL_HPP
@@ -386,6 +387,20 @@ class Generator
     bool UseGramSchedule() const;
     void EmitGram(HipKernelPlan &plan);
     void EmitTranspose(HipKernelPlan &plan);
+
+    // "A_e_r_c = R_e_{r,k} C_e_{k,c}": products of element matrices on the FP64 matrix cores (codegen_product.cpp)
+    struct ProductShape
+    {
+        const VarRef *row = nullptr, *col = nullptr;   // the factor that carries the result's row / column index
+        bool rowKFast = false, colKFast = false;       // the contracted index is the factor's fastest dimension
+        long M = 0, N = 0, K = 0, E = 0;
+        bool pairMap = false;                          // the terms of a step are permuted so that 16-byte loads feed two steps
+        int rowMode = 0;                               // how the row factor reaches the registers, see ProductPattern
+        long steps = 0, TI = 0, TJ = 0, NBE = 1, ldsPerEntry = 0;
+    };
+    bool ProductPattern(const Sub &s, ProductShape &p) const;
+    bool UseProductSchedule() const;
+    void EmitProduct(HipKernelPlan &plan);
 
     // ------------------------------------------------------------------------------ operator schedule
     // One dense operator applied to every batch entry: "A_e_i = B_i_j X_e_j" with B too large for scalar operands or a

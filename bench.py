@@ -224,6 +224,14 @@ KERNEL_SHAPES = [
     ("A_e_i_j = B_e_i_k C_e_k_j", [(138654, 11, 11), (138654, 11, 11)], (138654, 11, 11)),
     ("A_e_i_j = B_e_i_k C_e_k_j", [(26843, 25, 25), (26843, 25, 25)], (26843, 25, 25)),
     ("A_e_i_j = B_e_i_k C_e_k_j", [(10485, 40, 40), (10485, 40, 40)], (10485, 40, 40)),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(15406, 33, 33), (15406, 33, 33)], (15406, 33, 33)),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(12255, 37, 37), (12255, 37, 37)], (12255, 37, 37)),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(7281, 48, 48), (7281, 48, 48)], (7281, 48, 48)),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(5972, 53, 53), (5972, 53, 53)], (5972, 53, 53)),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(5546, 55, 55), (5546, 55, 55)], (5546, 55, 55)),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(4227, 63, 63), (4227, 63, 63)], (4227, 63, 63)),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(4096, 64, 64), (4096, 64, 64)], (4096, 64, 64)),
+    ("A_e_i_j = B_e_i_k C_e_j_k", [(4096, 64, 64), (4096, 64, 64)], (4096, 64, 64)),
     ("A_i = C_i_j B_j", [(1 << 20, 64), (64,)], (1 << 20,)),
     ("M_e_i1_i2_j1_j2 = B_k1_i1 B_k1_j1 B_k2_i2 B_k2_j2 D_e_k1_k2", [(5, 4)] * 4 + [(1 << 19, 5, 5)], (1 << 19, 4, 4, 4, 4)),
     ("A_i_j = B_j_i", [(1 << 22, 16)], (16, 1 << 22)),
@@ -240,6 +248,17 @@ KERNEL_SHAPES = [
     ("Y_e_i_j = B_q_i B_r_j D_e_q_r U_e_q_r", [(5, 4), (5, 4), (1 << 20, 5, 5), (1 << 20, 5, 5)], (1 << 20, 4, 4)),
     ("U_e_q_r_s = B_q_i B_r_j B_s_k X_e_i_j_k", [(5, 4), (5, 4), (5, 4), (1 << 18, 4, 4, 4)], (1 << 18, 5, 5, 5)),
 ]
+
+
+def schedule_line(source):
+    """The first line of the schedule comment of a generated kernel (after "// Generated by ...", past notes in
+    brackets)."""
+    lines = source.splitlines()
+    for i, line in enumerate(lines):
+        if line.startswith("// Generated by"):
+            rest = [l for l in lines[i + 1:i + 4] if not l.startswith("// (")]
+            return rest[0][3:] if rest else ""
+    return ""
 
 
 def kernel_shapes(at, args):
@@ -283,7 +302,7 @@ def kernel_shapes(at, args):
                         "algorithmic_bytes": abytes, "frac": abytes / launch_s * 1e-9 / HBM_PEAK_GBS,
                         "buffer_sets": n_sets, "launch_us_cold": cold_s * 1e6,
                         "frac_cold": abytes / cold_s * 1e-9 / HBM_PEAK_GBS,
-                        "schedule": engine.GetLastImplementation().splitlines()[1][3:]})
+                        "schedule": schedule_line(engine.GetLastImplementation())})
         del sets, tensors
     mean = math.exp(sum(math.log(r["frac"]) for r in results) / len(results))
     mean_cold = math.exp(sum(math.log(r["frac_cold"]) for r in results) / len(results))

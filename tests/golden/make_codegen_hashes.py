@@ -28,6 +28,8 @@ SINGLES = [
     ("operator_entries_fastest", "A_i_e = B_i_j X_j_e", [(32, 1 << 18), (32, 32), (32, 1 << 18)]),
     ("copy_out_tile", "A_e_i = B_i_j X_e_j", [(1 << 21, 27), (27, 3), (1 << 21, 3)]),
     ("transpose", "A_i_j = B_j_i", [(8192, 8192), (8192, 8192)]),
+    ("product_mfma_rows_in_pairs", "A_e_i_j = B_e_i_k C_e_k_j", [(4096, 64, 64), (4096, 64, 64), (4096, 64, 64)]),
+    ("product_mfma_strips_through_lds", "A_e_i_j = B_e_i_k C_e_j_k", [(5546, 55, 55), (5546, 55, 55), (5546, 55, 55)]),
     ("row_reduction", "S_i = A_i_n", [(64,), (64, 1 << 20)]),
     ("dsetup", "D_e_m_n_k1_k2_k3 = W_k1_k2_k3 C_e_k1_k2_k3 Jdet_e_k1_k2_k3 Jinv_e_k1_k2_k3_n_j Jinv_e_k1_k2_k3_m_j",
      [(16384, 3, 3, 10, 10, 10), (10, 10, 10), (16384, 10, 10, 10), (16384, 10, 10, 10), (16384, 10, 10, 10, 3, 3),

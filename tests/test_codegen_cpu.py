@@ -284,7 +284,7 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     assert "operator schedule" not in TE.GetImplementation("A_e_i = B_j_i X_e_j", at.Tensor(500, 64), at.Tensor(64, 64), at.Tensor(500, 64))
 
 
-def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE):
+def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE, monkeypatch):
     # one lane per matrix product would read 128-byte pieces 128 bytes apart; tiny entries get one output per lane
     src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 4, 4), at.Tensor(4096, 4, 4), at.Tensor(4096, 4, 4))
     assert "lanes(i,k)=16 tile()=1" in src
@@ -305,10 +305,14 @@ def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE):
     assert "operands staged in LDS" in src and "lanes(ihi,k)=125 tile(ilo)=5" in src
     src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 35, 35), at.Tensor(4096, 35, 35), at.Tensor(4096, 35, 35))
     assert "operands staged in LDS" in src and "lanes(ihi,k)=245 tile(ilo)=5" in src and "1 per workgroup of 256 lanes" in src
-    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 62, 62), at.Tensor(4096, 62, 62), at.Tensor(4096, 62, 62))
+    # (beyond 36 x 36, and for extents without a divisor 2, 3 or 5, products run on the matrix cores: see the test of
+    # the product schedule; this is what the staged schedule does with them when that is switched off)
+    monkeypatch.setenv("ACRO_HIP_PRODUCT", "-1")
+    src = at.TensorEngine("HIP").GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 62, 62), at.Tensor(4096, 62, 62), at.Tensor(4096, 62, 62))
     assert "operands staged in LDS" in src and "LDS 61504 bytes" in src
-    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 64, 64), at.Tensor(4096, 64, 64), at.Tensor(4096, 64, 64))
+    src = at.TensorEngine("HIP").GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 64, 64), at.Tensor(4096, 64, 64), at.Tensor(4096, 64, 64))
     assert "operands staged in LDS" not in src
+    monkeypatch.delenv("ACRO_HIP_PRODUCT")
     # second factor transposed: its copy in LDS has the contracted index in front, the copying lanes follow the operand
     src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_k_j", at.Tensor(4096, 24, 24), at.Tensor(4096, 24, 24), at.Tensor(4096, 24, 24))
     assert "_S2_e_j_khi_klo = C_e_khi_klo_j : lanes(khi,klo,j)=576" in src
@@ -554,3 +558,54 @@ def test_bad_kernel_strings_fail_before_code_generation():
     TE = at.TensorEngine("HIP")
     with pytest.raises(at.AcroError):
         TE.GetImplementation("A_i = b_i", at.Tensor(3), at.Tensor(3))
+
+
+def test_products_of_element_matrices_run_on_the_matrix_cores(TE, monkeypatch):
+    """The product schedule (codegen_product.cpp): which products take it, how each factor reaches the instruction's
+    operand layout, and what does not qualify."""
+    def product(kernel, M, N, K, E=4096):
+        ext = {"e": E, "i": M, "j": N, "k": K}
+        lhs, rhs = kernel.replace("+=", "=").replace("-=", "=").split("=")
+        tensors = [at.Tensor(*[ext[x] for x in tok.split("_")[1:]]) for tok in [lhs.split()[0]] + rhs.split()]
+        return at.TensorEngine("HIP").GetImplementation(kernel, *tensors)
+
+    # rows of a multiple of 128 bytes along the contracted index: the row factor straight into registers in pairs
+    # (terms permuted), the column factor through LDS; four strips, one entry per workgroup of 256 lanes
+    src = product("A_e_i_j = B_e_i_k C_e_k_j", 64, 64, 64)
+    assert "product schedule on the FP64 matrix cores: 64 x 64 by 64 x 64 per entry" in src
+    assert "read straight into registers" in src and "(terms in pairs)" in src and "1 entry per workgroup of 256 lanes, LDS 32768 bytes" in src
+    assert "const int k = 8 * u + 2 * g;" in src and src.count("__syncthreads()") == 3
+    assert "acc[J] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[s], frag[(J * 16 + s) * 64 + q], acc[J], 0, 0, 0);" in src
+    assert "__builtin_nontemporal_store(v, d);" in src
+    # other rows along the contracted index: every wavefront passes its strip, a contiguous range, through LDS
+    src = product("A_e_i_j = B_e_i_k C_e_k_j", 53, 53, 53)
+    assert "strips through LDS" in src and "14 steps of four terms," in src and "LDS 28672 bytes" in src
+    assert "const int x = j / 53, k = j % 53;" in src and '__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");' in src
+    assert src.count("__syncthreads()") == 4
+    # terms past the end are zero in both factors' fragments (53 = 13 * 4 + 1: three places of the last step)
+    assert "fr[(13) * 64 + (1 + w) * 16 + (z & 15)] = 0.0;" in src and "fr[(blk * 14 + 13) * 64 + (1 + w) * 16 + (z & 15)] = 0.0;" in src
+    # the row factor with the contracted index first: 128 contiguous bytes per term, straight into registers
+    src = product("A_e_i_j = B_e_k_i C_e_k_j", 40, 40, 40)
+    assert "row factor with the contracted index first, read straight into registers" in src and "a[s] = k < 40 ? rm[k * 40 + m] : 0.0;" in src
+    # the column factor either way round, the factors in either order, accumulation into the result
+    src = product("A_e_i_j -= C_e_j_k B_e_i_k", 37, 45, 20)
+    assert "37 x 20 by 20 x 45 per entry" in src and "column factor with the contracted index last" in src
+    assert "*d = *d - v;" in src and "nontemporal" not in src
+    # small matrices: two entries per workgroup
+    src = product("A_e_i_j = B_e_i_k C_e_k_j", 31, 31, 31)
+    assert "2 strips of 16 rows x 2 blocks of 16 columns" in src and "2 entries per workgroup of 256 lanes" in src
+    # an odd number of doubles in the whole tensor: its last one is read on its own
+    src = product("A_e_i_j = B_e_i_k C_e_k_j", 17, 17, 17, E=4097)
+    assert "if (it == " in src and "cv[it].x = T2[1184032L];" in src
+    # not this schedule: small matrices whose extents the staged schedule can split into blocks, 16 x 16 and smaller,
+    # a shared factor, more than two factors, too few entries for e to be the batch index
+    assert "product schedule" not in product("A_e_i_j = B_e_i_k C_e_k_j", 24, 24, 24)
+    assert "product schedule" not in product("A_e_i_j = B_e_i_k C_e_k_j", 16, 16, 16)
+    assert "product schedule" not in TE.GetImplementation("A_e_i_j = B_e_i_k C_k_j", at.Tensor(4096, 40, 40), at.Tensor(4096, 40, 40), at.Tensor(40, 40))
+    assert "product schedule" not in TE.GetImplementation("A_e_i_j = B_e_i_k C_e_k_j D_e", at.Tensor(4096, 40, 40), at.Tensor(4096, 40, 40),
+                                                          at.Tensor(4096, 40, 40), at.Tensor(4096))
+    assert "product schedule" not in product("A_e_i_j = B_e_i_k C_e_k_j", 50, 50, 50, E=30)
+    # ... and it is a matrix-core schedule: off where those are refused
+    monkeypatch.setenv("ACRO_HIP_TEST_PRIVATE_BYTES", "8,8")
+    src = product("A_e_i_j = B_e_i_k C_e_k_j", 64, 64, 64)
+    assert "product schedule" not in src and "was refused" in src

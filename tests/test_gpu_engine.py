@@ -223,14 +223,11 @@ def test_products_of_element_matrices_stage_their_operands_in_lds(at, engine, ch
     ("A_e_i_j = B_e_i_k C_e_k_j D_e_i_j", [(31, 24, 8), (31, 8, 25), (31, 24, 25)], "tile(ilo)=2"),
     # no blocks: one output per lane, several entries per workgroup; rows of odd length are padded in LDS
     ("A_e_i_j = B_e_i_k C_e_k_j", [(203, 11, 11), (203, 11, 11)], "8 per workgroup of 256 lanes"),
-    ("A_e_i_j += B_e_i_k C_e_k_j", [(29, 23, 23), (29, 23, 23)], "LDS 8832 bytes"),
     # divisible by five only: blocks of five along one index while a hundred lane items are left per entry
     ("A_e_i_j += B_e_i_k C_e_k_j", [(29, 25, 25), (29, 25, 25)], "lanes(ihi,j)=125 tile(ilo)=5"),
     ("A_e_i_j = B_e_i_k C_e_k_j", [(41, 25, 15), (41, 15, 20)], "lanes(ihi,jhi)=50 tile(ilo,jlo)=10"),
     # larger than 32 x 32: an entry's operands fill most of a workgroup's LDS
     ("A_e_i_j -= B_e_i_k C_e_k_j", [(39, 35, 35), (39, 35, 35)], "lanes(ihi,j)=245 tile(ilo)=5"),
-    ("A_e_i_j = B_e_k_i C_e_j_k", [(51, 47, 45), (51, 40, 47)], "1 per workgroup of 256 lanes"),
-    ("A_e_i_j = B_e_i_k C_e_k_j", [(67, 62, 62), (67, 62, 62)], "LDS 61504 bytes"),
 ])
 def test_products_of_small_element_matrices(at, engine, checker, kernel, shapes, expect):
     rng = np.random.default_rng(len(kernel) + shapes[0][0])
@@ -242,6 +239,73 @@ def test_products_of_small_element_matrices(at, engine, checker, kernel, shapes,
     if "-=" in kernel:
         expected = 2.0 * out0 - expected
     assert rel_err(got, expected) <= TOL
+
+
+PRODUCTS_ON_THE_MATRIX_CORES = [
+    # (kernel, shapes of the inputs in the order written): square and rectangular, every combination of layouts,
+    # extents that are multiples of 16 and extents that are not, odd tensors, the factors in either order
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(67, 64, 64), (67, 64, 64)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(129, 63, 63), (129, 63, 63)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(71, 55, 55), (71, 55, 55)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(64, 53, 53), (64, 53, 53)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(100, 37, 37), (100, 37, 37)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(101, 33, 29), (101, 29, 41)]),
+    ("A_e_i_j = B_e_i_k C_e_j_k", [(75, 62, 62), (75, 62, 62)]),
+    ("A_e_i_j = B_e_k_i C_e_k_j", [(80, 48, 56), (80, 48, 40)]),
+    ("A_e_i_j = B_e_k_i C_e_j_k", [(51, 47, 45), (51, 40, 47)]),
+    ("A_e_i_j += B_e_i_k C_e_k_j", [(29, 23, 23), (29, 23, 23)]),
+    ("A_e_i_j -= C_e_j_k B_e_i_k", [(90, 45, 20), (90, 37, 20)]),
+    ("A_e_i_j += B_e_k_i C_e_k_j", [(1001, 9, 17), (1001, 9, 64)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(333, 19, 128), (333, 128, 8)]),
+    ("A_e_i_j -= B_e_i_k C_e_j_k", [(257, 31, 31), (257, 31, 31)]),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kernel,shapes", PRODUCTS_ON_THE_MATRIX_CORES)
+def test_products_of_element_matrices_on_the_matrix_cores_random(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(len(kernel) + shapes[0][0])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "product schedule on the FP64 matrix cores" in engine.GetLastImplementation()
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kernel,shapes", PRODUCTS_ON_THE_MATRIX_CORES)
+def test_products_of_element_matrices_on_the_matrix_cores_integer_exact(at, engine, checker, kernel, shapes):
+    """Integer-valued data: sums in any order are exact, so every entry, row, column and term must be in its place
+    (also the ones next to the padding of blocks of 16 rows or columns and of steps of four terms)."""
+    rng = np.random.default_rng(7 * len(kernel) + shapes[0][1])
+    ins = [rng.integers(-5, 6, s).astype(np.float64) for s in shapes]
+    out0 = rng.integers(-5, 6, output_shape(kernel, shapes)).astype(np.float64)
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "product schedule on the FP64 matrix cores" in engine.GetLastImplementation()
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert np.array_equal(got, expected)
+
+
+@pytest.mark.gpu
+def test_products_of_element_matrices_on_the_matrix_cores_views_and_odd_tensors(at, engine, checker):
+    """Factors and results that are slices at odd offsets of larger tensors, and tensors with an odd number of
+    doubles (whose last one cannot be read as part of a pair)."""
+    rng = np.random.default_rng(99)
+    E, n = 65, 19                                           # 65 * 19 * 19 doubles: odd; slices start at odd offsets
+    B3, C3, A3 = (rng.integers(-4, 5, (3, E, n, n)).astype(np.float64) for _ in range(3))
+    tB, tC, tA = (to_tensor(at, x) for x in (B3, C3, A3))
+    for which in (1, 2):
+        sB, sC, sA = (at.SliceTensor(t, which) for t in (tB, tC, tA))
+        engine("A_e_i_j = B_e_i_k C_e_j_k", sA, sB, sC)
+        assert "product schedule on the FP64 matrix cores" in engine.GetLastImplementation()
+    tA.MoveFromGPU()
+    expected = A3.copy()
+    for which in (1, 2):
+        checker.contract("A_e_i_j = B_e_i_k C_e_j_k", expected[which], np.ascontiguousarray(B3[which]), np.ascontiguousarray(C3[which]))
+    assert np.array_equal(tA.data, expected)                # also: nothing outside the slices was touched
 
 
 def test_product_of_slices_keeps_its_indices(at, engine, checker):
