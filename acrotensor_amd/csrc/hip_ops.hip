@@ -3,10 +3,11 @@
 // inverse+determinant (reference ops/CudaGPUOps.cpp:13-80,108-275), indexed scatter and compressed-row sum-gather
 // (reference ops/CudaGPUOps.cpp:83-105,278-302).
 //
-// Layout: matrices are stored one after the other (9, 4 or 1 doubles each).  A workgroup of 256 lanes owns 256
-// consecutive matrices; it moves their doubles between HBM and LDS with unit-stride 16-byte accesses and each
-// lane then works on "its" matrix out of LDS, so HBM only sees full, contiguous lines.  The lane stride in LDS is
-// 9 (or 4+1 padded to 5) doubles, which maps the 32 lanes of a half wave onto distinct banks.
+// Layout: matrices are stored one after the other (9, 4 or 1 doubles each).  A workgroup of 64 lanes (one wavefront,
+// so its barriers cost nothing) owns 64 consecutive matrices; it moves their doubles between HBM and LDS with
+// unit-stride 16-byte accesses and each lane then works on "its" matrix out of LDS, so HBM only sees full,
+// contiguous lines.  The lane stride in LDS is 9 (or 4+1 padded to 5) doubles, which maps the lanes onto distinct
+// banks.  1 x 1 "matrices" have a plain streaming kernel of their own (256 lanes, four entries each).
 //
 // Arithmetic is written term by term in the order of the reference's ops/NativeCPUOps.hpp:38-86 and compiled
 // without multiply-add contraction, so results are bit-identical to the host formulas.

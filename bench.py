@@ -32,6 +32,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+ONLY_ROTATED = False   # --only-rotated
 METRIC = "GDOF/s + % HBM peak, p=3 sum-factorised hex mass apply fp64 (1 GPU)"
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the same counter
@@ -39,12 +40,16 @@ METRIC = "GDOF/s + % HBM peak, p=3 sum-factorised hex mass apply fp64 (1 GPU)"
 # function, first 16 hex digits of the SHA-1 of the generated source).  A generator change that alters the source of
 # a kernel therefore drops its figure (the line then says null) until the counters are taken again.
 TRAFFIC_BY_KERNEL = {
-    ("acro_mk_4ceea56515f0c53c", "7b71a034a2a078a5"): 541797694,            # cfg4, intermediates transient
-    ("acro_mk_664cf228dc3d274e", "bb5ff2ad54f2a970"): 1815899708,           # cfg4, every intermediate stored
-    ("acro_red_35ac69981569e511_partial", "1698cfe138e16625"): 83942935,    # cfg1 (first of its two launches)
-    ("batchMatrixKernel<3,inv,det>", "ad5dc2a53b830c72"): 637584186,        # cfg2 (precompiled: hash of hip_ops.hip)
-    ("acro_mk_c7f1f43821aef74f", "19c88bbbd31b17c8"): 208703260,            # cfg3
-    ("acro_mk_e688ac87da28a7bd", "018c1f37edc57625"): 5258953433,           # cfg5
+    ("acro_mk_4ceea56515f0c53c", "7b71a034a2a078a5"): 541935762,            # cfg4, intermediates transient
+    ("acro_mk_664cf228dc3d274e", "bb5ff2ad54f2a970"): 1815908764,           # cfg4, every intermediate stored
+    ("acro_red_35ac69981569e511_partial", "1698cfe138e16625"): 83942611,    # cfg1 (first of its two launches)
+    ("batchMatrixKernel<3,inv,det>", "bc2ddd23143ef404"): 637579842,        # cfg2 (precompiled: hash of hip_ops.hip)
+    ("acro_mk_567e3a4d341f4dc2", "663c472f29b65c65"): 210843823,            # cfg3
+    ("acro_mk_e688ac87da28a7bd", "018c1f37edc57625"): 5258883071,           # cfg5
+    ("scatterKernel2", "bc2ddd23143ef404"): 261167030,                      # node vector -> element vector
+    ("sumGatherKernel", "bc2ddd23143ef404"): 317995671,                     # element vector -> node vector
+    ("acro_mk_e5e3c68e773e2587", "2f278ec4d44c8ab3"): 2517040325,           # geometric factors from the Jacobians, one launch
+    ("acro_mk_ff9b33d31033d4fa", "810d4b7e198a2fdb"): 609195587,            # scatter read through the map by the mass apply
 }
 
 
@@ -282,12 +287,13 @@ def kernel_shapes(at, args):
                 t.Set(0.5)
             sets.append(tensors)
         step = lambda i=0: engine(kernel, sets[i][-1], *sets[i][:-1])
-        for _ in range(5):
-            step()
+        same = (lambda k: k % n_sets) if ONLY_ROTATED else (lambda k: 0)
+        for k in range(5):
+            step(same(k))
         at.synchronize()
         with at.hip_event_timer() as ev:
-            for _ in range(steps):
-                step()
+            for k in range(steps):
+                step(same(k))
         launch_s = ev.ms * 1e-3 / steps
         rounds = max(2, -(-steps // n_sets))
         for i in range(n_sets):
@@ -330,7 +336,8 @@ def next_rows(at, workloads, args):
             "workload": label, "launch_us": launch_s * 1e6, "algorithmic_bytes": abytes, "frac": roofline["frac"],
             "buffer_sets": roofline["buffer_sets"], "launch_us_cold": roofline["launch_us_cold"],
             "frac_cold": roofline["frac_cold"], "value_cold": units / (roofline["launch_us_cold"] * 1e-6) * 1e-9,
-            "unit": unit_name, "kernel": roofline["kernel"], "kernel_source_sha1_16": roofline["kernel_source_sha1_16"],
+            "unit": unit_name, "traffic": roofline["traffic"], "kernel": roofline["kernel"],
+            "kernel_source_sha1_16": roofline["kernel_source_sha1_16"],
         }
         del engine, steps_list
         if args.no_cpu_baseline:
@@ -590,6 +597,14 @@ def measure_case(at, engine, steps_list, abytes, flops, steps, warmup, settle_se
     if callable(steps_list):
         steps_list = [steps_list]
     step = steps_list[0]
+    if ONLY_ROTATED and len(steps_list) > 1:
+        # every launch of the run, settling and warm-up included, goes round-robin over the buffer sets (for kernel
+        # traces, whose per-kernel averages then are those of launches on data that comes from HBM)
+        turn = [0]
+
+        def step():
+            turn[0] += 1
+            steps_list[turn[0] % len(steps_list)]()
     # sustained load before anything is timed (see settle_clocks): bursts of launches, not one launch per
     # synchronisation, or the device drops back to idle clocks between them
     for s in steps_list:
@@ -742,6 +757,10 @@ def main():
     ap.add_argument("--rotate", type=int, default=0,
                     help="buffer sets that the cold figures rotate over: 0 (default) as many as it takes to exceed 1 GiB "
                          "together, 1 none (cold figures then repeat the ordinary ones), N that many")
+    ap.add_argument("--only-rotated", action="store_true",
+                    help="every launch of the run (settling, warm-up, timed) goes round-robin over the buffer sets, so a "
+                         "kernel trace of the run averages launches on data from HBM only; the same-buffer figures of "
+                         "the line then repeat the rotated ones")
     ap.add_argument("--elements", type=int, default=262144)
     ap.add_argument("--cpu-sample-elems", type=int, default=262144)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -759,6 +778,8 @@ def main():
                     help="also run one scale-by-1.0 kernel over X (reads and writes E*512 bytes): the known-size "
                          "kernel that hardware-counter runs are scaled by")
     args = ap.parse_args()
+    global ONLY_ROTATED
+    ONLY_ROTATED = args.only_rotated
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the workload shards over elements "
                  "without any exchange, so N GPUs would each run this same kernel on 1/N of them).  Run with --gpus 1.")
@@ -797,8 +818,14 @@ def main():
         tensors["X"].Mult(1.0)
         at.synchronize()
 
-    settle_clocks(at, workloads, wl, engine, tensors, args.settle_seconds)
-    wall, dev = time_steps(at, workloads, wl, engine, tensors, args.steps, args.warmup)
+    if ONLY_ROTATED:
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < args.settle_seconds:
+            time_steps_rotating(at, workloads, wl, engine, sets, 100, 0)
+        wall, dev = time_steps_rotating(at, workloads, wl, engine, sets, args.steps, args.warmup)
+    else:
+        settle_clocks(at, workloads, wl, engine, tensors, args.settle_seconds)
+        wall, dev = time_steps(at, workloads, wl, engine, tensors, args.steps, args.warmup)
     ms_per_step = wall / args.steps * 1e3
     launch_s = dev / args.steps
     achieved = wl.algorithmic_bytes / launch_s * 1e-9
@@ -861,8 +888,11 @@ def main():
         # The first launch compiles the other kernel while the device idles: settle again before timing.
         workloads.launch(wl, engine, tensors)
         at.synchronize()
-        settle_clocks(at, workloads, wl, engine, tensors, args.settle_seconds)
-        wall2, dev2 = time_steps(at, workloads, wl, engine, tensors, n2, max(5, args.warmup // 4))
+        if ONLY_ROTATED:
+            wall2, dev2 = time_steps_rotating(at, workloads, wl, engine, sets, n2, max(5, args.warmup // 4))
+        else:
+            settle_clocks(at, workloads, wl, engine, tensors, args.settle_seconds)
+            wall2, dev2 = time_steps(at, workloads, wl, engine, tensors, n2, max(5, args.warmup // 4))
         wall2c, dev2c = time_steps_rotating(at, workloads, wl, engine, sets, n2, max(5, args.warmup // 4))
         stored_bytes = args.elements * (64 + 125 + 64 + 610) * 8
         moved = stored_bytes / (dev2 / n2) * 1e-9

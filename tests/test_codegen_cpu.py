@@ -575,7 +575,7 @@ def test_products_of_element_matrices_run_on_the_matrix_cores(TE, monkeypatch):
     assert "product schedule on the FP64 matrix cores: 64 x 64 by 64 x 64 per entry" in src
     assert "read straight into registers" in src and "(terms in pairs)" in src and "1 entry per workgroup of 256 lanes, LDS 32768 bytes" in src
     assert "const int k = 8 * u + 2 * g;" in src and src.count("__syncthreads()") == 3
-    assert "acc[J] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[s], frag[(J * 16 + s) * 64 + q], acc[J], 0, 0, 0);" in src
+    assert "acc[J] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[s], frag[(J * 16 + s) * 64 + g * 16 + acro_place(16 * J + c, k)], acc[J], 0, 0, 0);" in src
     assert "__builtin_nontemporal_store(v, d);" in src
     # other rows along the contracted index: every wavefront passes its strip, a contiguous range, through LDS
     src = product("A_e_i_j = B_e_i_k C_e_k_j", 53, 53, 53)
@@ -596,7 +596,7 @@ def test_products_of_element_matrices_run_on_the_matrix_cores(TE, monkeypatch):
     assert "2 strips of 16 rows x 2 blocks of 16 columns" in src and "2 entries per workgroup of 256 lanes" in src
     # an odd number of doubles in the whole tensor: its last one is read on its own
     src = product("A_e_i_j = B_e_i_k C_e_k_j", 17, 17, 17, E=4097)
-    assert "if (it == " in src and "cv[it].x = T2[1184032L];" in src
+    assert "if (at == 1184032L) cv[it].x = T2[1184032L];" in src
     # not this schedule: small matrices whose extents the staged schedule can split into blocks, 16 x 16 and smaller,
     # a shared factor, more than two factors, too few entries for e to be the batch index
     assert "product schedule" not in product("A_e_i_j = B_e_i_k C_e_k_j", 24, 24, 24)
