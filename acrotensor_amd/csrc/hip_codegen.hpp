@@ -119,6 +119,20 @@
 //   ACRO_HIP_ONE_PASS=1         split contractions: the workgroup that finishes last adds the per-workgroup partials
 //                               instead of a second kernel (measured 18.4 against 16.3 us: the device-scope release
 //                               writes back the XCD's L2 once per workgroup)
+//   ACRO_HIP_RED_GROUPS=<n> / ACRO_HIP_RED_UNROLL=<n>
+//                               split contractions where a lane owns whole slices: number of workgroups (default 256, one per
+//                               compute unit) and slices a lane requests before it adds them (default 1)
+//   ACRO_HIP_PRODUCT=-1 / =2    products of two element matrices never / whenever they fit take the product schedule on the
+//                               matrix cores (default: from 17 rows or columns on, except sizes up to 36 that 2, 3 or 5 divide)
+//   ACRO_HIP_PRODUCT_FROM=<n> / ACRO_HIP_PRODUCT_TO=<n>   smallest and largest "larger of rows and columns" it takes (17, 128)
+//   ACRO_HIP_PRODUCT_ENTRIES=<n>  entries per workgroup of the product schedule (default: up to 4 wavefronts, 8 192 LDS values)
+//   ACRO_HIP_PRODUCT_DIRECT=-1  the row factor always passes through LDS, also where lanes could load their operands directly
+//   ACRO_HIP_COPY_OUT_COVERAGE=<percent>  share of the touched lines below which the last kernel's stores leave through an
+//                               LDS tile (default 30);  ACRO_HIP_COPY_OUT_WRITERS=-1: launches whose stores dominate no
+//                               longer do so below 95 %
+//   ACRO_HIP_WRITE_BATCH_FROM=<n>  write-heavy launches that copy out of LDS tiles double their batch from this batch size on (1)
+//   ACRO_HIP_NT_COPY_OUT=-1     copies out of LDS tiles use non-temporal stores only for tiles of at most 20 KB
+//   ACRO_HIP_NT_STORE=2         non-temporal stores from registers also in launches that hold more than 20 KB of LDS per workgroup
 #ifndef ACRO_HIP_CODEGEN_HPP
 #define ACRO_HIP_CODEGEN_HPP
 
