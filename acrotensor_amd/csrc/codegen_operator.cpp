@@ -339,6 +339,18 @@ auto Generator::OperatorPair(OperatorShape &first, OperatorShape &second) const 
 
 // Index of the operator's entry (row, j) in its own memory: rows by columns, columns by rows, or any order of its
 // dimensions (then `row` and `j` are taken apart into the indices they number).
+// Head of the loop in which the 256 lanes of a workgroup fill `count` doubles of LDS (the body follows, then the closing
+// brace).  A counted loop that the compiler unrolls: all loads of a lane are in flight together.  Written as
+// "for (f = threadIdx.x; f < count; f += 256)" it stayed a loop of one load and one wait per turn, 16 round trips to
+// L2 for a 64 x 64 operator before a workgroup's first trip.
+static void FillLoopHead(std::ostream &out, long count)
+{
+    const long turns = (count + 255) / 256;
+    out << "#pragma unroll\n    for (int turn = 0; turn < " << turns << "; ++turn)\n    {\n";
+    out << "        const int f = threadIdx.x + 256 * turn;\n";
+    if (count % 256 != 0) out << "        if (f >= " << count << ") continue;\n";
+}
+
 auto Generator::OperatorEntry(const OperatorShape &shape, const std::string &row, const std::string &j, long allRows) const -> std::string
 {
     if (!shape.mixed) return shape.transposed ? j + " * " + str(allRows) + " + " + row : row + " * " + str(shape.cols) + " + " + j;
@@ -563,13 +575,22 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     const long midStride = nI % 2 == 0 ? nI + 1 : nI; // odd: the lanes' rows of the hand-over buffer start in different banks
     const long tiles = (E + 15) / 16;
     const bool ragged = E % 16 != 0;
-    // Equal work per CU matters more than the number of wavefronts: 256 CUs, one or two workgroups each.
-    // With one or two loads per lane and trip a wavefront has little in flight, and twice the wavefronts help
-    // once the tensors exceed the 256 MB of last-level cache (8 x 8 on 2^23 entries: 227 us with 512
-    // workgroups, 185 us with 1 024, 216 us with 2 048; 64 x 64 on 2^18: 47 / 54 / 62 us).
+    // Equal work per CU matters more than the number of wavefronts: 256 CUs, a whole number of workgroups each
+    // (640 workgroups: 10 - 15 % slower than 512 or 768 at every size).  How many is a matter of bytes in flight: a
+    // wavefront requests 128 x columns bytes per trip, and a CU needs some 20 KB of loads outstanding to keep its
+    // share of the memory system busy.  Measured on tensors that exceed the memory-side cache, % of the HBM peak with
+    // 256 / 512 / 768 / 1 024 workgroups: 8 x 8 - / 56 / 70 / 73, 10 x 10 - / 57 / 70 / 75, 12 x 12 - / 66 / 75 / 73,
+    // 8 x 16 - / 70 / 74 / 72, 17 x 17 43 / 65 / 74 / 73, 19 x 19 - / 71 / 75 / 72, 21 x 21 - / 69 / 73 / 68,
+    // 40 x 12 - / 66 / 71 / 67, 27 x 27 55 / 74 / 71 / 67, 32 x 32 66 / 74 / 72 / 72, 48 x 48 66 / 71 / 67 / 67,
+    // 64 x 64 on 2^18 entries 67 / 63 / - / 60, on 2^20 74 / 67 / - / 68, 128 x 32 78 / 72 / - / 74.
     // (An operator above 32 KB: one workgroup per CU, since every workgroup reads all of it.  192 x 64 on 2^15 entries:
-    // 34.6 -> 26.9 us; 375 x 125 on 2^17: 410 -> 320 us; 1 024 workgroups: 558 us.)
-    const long most = nIp * nJp > 4096 ? 256 : (pairs && nJp <= 16 ? 1024 : 512);
+    // 34.6 -> 26.9 us; 375 x 125 on 2^17: 410 -> 320 us; 1 024 workgroups: 558 us.  Results that leave through the
+    // LDS stage keep two: 60 x 60 59 against 50 %.)
+    long most = 512;
+    if (nIp * nJp > 4096 || (nIp * nJp == 4096 && nIp >= 32 && !viaStage)) most = 256;
+    else if (nJ <= 10) most = 1024;
+    else if (nJ <= 24) most = 768;
+    if (envInt("ACRO_HIP_OPERATOR_GROUPS") > 0) most = envInt("ACRO_HIP_OPERATOR_GROUPS");
     const long blocks = std::max<long>(1, std::min<long>(most, (tiles + 3) / 4));
     for (const auto &st : stores)
     {
@@ -614,7 +635,7 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
     out << "typedef double acro_pair __attribute__((ext_vector_type(2), aligned(8)));\n";
     out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << plan.module_name << "(" << ParamList() << ")\n{\n";
     out << "    __shared__ double frag[" << nIp * nJp << "];\n";
-    out << "    for (int f = threadIdx.x; f < " << nIp * nJp << "; f += 256)\n    {\n";
+    FillLoopHead(out, nIp * nJp);
     out << "        const int l = f & 63, step = (f >> 6) % " << steps << ", t = (f >> 6) / " << steps << ";\n";
     out << "        const int row = 16 * t + (l & 15), j = " << termOf << ";\n";
     const std::string rowHere = row0 > 0 ? "(row + " + str(row0) + ")" : std::string("row");
@@ -630,7 +651,7 @@ auto Generator::EmitOperatorMatrixCores(HipKernelPlan &plan, const OperatorShape
         const long rows2P = (next->rows + 15) / 16 * 16;
         out << "    __shared__ double frag2[" << rows2P * steps2 * 4 << "];\n";
         out << "    __shared__ double stage[" << 4 * 16 * midStride << "];\n";
-        out << "    for (int f = threadIdx.x; f < " << rows2P * steps2 * 4 << "; f += 256)\n    {\n";
+        FillLoopHead(out, rows2P * steps2 * 4);
         out << "        const int l = f & 63, step = (f >> 6) % " << steps2 << ", t = (f >> 6) / " << steps2 << ";\n";
         out << "        const int row = 16 * t + (l & 15), j = 4 * step + (l >> 4);\n";
         out << "        frag2[f] = row < " << next->rows << " && j < " << nI << " ? " << PtrName(next->op->uvar) << "[" << Lit(uvars[next->op->uvar].viewOffset)
@@ -881,7 +902,10 @@ auto Generator::ComponentsTogether(const OperatorShape &o) const -> bool
     if (o.comp <= 1 || o.comp > 16 || o.trailing || envInt("ACRO_HIP_OPERATOR_COMPONENTS") >= 2) return false;
     if (o.outMixed) return true;
     const long padded = ((o.rows + 15) / 16 * 16) * ((o.cols + 3) / 4 * 4);
-    return padded <= 1024 || (o.rows * o.cols > 4096 && o.cols <= 64);
+    // (on tensors that exceed the memory-side cache, entries (entry, component) against the components together:
+    // 64 x 27 x 3 58 -> 64 %, 48 x 48 x 2 66 -> 66 % (re-launched on the same tensors 66 -> 74 %), 64 x 64 x 3 67 -> 58 %;
+    // non-temporal stores of the single doubles C apart: slower everywhere, 27 x 27 x 3 62 -> 56 %)
+    return padded <= 2304 || (o.rows * o.cols > 4096 && o.cols <= 64);
 }
 
 auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape &shape) -> void
@@ -939,7 +963,7 @@ auto Generator::EmitOperatorComponents(HipKernelPlan &plan, const OperatorShape 
     out << (first ? "" : "\n") << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
     out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << plan.module_name << "(" << ParamList() << ")\n{\n";
     out << "    __shared__ double frag[" << nIp * nJp << "];\n";
-    out << "    for (int f = threadIdx.x; f < " << nIp * nJp << "; f += 256)\n    {\n";
+    FillLoopHead(out, nIp * nJp);
     out << "        const int l = f & 63, step = (f >> 6) % " << steps << ", t = (f >> 6) / " << steps << ";\n";
     out << "        const int row = 16 * t + (l & 15), j = 4 * step + (l >> 4);\n";
     const std::string rowHere = row0 > 0 ? "(row + " + str(row0) + ")" : std::string("row");
@@ -1100,7 +1124,7 @@ auto Generator::EmitOperatorEntriesFastest(HipKernelPlan &plan, const OperatorSh
     out << "typedef double acro_double2 __attribute__((ext_vector_type(2), aligned(8)));\n";
     out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << plan.module_name << "(" << ParamList() << ")\n{\n";
     out << "    __shared__ double frag[" << nIp * nJp << "];\n";
-    out << "    for (int f = threadIdx.x; f < " << nIp * nJp << "; f += 256)\n    {\n";
+    FillLoopHead(out, nIp * nJp);
     out << "        const int l = f & 63, step = (f >> 6) % " << steps << ", t = (f >> 6) / " << steps << ";\n";
     out << "        const int row = 16 * t + (l & 15), j = 4 * step + (l >> 4);\n";
     const std::string element = B + "[" + offsetOf(opr) + " + " + OperatorEntry(shape, "row", "j", nI) + "]";
