@@ -14,6 +14,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <cstdlib>
 
 #include "HipRuntime.hpp"
 #include "NonContractionOps.hpp"
@@ -297,8 +298,13 @@ __global__ __launch_bounds__(kLanes) void scatterKernel2(double *__restrict__ Ao
 // flight per lane whatever the row lengths are), then the lane of each row adds the part of its row that lies in
 // the chunk, in row order.  Rows are short on average (2.3 entries for a hexahedral mesh) and uneven (1 to 8), so
 // one lane walking its own row leaves most of a wavefront's gather slots empty.
-constexpr int kGatherChunk = 8 * kLanes;
-constexpr int kGatherRows = 4;  // rows per lane: a workgroup's range of entries should fill a chunk
+// A chunk should hold all entries of the workgroup's rows: every further chunk is another chain of dependent loads (map,
+// then values) behind a barrier.  Lines of mesh nodes that lie on element faces have 3.6 entries per row; with 1 024 rows
+// and chunks of 2 048 those workgroups took two chunks (64^3 hexahedra of degree 3, tensors that exceed the memory-side
+// cache: 59.5 us); 512 rows per chunk of 2 048, or 1 024 per 4 096: 55.2 us; 256 rows: 57.9 us; 2 048 rows: 64 us.
+constexpr int kGatherPerLane = 8;
+constexpr int kGatherChunk = kGatherPerLane * kLanes;
+constexpr int kGatherRows = 2;  // rows per lane
 
 __global__ __launch_bounds__(kLanes) void sumGatherKernel(double *__restrict__ Aout, const double *__restrict__ Ain,
                                                           const int *__restrict__ InvM,
@@ -322,18 +328,18 @@ __global__ __launch_bounds__(kLanes) void sumGatherKernel(double *__restrict__ A
     for (int c = first; c < last; c += kGatherChunk)
     {
         const int n = last - c < kGatherChunk ? last - c : kGatherChunk;
-        int idx[8];
-        double a[8];
+        int idx[kGatherPerLane];
+        double a[kGatherPerLane];
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
+        for (int u = 0; u < kGatherPerLane; ++u)
         {
             const int j = threadIdx.x + u * kLanes;
             idx[u] = j < n ? InvM[c + j] : -1;
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) a[u] = idx[u] >= 0 ? Ain[idx[u]] : 0.0;
+        for (int u = 0; u < kGatherPerLane; ++u) a[u] = idx[u] >= 0 ? Ain[idx[u]] : 0.0;
 #pragma unroll
-        for (int u = 0; u < 8; ++u) vals[threadIdx.x + u * kLanes] = a[u];
+        for (int u = 0; u < kGatherPerLane; ++u) vals[threadIdx.x + u * kLanes] = a[u];
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < kGatherRows; ++r)
