@@ -59,7 +59,7 @@ auto Generator::ProductPattern(const Sub &s, ProductShape &p) const -> bool
     p.E = extent[batch];
     // From 17 rows or columns on (up to 16 x 16 the staged schedule has a lane per output and is bound by memory);
     // a wavefront holds one strip of at most eight column blocks, an entry at most eight strips.
-    const long lo = envInt("ACRO_HIP_PRODUCT_FROM", 17), hi = envInt("ACRO_HIP_PRODUCT_TO", 128);
+    const long lo = envInt("ACRO_HIP_PRODUCT_FROM", 17), hi = envInt("ACRO_HIP_PRODUCT_TO", 64);
     if (std::max(p.M, p.N) < lo || p.M > hi || p.N > hi || p.K > 128 || p.K < 8 || p.M < 8 || p.N < 8) return false;
     // Up to 36 x 36 the staged vector-ALU schedule is as fast or a little faster where it can give a lane a block of
     // outputs, i.e. where both extents have a divisor 2, 3 or 5 (rotated buffers, % of the HBM peak, staged / here:
@@ -353,6 +353,233 @@ auto Generator::EmitProduct(HipKernelPlan &plan) -> void
     plan.source = out.str();
     plan.nb = static_cast<int>(NBE);
     plan.lds_bytes = static_cast<int>(ldsDoublesHere * 8);
+    FillParams(plan, false);
+    HipLaunch launch;
+    launch.function_name = plan.module_name;
+    launch.grid = static_cast<unsigned>(groups);
+    launch.block = static_cast<unsigned>(NT);
+    for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
+    plan.launches.push_back(launch);
+}
+
+// ---------------------------------------------------------------------------------------------- tiled products
+// Matrix products beyond what one workgroup can hold: "A_e_r_c (=|+=|-=) R_e_{r,k} C_e_{k,c}" with more than 64 rows or
+// columns or more than 128 terms, and the same without a batch index ("A_i_j = B_i_k C_k_j", a plain matrix product).
+// The reference gives every output a thread that walks the contracted index through device memory
+// (exec/CudaExecutor.cpp:193-263); so did the generic schedule here (128 x 128 per entry: 6 % of the HBM peak,
+// 2 048 x 2 048 unbatched: 4.8 TFLOP/s).
+//
+// A workgroup of W wavefronts owns a tile of 16 W rows by 16 TJ columns of one entry's result: wavefront w the strip of 16
+// rows number w, TJ accumulator blocks of v_mfma_f64_16x16x4.  The contracted index is walked in chunks of KC terms.  Per
+// chunk the workgroup reads a 16 W x KC piece of the row factor and a KC x 16 TJ piece of the column factor, each lane
+// single doubles with the lanes along the factor's fastest dimension, into registers; writes them to LDS in the order
+// the instruction wants its operands (fragment = block of 16 rows or columns and step of four terms; within a group of
+// 16 the place (x + k) mod 16, which keeps the 16 lanes that write a run along either dimension, and the 16 that read,
+// on different banks); and requests the next chunk before it multiplies this one, so that device memory is busy while
+// the matrix cores are.  Rows, columns and terms past the end are zero in LDS; results past the end are not stored.
+// Result register q of a lane holds row 4 q + lane / 16 and column lane % 16 of its block: a store instruction
+// writes four runs of 128 bytes.
+auto Generator::TiledProductPattern(const Sub &s, TiledProductShape &p) const -> bool
+{
+    if (envInt("ACRO_HIP_TILED_PRODUCT") < 0 || opt.no_matrix_cores || !opt.noalias || NumGatherSlots() > 0) return false;
+    if (mk.GetNumKernels() != 1 || s.matrixOp != 0 || s.out.repeated || s.in.size() != 2 || s.contr.size() != 1) return false;
+    const size_t rank = s.out.idx.size();
+    if (rank != 2 && rank != 3) return false;
+    p.batched = rank == 3;
+    const int entry = p.batched ? s.out.idx[0] : -1;   // (need not be the index that the other schedules would batch over)
+    const int k = s.contr[0], r = s.out.idx[rank - 2], c = s.out.idx[rank - 1];
+    for (const auto &v : s.in)
+    {
+        if (v.repeated || v.idx.size() != rank || (p.batched && v.idx[0] != entry)) return false;
+        if (v.uvar == s.out.uvar || (uvars[v.uvar].storage >= 0 && uvars[v.uvar].storage == uvars[s.out.uvar].storage)) return false;
+        const bool kLast = v.idx[rank - 1] == k, kFirst = v.idx[rank - 2] == k;
+        if (!kLast && !kFirst) return false;
+        const int other = kLast ? v.idx[rank - 2] : v.idx[rank - 1];
+        if (other == r && !p.row)
+        {
+            p.row = &v;
+            p.rowKFast = kLast;
+        }
+        else if (other == c && !p.col)
+        {
+            p.col = &v;
+            p.colKFast = kLast;
+        }
+        else
+            return false;
+    }
+    if (!p.row || !p.col) return false;
+    p.M = extent[r];
+    p.N = extent[c];
+    p.K = extent[k];
+    p.E = p.batched ? extent[entry] : 1;
+    if (p.M < 16 || p.N < 16 || p.K < 16 || p.M * p.K >= (1L << 31) || p.N * p.K >= (1L << 31) || p.M * p.N >= (1L << 31)) return false;
+    // (smaller matrices per entry have the schedules above; an unbatched product must be worth a launch of its own)
+    const long from = envInt("ACRO_HIP_TILED_PRODUCT_FROM", 65);
+    if (p.batched && std::max(p.M, p.N) < from && p.K <= 128) return false;
+    if (!p.batched && p.M * p.N < 64 * 64) return false;
+    // (one factor small enough for LDS in one piece: that is a dense operator applied to many vectors, "A_e_i = B_i_j X_e_j",
+    // which the operator schedule streams at 64 - 86 % of the HBM peak)
+    if (!p.batched && std::min(p.M, p.N) * p.K <= envInt("ACRO_HIP_TILED_PRODUCT_OPERATOR", 4096)) return false;
+    // strips per workgroup and blocks per strip: as even a split of the result as eight of each allow
+    const long strips = (p.M + 15) / 16, blocks = (p.N + 15) / 16;
+    // The split wastes as little of the matrix instruction on padding as it can.  Among equals: four blocks per strip
+    // rather than more (32 accumulator registers: two workgroups of eight wavefronts fit a compute unit, and one starts
+    // or drains while the other multiplies; with eight blocks one fits.  128 x 128 x 128 per entry: 52 against 43 % of
+    // the HBM peak), and as many strips as possible (128 x 64 against 64 x 64 tiles: 52 against 49 %).
+    auto split = [](long units, long lo, long hi, long preferred, long &parts, long &each) {
+        double best = 1e30;
+        for (long n = lo; n <= hi; ++n)
+        {
+            const long m = (units + n - 1) / n;
+            const double cost = static_cast<double>(m * n) * (n > preferred ? 1.15 : 1.0) - 1e-3 * n;
+            if (units <= n && n > units) continue;   // (never more than there is)
+            if (cost < best)
+            {
+                best = cost;
+                parts = m;
+                each = n;
+            }
+        }
+        if (units < lo)
+        {
+            parts = 1;
+            each = units;
+        }
+    };
+    const long mostW = envInt("ACRO_HIP_TILED_PRODUCT_STRIPS") > 0 ? envInt("ACRO_HIP_TILED_PRODUCT_STRIPS") : 8;
+    const long mostJ = envInt("ACRO_HIP_TILED_PRODUCT_BLOCKS") > 0 ? envInt("ACRO_HIP_TILED_PRODUCT_BLOCKS") : 8;
+    split(blocks, std::min<long>(3, mostJ), mostJ, 4, p.panels, p.TJ);
+    split(strips, std::min<long>(4, mostW), mostW, 8, p.tilesM, p.W);
+    // (few workgroups, a product without a batch index of moderate size: tiles of half the height fill the device better;
+    // 1 024 x 1 024 x 1 024: 14.5 -> 31.6 TFLOP/s)
+    if (p.E * p.tilesM * p.panels < 512 && p.W > 4 && mostW > 4) split(strips, 4, 4, 4, p.tilesM, p.W);
+    p.KC = envInt("ACRO_HIP_TILED_PRODUCT_CHUNK") > 0 ? envInt("ACRO_HIP_TILED_PRODUCT_CHUNK") : 16;
+    if (p.KC % 4 != 0 || p.KC > 64) return false;
+    return true;
+}
+
+auto Generator::UseTiledProductSchedule() const -> bool
+{
+    TiledProductShape p;
+    return subs.size() == 1 && TiledProductPattern(subs[0], p);
+}
+
+auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
+{
+    const Sub &s = subs[0];
+    TiledProductShape p;
+    TiledProductPattern(s, p);
+    const long M = p.M, N = p.N, K = p.K, E = p.E, W = p.W, TJ = p.TJ, KC = p.KC, KS = KC / 4, NT = 64 * W;
+    const long tiles = p.tilesM * p.panels, groups = tiles * E;
+    const long rowTile = 16 * W * KC, colTile = 16 * TJ * KC;
+    const long UA = (rowTile + NT - 1) / NT, UB = (colTile + NT - 1) / NT;
+    const std::string dimName = mk.GetDimensionedNameString();
+    char hex[32];
+    std::snprintf(hex, sizeof(hex), "%016llx",
+                  static_cast<unsigned long long>(hashString(dimName + "/tiled-product/" + (Positional() ? "p" : "u") + str(KC) + "/" + str(W) + "/" + str(TJ))));
+    plan.module_name = std::string("acro_tprod_") + hex;
+
+    std::ostringstream sched;
+    sched << "tiled product schedule on the FP64 matrix cores: " << M << " x " << K << " by " << K << " x " << N
+          << (p.batched ? " per entry, " + str(E) + " entries" : std::string(", no batch index")) << " (row factor "
+          << (p.rowKFast ? "with the contracted index last" : "with the contracted index first") << ", column factor "
+          << (p.colKFast ? "with the contracted index last" : "with the contracted index first") << "), tiles of " << 16 * W << " rows x "
+          << 16 * TJ << " columns (" << p.tilesM << " x " << p.panels << " per entry), chunks of " << KC << " terms through "
+          << (rowTile + colTile) * 8 << " bytes of LDS, " << groups << " workgroups of " << NT << " lanes\n  [0] " << s.text << "\n";
+    plan.schedule = sched.str();
+    out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
+    {
+        std::istringstream lines(plan.schedule);
+        std::string l;
+        while (std::getline(lines, l)) out << "// " << l << "\n";
+    }
+    const std::string R = PtrName(p.row->uvar), C = PtrName(p.col->uvar), A = PtrName(s.out.uvar);
+    const long rOff = uvars[p.row->uvar].viewOffset, cOff = uvars[p.col->uvar].viewOffset, aOff = uvars[s.out.uvar].viewOffset;
+    const bool streams = s.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0;
+
+    out << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
+    out << "\nextern \"C\" __global__ __launch_bounds__(" << NT << ") ";
+    if (envInt("ACRO_HIP_TILED_PRODUCT_WAVES") > 0) out << "__attribute__((amdgpu_waves_per_eu(" << envInt("ACRO_HIP_TILED_PRODUCT_WAVES") << "))) ";
+    out << "void " << plan.module_name << "(" << ParamList() << ")\n{\n";
+    // (padded to a whole number of values per lane: lanes without a value of the tile write into the padding, no branch)
+    out << "    __shared__ double fragA[" << UA * NT << "];\n";
+    out << "    __shared__ double fragB[" << UB * NT << "];\n";
+    out << "    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;\n";
+    out << "    const long e = (long)blockIdx.x / " << tiles << ";\n";
+    out << "    const int tile = (int)((long)blockIdx.x % " << tiles << "), r0 = tile / " << p.panels << " * " << 16 * W << ", c0 = tile % " << p.panels
+        << " * " << 16 * TJ << ";\n";
+    out << "    const double *Rm = " << R << " + " << rOff << "L + e * " << M * K << "L;\n";
+    out << "    const double *Cm = " << C << " + " << cOff << "L + e * " << K * N << "L;\n";
+    out << "    double *Am = " << A << " + " << aOff << "L + e * " << M * N << "L;\n";
+    // where this lane's values of a chunk come from and go to (the same for every chunk but for the term offset)
+    out << "    int aFrom[" << UA << "], aTo[" << UA << "], bFrom[" << UB << "], bTo[" << UB << "];\n";
+    out << "    int aK[" << UA << "], bK[" << UB << "];\n";
+    out << "#pragma unroll\n    for (int u = 0; u < " << UA << "; ++u)\n    {\n";
+    out << "        const int i = threadIdx.x + " << NT << " * u;\n";
+    if (p.rowKFast)
+        out << "        const int kk = i % " << KC << ", rr = i / " << KC << ";\n";
+    else
+        out << "        const int rr = i % " << 16 * W << ", kk = i / " << 16 * W << ";\n";
+    out << "        aK[u] = i < " << rowTile << " && r0 + rr < " << M << " ? kk : " << (1 << 28) << ";   // (never below K: reads as zero)\n";
+    out << "        aFrom[u] = " << (p.rowKFast ? "(r0 + rr) * " + str(K) + " + kk" : "kk * " + str(M) + " + r0 + rr") << ";\n";
+    out << "        aTo[u] = i < " << rowTile << " ? ((rr / 16) * " << KS << " + kk / 4) * 64 + (kk % 4) * 16 + ((rr + kk) & 15) : i;\n";
+    out << "    }\n";
+    out << "#pragma unroll\n    for (int u = 0; u < " << UB << "; ++u)\n    {\n";
+    out << "        const int i = threadIdx.x + " << NT << " * u;\n";
+    if (p.colKFast)
+        out << "        const int kk = i % " << KC << ", cc = i / " << KC << ";\n";
+    else
+        out << "        const int cc = i % " << 16 * TJ << ", kk = i / " << 16 * TJ << ";\n";
+    out << "        bK[u] = i < " << colTile << " && c0 + cc < " << N << " ? kk : " << (1 << 28) << ";\n";
+    out << "        bFrom[u] = " << (p.colKFast ? "(c0 + cc) * " + str(K) + " + kk" : "kk * " + str(N) + " + c0 + cc") << ";\n";
+    out << "        bTo[u] = i < " << colTile << " ? ((cc / 16) * " << KS << " + kk / 4) * 64 + (kk % 4) * 16 + ((cc + kk) & 15) : i;\n";
+    out << "    }\n";
+    const std::string aStep = p.rowKFast ? "k0" : "(long)k0 * " + str(M);
+    const std::string bStep = p.colKFast ? "k0" : "(long)k0 * " + str(N);
+    out << "    double ra[" << UA << "], rb[" << UB << "];\n";
+    auto emitLoads = [&](const std::string &ind) {
+        // (no branches around the loads and no use of their values here, so that all of them are in flight together and
+        // stay so while the previous chunk is multiplied: a value that does not exist is read from the entry's first
+        // element and replaced by zero when it is written to LDS)
+        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UA << "; ++u) ra[u] = Rm[k0 + aK[u] < " << K << " ? " << aStep << " + aFrom[u] : 0];\n";
+        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UB << "; ++u) rb[u] = Cm[k0 + bK[u] < " << K << " ? " << bStep << " + bFrom[u] : 0];\n";
+    };
+    out << "    {\n        const int k0 = 0;\n";
+    emitLoads("        ");
+    out << "    }\n";
+    out << "    acro_double4 acc[" << TJ << "];\n";
+    out << "#pragma unroll\n    for (int J = 0; J < " << TJ << "; ++J) acc[J] = acro_double4{0.0, 0.0, 0.0, 0.0};\n";
+    out << "    for (int kc = 0; kc < " << K << "; kc += " << KC << ")\n    {\n";
+    out << "#pragma unroll\n        for (int u = 0; u < " << UA << "; ++u) fragA[aTo[u]] = kc + aK[u] < " << K << " ? ra[u] : 0.0;\n";
+    out << "#pragma unroll\n        for (int u = 0; u < " << UB << "; ++u) fragB[bTo[u]] = kc + bK[u] < " << K << " ? rb[u] : 0.0;\n";
+    out << "        __syncthreads();\n";
+    out << "        {\n            const int k0 = kc + " << KC << ";   // the next chunk is on its way while this one is multiplied (past the end: zeros, no loads)\n";
+    emitLoads("            ");
+    out << "        }\n";
+    out << "#pragma unroll\n        for (int s = 0; s < " << KS << "; ++s)\n        {\n";
+    out << "            const int at = s * 64 + g * 16 + ((c + 4 * s + g) & 15);\n";
+    out << "            const double a = fragA[wave * " << KS * 64 << " + at];\n";
+    out << "#pragma unroll\n            for (int J = 0; J < " << TJ << "; ++J)\n";
+    out << "                acc[J] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, fragB[J * " << KS * 64 << " + at], acc[J], 0, 0, 0);\n";
+    out << "        }\n";
+    out << "        __syncthreads();\n";
+    out << "    }\n";
+    out << "#pragma unroll\n    for (int J = 0; J < " << TJ << "; ++J)\n";
+    out << "#pragma unroll\n        for (int q = 0; q < 4; ++q)\n        {\n";
+    out << "            const int m = r0 + 16 * wave + 4 * q + g, n = c0 + 16 * J + c;\n";
+    if (M % (16 * W) != 0 || N % (16 * TJ) != 0) out << "            if (m >= " << M << " || n >= " << N << ") continue;\n";
+    out << "            double *d = Am + (long)m * " << N << " + n;\n";
+    if (s.op == '=')
+        out << "            " << (streams ? "__builtin_nontemporal_store(acc[J][q], d);" : "*d = acc[J][q];") << "\n";
+    else
+        out << "            *d " << (s.op == '+' ? "+=" : "-=") << " acc[J][q];\n";
+    out << "        }\n";
+    out << "}\n";
+
+    plan.source = out.str();
+    plan.nb = 1;
+    plan.lds_bytes = static_cast<int>((rowTile + colTile) * 8);
     FillParams(plan, false);
     HipLaunch launch;
     launch.function_name = plan.module_name;

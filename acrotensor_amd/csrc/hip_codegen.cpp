@@ -41,6 +41,11 @@ auto Generator::Run() -> HipKernelPlan
         EmitProduct(plan);
         return plan;
     }
+    if (UseTiledProductSchedule())
+    {
+        EmitTiledProduct(plan);
+        return plan;
+    }
     if (UseOperatorSchedule())
     {
         EmitOperator(plan);

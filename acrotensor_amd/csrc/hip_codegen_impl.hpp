@@ -402,6 +402,18 @@ class Generator
     bool UseProductSchedule() const;
     void EmitProduct(HipKernelPlan &plan);
 
+    // Products of matrices too large for one workgroup, with or without a batch index (codegen_product.cpp).
+    struct TiledProductShape
+    {
+        const VarRef *row = nullptr, *col = nullptr;
+        bool rowKFast = false, colKFast = false, batched = false;
+        long M = 0, N = 0, K = 0, E = 1;
+        long W = 0, TJ = 0, tilesM = 0, panels = 0, KC = 16;   // strips per workgroup, blocks per strip, tiles per entry, terms per chunk
+    };
+    bool TiledProductPattern(const Sub &s, TiledProductShape &p) const;
+    bool UseTiledProductSchedule() const;
+    void EmitTiledProduct(HipKernelPlan &plan);
+
     // ------------------------------------------------------------------------------ operator schedule
     // One dense operator applied to every batch entry: "A_e_i = B_i_j X_e_j" with B too large for scalar operands or a
     // register tile (16 <= rows, columns; at most 4 096 entries), also with several row or column indices

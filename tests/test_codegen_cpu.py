@@ -609,3 +609,52 @@ def test_products_of_element_matrices_run_on_the_matrix_cores(TE, monkeypatch):
     monkeypatch.setenv("ACRO_HIP_TEST_PRIVATE_BYTES", "8,8")
     src = product("A_e_i_j = B_e_i_k C_e_k_j", 64, 64, 64)
     assert "product schedule" not in src and "was refused" in src
+
+
+def test_products_of_large_matrices_run_in_tiles_on_the_matrix_cores(TE, monkeypatch):
+    """The tiled product schedule (codegen_product.cpp): products beyond one workgroup's reach and products without a
+    batch index; how the result is split into tiles and what each form of the factors turns into."""
+    def product(kernel, M, N, K, E=2048):
+        ext = {"e": E, "i": M, "j": N, "k": K}
+        lhs, rhs = kernel.replace("+=", "=").replace("-=", "=").split("=")
+        tensors = [at.Tensor(*[ext[x] for x in tok.split("_")[1:]]) for tok in [lhs.split()[0]] + rhs.split()]
+        return at.TensorEngine("HIP").GetImplementation(kernel, *tensors)
+
+    # 128 x 128 per entry: eight strips by four blocks per workgroup, two tiles per entry, chunks of 16 terms
+    src = product("A_e_i_j = B_e_i_k C_e_k_j", 128, 128, 128)
+    assert "tiled product schedule on the FP64 matrix cores: 128 x 128 by 128 x 128 per entry, 2048 entries" in src
+    assert "tiles of 128 rows x 64 columns (1 x 2 per entry), chunks of 16 terms through 24576 bytes of LDS, 4096 workgroups of 512 lanes" in src
+    assert "__shared__ double fragA[2048];" in src and "__shared__ double fragB[1024];" in src
+    # the lanes run along each factor's fastest dimension; values land in the instruction's operand order
+    assert "const int kk = i % 16, rr = i / 16;" in src and "const int cc = i % 64, kk = i / 64;" in src
+    assert "((rr / 16) * 4 + kk / 4) * 64 + (kk % 4) * 16 + ((rr + kk) & 15)" in src
+    # loads without branches, zeros written to LDS for what does not exist, the next chunk requested before the products
+    assert "ra[u] = Rm[k0 + aK[u] < 128 ? k0 + aFrom[u] : 0];" in src and "fragA[aTo[u]] = kc + aK[u] < 128 ? ra[u] : 0.0;" in src
+    assert src.index("const int k0 = kc + 16;") < src.index("__builtin_amdgcn_mfma_f64_16x16x4f64")
+    assert src.count("__syncthreads()") == 2 and "__builtin_nontemporal_store(acc[J][q], d);" in src
+    assert "if (m >= 128" not in src                       # tiles without padding store without guards
+    # extents that 16 does not divide, the factors stored the other way round, accumulation
+    src = product("A_e_i_j += B_e_k_i C_e_j_k", 100, 70, 150)
+    assert "100 x 150 by 150 x 70 per entry" in src and "row factor with the contracted index first, column factor with the contracted index last" in src
+    assert "tiles of 112 rows x 80 columns (1 x 1 per entry)" in src and "workgroups of 448 lanes" in src
+    assert "const int rr = i % 112, kk = i / 112;" in src and "const int kk = i % 16, cc = i / 16;" in src
+    assert "if (m >= 100 || n >= 70) continue;" in src and "*d += acc[J][q];" in src and "nontemporal" not in src
+    # no batch index: a plain matrix product; few tiles take half the height to fill the device
+    src = TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(2048, 2048), at.Tensor(2048, 2048), at.Tensor(2048, 2048))
+    assert "2048 x 2048 by 2048 x 2048, no batch index" in src and "tiles of 128 rows x 64 columns (16 x 32 per entry)" in src and "512 workgroups" in src
+    src = TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(1024, 1024), at.Tensor(1024, 1024), at.Tensor(1024, 1024))
+    assert "tiles of 64 rows x 64 columns (16 x 16 per entry)" in src and "256 workgroups of 256 lanes" in src
+    # 65 to 128 rows or columns per entry, and small matrices with more than 128 terms
+    assert "tiled product schedule" in product("A_e_i_j = B_e_i_k C_e_k_j", 72, 72, 72)
+    assert "tiled product schedule" in product("A_e_i_j = B_e_i_k C_e_k_j", 32, 48, 200)
+    # entries fewer than rows: the entry index is still the first one
+    assert "tiled product schedule" in product("A_e_i_j = B_e_i_k C_e_k_j", 128, 128, 128, E=10)
+    # not this schedule: what the product schedule takes, tiny matrices, a shared factor
+    assert "tiled" not in product("A_e_i_j = B_e_i_k C_e_k_j", 64, 64, 64)
+    assert "tiled" not in product("A_e_i_j = B_e_i_k C_e_k_j", 8, 100, 100)
+    assert "tiled" not in TE.GetImplementation("A_e_i_j = B_e_i_k C_k_j", at.Tensor(64, 100, 100), at.Tensor(64, 100, 100), at.Tensor(100, 100))
+    assert "tiled" not in TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(32, 32), at.Tensor(32, 32), at.Tensor(32, 32))
+    # ... and it is a matrix-core schedule: off where those are refused
+    monkeypatch.setenv("ACRO_HIP_TEST_PRIVATE_BYTES", "8,8")
+    src = product("A_e_i_j = B_e_i_k C_e_k_j", 128, 128, 128)
+    assert "tiled product schedule" not in src and "was refused" in src

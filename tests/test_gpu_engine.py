@@ -311,6 +311,82 @@ def test_products_of_element_matrices_on_the_matrix_cores_views_and_odd_tensors(
     assert np.array_equal(tA.data, expected)                # also: nothing outside the slices was touched
 
 
+TILED_PRODUCTS = [
+    # (kernel, shapes of the inputs in the order written): matrices beyond 64 rows or columns or 128 terms per entry, and
+    # products without a batch index; every combination of layouts, extents that 16 divides and extents that it does
+    # not, tiles with and without padding, more than one tile per entry either way, the factors in either order
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(7, 128, 128), (7, 128, 128)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(5, 100, 150), (5, 150, 70)]),
+    ("A_e_i_j += B_e_k_i C_e_j_k", [(5, 150, 100), (5, 70, 150)]),
+    ("A_e_i_j -= B_e_k_i C_e_k_j", [(3, 17, 65), (3, 17, 129)]),
+    ("A_e_i_j = C_e_j_k B_e_i_k", [(3, 33, 64), (3, 200, 64)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(2, 300, 40), (2, 40, 260)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(80, 72, 72), (80, 72, 72)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(130, 125, 125), (130, 125, 125)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(64, 32, 200), (64, 200, 48)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(4, 16, 16), (4, 16, 400)]),
+    ("A_i_j = B_i_k C_k_j", [(256, 100), (100, 192)]),
+    ("A_i_j += B_k_i C_j_k", [(333, 129), (65, 333)]),
+    ("A_i_j = B_i_k C_j_k", [(96, 80), (112, 80)]),
+    ("A_i_j -= C_k_j B_i_k", [(77, 301), (515, 77)]),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kernel,shapes", TILED_PRODUCTS)
+def test_products_of_large_matrices_in_tiles_on_the_matrix_cores_random(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(len(kernel) + shapes[0][0])
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "tiled product schedule on the FP64 matrix cores" in engine.GetLastImplementation()
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kernel,shapes", TILED_PRODUCTS)
+def test_products_of_large_matrices_in_tiles_on_the_matrix_cores_integer_exact(at, engine, checker, kernel, shapes):
+    """Integer-valued data: sums in any order are exact, so every row, column and term must be in its place (also the
+    ones next to the padding of tiles, of blocks of 16 and of chunks of terms)."""
+    rng = np.random.default_rng(11 * len(kernel) + shapes[0][1])
+    ins = [rng.integers(-5, 6, s).astype(np.float64) for s in shapes]
+    out0 = rng.integers(-5, 6, output_shape(kernel, shapes)).astype(np.float64)
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "tiled product schedule on the FP64 matrix cores" in engine.GetLastImplementation()
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert np.array_equal(got, expected)
+
+
+@pytest.mark.gpu
+def test_products_of_large_matrices_in_tiles_views_and_special_values(at, engine, checker):
+    """Factors and results that are slices at odd offsets of larger tensors; and a NaN in an entry's first element,
+    the element that stands in for values past the end of a matrix, must stay where it belongs."""
+    rng = np.random.default_rng(41)
+    E, m, k, n = 3, 81, 37, 70
+    B3, C3, A3 = (rng.integers(-4, 5, (3, E) + s).astype(np.float64) for s in ((m, k), (k, n), (m, n)))
+    tB, tC, tA = (to_tensor(at, x) for x in (B3, C3, A3))
+    for which in (1, 2):
+        engine("A_e_i_j = B_e_i_k C_e_k_j", at.SliceTensor(tA, which), at.SliceTensor(tB, which), at.SliceTensor(tC, which))
+        assert "tiled product schedule on the FP64 matrix cores" in engine.GetLastImplementation()
+    tA.MoveFromGPU()
+    expected = A3.copy()
+    for which in (1, 2):
+        expected[which] = np.einsum("eik,ekj->eij", B3[which], C3[which])
+    assert np.array_equal(tA.data, expected)                # also: nothing outside the slices was touched
+    B = rng.integers(-4, 5, (E, m, k)).astype(np.float64)
+    C = rng.integers(-4, 5, (E, k, n)).astype(np.float64)
+    B[1, 0, 0] = np.nan
+    tB, tC, tA = to_tensor(at, B), to_tensor(at, C), at.Tensor(E, m, n)
+    engine("A_e_i_j = B_e_i_k C_e_k_j", tA, tB, tC)
+    tA.MoveFromGPU()
+    expected = np.einsum("eik,ekj->eij", B, C)
+    assert np.isnan(tA.data[1, 0]).all() and np.isnan(tA.data).sum() == n
+    assert np.array_equal(np.nan_to_num(tA.data), np.nan_to_num(expected))
+
+
 def test_product_of_slices_keeps_its_indices(at, engine, checker):
     # operands that are views into larger tensors are not described by split dimensions
     rng = np.random.default_rng(12)
