@@ -456,6 +456,18 @@ auto Generator::TiledProductPattern(const Sub &s, TiledProductShape &p) const ->
     if (p.E * p.tilesM * p.panels < 512 && p.W > 4 && mostW > 4) split(strips, 4, 4, 4, p.tilesM, p.W);
     p.KC = envInt("ACRO_HIP_TILED_PRODUCT_CHUNK") > 0 ? envInt("ACRO_HIP_TILED_PRODUCT_CHUNK") : 16;
     if (p.KC % 4 != 0 || p.KC > 64) return false;
+    // Few tiles and a long contraction (normal equations "A_i_j = B_n_i C_n_j" with many columns, a product of two wide
+    // matrices): the contracted range is split over workgroups as well, each writes its tile of partial sums to the
+    // scratch buffer, and a second kernel adds them in a fixed order (reproducible, no atomics).  As many shares as
+    // fill the device twice, at least 32 chunks each, at most 64 MB of partial sums.
+    p.splits = 1;
+    const long groups = p.E * p.tilesM * p.panels, chunks = (p.K + p.KC - 1) / p.KC;
+    if (groups < 256 && chunks >= 64 && envInt("ACRO_HIP_TILED_PRODUCT_SPLIT") >= 0)
+    {
+        p.splits = std::min<long>(std::min<long>((512 + groups - 1) / groups, chunks / 32), 256);
+        while (p.splits > 1 && p.splits * p.E * p.M * p.N > (1L << 23)) --p.splits;
+        if (envInt("ACRO_HIP_TILED_PRODUCT_SPLIT") > 0) p.splits = std::min<long>(envInt("ACRO_HIP_TILED_PRODUCT_SPLIT"), chunks);
+    }
     return true;
 }
 
@@ -471,13 +483,14 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
     TiledProductShape p;
     TiledProductPattern(s, p);
     const long M = p.M, N = p.N, K = p.K, E = p.E, W = p.W, TJ = p.TJ, KC = p.KC, KS = KC / 4, NT = 64 * W;
-    const long tiles = p.tilesM * p.panels, groups = tiles * E;
+    const long tiles = p.tilesM * p.panels, groups = tiles * E, splits = p.splits;
+    const long span = ((K + splits - 1) / splits + KC - 1) / KC * KC;   // terms per share of the contracted range
     const long rowTile = 16 * W * KC, colTile = 16 * TJ * KC;
     const long UA = (rowTile + NT - 1) / NT, UB = (colTile + NT - 1) / NT;
     const std::string dimName = mk.GetDimensionedNameString();
     char hex[32];
     std::snprintf(hex, sizeof(hex), "%016llx",
-                  static_cast<unsigned long long>(hashString(dimName + "/tiled-product/" + (Positional() ? "p" : "u") + str(KC) + "/" + str(W) + "/" + str(TJ))));
+                  static_cast<unsigned long long>(hashString(dimName + "/tiled-product/" + (Positional() ? "p" : "u") + str(KC) + "/" + str(W) + "/" + str(TJ) + "/" + str(splits))));
     plan.module_name = std::string("acro_tprod_") + hex;
 
     std::ostringstream sched;
@@ -486,7 +499,9 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
           << (p.rowKFast ? "with the contracted index last" : "with the contracted index first") << ", column factor "
           << (p.colKFast ? "with the contracted index last" : "with the contracted index first") << "), tiles of " << 16 * W << " rows x "
           << 16 * TJ << " columns (" << p.tilesM << " x " << p.panels << " per entry), chunks of " << KC << " terms through "
-          << (rowTile + colTile) * 8 << " bytes of LDS, " << groups << " workgroups of " << NT << " lanes\n  [0] " << s.text << "\n";
+          << (rowTile + colTile) * 8 << " bytes of LDS, " << groups * splits << " workgroups of " << NT << " lanes";
+    if (splits > 1) sched << ", the contracted range in " << splits << " shares of " << span << " terms whose partial sums a second kernel adds";
+    sched << "\n  [0] " << s.text << "\n";
     plan.schedule = sched.str();
     out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
     {
@@ -496,18 +511,28 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
     }
     const std::string R = PtrName(p.row->uvar), C = PtrName(p.col->uvar), A = PtrName(s.out.uvar);
     const long rOff = uvars[p.row->uvar].viewOffset, cOff = uvars[p.col->uvar].viewOffset, aOff = uvars[s.out.uvar].viewOffset;
-    const bool streams = s.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0;
+    // Non-temporal stores where a store instruction's four runs of 16 doubles are whole lines; rows that 16 does not divide
+    // start anywhere in a line, and the pieces of a line then meet in L2 (125 x 125: 36 -> 40 % of the HBM peak, 65 x 65 39 -> 42 %).
+    const bool streams = s.op == '=' && envInt("ACRO_HIP_NT_STORE") >= 0 && N % 16 == 0 && aOff % 16 == 0;
 
     out << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
     out << "\nextern \"C\" __global__ __launch_bounds__(" << NT << ") ";
     if (envInt("ACRO_HIP_TILED_PRODUCT_WAVES") > 0) out << "__attribute__((amdgpu_waves_per_eu(" << envInt("ACRO_HIP_TILED_PRODUCT_WAVES") << "))) ";
-    out << "void " << plan.module_name << "(" << ParamList() << ")\n{\n";
+    const std::string fMain = splits > 1 ? plan.module_name + "_partial" : plan.module_name, fFinal = plan.module_name + "_final";
+    out << "void " << fMain << "(" << ParamList() << (splits > 1 ? ", double *__restrict__ scratch" : "") << ")\n{\n";
     // (padded to a whole number of values per lane: lanes without a value of the tile write into the padding, no branch)
     out << "    __shared__ double fragA[" << UA * NT << "];\n";
     out << "    __shared__ double fragB[" << UB * NT << "];\n";
     out << "    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;\n";
-    out << "    const long e = (long)blockIdx.x / " << tiles << ";\n";
-    out << "    const int tile = (int)((long)blockIdx.x % " << tiles << "), r0 = tile / " << p.panels << " * " << 16 * W << ", c0 = tile % " << p.panels
+    if (splits > 1)
+    {
+        out << "    const int split = blockIdx.x / " << groups << ";\n    const long group = blockIdx.x % " << groups << ";\n";
+        out << "    const int kBegin = split * " << span << ", kEnd = kBegin + " << span << " < " << K << " ? kBegin + " << span << " : " << K << ";\n";
+    }
+    else
+        out << "    const long group = blockIdx.x;\n    const int kBegin = 0, kEnd = " << K << ";\n";
+    out << "    const long e = group / " << tiles << ";\n";
+    out << "    const int tile = (int)(group % " << tiles << "), r0 = tile / " << p.panels << " * " << 16 * W << ", c0 = tile % " << p.panels
         << " * " << 16 * TJ << ";\n";
     out << "    const double *Rm = " << R << " + " << rOff << "L + e * " << M * K << "L;\n";
     out << "    const double *Cm = " << C << " + " << cOff << "L + e * " << K * N << "L;\n";
@@ -542,17 +567,17 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
         // (no branches around the loads and no use of their values here, so that all of them are in flight together and
         // stay so while the previous chunk is multiplied: a value that does not exist is read from the entry's first
         // element and replaced by zero when it is written to LDS)
-        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UA << "; ++u) ra[u] = Rm[k0 + aK[u] < " << K << " ? " << aStep << " + aFrom[u] : 0];\n";
-        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UB << "; ++u) rb[u] = Cm[k0 + bK[u] < " << K << " ? " << bStep << " + bFrom[u] : 0];\n";
+        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UA << "; ++u) ra[u] = Rm[k0 + aK[u] < kEnd ? " << aStep << " + aFrom[u] : 0];\n";
+        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UB << "; ++u) rb[u] = Cm[k0 + bK[u] < kEnd ? " << bStep << " + bFrom[u] : 0];\n";
     };
-    out << "    {\n        const int k0 = 0;\n";
+    out << "    {\n        const int k0 = kBegin;\n";
     emitLoads("        ");
     out << "    }\n";
     out << "    acro_double4 acc[" << TJ << "];\n";
     out << "#pragma unroll\n    for (int J = 0; J < " << TJ << "; ++J) acc[J] = acro_double4{0.0, 0.0, 0.0, 0.0};\n";
-    out << "    for (int kc = 0; kc < " << K << "; kc += " << KC << ")\n    {\n";
-    out << "#pragma unroll\n        for (int u = 0; u < " << UA << "; ++u) fragA[aTo[u]] = kc + aK[u] < " << K << " ? ra[u] : 0.0;\n";
-    out << "#pragma unroll\n        for (int u = 0; u < " << UB << "; ++u) fragB[bTo[u]] = kc + bK[u] < " << K << " ? rb[u] : 0.0;\n";
+    out << "    for (int kc = kBegin; kc < kEnd; kc += " << KC << ")\n    {\n";
+    out << "#pragma unroll\n        for (int u = 0; u < " << UA << "; ++u) fragA[aTo[u]] = kc + aK[u] < kEnd ? ra[u] : 0.0;\n";
+    out << "#pragma unroll\n        for (int u = 0; u < " << UB << "; ++u) fragB[bTo[u]] = kc + bK[u] < kEnd ? rb[u] : 0.0;\n";
     out << "        __syncthreads();\n";
     out << "        {\n            const int k0 = kc + " << KC << ";   // the next chunk is on its way while this one is multiplied (past the end: zeros, no loads)\n";
     emitLoads("            ");
@@ -569,24 +594,58 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
     out << "#pragma unroll\n        for (int q = 0; q < 4; ++q)\n        {\n";
     out << "            const int m = r0 + 16 * wave + 4 * q + g, n = c0 + 16 * J + c;\n";
     if (M % (16 * W) != 0 || N % (16 * TJ) != 0) out << "            if (m >= " << M << " || n >= " << N << ") continue;\n";
-    out << "            double *d = Am + (long)m * " << N << " + n;\n";
-    if (s.op == '=')
-        out << "            " << (streams ? "__builtin_nontemporal_store(acc[J][q], d);" : "*d = acc[J][q];") << "\n";
+    if (splits > 1)
+    {
+        out << "            scratch[((long)split * " << E << " + e) * " << M * N << "L + (long)m * " << N << " + n] = acc[J][q];\n";
+        out << "        }\n}\n";
+        // ---- the partial sums of all shares, added in a fixed order, one lane per output
+        const long O = E * M * N;
+        out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << fFinal << "(double *" << (opt.noalias ? "__restrict__ " : "")
+            << "result, const double *__restrict__ scratch)\n{\n";
+        out << "    const long o = (long)blockIdx.x * 256 + threadIdx.x;\n";
+        out << "    if (o >= " << O << "L) return;\n";
+        out << "    double t = 0.0;\n";
+        out << "#pragma unroll 8\n    for (int w = 0; w < " << splits << "; ++w) t += scratch[w * " << O << "L + o];\n";
+        const std::string dst = "result[" + str(aOff) + "L + o]";
+        if (s.op == '=')
+            out << "    " << dst << " = t;\n";
+        else
+            out << "    " << dst << " = " << dst << (s.op == '+' ? " + t;\n" : " - t;\n");
+        out << "}\n";
+    }
     else
-        out << "            *d " << (s.op == '+' ? "+=" : "-=") << " acc[J][q];\n";
-    out << "        }\n";
-    out << "}\n";
+    {
+        out << "            double *d = Am + (long)m * " << N << " + n;\n";
+        if (s.op == '=')
+            out << "            " << (streams ? "__builtin_nontemporal_store(acc[J][q], d);" : "*d = acc[J][q];") << "\n";
+        else
+            out << "            *d " << (s.op == '+' ? "+=" : "-=") << " acc[J][q];\n";
+        out << "        }\n";
+        out << "}\n";
+    }
 
     plan.source = out.str();
     plan.nb = 1;
     plan.lds_bytes = static_cast<int>((rowTile + colTile) * 8);
     FillParams(plan, false);
     HipLaunch launch;
-    launch.function_name = plan.module_name;
-    launch.grid = static_cast<unsigned>(groups);
+    launch.function_name = fMain;
+    launch.grid = static_cast<unsigned>(groups * splits);
     launch.block = static_cast<unsigned>(NT);
     for (int si = 0; si < NumParamStores(); ++si) launch.params.push_back(si);
+    if (splits > 1) launch.params.push_back(-1);
     plan.launches.push_back(launch);
+    if (splits > 1)
+    {
+        plan.scratch_doubles = static_cast<size_t>(splits * E * M * N);
+        HipLaunch fin;
+        fin.function_name = fFinal;
+        fin.grid = static_cast<unsigned>((E * M * N + 255) / 256);
+        fin.block = 256;
+        fin.params.push_back(uvars[s.out.uvar].storage);
+        fin.params.push_back(-1);
+        plan.launches.push_back(fin);
+    }
 }
 
 }  // namespace codegen

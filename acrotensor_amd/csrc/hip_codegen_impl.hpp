@@ -409,6 +409,7 @@ class Generator
         bool rowKFast = false, colKFast = false, batched = false;
         long M = 0, N = 0, K = 0, E = 1;
         long W = 0, TJ = 0, tilesM = 0, panels = 0, KC = 16;   // strips per workgroup, blocks per strip, tiles per entry, terms per chunk
+        long splits = 1;                                        // shares of the contracted range (more than one: partial sums through scratch)
     };
     bool TiledProductPattern(const Sub &s, TiledProductShape &p) const;
     bool UseTiledProductSchedule() const;

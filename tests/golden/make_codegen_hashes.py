@@ -32,6 +32,7 @@ SINGLES = [
     ("product_mfma_strips_through_lds", "A_e_i_j = B_e_i_k C_e_j_k", [(5546, 55, 55), (5546, 55, 55), (5546, 55, 55)]),
     ("product_mfma_tiled_batched", "A_e_i_j = B_e_i_k C_e_k_j", [(1024, 128, 128), (1024, 128, 128), (1024, 128, 128)]),
     ("product_mfma_tiled_plain", "A_i_j += B_k_i C_j_k", [(1000, 700), (333, 1000), (700, 333)]),
+    ("product_mfma_tiled_shares", "A_i_j = B_n_i C_n_j", [(96, 80), (100000, 96), (100000, 80)]),
     ("row_reduction", "S_i = A_i_n", [(64,), (64, 1 << 20)]),
     ("dsetup", "D_e_m_n_k1_k2_k3 = W_k1_k2_k3 C_e_k1_k2_k3 Jdet_e_k1_k2_k3 Jinv_e_k1_k2_k3_n_j Jinv_e_k1_k2_k3_m_j",
      [(16384, 3, 3, 10, 10, 10), (10, 10, 10), (16384, 10, 10, 10), (16384, 10, 10, 10), (16384, 10, 10, 10, 3, 3),

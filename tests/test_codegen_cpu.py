@@ -629,7 +629,8 @@ def test_products_of_large_matrices_run_in_tiles_on_the_matrix_cores(TE, monkeyp
     assert "const int kk = i % 16, rr = i / 16;" in src and "const int cc = i % 64, kk = i / 64;" in src
     assert "((rr / 16) * 4 + kk / 4) * 64 + (kk % 4) * 16 + ((rr + kk) & 15)" in src
     # loads without branches, zeros written to LDS for what does not exist, the next chunk requested before the products
-    assert "ra[u] = Rm[k0 + aK[u] < 128 ? k0 + aFrom[u] : 0];" in src and "fragA[aTo[u]] = kc + aK[u] < 128 ? ra[u] : 0.0;" in src
+    assert "const int kBegin = 0, kEnd = 128;" in src
+    assert "ra[u] = Rm[k0 + aK[u] < kEnd ? k0 + aFrom[u] : 0];" in src and "fragA[aTo[u]] = kc + aK[u] < kEnd ? ra[u] : 0.0;" in src
     assert src.index("const int k0 = kc + 16;") < src.index("__builtin_amdgcn_mfma_f64_16x16x4f64")
     assert src.count("__syncthreads()") == 2 and "__builtin_nontemporal_store(acc[J][q], d);" in src
     assert "if (m >= 128" not in src                       # tiles without padding store without guards
@@ -644,6 +645,13 @@ def test_products_of_large_matrices_run_in_tiles_on_the_matrix_cores(TE, monkeyp
     assert "2048 x 2048 by 2048 x 2048, no batch index" in src and "tiles of 128 rows x 64 columns (16 x 32 per entry)" in src and "512 workgroups" in src
     src = TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(1024, 1024), at.Tensor(1024, 1024), at.Tensor(1024, 1024))
     assert "tiles of 64 rows x 64 columns (16 x 16 per entry)" in src and "256 workgroups of 256 lanes" in src
+    # few tiles, many terms (normal equations with more columns than the Gram schedule takes): the contracted range is
+    # shared out as well, partial tiles go to the scratch buffer and a second kernel adds them in a fixed order
+    src = TE.GetImplementation("A_i_j += B_n_i C_n_j", at.Tensor(128, 128), at.Tensor(262144, 128), at.Tensor(262144, 128))
+    assert "tiles of 64 rows x 64 columns (2 x 2 per entry)" in src and "512 workgroups of 256 lanes, the contracted range in 128 shares of 2048 terms" in src
+    assert "_partial(" in src and "double *__restrict__ scratch)" in src and "const int split = blockIdx.x / 4;" in src
+    assert "scratch[((long)split * 1 + e) * 16384L + (long)m * 128 + n] = acc[J][q];" in src
+    assert "for (int w = 0; w < 128; ++w) t += scratch[w * 16384L + o];" in src and "result[0L + o] = result[0L + o] + t;" in src
     # 65 to 128 rows or columns per entry, and small matrices with more than 128 terms
     assert "tiled product schedule" in product("A_e_i_j = B_e_i_k C_e_k_j", 72, 72, 72)
     assert "tiled product schedule" in product("A_e_i_j = B_e_i_k C_e_k_j", 32, 48, 200)

@@ -329,6 +329,10 @@ TILED_PRODUCTS = [
     ("A_i_j += B_k_i C_j_k", [(333, 129), (65, 333)]),
     ("A_i_j = B_i_k C_j_k", [(96, 80), (112, 80)]),
     ("A_i_j -= C_k_j B_i_k", [(77, 301), (515, 77)]),
+    # few tiles and a long contracted range: shares of the range per workgroup, partial sums added by a second kernel
+    ("A_i_j = B_e_i C_e_j", [(3000, 96), (3000, 100)]),
+    ("A_i_j -= B_i_k C_k_j", [(65, 4099), (4099, 96)]),
+    ("A_e_i_j += B_e_i_k C_e_k_j", [(3, 70, 1500), (3, 1500, 66)]),
 ]
 
 
