@@ -124,7 +124,7 @@
 //                               compute unit) and slices a lane requests before it adds them (default 1)
 //   ACRO_HIP_PRODUCT=-1 / =2    products of two element matrices never / whenever they fit take the product schedule on the
 //                               matrix cores (default: from 17 rows or columns on, except sizes up to 36 that 2, 3 or 5 divide)
-//   ACRO_HIP_PRODUCT_FROM=<n> / ACRO_HIP_PRODUCT_TO=<n>   smallest and largest "larger of rows and columns" it takes (17, 128)
+//   ACRO_HIP_PRODUCT_FROM=<n> / ACRO_HIP_PRODUCT_TO=<n>   smallest and largest "larger of rows and columns" it takes (17, 64)
 //   ACRO_HIP_PRODUCT_ENTRIES=<n>  entries per workgroup of the product schedule (default: up to 4 wavefronts, 8 192 LDS values)
 //   ACRO_HIP_PRODUCT_DIRECT=-1  the row factor always passes through LDS, also where lanes could load their operands directly
 //   ACRO_HIP_COPY_OUT_COVERAGE=<percent>  share of the touched lines below which the last kernel's stores leave through an
@@ -133,6 +133,17 @@
 //   ACRO_HIP_WRITE_BATCH_FROM=<n>  write-heavy launches that copy out of LDS tiles double their batch from this batch size on (1)
 //   ACRO_HIP_NT_COPY_OUT=-1     copies out of LDS tiles use non-temporal stores only for tiles of at most 20 KB
 //   ACRO_HIP_NT_STORE=2         non-temporal stores from registers also in launches that hold more than 20 KB of LDS per workgroup
+//   ACRO_HIP_OPERATOR_GROUPS=<n>  workgroups of the matrix-core operator kernel (default: 256 - 1 024 by the operator's size)
+//   ACRO_HIP_XCD_RUN=-1 / =<n>  fused launches that read an operand through an index map number their workgroups as the hardware
+//                               deals them / in runs of n per XCD (default 16)
+//   ACRO_HIP_TILED_PRODUCT=-1   large matrix products (more than 64 rows or columns or 128 terms per entry, or no batch index) keep
+//                               the generic schedule;  ACRO_HIP_TILED_PRODUCT_FROM=<n>: smallest "larger of rows and columns" (65)
+//   ACRO_HIP_TILED_PRODUCT_CHUNK=<terms> / _STRIPS=<n> / _BLOCKS=<n> / _WAVES=<n>
+//                               terms per chunk (16), most strips per workgroup and blocks per strip (8, 8), waves per SIMD asked of
+//                               the compiler (none)
+//   ACRO_HIP_TILED_PRODUCT_SPLIT=-1 / =<n>  never share out the contracted range / share it out n ways
+//   ACRO_HIP_TILED_PRODUCT_OPERATOR=<entries>  a product without a batch index one of whose factors has at most this many entries
+//                               is left to the operator schedule (4 096)
 #ifndef ACRO_HIP_CODEGEN_HPP
 #define ACRO_HIP_CODEGEN_HPP
 
