@@ -81,9 +81,14 @@ auto Generator::EmitGram(HipKernelPlan &plan) -> void
     const long nI = g.rows, nJ = g.cols, N = g.range, O = nI * nJ;
     const long TI = (nI + 15) / 16, TJ = (nJ + 15) / 16;
     const long groups = (N + 3) / 4;                      // four rows of N per instruction
-    // One workgroup of four wavefronts per CU and as many again: each wavefront strides over the groups of rows.
-    // (256 workgroups: 269 / 207 us for 64 x 64 / 32 x 32 outputs, 512: 280 / 195 us, 1 024: 312 / 262 us)
-    const long G = std::max<long>(1, std::min<long>(512, groups / 16));
+    // One workgroup of four wavefronts per CU, or two: each wavefront strides over the groups of rows.  Whole blocks of
+    // outputs, four or more of them: one (the loop then has no selects for a second wavefront to hide, and with 16
+    // blocks only one wavefront fits a SIMD anyway, so 512 workgroups ran as two rounds of 256); outputs that 16 does
+    // not divide, and a single block: two.  512 MB of operands, tensors rotated, % of the HBM peak with 256 / 512 / 768
+    // workgroups: 64 x 64 63 / 55 / 49, 64 x 48 68 / 60 / 56, 64 x 32 72 / 61 / 61, 32 x 32 71 / 64 / 61; 48 x 40 56 / 64 / 50,
+    // 40 x 40 54 / 63 / 49, 24 x 24 60 / 65 / 59, 16 x 16 66 / 70 / 62, 12 x 12 63 / 65 / 59.
+    const bool wholeBlocks = nI % 16 == 0 && nJ % 16 == 0 && TI * TJ >= 4;
+    const long G = envInt("ACRO_HIP_GRAM_GROUPS") > 0 ? envInt("ACRO_HIP_GRAM_GROUPS") : std::max<long>(1, std::min<long>(wholeBlocks ? 256 : 512, groups / 16));
 
     const std::string dimName = mk.GetDimensionedNameString();
     char hex[32];
@@ -118,35 +123,62 @@ auto Generator::EmitGram(HipKernelPlan &plan) -> void
     // (48 x 40 with a weight per row: 157 us with 2 groups, 181 us with 4)
     const long U = TI + TJ >= 8 ? 4 : std::max<long>(1, 16 / (TI + TJ));
     const long stride = G * 4;
-    out << "    auto fetch = [&](long g0, double (&bq)[" << U << "][" << TI << "], double (&cq)[" << U << "][" << TJ << "]) {\n";
-    out << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u)\n        {\n";
-    out << "            const long n = (g0 + u * " << stride << ") * 4 + k;\n";
-    out << "            const bool inRange = n < " << N << ";\n";
-    out << "            const double *b = " << B << " + " << Lit(uvars[g.b->uvar].viewOffset) << " + (inRange ? n : 0) * " << nI << " + r;\n";
-    out << "            const double *c = " << C << " + " << Lit(uvars[g.c->uvar].viewOffset) << " + (inRange ? n : 0) * " << nJ << " + r;\n";
-    out << "#pragma unroll\n            for (int ti = 0; ti < " << TI << "; ++ti) bq[u][ti] = (inRange"
-        << (nI % 16 != 0 ? " && 16 * ti + r < " + str(nI) : std::string()) << ") ? b[16 * ti] : 0.0;\n";
-    out << "#pragma unroll\n            for (int tj = 0; tj < " << TJ << "; ++tj) cq[u][tj] = (inRange"
-        << (nJ % 16 != 0 ? " && 16 * tj + r < " + str(nJ) : std::string()) << ") ? c[16 * tj] : 0.0;\n";
-    if (g.w)
+    // Two forms of the loads of a step: `fetch` serves any rows (rows past the end of the range read as zero, their
+    // addresses fall back to row 0), `fetchInside` only rows that all exist: no selects on the loaded values, which the
+    // first form needs one or two of per value.  The main loop takes two steps per turn, the operands of the one in the
+    // registers that the other has just used up (no copies), and runs while both steps' rows are inside the range; the
+    // steps near the end go one at a time through `fetch`.  With one wavefront per SIMD (16 blocks of sums are 128
+    // registers, the operands of two steps as many again) nothing else hides those instructions: 64 x 64 over 2^20 rows
+    // 53 -> 67 % of the HBM peak with both changes and one workgroup per CU, 5.9 -> 2.6 vector instructions per
+    // matrix instruction.
+    for (int inside = 0; inside < 2; ++inside)
     {
-        out << "            const double w = " << PtrName(g.w->uvar) << "[" << Lit(uvars[g.w->uvar].viewOffset) << " + (inRange ? n : 0)];\n";
-        // on the side with fewer blocks
-        if (TI <= TJ)
-            out << "#pragma unroll\n            for (int ti = 0; ti < " << TI << "; ++ti) bq[u][ti] *= w;\n";
-        else
-            out << "#pragma unroll\n            for (int tj = 0; tj < " << TJ << "; ++tj) cq[u][tj] *= w;\n";
+        out << "    auto " << (inside ? "fetchInside" : "fetch") << " = [&](long g0, double (&bq)[" << U << "][" << TI << "], double (&cq)[" << U << "][" << TJ << "]) {\n";
+        out << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u)\n        {\n";
+        out << "            const long n = (g0 + u * " << stride << ") * 4 + k;\n";
+        const std::string row = inside ? "n" : "(inRange ? n : 0)";
+        const std::string ok = inside ? "" : "inRange";
+        if (!inside) out << "            const bool inRange = n < " << N << ";\n";
+        out << "            const double *b = " << B << " + " << Lit(uvars[g.b->uvar].viewOffset) << " + " << row << " * " << nI << " + r;\n";
+        out << "            const double *c = " << C << " + " << Lit(uvars[g.c->uvar].viewOffset) << " + " << row << " * " << nJ << " + r;\n";
+        auto guarded = [&](long extentHere, const std::string &t, const std::string &load) {
+            std::string cond = ok;
+            if (extentHere % 16 != 0) cond += (cond.empty() ? "" : " && ") + std::string("16 * ") + t + " + r < " + str(extentHere);
+            return cond.empty() ? load : "(" + cond + ") ? " + load + " : 0.0";
+        };
+        out << "#pragma unroll\n            for (int ti = 0; ti < " << TI << "; ++ti) bq[u][ti] = " << guarded(nI, "ti", "b[16 * ti]") << ";\n";
+        out << "#pragma unroll\n            for (int tj = 0; tj < " << TJ << "; ++tj) cq[u][tj] = " << guarded(nJ, "tj", "c[16 * tj]") << ";\n";
+        if (g.w)
+        {
+            out << "            const double w = " << PtrName(g.w->uvar) << "[" << Lit(uvars[g.w->uvar].viewOffset) << " + " << row << "];\n";
+            // on the side with fewer blocks
+            if (TI <= TJ)
+                out << "#pragma unroll\n            for (int ti = 0; ti < " << TI << "; ++ti) bq[u][ti] *= w;\n";
+            else
+                out << "#pragma unroll\n            for (int tj = 0; tj < " << TJ << "; ++tj) cq[u][tj] *= w;\n";
+        }
+        out << "        }\n    };\n";
     }
-    out << "        }\n    };\n";
+    auto emitProducts = [&](const std::string &bName, const std::string &cName, const std::string &ind) {
+        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << U << "; ++u)\n";
+        out << "#pragma unroll\n" << ind << "    for (int ti = 0; ti < " << TI << "; ++ti)\n";
+        out << "#pragma unroll\n" << ind << "        for (int tj = 0; tj < " << TJ << "; ++tj)\n";
+        out << ind << "            acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(" << bName << "[u][ti], " << cName << "[u][tj], acc[ti][tj], 0, 0, 0);\n";
+    };
+    const long step = U * stride, fullGroups = N / 4;   // groups of four rows that all exist
     out << "    double bv[" << U << "][" << TI << "], cv[" << U << "][" << TJ << "], bn[" << U << "][" << TI << "], cn[" << U << "][" << TJ << "];\n";
-    out << "    const long first = (long)blockIdx.x * 4 + wave;\n";
-    out << "    fetch(first, bv, cv);\n";
-    out << "    for (long g0 = first; g0 < " << groups << "; g0 += " << U * stride << ")\n    {\n";
-    out << "        fetch(g0 + " << U * stride << ", bn, cn);\n";
-    out << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u)\n";
-    out << "#pragma unroll\n            for (int ti = 0; ti < " << TI << "; ++ti)\n";
-    out << "#pragma unroll\n                for (int tj = 0; tj < " << TJ << "; ++tj)\n";
-    out << "                    acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(bv[u][ti], cv[u][tj], acc[ti][tj], 0, 0, 0);\n";
+    out << "    long g0 = (long)blockIdx.x * 4 + wave;\n";
+    out << "    fetch(g0, bv, cv);\n";
+    // (the last group that the second fetch of a turn touches is g0 + 2 * step + (U - 1) * stride)
+    out << "    for (; g0 + " << 2 * step + (U - 1) * stride << " < " << fullGroups << "; g0 += " << 2 * step << ")\n    {\n";
+    out << "        fetchInside(g0 + " << step << ", bn, cn);\n";
+    emitProducts("bv", "cv", "        ");
+    out << "        fetchInside(g0 + " << 2 * step << ", bv, cv);\n";
+    emitProducts("bn", "cn", "        ");
+    out << "    }\n";
+    out << "    for (; g0 < " << groups << "; g0 += " << step << ")\n    {\n";
+    out << "        fetch(g0 + " << step << ", bn, cn);\n";
+    emitProducts("bv", "cv", "        ");
     out << "#pragma unroll\n        for (int u = 0; u < " << U << "; ++u)\n        {\n";
     out << "#pragma unroll\n            for (int ti = 0; ti < " << TI << "; ++ti) bv[u][ti] = bn[u][ti];\n";
     out << "#pragma unroll\n            for (int tj = 0; tj < " << TJ << "; ++tj) cv[u][tj] = cn[u][tj];\n";
@@ -197,7 +229,7 @@ auto Generator::EmitGram(HipKernelPlan &plan) -> void
     HipLaunch partial;
     partial.function_name = fPartial;
     partial.grid = static_cast<unsigned>(G);
-    partial.block = 256;
+    partial.block = envInt("ACRO_HIP_GRAM_BLOCK") > 0 ? envInt("ACRO_HIP_GRAM_BLOCK") : 256;
     for (int si = 0; si < S; ++si) partial.params.push_back(si);
     partial.params.push_back(-1);
     plan.launches.push_back(partial);
