@@ -486,6 +486,10 @@ auto Generator::ProductThenRowSums(int ki, const Sub &orig, std::vector<Sub> &re
 {
     if (envInt("ACRO_HIP_ROW_SUMS") < 0 || batch < 0 || orig.in.size() != 2 || orig.contr.empty() || !opt.noalias) return false;
     if (orig.out.repeated || orig.matrixOp != 0) return false;
+    {
+        ProductShape onMatrixCores;  // (the product schedule takes matrices of up to 128 x 128 with such rows)
+        if (ProductPattern(orig, onMatrixCores)) return false;
+    }
     const VarRef *matrix = nullptr, *vec = nullptr;
     for (const auto &r : orig.in)
     {

@@ -29,10 +29,19 @@ auto Generator::ProductPattern(const Sub &s, ProductShape &p) const -> bool
 {
     if (envInt("ACRO_HIP_PRODUCT") < 0 || opt.no_matrix_cores || batch < 0 || !opt.noalias || NumGatherSlots() > 0) return false;
     if (mk.GetNumKernels() != 1 || s.matrixOp != 0 || s.out.repeated || s.in.size() != 2 || s.contr.size() != 1) return false;
-    if (s.out.idx.size() != 3 || s.out.idx[0] != batch) return false;
-    const int k = s.contr[0], r = s.out.idx[1], c = s.out.idx[2];
+    // (an element matrix applied to an element vector, "A_e_r = R_e_r_k X_e_k", is the product with a single column)
+    const bool vectorForm = s.out.idx.size() == 2;
+    if ((s.out.idx.size() != 3 && !vectorForm) || s.out.idx[0] != batch) return false;
+    const int k = s.contr[0], r = s.out.idx[1], c = vectorForm ? -1 : s.out.idx[2];
     for (const auto &v : s.in)
     {
+        if (vectorForm && !v.repeated && v.idx.size() == 2 && v.idx[0] == batch && v.idx[1] == k && !p.col && v.uvar != s.out.uvar &&
+            !(uvars[v.uvar].storage >= 0 && uvars[v.uvar].storage == uvars[s.out.uvar].storage))
+        {
+            p.col = &v;
+            p.colKFast = true;
+            continue;
+        }
         if (v.repeated || v.idx.size() != 3 || v.idx[0] != batch) return false;
         // (the pattern is also asked for while the model is being built, before storages are known)
         if (v.uvar == s.out.uvar || (uvars[v.uvar].storage >= 0 && uvars[v.uvar].storage == uvars[s.out.uvar].storage)) return false;
@@ -54,20 +63,34 @@ auto Generator::ProductPattern(const Sub &s, ProductShape &p) const -> bool
     }
     if (!p.row || !p.col) return false;
     p.M = extent[r];
-    p.N = extent[c];
+    p.N = vectorForm ? 1 : extent[c];
     p.K = extent[k];
     p.E = extent[batch];
+    if (vectorForm)
+    {
+        // Rows that are no whole number of 32-byte pieces (27 x 27, 25 x 25, 45 x 45): with the lanes along the rows a
+        // wavefront reads its matrices in pieces of a row that start anywhere in a line (47 - 59 % of the HBM peak with
+        // any of the vector-ALU schedules).  Here every strip of 16 rows is one contiguous range read front to back, and
+        // the 15 unused columns of the matrix instruction cost nothing that shows: 27 x 27 needs 14 instructions per
+        // entry, 48 us of matrix time for 127 us of memory time.  Rows of a multiple of four doubles keep the lanes that
+        // share a contraction (69 - 76 %).
+        if (!p.rowKFast || envInt("ACRO_HIP_PRODUCT_VECTOR") < 0) return false;
+        // (rotated tensors, % of the HBM peak, two-step vector-ALU schedule / this one: 27 x 27 57 / 67, 25 x 25 58 / 63,
+        // 31 x 31 57 / 70, 45 x 45 59 / 70, 63 x 63 58 / 73, 64 x 27 60 / 74, 27 x 45 58 / 72; short rows the other way
+        // round: 21 x 21 62 / 52, 17 x 17 60 / 38, 13 x 13 59 / 56, 9 x 9 63 / 35)
+        if (p.K % 4 == 0 || p.K < 25 || p.K > 128 || p.M < 16 || p.M > 128) return false;
+    }
     // From 17 rows or columns on (up to 16 x 16 the staged schedule has a lane per output and is bound by memory);
     // a wavefront holds one strip of at most eight column blocks, an entry at most eight strips.
     const long lo = envInt("ACRO_HIP_PRODUCT_FROM", 17), hi = envInt("ACRO_HIP_PRODUCT_TO", 64);
-    if (std::max(p.M, p.N) < lo || p.M > hi || p.N > hi || p.K > 128 || p.K < 8 || p.M < 8 || p.N < 8) return false;
+    if (!vectorForm && (std::max(p.M, p.N) < lo || p.M > hi || p.N > hi || p.K > 128 || p.K < 8 || p.M < 8 || p.N < 8)) return false;
     // Up to 36 x 36 the staged vector-ALU schedule is as fast or a little faster where it can give a lane a block of
     // outputs, i.e. where both extents have a divisor 2, 3 or 5 (rotated buffers, % of the HBM peak, staged / here:
     // 20 x 20 75 / 71, 24 x 24 75 / 72, 25 x 25 74 / 71, 28 x 28 74 / 73, 33 x 33 67 / 64, 36 x 36 71 / 70; without such
     // a divisor 17 x 17 59 / 67, 31 x 31 42 / 71, 37 x 37 37 / 70; larger: 40 x 40 69 / 69, 45 x 45 67 / 69, 48 x 48 69 / 70,
     // 53 x 53 28 / 68, 55 x 55 23 / 68, 56 x 56 58 / 69, 63 x 63 32 / 67, 64 x 64 15 / 70).
     auto blocks = [](long n) { return n % 2 == 0 || n % 3 == 0 || n % 5 == 0; };
-    if (std::max(p.M, p.N) <= 36 && blocks(p.M) && blocks(p.N) && envInt("ACRO_HIP_PRODUCT") < 2) return false;
+    if (!vectorForm && std::max(p.M, p.N) <= 36 && blocks(p.M) && blocks(p.N) && envInt("ACRO_HIP_PRODUCT") < 2) return false;
     p.TI = (p.M + 15) / 16;
     p.TJ = (p.N + 15) / 16;
     if (p.TI > 8 || p.TJ > 8) return false;

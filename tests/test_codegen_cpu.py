@@ -597,6 +597,12 @@ def test_products_of_element_matrices_run_on_the_matrix_cores(TE, monkeypatch):
     # an odd number of doubles in the whole tensor: its last one is read on its own
     src = product("A_e_i_j = B_e_i_k C_e_k_j", 17, 17, 17, E=4097)
     assert "if (at == 1184032L) cv[it].x = T2[1184032L];" in src
+    # an element matrix applied to an element vector, rows that are no whole number of 32-byte pieces: a single column
+    src = TE.GetImplementation("A_e_i = B_e_i_j C_e_j", at.Tensor(4096, 27), at.Tensor(4096, 27, 27), at.Tensor(4096, 27))
+    assert "product schedule on the FP64 matrix cores: 27 x 27 by 27 x 1 per entry" in src and "2 strips of 16 rows x 1 blocks of 16 columns" in src
+    for rows, cols in ((27, 32), (21, 21), (9, 45)):     # rows of whole pieces, short rows, few rows: the vector-ALU schedules
+        assert "product schedule" not in TE.GetImplementation("A_e_i = B_e_i_j C_e_j", at.Tensor(4096, rows), at.Tensor(4096, rows, cols), at.Tensor(4096, cols))
+    assert "product schedule" not in TE.GetImplementation("A_e_i = B_e_i_j C_j", at.Tensor(4096, 27), at.Tensor(4096, 27, 27), at.Tensor(27))
     # not this schedule: small matrices whose extents the staged schedule can split into blocks, 16 x 16 and smaller,
     # a shared factor, more than two factors, too few entries for e to be the batch index
     assert "product schedule" not in product("A_e_i_j = B_e_i_k C_e_k_j", 24, 24, 24)

@@ -261,6 +261,11 @@ PRODUCTS_ON_THE_MATRIX_CORES = [
     # tensors of odd length whose last double sits in a 16-byte piece that is not a lane's last one
     ("A_e_i_j = C_e_k_j B_e_k_i", [(129, 93, 11), (129, 93, 49)]),
     ("A_e_i_j = B_e_i_k C_e_k_j", [(145, 27, 67), (145, 67, 19)]),
+    # an element matrix applied to an element vector, rows that are no multiple of four doubles: a single column
+    ("A_e_i = B_e_i_j C_e_j", [(1001, 27, 27), (1001, 27)]),
+    ("A_e_i += B_e_i_j C_e_j", [(333, 45, 31), (333, 31)]),
+    ("A_e_i -= C_e_j B_e_i_j", [(129, 27), (129, 64, 27)]),
+    ("A_e_i = B_e_i_j C_e_j", [(177, 125, 63), (177, 63)]),
 ]
 
 
@@ -1083,7 +1088,7 @@ def test_long_output_runs_leave_through_an_lds_tile(at, engine, checker, kernel,
 
 
 @pytest.mark.parametrize("kernel,shapes", [
-    ("A_e_i = B_e_i_j C_e_j", [(300, 27, 27), (300, 27)]),        # rows of 27: products into LDS, then row sums
+    ("A_e_i = B_e_i_j C_e_j", [(300, 21, 21), (300, 21)]),        # rows of 21: products into LDS, then row sums (from 25 on: matrix cores)
     ("A_e_i += B_e_i_j C_e_j", [(77, 9, 25), (77, 25)]),
     ("A_e_i -= C_e_j B_e_i_j", [(50, 33), (50, 12, 33)]),
     ("A_e_i = B_e_i_j_k C_e_j_k", [(40, 6, 3, 7), (40, 3, 7)]),   # two contraction indices, 21 terms
