@@ -78,7 +78,7 @@ auto Generator::ProductPattern(const Sub &s, ProductShape &p) const -> bool
         // (rotated tensors, % of the HBM peak, two-step vector-ALU schedule / this one: 27 x 27 57 / 67, 25 x 25 58 / 63,
         // 31 x 31 57 / 70, 45 x 45 59 / 70, 63 x 63 58 / 73, 64 x 27 60 / 74, 27 x 45 58 / 72; short rows the other way
         // round: 21 x 21 62 / 52, 17 x 17 60 / 38, 13 x 13 59 / 56, 9 x 9 63 / 35)
-        if (p.K % 4 == 0 || p.K < 25 || p.K > 128 || p.M < 16 || p.M > 128) return false;
+        if ((p.K % 4 == 0 && envInt("ACRO_HIP_PRODUCT_VECTOR") < 2) || p.K < 25 || p.K > 128 || p.M < 16 || p.M > 128) return false;
     }
     // From 17 rows or columns on (up to 16 x 16 the staged schedule has a lane per output and is bound by memory);
     // a wavefront holds one strip of at most eight column blocks, an entry at most eight strips.

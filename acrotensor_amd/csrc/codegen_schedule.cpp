@@ -786,7 +786,12 @@ auto Generator::ChooseCopyOutTile() -> void
     // lanes (i2, j2) and tile (i1, j1) writes pieces of 32 bytes 128 bytes apart (52 % of the HBM peak; through the
     // tile see the schedule comment).
     bool scattered = false;
-    if (run < 8 && envInt("ACRO_HIP_COPY_OUT_TILE") < 2)
+    // (a run of four doubles per lane is enough: the lanes' pieces are 32 - 56 bytes long and as far apart, every store
+    // instruction touches every line of the wavefront's range, and from HBM that costs more than it does out of the
+    // memory-side cache.  Rotated tensors, by the lanes / through the tile: 7 x 9 operator 59 -> 72 %, 7 x 7 59 -> 75 %,
+    // 5 x 5 64 -> 75 %, 4 x 4 69 -> 75 %, outer product of two 8-vectors 78 -> 91 %.)
+    const long longRun = envInt("ACRO_HIP_COPY_OUT_RUN", 4);
+    if (run < longRun && envInt("ACRO_HIP_COPY_OUT_TILE") < 2)
     {
         const int entries = static_cast<int>(std::max<long>(1, 64 / std::max<long>(1, s.laneCount)));
         const double coverage = WaveStoreLineCoverage(k, entries);
@@ -794,7 +799,7 @@ auto Generator::ChooseCopyOutTile() -> void
                                          (coverage < 0.95 && envInt("ACRO_HIP_COPY_OUT_WRITERS") >= 0 && WritesDominate()));
     }
     if (subs.size() != 1 && !scattered) return;
-    if (run < 8 && !scattered) return;
+    if (run < longRun && !scattered) return;
     st.copyOutOnly = true;
     st.wantLds = true;
     st.liveTo = k;
