@@ -129,7 +129,7 @@ auto Generator::EmitGram(HipKernelPlan &plan) -> void
     // registers that the other has just used up (no copies), and runs while both steps' rows are inside the range; the
     // steps near the end go one at a time through `fetch`.  With one wavefront per SIMD (16 blocks of sums are 128
     // registers, the operands of two steps as many again) nothing else hides those instructions: 64 x 64 over 2^20 rows
-    // 53 -> 67 % of the HBM peak with both changes and one workgroup per CU, 5.9 -> 2.6 vector instructions per
+    // 54 -> 70 % of the HBM peak with both changes and one workgroup per CU, 5.8 -> 2.4 other vector instructions per
     // matrix instruction.
     for (int inside = 0; inside < 2; ++inside)
     {
