@@ -229,7 +229,7 @@ auto Generator::EmitGram(HipKernelPlan &plan) -> void
     HipLaunch partial;
     partial.function_name = fPartial;
     partial.grid = static_cast<unsigned>(G);
-    partial.block = envInt("ACRO_HIP_GRAM_BLOCK") > 0 ? envInt("ACRO_HIP_GRAM_BLOCK") : 256;
+    partial.block = 256;
     for (int si = 0; si < S; ++si) partial.params.push_back(si);
     partial.params.push_back(-1);
     plan.launches.push_back(partial);

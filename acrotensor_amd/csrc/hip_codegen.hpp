@@ -134,6 +134,11 @@
 //   ACRO_HIP_NT_COPY_OUT=-1     copies out of LDS tiles use non-temporal stores only for tiles of at most 20 KB
 //   ACRO_HIP_NT_STORE=2         non-temporal stores from registers also in launches that hold more than 20 KB of LDS per workgroup
 //   ACRO_HIP_OPERATOR_GROUPS=<n>  workgroups of the matrix-core operator kernel (default: 256 - 1 024 by the operator's size)
+//   ACRO_HIP_GRAM_GROUPS=<n>    workgroups of the Gram schedule's first kernel (default: 256 where the blocks of outputs are whole, else 512)
+//   ACRO_HIP_PRODUCT_VECTOR=-1 / =2  an element matrix applied to an element vector never takes the product schedule / takes it
+//                               whatever its row length (default: rows of 25 - 128 doubles that are no multiple of four, 16 - 128 rows)
+//   ACRO_HIP_COPY_OUT_RUN=<n>   a kernel on its own whose lanes each hold a run of n or more consecutive outputs writes them out
+//                               through an LDS tile (default 4)
 //   ACRO_HIP_XCD_RUN=-1 / =<n>  fused launches that read an operand through an index map number their workgroups as the hardware
 //                               deals them / in runs of n per XCD (default 16)
 //   ACRO_HIP_TILED_PRODUCT=-1   large matrix products (more than 64 rows or columns or 128 terms per entry, or no batch index) keep
