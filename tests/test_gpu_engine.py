@@ -396,6 +396,57 @@ def test_products_of_large_matrices_in_tiles_views_and_special_values(at, engine
     assert np.array_equal(np.nan_to_num(tA.data), np.nan_to_num(expected))
 
 
+@pytest.mark.gpu
+def test_large_matrix_product_in_tiles_through_properties(at, engine):
+    """A 2 048 x 1 536 x 2 560 product without a batch index (256 tiles, 160 chunks of terms each), too large for the
+    checker's loops: (B C) x must equal B (C x) for random x, rows and columns of ones must give the row and column sums,
+    and integer-valued factors must give the exact integer product in sampled entries."""
+    rng = np.random.default_rng(77)
+    m, k, n = 2048, 2560, 1536
+    B = rng.integers(-3, 4, (m, k)).astype(np.float64)
+    C = rng.integers(-3, 4, (k, n)).astype(np.float64)
+    tA, tB, tC = at.Tensor(m, n), to_tensor(at, B), to_tensor(at, C)
+    engine("A_i_j = B_i_k C_k_j", tA, tB, tC)
+    assert "tiled product schedule on the FP64 matrix cores" in engine.GetLastImplementation()
+    tA.MoveFromGPU()
+    A = tA.data
+    x = rng.integers(-2, 3, (n, 3)).astype(np.float64)
+    assert np.array_equal(A @ x, B @ (C @ x))                                   # integers: exact in any order
+    y = rng.integers(-2, 3, (3, m)).astype(np.float64)
+    assert np.array_equal(y @ A, (y @ B) @ C)
+    rows = rng.integers(0, m, 40)
+    assert np.array_equal(A[rows], B[rows] @ C)
+    # the same with the second factor transposed and accumulation, random data: <= 1e-12 against numpy in sampled rows
+    Bf, Cf = rng.uniform(-1, 1, (m, k)), rng.uniform(-1, 1, (n, k))
+    A0 = rng.uniform(-1, 1, (m, n))
+    tA, tB, tC = to_tensor(at, A0), to_tensor(at, Bf), to_tensor(at, Cf)
+    engine("A_i_j += B_i_k C_j_k", tA, tB, tC)
+    tA.MoveFromGPU()
+    assert rel_err(tA.data[rows], A0[rows] + Bf[rows] @ Cf.T) <= TOL
+
+
+@pytest.mark.gpu
+def test_normal_equations_with_many_columns_share_out_the_rows(at, engine):
+    """A_i_j = B_n_i C_n_j with 144 x 128 outputs over 2^17 rows: more blocks than the Gram schedule holds, so tiles with
+    the contracted range shared out over 86 workgroups per tile; against numpy, integer data exact, twice in a row
+    (the scratch buffer of partial tiles is reused)."""
+    rng = np.random.default_rng(78)
+    rows, ni, nj = 1 << 17, 144, 128
+    B = rng.integers(-3, 4, (rows, ni)).astype(np.float64)
+    C = rng.integers(-3, 4, (rows, nj)).astype(np.float64)
+    tA, tB, tC = at.Tensor(ni, nj), to_tensor(at, B), to_tensor(at, C)
+    expected = B.T @ C
+    for _ in range(2):
+        engine("A_i_j = B_n_i C_n_j", tA, tB, tC)
+        src = engine.GetLastImplementation()
+        assert "tiled product schedule" in src and "shares of" in src
+        tA.MoveFromGPU()
+        assert np.array_equal(tA.data, expected)
+    engine("A_i_j -= B_n_i C_n_j", tA, tB, tC)
+    tA.MoveFromGPU()
+    assert np.array_equal(tA.data, np.zeros((ni, nj)))
+
+
 def test_product_of_slices_keeps_its_indices(at, engine, checker):
     # operands that are views into larger tensors are not described by split dimensions
     rng = np.random.default_rng(12)
