@@ -522,7 +522,7 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
           << (p.rowKFast ? "with the contracted index last" : "with the contracted index first") << ", column factor "
           << (p.colKFast ? "with the contracted index last" : "with the contracted index first") << "), tiles of " << 16 * W << " rows x "
           << 16 * TJ << " columns (" << p.tilesM << " x " << p.panels << " per entry), chunks of " << KC << " terms through "
-          << (rowTile + colTile) * 8 << " bytes of LDS, " << groups * splits << " workgroups of " << NT << " lanes";
+          << (envInt("ACRO_HIP_TILED_PRODUCT_LDS") == 2 ? 2 : 1) * (UA + UB) * NT * 8 << " bytes of LDS, " << groups * splits << " workgroups of " << NT << " lanes";
     if (splits > 1) sched << ", the contracted range in " << splits << " shares of " << span << " terms whose partial sums a second kernel adds";
     sched << "\n  [0] " << s.text << "\n";
     plan.schedule = sched.str();
@@ -544,8 +544,9 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
     const std::string fMain = splits > 1 ? plan.module_name + "_partial" : plan.module_name, fFinal = plan.module_name + "_final";
     out << "void " << fMain << "(" << ParamList() << (splits > 1 ? ", double *__restrict__ scratch" : "") << ")\n{\n";
     // (padded to a whole number of values per lane: lanes without a value of the tile write into the padding, no branch)
-    out << "    __shared__ double fragA[" << UA * NT << "];\n";
-    out << "    __shared__ double fragB[" << UB * NT << "];\n";
+    const long ldsHalves = envInt("ACRO_HIP_TILED_PRODUCT_LDS") == 2 ? 2 : 1;
+    out << "    __shared__ double fragA[" << ldsHalves * UA * NT << "];\n";
+    out << "    __shared__ double fragB[" << ldsHalves * UB * NT << "];\n";
     out << "    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;\n";
     if (splits > 1)
     {
@@ -585,34 +586,59 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
     out << "    }\n";
     const std::string aStep = p.rowKFast ? "k0" : "(long)k0 * " + str(M);
     const std::string bStep = p.colKFast ? "k0" : "(long)k0 * " + str(N);
+    // One copy of a chunk's fragments in LDS and two barriers per chunk (before the fragments are overwritten and after).
+    // Measured against that and not kept as the default: two halves of LDS, the next chunk written to one while the other is
+    // multiplied, one barrier per chunk (ACRO_HIP_TILED_PRODUCT_LDS=2: 80^3 per entry 57 -> 62 %, 128 x 128 x 2^18 37 -> 41
+    // TFLOP/s, but 128^3 per entry 53 -> 50 %, 2 048^3 58 -> 53 TFLOP/s); two chunks on their way in two sets of registers
+    // (4 096^3 62 -> 53 TFLOP/s): neither the barriers nor the latency of the loads is what these kernels wait for.
+    const long halves = envInt("ACRO_HIP_TILED_PRODUCT_LDS") == 2 ? 2 : 1;
     out << "    double ra[" << UA << "], rb[" << UB << "];\n";
-    auto emitLoads = [&](const std::string &ind) {
+    auto emitLoads = [&](const std::string &ind, const std::string &k0) {
         // (no branches around the loads and no use of their values here, so that all of them are in flight together and
-        // stay so while the previous chunk is multiplied: a value that does not exist is read from the entry's first
+        // stay so while the chunk before is multiplied: a value that does not exist is read from the entry's first
         // element and replaced by zero when it is written to LDS)
-        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UA << "; ++u) ra[u] = Rm[k0 + aK[u] < kEnd ? " << aStep << " + aFrom[u] : 0];\n";
-        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UB << "; ++u) rb[u] = Cm[k0 + bK[u] < kEnd ? " << bStep << " + bFrom[u] : 0];\n";
+        out << ind << "{\n" << ind << "    const int k0 = " << k0 << ";\n";
+        out << "#pragma unroll\n" << ind << "    for (int u = 0; u < " << UA << "; ++u) ra[u] = Rm[k0 + aK[u] < kEnd ? " << aStep << " + aFrom[u] : 0];\n";
+        out << "#pragma unroll\n" << ind << "    for (int u = 0; u < " << UB << "; ++u) rb[u] = Cm[k0 + bK[u] < kEnd ? " << bStep << " + bFrom[u] : 0];\n";
+        out << ind << "}\n";
     };
-    out << "    {\n        const int k0 = kBegin;\n";
-    emitLoads("        ");
-    out << "    }\n";
+    auto emitToLds = [&](const std::string &ind, const std::string &kHere, const std::string &half) {
+        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UA << "; ++u) fragA[" << (half.empty() ? std::string() : half + str(UA * NT) + " + ") << "aTo[u]] = " << kHere << " + aK[u] < kEnd ? ra[u] : 0.0;\n";
+        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UB << "; ++u) fragB[" << (half.empty() ? std::string() : half + str(UB * NT) + " + ") << "bTo[u]] = " << kHere << " + bK[u] < kEnd ? rb[u] : 0.0;\n";
+    };
+    auto emitProducts = [&](const std::string &ind, const std::string &half) {
+        out << "#pragma unroll\n" << ind << "for (int s = 0; s < " << KS << "; ++s)\n" << ind << "{\n";
+        out << ind << "    const int at = s * 64 + g * 16 + ((c + 4 * s + g) & 15);\n";
+        out << ind << "    const double a = fragA[" << (half.empty() ? std::string() : half + str(UA * NT) + " + ") << "wave * " << KS * 64 << " + at];\n";
+        out << "#pragma unroll\n" << ind << "    for (int J = 0; J < " << TJ << "; ++J)\n";
+        out << ind << "        acc[J] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, fragB[" << (half.empty() ? std::string() : half + str(UB * NT) + " + ") << "J * " << KS * 64 << " + at], acc[J], 0, 0, 0);\n";
+        out << ind << "}\n";
+    };
+    emitLoads("    ", "kBegin");
     out << "    acro_double4 acc[" << TJ << "];\n";
     out << "#pragma unroll\n    for (int J = 0; J < " << TJ << "; ++J) acc[J] = acro_double4{0.0, 0.0, 0.0, 0.0};\n";
-    out << "    for (int kc = kBegin; kc < kEnd; kc += " << KC << ")\n    {\n";
-    out << "#pragma unroll\n        for (int u = 0; u < " << UA << "; ++u) fragA[aTo[u]] = kc + aK[u] < kEnd ? ra[u] : 0.0;\n";
-    out << "#pragma unroll\n        for (int u = 0; u < " << UB << "; ++u) fragB[bTo[u]] = kc + bK[u] < kEnd ? rb[u] : 0.0;\n";
-    out << "        __syncthreads();\n";
-    out << "        {\n            const int k0 = kc + " << KC << ";   // the next chunk is on its way while this one is multiplied (past the end: zeros, no loads)\n";
-    emitLoads("            ");
-    out << "        }\n";
-    out << "#pragma unroll\n        for (int s = 0; s < " << KS << "; ++s)\n        {\n";
-    out << "            const int at = s * 64 + g * 16 + ((c + 4 * s + g) & 15);\n";
-    out << "            const double a = fragA[wave * " << KS * 64 << " + at];\n";
-    out << "#pragma unroll\n            for (int J = 0; J < " << TJ << "; ++J)\n";
-    out << "                acc[J] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, fragB[J * " << KS * 64 << " + at], acc[J], 0, 0, 0);\n";
-    out << "        }\n";
-    out << "        __syncthreads();\n";
-    out << "    }\n";
+    if (halves == 2)
+    {
+        emitToLds("    ", "kBegin", "0 * ");
+        out << "    __syncthreads();\n";
+        out << "    int half = 0;\n";
+        out << "    for (int kc = kBegin; kc < kEnd; kc += " << KC << ", half ^= 1)\n    {\n";
+        emitLoads("        ", "kc + " + str(KC));   // (past the end: no loads)
+        emitProducts("        ", "half * ");
+        emitToLds("        ", "kc + " + str(KC), "(half ^ 1) * ");
+        out << "        __syncthreads();\n";
+        out << "    }\n";
+    }
+    else
+    {
+        out << "    for (int kc = kBegin; kc < kEnd; kc += " << KC << ")\n    {\n";
+        emitToLds("        ", "kc", "");
+        out << "        __syncthreads();\n";
+        emitLoads("        ", "kc + " + str(KC));
+        emitProducts("        ", "");
+        out << "        __syncthreads();\n";
+        out << "    }\n";
+    }
     out << "#pragma unroll\n    for (int J = 0; J < " << TJ << "; ++J)\n";
     out << "#pragma unroll\n        for (int q = 0; q < 4; ++q)\n        {\n";
     out << "            const int m = r0 + 16 * wave + 4 * q + g, n = c0 + 16 * J + c;\n";
@@ -649,7 +675,7 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
 
     plan.source = out.str();
     plan.nb = 1;
-    plan.lds_bytes = static_cast<int>((rowTile + colTile) * 8);
+    plan.lds_bytes = static_cast<int>(ldsHalves * (UA + UB) * NT * 8);
     FillParams(plan, false);
     HipLaunch launch;
     launch.function_name = fMain;
