@@ -553,6 +553,18 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
         out << "    const int split = blockIdx.x / " << groups << ";\n    const long group = blockIdx.x % " << groups << ";\n";
         out << "    const int kBegin = split * " << span << ", kEnd = kBegin + " << span << " < " << K << " ? kBegin + " << span << " : " << K << ";\n";
     }
+    else if (tiles > 1 && tiles <= 4 && p.batched && envInt("ACRO_HIP_TILED_PRODUCT_XCD") >= 0)
+    {
+        // The tiles of an entry read the same strips of the factors.  Hardware deals consecutive workgroup ids round-robin
+        // to the eight XCDs, each with an L2 of its own: numbered as they come, the tiles of an entry would each fetch
+        // their factors through another L2.  Workgroup b is on XCD b % 8 and is that XCD's number b / 8; the tiles of an
+        // entry take consecutive numbers of one XCD.  (Rotated tensors, % of the HBM peak: 125^3 per entry 41 -> 44,
+        // 216^3 26.5 -> 28, 100^3 37 -> 38.5, 128^3 53 -> 54; with eight tiles per entry, 256^3, 28 -> 26: left as it comes.)
+        const long whole = groups / (8 * tiles) * (8 * tiles);
+        out << "    const long b_ = blockIdx.x;\n";
+        out << "    const long group = b_ >= " << whole << "L ? b_ : ((b_ / 8) / " << tiles << " * 8 + b_ % 8) * " << tiles << " + (b_ / 8) % " << tiles << ";\n";
+        out << "    const int kBegin = 0, kEnd = " << K << ";\n";
+    }
     else
         out << "    const long group = blockIdx.x;\n    const int kBegin = 0, kEnd = " << K << ";\n";
     out << "    const long e = group / " << tiles << ";\n";
