@@ -248,11 +248,14 @@ auto Generator::StageReusedOperands(int ki, const Sub &asWritten, std::vector<Su
     const long outputs = product(orig.outIdx, extent) / extent[batch];
     const long stageMost = envInt("ACRO_HIP_STAGE_MOST", 8000);
     if (outputs < 4 || outputs > stageMost / 2) return false;
-    // Tiny matrices (fewer than 64 outputs) are staged as well unless every operand's entry is a power of two of
-    // doubles: those lie in whole lines and the lanes read them well from device memory (4 x 4 products with one
-    // output per lane: 90 % of the HBM peak, 51 % staged), the others do not (3 x 3: 64 -> 82 %, 5 x 5: 46 -> 77 %,
-    // 6 x 6: 48 -> 80 %, 7 x 7: 46 -> 77 %, with some 500 outputs per workgroup of 256 lanes).
+    // Tiny matrices (fewer than 64 outputs) are staged as well (3 x 3: 64 -> 82 %, 5 x 5: 46 -> 77 %, 6 x 6: 48 -> 80 %,
+    // 7 x 7: 46 -> 77 % of the HBM peak, with some 500 outputs per workgroup of 256 lanes), except those with fewer than
+    // 16 outputs whose operands' entries are all powers of two of doubles: those lie in whole lines and the lanes read
+    // them as well from device memory (with the launches rotated over tensors that no cache holds: 2 x 2 times 2 x 8
+    // 77 % straight and 68 % staged, 2 x 8 times 8 x 4 70 and 69 %, 2 x 2 times 2 x 2 75 and 76 %; from 16 outputs on
+    // the tiles win: 4 x 4 times 4 x 4 61 -> 76 %, 4 x 2 times 2 x 4 68 -> 76 %, 8 x 2 times 2 x 2 73 -> 77 %).
     const bool tiny = outputs < 64;
+    const long wholeLinesFrom = envInt("ACRO_HIP_STAGE_WHOLE_LINES", 16);  // -1: never
     bool wholeLines = true;
     std::vector<char> staged(orig.in.size(), 0);
     long total = 0;
@@ -276,7 +279,7 @@ auto Generator::StageReusedOperands(int ki, const Sub &asWritten, std::vector<Su
     }
     // Two such operands: products of element matrices.  With one (an element vector under an element matrix, the
     // vectors of a dense operator) the kernel has schedules of its own that read the big operand once and well.
-    if (count < 2 || total > stageMost || (tiny && wholeLines)) return false;
+    if (count < 2 || total > stageMost || (tiny && wholeLines && (wholeLinesFrom < 0 || outputs < wholeLinesFrom))) return false;
     // More than 1 024 outputs or 2 048 staged values per entry (products of 33 x 33 to 62 x 62 matrices, which the lanes
     // read straight from device memory at 9 - 12 % of the HBM peak: staged 49 - 66 %): only the two factors of a
     // product, each of which carries a contracted index

@@ -91,6 +91,8 @@
 //   ACRO_HIP_STAGE_TRANSPOSED=-1 ... and the copy of a factor whose fastest dimension is contracted keeps the operand's layout
 //   ACRO_HIP_SPLIT_FIVE=-1      ... and extents divisible by five only are not split in five
 //   ACRO_HIP_STAGE_MOST=<n>     ... at most n staged values per entry (default 8000; 2048: matrices up to 32 x 32 only)
+//   ACRO_HIP_STAGE_WHOLE_LINES=<n> / =-1  tiny products (fewer than 64 outputs per entry) whose operands' entries are powers of two
+//                               of doubles are staged from n outputs per entry on (16) / never
 //   ACRO_HIP_STAGE=-1           small invariant operands with lane-dependent addresses stay in device memory (not staged in LDS)
 //   ACRO_HIP_SPLIT_PAIRS=-1     lanes that share a contraction take its terms one at a time also where they have few of them
 //   ACRO_HIP_SPLIT_LANES=-1     one lane per batch entry also for kernels with one output per entry (no lane exchanges)
@@ -147,6 +149,9 @@
 //                               terms per chunk (16), most strips per workgroup and blocks per strip (8, 8), waves per SIMD asked of
 //                               the compiler (none)
 //   ACRO_HIP_TILED_PRODUCT_SPLIT=-1 / =<n>  never share out the contracted range / share it out n ways
+//   ACRO_HIP_TILED_PRODUCT_LDS=2  two halves of LDS for the chunks, one barrier per chunk (default: one half, two barriers)
+//   ACRO_HIP_TILED_PRODUCT_XCD=-1  the tiles of an entry are numbered as the hardware deals them (default: an entry's two to four
+//                               tiles on one XCD, so that the strips they share pass through one L2)
 //   ACRO_HIP_TILED_PRODUCT_OPERATOR=<entries>  a product without a batch index one of whose factors has at most this many entries
 //                               is left to the operator schedule (4 096)
 #ifndef ACRO_HIP_CODEGEN_HPP

@@ -285,9 +285,12 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
 
 
 def test_tile_choice_follows_how_the_lanes_reach_device_memory(TE, monkeypatch):
-    # one lane per matrix product would read 128-byte pieces 128 bytes apart; tiny entries get one output per lane
+    # one lane per matrix product would read 128-byte pieces 128 bytes apart; tiny entries get one output per lane, from
+    # tiles in LDS; entries of whole lines with fewer than 16 outputs are read as well straight from device memory
     src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 4, 4), at.Tensor(4096, 4, 4), at.Tensor(4096, 4, 4))
-    assert "lanes(i,k)=16 tile()=1" in src
+    assert "lanes(i,k)=16 tile()=1" in src and "operands staged in LDS" in src and "32 per workgroup of 256 lanes" in src
+    src = TE.GetImplementation("A_e_i_k = B_e_i_j C_e_j_k", at.Tensor(4096, 2, 2), at.Tensor(4096, 2, 8), at.Tensor(4096, 8, 2))
+    assert "lanes(i,k)=4 tile()=1" in src and "operands staged in LDS" not in src
     # one lane per entry would read 512-byte rows 512 bytes apart and overflow the vector cache: one lane per row
     src = TE.GetImplementation("A_e_i = B_e_i_j C_e_j", at.Tensor(4096, 8), at.Tensor(4096, 8, 8), at.Tensor(4096, 8))
     assert "lanes(i)=8 tile()=1" in src

@@ -215,6 +215,9 @@ def test_products_of_element_matrices_stage_their_operands_in_lds(at, engine, ch
     ("A_e_i_j = B_e_i_k C_e_k_j", [(1001, 3, 3), (1001, 3, 3)], "56 per workgroup of 256 lanes"),
     ("A_e_i_j -= B_e_k_i C_e_j_k", [(333, 5, 7), (333, 6, 5)], "lanes(i,j)=42 tile()=1"),
     ("A_e_i_j += B_e_i_k C_e_k_l D_e_l_j", [(77, 3, 3), (77, 3, 3), (77, 3, 3)], "operands staged in LDS"),
+    # entries of whole lines: staged from 16 outputs on (32 entries per workgroup, ragged end)
+    ("A_e_i_j += B_e_i_k C_e_k_j", [(1001, 4, 4), (1001, 4, 4)], "32 per workgroup of 256 lanes"),
+    ("A_e_i_j = B_e_i_k C_e_j_k", [(77, 8, 2), (77, 2, 2)], "lanes(i,j)=16 tile()=1"),
     # even extents: both output indices split in two, a 2 x 2 block of outputs per lane
     ("A_e_i_j = B_e_i_k C_e_k_j", [(203, 12, 12), (203, 12, 12)], "lanes(ihi,jhi)=36 tile(ilo,jlo)=4"),
     ("A_e_j_i += B_e_k_i C_e_j_k W_e", [(57, 9, 24), (57, 30, 9), (57,)], "tile(jlo,ilo)=4"),
