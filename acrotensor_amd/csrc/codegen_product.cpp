@@ -472,25 +472,43 @@ auto Generator::TiledProductPattern(const Sub &s, TiledProductShape &p) const ->
     };
     const long mostW = envInt("ACRO_HIP_TILED_PRODUCT_STRIPS") > 0 ? envInt("ACRO_HIP_TILED_PRODUCT_STRIPS") : 8;
     const long mostJ = envInt("ACRO_HIP_TILED_PRODUCT_BLOCKS") > 0 ? envInt("ACRO_HIP_TILED_PRODUCT_BLOCKS") : 8;
-    split(blocks, std::min<long>(3, mostJ), mostJ, 4, p.panels, p.TJ);
+    split(blocks, std::min<long>(3, mostJ), mostJ, envInt("ACRO_HIP_TILED_PRODUCT_PREFER", 4), p.panels, p.TJ);
     split(strips, std::min<long>(4, mostW), mostW, 8, p.tilesM, p.W);
     // (few workgroups, a product without a batch index of moderate size: tiles of half the height fill the device better;
     // 1 024 x 1 024 x 1 024: 14.5 -> 31.6 TFLOP/s)
-    if (p.E * p.tilesM * p.panels < 512 && p.W > 4 && mostW > 4) split(strips, 4, 4, 4, p.tilesM, p.W);
+    if (p.E * p.tilesM * p.panels < 512 && p.W > 4 && mostW > 4 && envInt("ACRO_HIP_TILED_PRODUCT_HALF") >= 0) split(strips, 4, 4, 4, p.tilesM, p.W);
     p.KC = envInt("ACRO_HIP_TILED_PRODUCT_CHUNK") > 0 ? envInt("ACRO_HIP_TILED_PRODUCT_CHUNK") : 16;
     if (p.KC % 4 != 0 || p.KC > 64) return false;
-    // Few tiles and a long contraction (normal equations "A_i_j = B_n_i C_n_j" with many columns, a product of two wide
-    // matrices): the contracted range is split over workgroups as well, each writes its tile of partial sums to the
-    // scratch buffer, and a second kernel adds them in a fixed order (reproducible, no atomics).  As many shares as
-    // fill the device twice, at least 32 chunks each, at most 64 MB of partial sums.
+    // Few tiles (normal equations "A_i_j = B_n_i C_n_j" with many columns, a product of two wide matrices, any product
+    // without a batch index up to some 1 000 rows and columns): a workgroup passes through its chunks one after the
+    // other, about a microsecond each while it has a SIMD to itself, and most of the device idles.  The contracted range
+    // is split over workgroups as well, each writes its tile of partial sums to the scratch buffer, and a second kernel
+    // adds them in a fixed order (reproducible, no atomics).  Every share costs a tile of partial sums written and read
+    // (some 3 TB/s, they stay in the caches), so the number of shares balances the two, and a second launch (some 4 us) must
+    // be worth it: no more shares than make three workgroups per compute unit (what its registers hold), at least two chunks each, at most 64 MB of
+    // partial sums.  512 x 512 x 512: 34.6 -> 17.9 us, 256 x 256 x 256: 18.1 -> 9.9 us, 768 x 768 x 768: 52 -> 35 us,
+    // 512 x 512 x 2048: 127 -> 35 us, 128 x 128 x 8192: 497 -> 20 us.
     p.splits = 1;
     const long groups = p.E * p.tilesM * p.panels, chunks = (p.K + p.KC - 1) / p.KC;
-    if (groups < 256 && chunks >= 64 && envInt("ACRO_HIP_TILED_PRODUCT_SPLIT") >= 0)
+    const long asked = envInt("ACRO_HIP_TILED_PRODUCT_SPLIT");
+    if (asked > 0) p.splits = std::min<long>(asked, chunks);
+    else if (groups < 512 && chunks >= 4 && asked == 0)
     {
-        p.splits = std::min<long>(std::min<long>((512 + groups - 1) / groups, chunks / 32), 256);
-        while (p.splits > 1 && p.splits * p.E * p.M * p.N > (1L << 23)) --p.splits;
-        if (envInt("ACRO_HIP_TILED_PRODUCT_SPLIT") > 0) p.splits = std::min<long>(envInt("ACRO_HIP_TILED_PRODUCT_SPLIT"), chunks);
+        // microseconds, roughly: one per chunk, the partial sums at 3 TB/s, four for the second launch
+        const double perShare = 16.0 * static_cast<double>(p.E * p.M * p.N) / 3.0e6;
+        const long most = std::min<long>(std::min<long>((768 + groups - 1) / groups, chunks / 2), 256);
+        double best = static_cast<double>(chunks);
+        for (long n = 2; n <= most; ++n)
+        {
+            const double cost = static_cast<double>((chunks + n - 1) / n) + static_cast<double>(n) * perShare + 4.0;
+            if (cost < best - 1.0)
+            {
+                best = cost;
+                p.splits = n;
+            }
+        }
     }
+    while (p.splits > 1 && p.splits * p.E * p.M * p.N > (1L << 23)) --p.splits;
     return true;
 }
 
@@ -664,14 +682,35 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
     {
         out << "            scratch[((long)split * " << E << " + e) * " << M * N << "L + (long)m * " << N << " + n] = acc[J][q];\n";
         out << "        }\n}\n";
-        // ---- the partial sums of all shares, added in a fixed order, one lane per output
+        // ---- the partial sums of all shares, added in a fixed order: one lane per output, or 4 or 16 lanes where the
+        // outputs alone are too few lanes to keep the loads of many shares in flight (64 x 64 outputs in 256 shares:
+        // 27 -> 6 us); the lanes of an output add their sums through LDS, in a fixed order again
         const long O = E * M * N;
+        long P = 1;
+        while (P < 16 && O * P < 65536 && 4 * P * 2 <= splits) P *= 4;
+        const long each = 256 / P;
         out << "\nextern \"C\" __global__ __launch_bounds__(256) void " << fFinal << "(double *" << (opt.noalias ? "__restrict__ " : "")
             << "result, const double *__restrict__ scratch)\n{\n";
-        out << "    const long o = (long)blockIdx.x * 256 + threadIdx.x;\n";
-        out << "    if (o >= " << O << "L) return;\n";
-        out << "    double t = 0.0;\n";
-        out << "#pragma unroll 8\n    for (int w = 0; w < " << splits << "; ++w) t += scratch[w * " << O << "L + o];\n";
+        if (P == 1)
+        {
+            out << "    const long o = (long)blockIdx.x * 256 + threadIdx.x;\n";
+            out << "    if (o >= " << O << "L) return;\n";
+            out << "    double t = 0.0;\n";
+            out << "#pragma unroll 8\n    for (int w = 0; w < " << splits << "; ++w) t += scratch[w * " << O << "L + o];\n";
+        }
+        else
+        {
+            out << "    __shared__ double red[256];\n";
+            out << "    const long o = (long)blockIdx.x * " << each << " + threadIdx.x % " << each << ";\n";
+            out << "    const int part = threadIdx.x / " << each << ";\n";
+            out << "    double t = 0.0;\n";
+            out << "    if (o < " << O << "L)\n    {\n";
+            out << "#pragma unroll 8\n        for (int w = part; w < " << splits << "; w += " << P << ") t += scratch[w * " << O << "L + o];\n    }\n";
+            out << "    red[threadIdx.x] = t;\n    __syncthreads();\n";
+            out << "    if (part != 0 || o >= " << O << "L) return;\n";
+            out << "    t = red[threadIdx.x];\n";
+            out << "#pragma unroll\n    for (int q = 1; q < " << P << "; ++q) t += red[threadIdx.x + " << each << " * q];\n";
+        }
         const std::string dst = "result[" + str(aOff) + "L + o]";
         if (s.op == '=')
             out << "    " << dst << " = t;\n";
@@ -706,7 +745,9 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
         plan.scratch_doubles = static_cast<size_t>(splits * E * M * N);
         HipLaunch fin;
         fin.function_name = fFinal;
-        fin.grid = static_cast<unsigned>((E * M * N + 255) / 256);
+        long P = 1;   // (lanes per output, as in the kernel above)
+        while (P < 16 && E * M * N * P < 65536 && 4 * P * 2 <= splits) P *= 4;
+        fin.grid = static_cast<unsigned>((E * M * N + 256 / P - 1) / (256 / P));
         fin.block = 256;
         fin.params.push_back(uvars[s.out.uvar].storage);
         fin.params.push_back(-1);

@@ -653,14 +653,25 @@ def test_products_of_large_matrices_run_in_tiles_on_the_matrix_cores(TE, monkeyp
     src = TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(2048, 2048), at.Tensor(2048, 2048), at.Tensor(2048, 2048))
     assert "2048 x 2048 by 2048 x 2048, no batch index" in src and "tiles of 128 rows x 64 columns (16 x 32 per entry)" in src and "512 workgroups" in src
     src = TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(1024, 1024), at.Tensor(1024, 1024), at.Tensor(1024, 1024))
-    assert "tiles of 64 rows x 64 columns (16 x 16 per entry)" in src and "256 workgroups of 256 lanes" in src
+    assert "tiles of 64 rows x 64 columns (16 x 16 per entry)" in src and "768 workgroups of 256 lanes, the contracted range in 3 shares of 352 terms" in src
+    # (a workgroup takes its chunks one after the other: with few tiles the contracted range is shared out as well, as far
+    # as the partial sums and the second launch are worth it)
+    src = TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(512, 512), at.Tensor(512, 512), at.Tensor(512, 512))
+    assert "256 workgroups of 256 lanes, the contracted range in 4 shares of 128 terms" in src
+    src = TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(512, 512), at.Tensor(512, 64), at.Tensor(64, 512))
+    assert "64 workgroups of 256 lanes" in src and "shares" not in src
+    src = TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(1536, 1536), at.Tensor(1536, 1536), at.Tensor(1536, 1536))
+    assert "576 workgroups of 256 lanes" in src and "shares" not in src
     # few tiles, many terms (normal equations with more columns than the Gram schedule takes): the contracted range is
     # shared out as well, partial tiles go to the scratch buffer and a second kernel adds them in a fixed order
     src = TE.GetImplementation("A_i_j += B_n_i C_n_j", at.Tensor(128, 128), at.Tensor(262144, 128), at.Tensor(262144, 128))
-    assert "tiles of 64 rows x 64 columns (2 x 2 per entry)" in src and "512 workgroups of 256 lanes, the contracted range in 128 shares of 2048 terms" in src
+    assert "tiles of 64 rows x 64 columns (2 x 2 per entry)" in src and "764 workgroups of 256 lanes, the contracted range in 191 shares of 1376 terms" in src
     assert "_partial(" in src and "double *__restrict__ scratch)" in src and "const int split = blockIdx.x / 4;" in src
     assert "scratch[((long)split * 1 + e) * 16384L + (long)m * 128 + n] = acc[J][q];" in src
-    assert "for (int w = 0; w < 128; ++w) t += scratch[w * 16384L + o];" in src and "result[0L + o] = result[0L + o] + t;" in src
+    # (the second kernel: four lanes per output where the outputs alone are too few to keep the loads in flight)
+    assert "for (int w = part; w < 191; w += 4) t += scratch[w * 16384L + o];" in src and "result[0L + o] = result[0L + o] + t;" in src
+    src = TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(512, 512), at.Tensor(512, 512), at.Tensor(512, 512))
+    assert "for (int w = 0; w < 4; ++w) t += scratch[w * 262144L + o];" in src
     # 65 to 128 rows or columns per entry, and small matrices with more than 128 terms
     assert "tiled product schedule" in product("A_e_i_j = B_e_i_k C_e_k_j", 72, 72, 72)
     assert "tiled product schedule" in product("A_e_i_j = B_e_i_k C_e_k_j", 32, 48, 200)

@@ -341,6 +341,13 @@ TILED_PRODUCTS = [
     ("A_i_j = B_e_i C_e_j", [(3000, 96), (3000, 100)]),
     ("A_i_j -= B_i_k C_k_j", [(65, 4099), (4099, 96)]),
     ("A_e_i_j += B_e_i_k C_e_k_j", [(3, 70, 1500), (3, 1500, 66)]),
+    # ... also products of moderate size (a workgroup takes its chunks one after the other, so few tiles leave most of the
+    # device idle): a few shares, one lane per output in the second kernel
+    ("A_i_j = B_i_k C_k_j", [(256, 256), (256, 256)]),
+    ("A_i_j += B_i_k C_k_j", [(300, 520), (520, 200)]),
+    # ... many shares of few outputs: four and sixteen lanes per output in the second kernel
+    ("A_i_j = B_n_i C_n_j", [(20000, 144), (20000, 128)]),
+    ("A_i_j -= B_i_k C_k_j", [(64, 60000), (60000, 64)]),
 ]
 
 
