@@ -479,6 +479,7 @@ auto Generator::TiledProductPattern(const Sub &s, TiledProductShape &p) const ->
     if (p.E * p.tilesM * p.panels < 512 && p.W > 4 && mostW > 4 && envInt("ACRO_HIP_TILED_PRODUCT_HALF") >= 0) split(strips, 4, 4, 4, p.tilesM, p.W);
     p.KC = envInt("ACRO_HIP_TILED_PRODUCT_CHUNK") > 0 ? envInt("ACRO_HIP_TILED_PRODUCT_CHUNK") : 16;
     if (p.KC % 4 != 0 || p.KC > 64) return false;
+    if (p.K < p.KC) p.KC = 16;   // (the end of a range is read as its last chunk's worth of terms)
     // Few tiles (normal equations "A_i_j = B_n_i C_n_j" with many columns, a product of two wide matrices, any product
     // without a batch index up to some 1 000 rows and columns): a workgroup passes through its chunks one after the
     // other, about a microsecond each while it has a SIMD to itself, and most of the device idles.  The contracted range
@@ -540,7 +541,7 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
           << (p.rowKFast ? "with the contracted index last" : "with the contracted index first") << ", column factor "
           << (p.colKFast ? "with the contracted index last" : "with the contracted index first") << "), tiles of " << 16 * W << " rows x "
           << 16 * TJ << " columns (" << p.tilesM << " x " << p.panels << " per entry), chunks of " << KC << " terms through "
-          << (envInt("ACRO_HIP_TILED_PRODUCT_LDS") == 2 ? 2 : 1) * (UA + UB) * NT * 8 << " bytes of LDS, " << groups * splits << " workgroups of " << NT << " lanes";
+          << (UA + UB) * NT * 8 << " bytes of LDS, " << groups * splits << " workgroups of " << NT << " lanes";
     if (splits > 1) sched << ", the contracted range in " << splits << " shares of " << span << " terms whose partial sums a second kernel adds";
     sched << "\n  [0] " << s.text << "\n";
     plan.schedule = sched.str();
@@ -562,9 +563,8 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
     const std::string fMain = splits > 1 ? plan.module_name + "_partial" : plan.module_name, fFinal = plan.module_name + "_final";
     out << "void " << fMain << "(" << ParamList() << (splits > 1 ? ", double *__restrict__ scratch" : "") << ")\n{\n";
     // (padded to a whole number of values per lane: lanes without a value of the tile write into the padding, no branch)
-    const long ldsHalves = envInt("ACRO_HIP_TILED_PRODUCT_LDS") == 2 ? 2 : 1;
-    out << "    __shared__ double fragA[" << ldsHalves * UA * NT << "];\n";
-    out << "    __shared__ double fragB[" << ldsHalves * UB * NT << "];\n";
+    out << "    __shared__ double fragA[" << UA * NT << "];\n";
+    out << "    __shared__ double fragB[" << UB * NT << "];\n";
     out << "    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;\n";
     if (splits > 1)
     {
@@ -591,87 +591,89 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
     out << "    const double *Rm = " << R << " + " << rOff << "L + e * " << M * K << "L;\n";
     out << "    const double *Cm = " << C << " + " << cOff << "L + e * " << K * N << "L;\n";
     out << "    double *Am = " << A << " + " << aOff << "L + e * " << M * N << "L;\n";
-    // where this lane's values of a chunk come from and go to (the same for every chunk but for the term offset)
-    out << "    int aFrom[" << UA << "], aTo[" << UA << "], bFrom[" << UB << "], bTo[" << UB << "];\n";
-    out << "    int aK[" << UA << "], bK[" << UB << "];\n";
+    // Where this lane's values of a chunk come from and go to (the same for every chunk but for the term offset).  Rows and
+    // columns past the end of the matrices read the last row or column instead: what they contribute to are results past
+    // the end, which are not stored.  Lanes without a value of the tile (a tile of fewer values than a whole number per
+    // lane) read the tile's first value and write into the padding of the LDS arrays.  So the loop has no lane-dependent
+    // condition, and its loads take a scalar base that moves with the chunk plus a 32-bit offset per lane
+    // (1 024 x 1 024 x 1 024 in 256 workgroups: 137 -> 75 other vector instructions per chunk, 67.6 -> 51.5 us).
+    out << "    unsigned aFrom[" << UA << "], bFrom[" << UB << "];\n    int aTo[" << UA << "], bTo[" << UB << "];\n";
     out << "#pragma unroll\n    for (int u = 0; u < " << UA << "; ++u)\n    {\n";
-    out << "        const int i = threadIdx.x + " << NT << " * u;\n";
+    out << "        const int i = threadIdx.x + " << NT << " * u, v = i < " << rowTile << " ? i : 0;\n";
     if (p.rowKFast)
-        out << "        const int kk = i % " << KC << ", rr = i / " << KC << ";\n";
+        out << "        const int kk = v % " << KC << ", rr = v / " << KC << ";\n";
     else
-        out << "        const int rr = i % " << 16 * W << ", kk = i / " << 16 * W << ";\n";
-    out << "        aK[u] = i < " << rowTile << " && r0 + rr < " << M << " ? kk : " << (1 << 28) << ";   // (never below K: reads as zero)\n";
-    out << "        aFrom[u] = " << (p.rowKFast ? "(r0 + rr) * " + str(K) + " + kk" : "kk * " + str(M) + " + r0 + rr") << ";\n";
+        out << "        const int rr = v % " << 16 * W << ", kk = v / " << 16 * W << ";\n";
+    out << "        const int row = r0 + rr < " << M << " ? r0 + rr : " << M - 1 << ";\n";
+    out << "        aFrom[u] = " << (p.rowKFast ? "row * " + str(K) + " + kk" : "kk * " + str(M) + " + row") << ";\n";
     out << "        aTo[u] = i < " << rowTile << " ? ((rr / 16) * " << KS << " + kk / 4) * 64 + (kk % 4) * 16 + ((rr + kk) & 15) : i;\n";
     out << "    }\n";
     out << "#pragma unroll\n    for (int u = 0; u < " << UB << "; ++u)\n    {\n";
-    out << "        const int i = threadIdx.x + " << NT << " * u;\n";
+    out << "        const int i = threadIdx.x + " << NT << " * u, v = i < " << colTile << " ? i : 0;\n";
     if (p.colKFast)
-        out << "        const int kk = i % " << KC << ", cc = i / " << KC << ";\n";
+        out << "        const int kk = v % " << KC << ", cc = v / " << KC << ";\n";
     else
-        out << "        const int cc = i % " << 16 * TJ << ", kk = i / " << 16 * TJ << ";\n";
-    out << "        bK[u] = i < " << colTile << " && c0 + cc < " << N << " ? kk : " << (1 << 28) << ";\n";
-    out << "        bFrom[u] = " << (p.colKFast ? "(c0 + cc) * " + str(K) + " + kk" : "kk * " + str(N) + " + c0 + cc") << ";\n";
+        out << "        const int cc = v % " << 16 * TJ << ", kk = v / " << 16 * TJ << ";\n";
+    out << "        const int col = c0 + cc < " << N << " ? c0 + cc : " << N - 1 << ";\n";
+    out << "        bFrom[u] = " << (p.colKFast ? "col * " + str(K) + " + kk" : "kk * " + str(N) + " + col") << ";\n";
     out << "        bTo[u] = i < " << colTile << " ? ((cc / 16) * " << KS << " + kk / 4) * 64 + (kk % 4) * 16 + ((cc + kk) & 15) : i;\n";
     out << "    }\n";
     const std::string aStep = p.rowKFast ? "k0" : "(long)k0 * " + str(M);
     const std::string bStep = p.colKFast ? "k0" : "(long)k0 * " + str(N);
     // One copy of a chunk's fragments in LDS and two barriers per chunk (before the fragments are overwritten and after).
-    // Measured against that and not kept as the default: two halves of LDS, the next chunk written to one while the other is
-    // multiplied, one barrier per chunk (ACRO_HIP_TILED_PRODUCT_LDS=2: 80^3 per entry 57 -> 62 %, 128 x 128 x 2^18 37 -> 41
-    // TFLOP/s, but 128^3 per entry 53 -> 50 %, 2 048^3 58 -> 53 TFLOP/s); two chunks on their way in two sets of registers
-    // (4 096^3 62 -> 53 TFLOP/s): neither the barriers nor the latency of the loads is what these kernels wait for.
-    const long halves = envInt("ACRO_HIP_TILED_PRODUCT_LDS") == 2 ? 2 : 1;
+    // Measured against that and not kept: two halves of LDS, the next chunk written to one while the other is
+    // multiplied, one barrier per chunk (80^3 per entry 57 -> 62 %, 128 x 128 x 2^18 37 -> 41 TFLOP/s, but 128^3 per entry
+    // 53 -> 50 %, 2 048^3 58 -> 53 TFLOP/s); two chunks on their way in two sets of registers (4 096^3 62 -> 53 TFLOP/s):
+    // neither the barriers nor the latency of the loads is what these kernels wait for.
     out << "    double ra[" << UA << "], rb[" << UB << "];\n";
     auto emitLoads = [&](const std::string &ind, const std::string &k0) {
         // (no branches around the loads and no use of their values here, so that all of them are in flight together and
-        // stay so while the chunk before is multiplied: a value that does not exist is read from the entry's first
-        // element and replaced by zero when it is written to LDS)
+        // stay so while the chunk before is multiplied)
         out << ind << "{\n" << ind << "    const int k0 = " << k0 << ";\n";
-        out << "#pragma unroll\n" << ind << "    for (int u = 0; u < " << UA << "; ++u) ra[u] = Rm[k0 + aK[u] < kEnd ? " << aStep << " + aFrom[u] : 0];\n";
-        out << "#pragma unroll\n" << ind << "    for (int u = 0; u < " << UB << "; ++u) rb[u] = Cm[k0 + bK[u] < kEnd ? " << bStep << " + bFrom[u] : 0];\n";
+        out << ind << "    const double *rk = Rm + " << aStep << ", *ck = Cm + " << bStep << ";\n";
+        out << "#pragma unroll\n" << ind << "    for (int u = 0; u < " << UA << "; ++u) ra[u] = rk[aFrom[u]];\n";
+        out << "#pragma unroll\n" << ind << "    for (int u = 0; u < " << UB << "; ++u) rb[u] = ck[bFrom[u]];\n";
         out << ind << "}\n";
     };
-    auto emitToLds = [&](const std::string &ind, const std::string &kHere, const std::string &half) {
-        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UA << "; ++u) fragA[" << (half.empty() ? std::string() : half + str(UA * NT) + " + ") << "aTo[u]] = " << kHere << " + aK[u] < kEnd ? ra[u] : 0.0;\n";
-        out << "#pragma unroll\n" << ind << "for (int u = 0; u < " << UB << "; ++u) fragB[" << (half.empty() ? std::string() : half + str(UB * NT) + " + ") << "bTo[u]] = " << kHere << " + bK[u] < kEnd ? rb[u] : 0.0;\n";
-    };
-    auto emitProducts = [&](const std::string &ind, const std::string &half) {
-        const std::string baseA = (half.empty() ? std::string() : half + str(UA * NT) + " + ") + "wave * " + str(KS * 64);
-        const std::string baseB = half.empty() ? std::string() : half + str(UB * NT) + " + ";
+    auto emitProducts = [&](const std::string &ind) {
         // (Reading the next step's fragments from LDS before this step's products, the order held by scheduling barriers,
         // changed nothing: 4 096^3 61 -> 59 TFLOP/s, 128^3 per entry 53 -> 49 %.  The wavefronts of a SIMD hide each other's
         // LDS latency already.)
         out << "#pragma unroll\n" << ind << "for (int s = 0; s < " << KS << "; ++s)\n" << ind << "{\n";
         out << ind << "    const int at = s * 64 + g * 16 + ((c + 4 * s + g) & 15);\n";
-        out << ind << "    const double a = fragA[" << baseA << " + at];\n";
+        out << ind << "    const double a = fragA[wave * " << KS * 64 << " + at];\n";
         out << "#pragma unroll\n" << ind << "    for (int J = 0; J < " << TJ << "; ++J)\n";
-        out << ind << "        acc[J] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, fragB[" << baseB << "J * " << KS * 64 << " + at], acc[J], 0, 0, 0);\n";
+        out << ind << "        acc[J] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, fragB[J * " << KS * 64 << " + at], acc[J], 0, 0, 0);\n";
         out << ind << "}\n";
     };
-    emitLoads("    ", "kBegin");
+    // The whole chunks of the range run in the loop.  What is left of a range that is no whole number of chunks is read as
+    // the range's last 16 terms (the factors have at least that many), and the terms among them that the loop has added
+    // already become zero on their way to LDS: both factors', so that a NaN or an infinity there stays out.
+    const bool tail = K % KC != 0 || (splits > 1 && span % KC != 0);
+    out << "    const int kWhole = kBegin + (kEnd - kBegin) / " << KC << " * " << KC << ";   // where the whole chunks end\n";
+    emitLoads("    ", "kBegin < kWhole ? kBegin : kEnd - " + str(KC));
     out << "    acro_double4 acc[" << TJ << "];\n";
     out << "#pragma unroll\n    for (int J = 0; J < " << TJ << "; ++J) acc[J] = acro_double4{0.0, 0.0, 0.0, 0.0};\n";
-    if (halves == 2)
+    out << "    for (int kc = kBegin; kc < kWhole; kc += " << KC << ")\n    {\n";
+    out << "#pragma unroll\n        for (int u = 0; u < " << UA << "; ++u) fragA[aTo[u]] = ra[u];\n";
+    out << "#pragma unroll\n        for (int u = 0; u < " << UB << "; ++u) fragB[bTo[u]] = rb[u];\n";
+    out << "        __syncthreads();\n";
+    emitLoads("        ", "kc + " + str(KC) + " < kWhole ? kc + " + str(KC) + " : kEnd - " + str(KC));
+    emitProducts("        ");
+    out << "        __syncthreads();\n";
+    out << "    }\n";
+    if (tail)
     {
-        emitToLds("    ", "kBegin", "0 * ");
-        out << "    __syncthreads();\n";
-        out << "    int half = 0;\n";
-        out << "    for (int kc = kBegin; kc < kEnd; kc += " << KC << ", half ^= 1)\n    {\n";
-        emitLoads("        ", "kc + " + str(KC));   // (past the end: no loads)
-        emitProducts("        ", "half * ");
-        emitToLds("        ", "kc + " + str(KC), "(half ^ 1) * ");
+        out << "    if (kWhole < kEnd)\n    {\n";
+        out << "        const int done = kWhole - (kEnd - " << KC << ");   // terms of the last 16 that the loop has added\n";
+        out << "#pragma unroll\n        for (int u = 0; u < " << UA << "; ++u)\n        {\n";
+        out << "            const int i = threadIdx.x + " << NT << " * u, v = i < " << rowTile << " ? i : 0;\n";
+        out << "            fragA[aTo[u]] = " << (p.rowKFast ? "v % " + str(KC) : "v / " + str(16 * W)) << " >= done ? ra[u] : 0.0;\n        }\n";
+        out << "#pragma unroll\n        for (int u = 0; u < " << UB << "; ++u)\n        {\n";
+        out << "            const int i = threadIdx.x + " << NT << " * u, v = i < " << colTile << " ? i : 0;\n";
+        out << "            fragB[bTo[u]] = " << (p.colKFast ? "v % " + str(KC) : "v / " + str(16 * TJ)) << " >= done ? rb[u] : 0.0;\n        }\n";
         out << "        __syncthreads();\n";
-        out << "    }\n";
-    }
-    else
-    {
-        out << "    for (int kc = kBegin; kc < kEnd; kc += " << KC << ")\n    {\n";
-        emitToLds("        ", "kc", "");
-        out << "        __syncthreads();\n";
-        emitLoads("        ", "kc + " + str(KC));
-        emitProducts("        ", "");
-        out << "        __syncthreads();\n";
+        emitProducts("        ");
         out << "    }\n";
     }
     out << "#pragma unroll\n    for (int J = 0; J < " << TJ << "; ++J)\n";
@@ -731,7 +733,7 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
 
     plan.source = out.str();
     plan.nb = 1;
-    plan.lds_bytes = static_cast<int>(ldsHalves * (UA + UB) * NT * 8);
+    plan.lds_bytes = static_cast<int>((UA + UB) * NT * 8);
     FillParams(plan, false);
     HipLaunch launch;
     launch.function_name = fMain;

@@ -151,7 +151,6 @@
 //   ACRO_HIP_TILED_PRODUCT_SPLIT=-1 / =<n>  never share out the contracted range / share it out n ways
 //   ACRO_HIP_TILED_PRODUCT_HALF=-1 / _PREFER=<n>  few tiles keep eight strips per workgroup (default: four) / blocks per strip
 //                               that the split of the columns prefers (4)
-//   ACRO_HIP_TILED_PRODUCT_LDS=2  two halves of LDS for the chunks, one barrier per chunk (default: one half, two barriers)
 //   ACRO_HIP_TILED_PRODUCT_XCD=-1  the tiles of an entry are numbered as the hardware deals them (default: an entry's two to four
 //                               tiles on one XCD, so that the strips they share pass through one L2)
 //   ACRO_HIP_TILED_PRODUCT_OPERATOR=<entries>  a product without a batch index one of whose factors has at most this many entries
