@@ -89,8 +89,14 @@ auto Generator::ProductPattern(const Sub &s, ProductShape &p) const -> bool
     // 20 x 20 75 / 71, 24 x 24 75 / 72, 25 x 25 74 / 71, 28 x 28 74 / 73, 33 x 33 67 / 64, 36 x 36 71 / 70; without such
     // a divisor 17 x 17 59 / 67, 31 x 31 42 / 71, 37 x 37 37 / 70; larger: 40 x 40 69 / 69, 45 x 45 67 / 69, 48 x 48 69 / 70,
     // 53 x 53 28 / 68, 55 x 55 23 / 68, 56 x 56 58 / 69, 63 x 63 32 / 67, 64 x 64 15 / 70).
+    // Blocks of 3 x 3 are the staged schedule's weakest, and up to 32 x 32 (two strips of two blocks here) extents that only
+    // three divides do better on the matrix cores: 21 x 21 64 / 70, 27 x 27 61 / 71, 27 x 27 x 9 terms 54 / 73,
+    // 21 x 33 x 27 terms 69 / 72.
     auto blocks = [](long n) { return n % 2 == 0 || n % 3 == 0 || n % 5 == 0; };
-    if (!vectorForm && std::max(p.M, p.N) <= 36 && blocks(p.M) && blocks(p.N) && envInt("ACRO_HIP_PRODUCT") < 2) return false;
+    auto byThreeOnly = [](long n) { return n % 3 == 0 && n % 2 != 0 && n % 5 != 0; };
+    const bool staged = std::max(p.M, p.N) <= 36 && blocks(p.M) && blocks(p.N) &&
+                        !(std::max(p.M, p.N) <= 32 && (byThreeOnly(p.M) || byThreeOnly(p.N)));
+    if (!vectorForm && staged && envInt("ACRO_HIP_PRODUCT") < 2) return false;
     p.TI = (p.M + 15) / 16;
     p.TJ = (p.N + 15) / 16;
     if (p.TI > 8 || p.TJ > 8) return false;

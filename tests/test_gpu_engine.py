@@ -261,6 +261,9 @@ PRODUCTS_ON_THE_MATRIX_CORES = [
     ("A_e_i_j += B_e_k_i C_e_k_j", [(1001, 9, 17), (1001, 9, 64)]),
     ("A_e_i_j = B_e_i_k C_e_k_j", [(333, 19, 128), (333, 128, 8)]),
     ("A_e_i_j -= B_e_i_k C_e_j_k", [(257, 31, 31), (257, 31, 31)]),
+    # extents up to 32 that only three divides
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(301, 27, 27), (301, 27, 27)]),
+    ("A_e_i_j += B_e_k_i C_e_j_k", [(111, 9, 21), (111, 27, 9)]),
     # tensors of odd length whose last double sits in a 16-byte piece that is not a lane's last one
     ("A_e_i_j = C_e_k_j B_e_k_i", [(129, 93, 11), (129, 93, 49)]),
     ("A_e_i_j = B_e_i_k C_e_k_j", [(145, 27, 67), (145, 67, 19)]),
