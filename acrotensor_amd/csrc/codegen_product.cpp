@@ -94,8 +94,10 @@ auto Generator::ProductPattern(const Sub &s, ProductShape &p) const -> bool
     // 21 x 33 x 27 terms 69 / 72.
     auto blocks = [](long n) { return n % 2 == 0 || n % 3 == 0 || n % 5 == 0; };
     auto byThreeOnly = [](long n) { return n % 3 == 0 && n % 2 != 0 && n % 5 != 0; };
+    // Whole blocks of 16 (32 x 32, 32 x 16) leave nothing of the matrix instruction unused and take it too: 32 x 32 72 / 74,
+    // with the second factor transposed 61 / 73, with both 67 / 73.
     const bool staged = std::max(p.M, p.N) <= 36 && blocks(p.M) && blocks(p.N) &&
-                        !(std::max(p.M, p.N) <= 32 && (byThreeOnly(p.M) || byThreeOnly(p.N)));
+                        !(std::max(p.M, p.N) <= 32 && (byThreeOnly(p.M) || byThreeOnly(p.N))) && !(p.M % 16 == 0 && p.N % 16 == 0);
     if (!vectorForm && staged && envInt("ACRO_HIP_PRODUCT") < 2) return false;
     p.TI = (p.M + 15) / 16;
     p.TJ = (p.N + 15) / 16;

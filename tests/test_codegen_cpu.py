@@ -610,7 +610,8 @@ def test_products_of_element_matrices_run_on_the_matrix_cores(TE, monkeypatch):
     # a shared factor, more than two factors, too few entries for e to be the batch index
     assert "product schedule" not in product("A_e_i_j = B_e_i_k C_e_k_j", 24, 24, 24)
     assert "product schedule" not in product("A_e_i_j = B_e_i_k C_e_k_j", 33, 33, 33)
-    # (extents up to 32 that only three divides would get blocks of 3 x 3 there: those are taken)
+    # (extents up to 32 that only three divides would get blocks of 3 x 3 there: those are taken, and so are whole blocks of 16)
+    assert "product schedule on the FP64 matrix cores: 32 x 32 by 32 x 32" in product("A_e_i_j = B_e_i_k C_e_j_k", 32, 32, 32)
     assert "product schedule on the FP64 matrix cores: 27 x 27 by 27 x 27" in product("A_e_i_j = B_e_i_k C_e_k_j", 27, 27, 27)
     assert "product schedule on the FP64 matrix cores: 21 x 27 by 27 x 30" in product("A_e_i_j = B_e_i_k C_e_k_j", 21, 30, 27)
     assert "product schedule" not in product("A_e_i_j = B_e_i_k C_e_k_j", 16, 16, 16)

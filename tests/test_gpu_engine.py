@@ -261,6 +261,9 @@ PRODUCTS_ON_THE_MATRIX_CORES = [
     ("A_e_i_j += B_e_k_i C_e_k_j", [(1001, 9, 17), (1001, 9, 64)]),
     ("A_e_i_j = B_e_i_k C_e_k_j", [(333, 19, 128), (333, 128, 8)]),
     ("A_e_i_j -= B_e_i_k C_e_j_k", [(257, 31, 31), (257, 31, 31)]),
+    # whole blocks of 16 below 36 x 36
+    ("A_e_i_j = B_e_i_k C_e_j_k", [(77, 32, 32), (77, 32, 32)]),
+    ("A_e_i_j += B_e_k_i C_e_k_j", [(55, 24, 32), (55, 24, 16)]),
     # extents up to 32 that only three divides
     ("A_e_i_j = B_e_i_k C_e_k_j", [(301, 27, 27), (301, 27, 27)]),
     ("A_e_i_j += B_e_k_i C_e_j_k", [(111, 9, 21), (111, 27, 9)]),
