@@ -634,17 +634,17 @@ def test_products_of_large_matrices_run_in_tiles_on_the_matrix_cores(TE, monkeyp
         tensors = [at.Tensor(*[ext[x] for x in tok.split("_")[1:]]) for tok in [lhs.split()[0]] + rhs.split()]
         return at.TensorEngine("HIP").GetImplementation(kernel, *tensors)
 
-    # 128 x 128 per entry: eight strips by four blocks per workgroup, two tiles per entry, chunks of 16 terms
+    # 128 x 128 per entry: four strips by four blocks per workgroup, four tiles per entry, chunks of 16 terms
     src = product("A_e_i_j = B_e_i_k C_e_k_j", 128, 128, 128)
     assert "tiled product schedule on the FP64 matrix cores: 128 x 128 by 128 x 128 per entry, 2048 entries" in src
-    assert "tiles of 128 rows x 64 columns (1 x 2 per entry), chunks of 16 terms through 24576 bytes of LDS, 4096 workgroups of 512 lanes" in src
-    assert "__shared__ double fragA[2048];" in src and "__shared__ double fragB[1024];" in src
+    assert "tiles of 64 rows x 64 columns (2 x 2 per entry), chunks of 16 terms through 16384 bytes of LDS, 8192 workgroups of 256 lanes" in src
+    assert "__shared__ double fragA[1024];" in src and "__shared__ double fragB[1024];" in src
     # the lanes run along each factor's fastest dimension; values land in the instruction's operand order
     assert "const int kk = v % 16, rr = v / 16;" in src and "const int cc = v % 64, kk = v / 64;" in src
     assert "((rr / 16) * 4 + kk / 4) * 64 + (kk % 4) * 16 + ((rr + kk) & 15)" in src
     # nothing in the loop depends on the lane but a 32-bit offset: loads from a base that moves with the chunk, values
     # straight to LDS, the next chunk requested before the products; 16 divides the range, so no code for what is left
-    assert "const int kBegin = 0, kEnd = 128;" in src and "unsigned aFrom[4], bFrom[2];" in src
+    assert "const int kBegin = 0, kEnd = 128;" in src and "unsigned aFrom[4], bFrom[4];" in src
     assert "const double *rk = Rm + k0, *ck = Cm + (long)k0 * 128;" in src and "ra[u] = rk[aFrom[u]];" in src and "fragA[aTo[u]] = ra[u];" in src
     assert src.index("const int k0 = kc + 16 < kWhole ? kc + 16 : kEnd - 16;") < src.index("__builtin_amdgcn_mfma_f64_16x16x4f64")
     assert src.count("__syncthreads()") == 2 and "__builtin_nontemporal_store(acc[J][q], d);" in src and "done" not in src
@@ -652,12 +652,12 @@ def test_products_of_large_matrices_run_in_tiles_on_the_matrix_cores(TE, monkeyp
     # extents that 16 does not divide, the factors stored the other way round, accumulation
     src = product("A_e_i_j += B_e_k_i C_e_j_k", 100, 70, 150)
     assert "100 x 150 by 150 x 70 per entry" in src and "row factor with the contracted index first, column factor with the contracted index last" in src
-    assert "tiles of 112 rows x 80 columns (1 x 1 per entry)" in src and "workgroups of 448 lanes" in src
-    assert "const int rr = v % 112, kk = v / 112;" in src and "const int kk = v % 16, cc = v / 16;" in src
+    assert "tiles of 64 rows x 80 columns (2 x 1 per entry)" in src and "workgroups of 256 lanes" in src
+    assert "const int rr = v % 64, kk = v / 64;" in src and "const int kk = v % 16, cc = v / 16;" in src
     # rows and columns past the end read the last one (their results are not stored); the 6 terms after the whole chunks
     # are read as the last 16, and the 10 of them that the loop has added become zero on their way to LDS
     assert "const int row = r0 + rr < 100 ? r0 + rr : 99;" in src and "const int col = c0 + cc < 70 ? c0 + cc : 69;" in src
-    assert "const int done = kWhole - (kEnd - 16);" in src and "fragA[aTo[u]] = v / 112 >= done ? ra[u] : 0.0;" in src
+    assert "const int done = kWhole - (kEnd - 16);" in src and "fragA[aTo[u]] = v / 64 >= done ? ra[u] : 0.0;" in src
     assert "fragB[bTo[u]] = v % 16 >= done ? rb[u] : 0.0;" in src and src.count("__syncthreads()") == 3
     assert "if (m >= 100 || n >= 70) continue;" in src and "*d += acc[J][q];" in src and "nontemporal" not in src
     # no batch index: a plain matrix product; few tiles take half the height to fill the device
