@@ -553,6 +553,18 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
           << 16 * TJ << " columns (" << p.tilesM << " x " << p.panels << " per entry), chunks of " << KC << " terms through "
           << (UA + UB) * NT * 8 << " bytes of LDS, " << groups * splits << " workgroups of " << NT << " lanes";
     if (splits > 1) sched << ", the contracted range in " << splits << " shares of " << span << " terms whose partial sums a second kernel adds";
+    // Few workgroups per compute unit: a wavefront has its SIMD almost to itself, and what it issues beside the matrix
+    // instructions shows.  By the compiler's default the accumulators live in the accumulation half of the register file
+    // inside the loop and in the other half around its back edge, 64 copies per chunk; told to keep the matrix
+    // instruction's operands in ordinary vector registers it makes none.  512^3 17.4 -> 15.8 us, 1 024^3 53.3 -> 47.3 us,
+    // 144 x 128 x 100 000 105 -> 94 us; with many workgroups per compute unit the copies hide behind other wavefronts and
+    // the option loses a little (128^3 per entry 56.5 -> 54.6 % of the HBM peak), so those keep the default.
+    const bool vgprForm = groups * splits <= 1024 && W <= 4 && envInt("ACRO_HIP_TILED_PRODUCT_VGPR_FORM") >= 0;
+    if (vgprForm)
+    {
+        plan.compile_options = {"-mllvm", "-amdgpu-mfma-vgpr-form"};
+        sched << ", compiled with -amdgpu-mfma-vgpr-form";
+    }
     sched << "\n  [0] " << s.text << "\n";
     plan.schedule = sched.str();
     out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
