@@ -132,6 +132,8 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     const bool wide = !pencil && !byRows && O > NTr;   // (up to 256 outputs: a lane per output in every workgroup, below)
     ACROBATIC_ASSERT(!wide || outputsFastest || O <= NTr, "HIP generator: too many outputs for the reduction schedule.");
     const long Sn = pencil ? NTr : (byRows ? 64 : (wide ? 1 : NTr / O));  // contraction slices per workgroup and step
+    // (Two neighbouring outputs per lane, read as one 16-byte piece, measured slower: "S_i_j = A_e_i_j" with 32 x 32
+    // outputs over 131 072 entries 70 -> 60 % of the HBM peak.)
     const long Ow = NTr / Sn, Go = (byRows || wide) ? (O + Ow - 1) / Ow : 1;  // outputs per workgroup, groups of outputs
     // First-stage workgroups.  Pencil: one per CU (256 on this device) without unrolling, i.e. about 20 KB of
     // loads in flight per CU and one 4.7 MB window moving through the operands; more workgroups or deeper
@@ -156,6 +158,8 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         while (NTf < 1024 && (G * O > NTf * 4 || NTf < O)) NTf *= 2;
     }
     const long S2 = wide ? 1 : NTf / O;
+    long wideParts = 1;   // lanes per output in the finishing kernel of the wide form
+    while (wide && wideParts < 16 && O * wideParts < 65536 && 8 * wideParts * 4 <= G) wideParts *= 4;
 
     const std::string dimName = mk.GetDimensionedNameString();
     char hex[32];
@@ -382,13 +386,30 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     };
     if (wide)
     {
-        // a lane per output adds its partials in order
+        // a lane per output adds its partials in order; with few outputs and many shares, 4 or 16 lanes per output, each a
+        // share of the partials, added through LDS in a fixed order again (1 024 outputs in 256 shares: 16.2 -> 4 us)
         out << "\nextern \"C\" __global__ __launch_bounds__(" << NTf << ") void " << fFinal << "(double *"
             << (opt.noalias ? "__restrict__ " : "") << "result, const double *__restrict__ scratch)\n{\n";
-        out << "    const int o = blockIdx.x * " << NTf << " + threadIdx.x;\n";
-        out << "    if (o < " << O << ")\n    {\n        double t = 0.0;\n";
-        out << "#pragma unroll 8\n";
-        out << "        for (long g = 0; g < " << G << "; ++g) t += scratch[g * " << O << " + o];\n";
+        const long each = NTf / wideParts;
+        if (wideParts > 1)
+        {
+            out << "    __shared__ double red[" << NTf << "];\n";
+            out << "    const int o = blockIdx.x * " << each << " + threadIdx.x % " << each << ", part = threadIdx.x / " << each << ";\n";
+            out << "    double t = 0.0;\n";
+            out << "    if (o < " << O << ")\n    {\n";
+            out << "#pragma unroll 8\n";
+            out << "        for (long g = part; g < " << G << "; g += " << wideParts << ") t += scratch[g * " << O << " + o];\n    }\n";
+            out << "    red[threadIdx.x] = t;\n    __syncthreads();\n";
+            out << "    if (part == 0 && o < " << O << ")\n    {\n";
+            out << "#pragma unroll\n        for (int q = 1; q < " << wideParts << "; ++q) t += red[threadIdx.x + " << each << " * q];\n";
+        }
+        else
+        {
+            out << "    const int o = blockIdx.x * " << NTf << " + threadIdx.x;\n";
+            out << "    if (o < " << O << ")\n    {\n        double t = 0.0;\n";
+            out << "#pragma unroll 8\n";
+            out << "        for (long g = 0; g < " << G << "; ++g) t += scratch[g * " << O << " + o];\n";
+        }
         decompose(s.outIdx, "o", "        ");
         const std::string dst = "result[" + FullOffset(s.out) + "]";
         if (s.op == '=')
@@ -445,7 +466,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     {
         HipLaunch fin;
         fin.function_name = fFinal;
-        fin.grid = wide ? static_cast<unsigned>((O + NTf - 1) / NTf) : 1;
+        fin.grid = wide ? static_cast<unsigned>((O + NTf / wideParts - 1) / (NTf / wideParts)) : 1;
         fin.block = NTf;
         fin.params.push_back(uvars[s.out.uvar].storage);
         fin.params.push_back(-1);

@@ -329,7 +329,13 @@ def test_sums_over_a_long_index_take_the_reduction_schedule_whatever_the_number_
     # a lane per output and workgroup, the summed range dealt out over the workgroups; a finishing workgroup per 256 outputs
     src = TE.GetImplementation("S_i_j = A_e_i_j", at.Tensor(32, 32), at.Tensor(32768, 32, 32))
     assert "reduction schedule: 1024 output entries, contraction of 32768 terms split over 256 workgroups x 1 slices (256 outputs per workgroup, a lane each)" in src
-    assert "for (long c = gc; c < 32768; c += 256)" in src and "const int o = blockIdx.x * 256 + threadIdx.x;" in src
+    assert "for (long c = gc; c < 32768; c += 256)" in src
+    # (the finishing kernel: 16 lanes per output, a share of the 256 partial sums each, added through LDS in a fixed order)
+    assert "const int o = blockIdx.x * 16 + threadIdx.x % 16, part = threadIdx.x / 16;" in src
+    assert "for (long g = part; g < 256; g += 16) t += scratch[g * 1024 + o];" in src
+    # (many outputs: a lane each)
+    src = TE.GetImplementation("S_i_j = A_e_i_j", at.Tensor(128, 128), at.Tensor(4000, 128, 128))
+    assert "const int o = blockIdx.x * 256 + threadIdx.x;" in src
     # up to 256 outputs every workgroup has them all; with the summed index fastest a workgroup takes four rows (up to 1 024)
     assert "output entries on adjacent lanes" in TE.GetImplementation("S_i = A_e_i", at.Tensor(200), at.Tensor(50000, 200))
     assert "four outputs per workgroup" in TE.GetImplementation("S_i = A_i_e", at.Tensor(1000), at.Tensor(1000, 50000))
