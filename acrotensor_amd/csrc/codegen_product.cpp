@@ -554,17 +554,17 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
           << (UA + UB) * NT * 8 << " bytes of LDS, " << groups * splits << " workgroups of " << NT << " lanes";
     if (splits > 1) sched << ", the contracted range in " << splits << " shares of " << span << " terms whose partial sums a second kernel adds";
     // Few workgroups per compute unit: a wavefront has its SIMD almost to itself, and what it issues beside the matrix
-    // instructions shows.  By the compiler's default the accumulators live in the accumulation half of the register file
-    // inside the loop and in the other half around its back edge, 64 copies per chunk; told to keep the matrix
-    // instruction's operands in ordinary vector registers it makes none.  512^3 17.4 -> 15.8 us, 1 024^3 53.3 -> 47.3 us,
-    // 144 x 128 x 100 000 105 -> 94 us; with many workgroups per compute unit the copies hide behind other wavefronts and
-    // the option loses a little (128^3 per entry 56.5 -> 54.6 % of the HBM peak), so those keep the default.
-    const bool vgprForm = groups * splits <= 1024 && W <= 4 && envInt("ACRO_HIP_TILED_PRODUCT_VGPR_FORM") >= 0;
-    if (vgprForm)
-    {
-        plan.compile_options = {"-mllvm", "-amdgpu-mfma-vgpr-form"};
-        sched << ", compiled with -amdgpu-mfma-vgpr-form";
-    }
+    // instructions shows.  Allowed all 512 registers of a SIMD lane (one wavefront per SIMD is enough for a workgroup of
+    // 256 lanes), the compiler keeps the accumulators in the accumulation half of the register file inside the loop and in
+    // the other half around its back edge, 64 copies per chunk; asked for at least two wavefronts per SIMD it has 256
+    // registers, all of them ordinary ones, uses about 100 and makes no copies.  512^3 16.5 -> 15.4 us, 1 024^3 54 -> 47 us,
+    // 1 536^3 183 -> 157 us, 144 x 128 x 100 000 105 -> 94 us; with many workgroups per compute unit the copies hide behind
+    // other wavefronts and the other form loses a little (128^3 per entry 56.5 -> 54.6 % of the HBM peak), so those are
+    // left to the compiler.
+    // Not for products that memory bounds (fewer than 9.8 operations per byte of the factors: 64 x 64 x 500 000 130 -> 157 us)
+    // nor for short ranges (128^3 on 16 entries: 8.7 -> 10.4 us).
+    const bool vgprForm = groups * splits <= 1024 && W <= 4 && M * N >= 40 * (M + N) && K >= 256 && envInt("ACRO_HIP_TILED_PRODUCT_VGPR_FORM") >= 0;
+    if (vgprForm) sched << ", at least two wavefronts per SIMD asked of the compiler";
     sched << "\n  [0] " << s.text << "\n";
     plan.schedule = sched.str();
     out << "// Generated by the acrotensor HIP code generator for gfx950.\n";
@@ -582,6 +582,7 @@ auto Generator::EmitTiledProduct(HipKernelPlan &plan) -> void
     out << "typedef double acro_double4 __attribute__((ext_vector_type(4)));\n";
     out << "\nextern \"C\" __global__ __launch_bounds__(" << NT << ") ";
     if (envInt("ACRO_HIP_TILED_PRODUCT_WAVES") > 0) out << "__attribute__((amdgpu_waves_per_eu(" << envInt("ACRO_HIP_TILED_PRODUCT_WAVES") << "))) ";
+    else if (vgprForm) out << "__attribute__((amdgpu_waves_per_eu(2))) ";
     const std::string fMain = splits > 1 ? plan.module_name + "_partial" : plan.module_name, fFinal = plan.module_name + "_final";
     out << "void " << fMain << "(" << ParamList() << (splits > 1 ? ", double *__restrict__ scratch" : "") << ")\n{\n";
     // (padded to a whole number of values per lane: lanes without a value of the tile write into the padding, no branch)

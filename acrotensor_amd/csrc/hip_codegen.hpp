@@ -149,8 +149,8 @@
 //                               terms per chunk (16), most strips per workgroup and blocks per strip (8, 8), waves per SIMD asked of
 //                               the compiler (none)
 //   ACRO_HIP_TILED_PRODUCT_SPLIT=-1 / =<n>  never share out the contracted range / share it out n ways
-//   ACRO_HIP_TILED_PRODUCT_VGPR_FORM=-1  launches of few workgroups are compiled like the others (default: with the matrix
-//                               instruction's accumulators in ordinary vector registers)
+//   ACRO_HIP_TILED_PRODUCT_VGPR_FORM=-1  launches of few workgroups are compiled like the others (default: for at least two
+//                               wavefronts per SIMD, which keeps the matrix instruction's accumulators in ordinary vector registers)
 //   ACRO_HIP_TILED_PRODUCT_HALF=-1 / _PREFER=<n>  few tiles keep eight strips per workgroup (default: four) / blocks per strip
 //                               that the split of the columns prefers (4)
 //   ACRO_HIP_TILED_PRODUCT_XCD=-1  the tiles of an entry are numbered as the hardware deals them (default: an entry's two to four
@@ -251,8 +251,6 @@ struct HipKernelPlan
     // the source that trades registers for LDS reads.
     std::vector<std::string> matrix_core_functions;
     std::string register_relief_macro;
-    // Further options for the run-time compiler that this source wants (beyond the library's own, which every source gets).
-    std::vector<std::string> compile_options;
     std::string schedule;          // human readable schedule summary (also a comment in the source)
 };
 

@@ -103,7 +103,7 @@ class HipExecutor : public KernelExecutor
             if (v->plan.fusable)
             {
                 v->kernel.reset(new HipKernel(v->plan.module_name, v->plan.source, v->plan.matrix_core_functions,
-                                              v->plan.register_relief_macro, v->plan.compile_options));
+                                              v->plan.register_relief_macro));
                 if (!v->kernel->PrivateMemoryRemains().empty())
                 {
                     // A matrix-core kernel that the compiler could only fit with register spills, also with the
@@ -120,7 +120,7 @@ class HipExecutor : public KernelExecutor
                         v->plan.source.insert(firstLine, "// (matrix-core kernel " + refused + " needed private memory, i.e. register spills, "
                                                          "and was refused: this is the schedule without the matrix cores)\n");
                         v->kernel.reset(new HipKernel(v->plan.module_name, v->plan.source, v->plan.matrix_core_functions,
-                                                      v->plan.register_relief_macro, v->plan.compile_options));
+                                                      v->plan.register_relief_macro));
                         ACROBATIC_ASSERT(v->kernel->PrivateMemoryRemains().empty(), "Internal error: matrix-core kernel in a plan without matrix cores.");
                     }
                 }

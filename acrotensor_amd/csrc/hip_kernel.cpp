@@ -86,7 +86,7 @@ bool makeDirs(const std::string &path)
     return true;
 }
 
-std::string cachePath(const std::string &name, const std::string &source, const std::vector<std::string> &own)
+std::string cachePath(const std::string &name, const std::string &source)
 {
     std::string dir = cacheDir();
     if (dir.empty()) return "";
@@ -94,7 +94,6 @@ std::string cachePath(const std::string &name, const std::string &source, const 
     hiprtcVersion(&major, &minor);
     std::string salt = std::to_string(major) + "." + std::to_string(minor);
     for (int i = 0; i < kNumCompileOptions; ++i) salt += std::string(" ") + kCompileOptions[i];
-    for (const std::string &option : own) salt += " " + option;
     for (const std::string &option : extraCompileOptions()) salt += " " + option;
     uint64_t h = fnv1a(source, fnv1a(salt + name));
     char hex[32];
@@ -191,9 +190,8 @@ std::string HipKernel::FirstKernelWithPrivateMemory() const
 }
 
 HipKernel::HipKernel(const std::string &module_name, const std::string &source,
-                     const std::vector<std::string> &no_private_memory, const std::string &relief_macro,
-                     const std::vector<std::string> &compile_options)
-    : FunctionName(module_name), Source(source), CacheHit(false), Options(compile_options), Guarded(no_private_memory), Module(nullptr)
+                     const std::vector<std::string> &no_private_memory, const std::string &relief_macro)
+    : FunctionName(module_name), Source(source), CacheHit(false), Guarded(no_private_memory), Module(nullptr)
 {
     // Experiment hook: $ACRO_HIP_KERNEL_OVERRIDE_DIR/<module name>.hip, when it exists, is compiled in place of the
     // generated source (same function names and parameters), e.g. a hand-edited copy of what GetImplementation printed.
@@ -228,7 +226,7 @@ HipKernel::~HipKernel()
 
 void HipKernel::Compile()
 {
-    const std::string path = cachePath(FunctionName, Source, Options);
+    const std::string path = cachePath(FunctionName, Source);
     if (!path.empty())
     {
         std::ifstream in(path, std::ios::binary | std::ios::ate);
@@ -251,7 +249,6 @@ void HipKernel::Compile()
              "hiprtcCreateProgram");
     const std::vector<std::string> extra = extraCompileOptions();
     std::vector<const char *> options(kCompileOptions, kCompileOptions + kNumCompileOptions);
-    for (const std::string &option : Options) options.push_back(option.c_str());
     for (const std::string &option : extra) options.push_back(option.c_str());
     hiprtcResult result = hiprtcCompileProgram(prog, static_cast<int>(options.size()), options.data());
     if (result != HIPRTC_SUCCESS)
@@ -298,7 +295,7 @@ void HipKernel::EnsureLoaded()
     {
         // A code object from the disk cache that does not load (damaged file, different driver): compile afresh.
         (void)hipGetLastError();
-        const std::string path = cachePath(FunctionName, Source, Options);
+        const std::string path = cachePath(FunctionName, Source);
         if (!path.empty()) std::remove(path.c_str());
         CacheHit = false;
         CodeObject.clear();

@@ -27,12 +27,10 @@ class HipKernel
     // segment size is read from the kernel descriptors of the code object, so the check needs no device.  When one
     // of them has private memory and relief_macro is not empty, the source is compiled once more with that macro
     // defined and checked again; what is left then is reported by PrivateMemoryRemains() and Launch refuses to run
-    // such a module (the caller generates another schedule).  compile_options are passed to the run-time compiler after
-    // the library's own options (and are part of the key of the on-disk cache).
+    // such a module (the caller generates another schedule).
     HipKernel(const std::string &module_name, const std::string &source,
               const std::vector<std::string> &no_private_memory = std::vector<std::string>(),
-              const std::string &relief_macro = std::string(),
-              const std::vector<std::string> &compile_options = std::vector<std::string>());
+              const std::string &relief_macro = std::string());
     ~HipKernel();
     HipKernel(const HipKernel &) = delete;
     HipKernel &operator=(const HipKernel &) = delete;
@@ -62,7 +60,6 @@ class HipKernel
     std::string Source;
     std::vector<char> CodeObject;
     bool CacheHit;
-    std::vector<std::string> Options;  // compiler options of this source's own
     std::vector<std::string> Guarded;  // kernels that must not have private memory
     std::string Spilling;              // one of them that has it all the same (after the relief macro, if any)
     bool Relieved = false;
