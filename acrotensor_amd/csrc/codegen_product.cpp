@@ -444,11 +444,18 @@ auto Generator::TiledProductPattern(const Sub &s, TiledProductShape &p) const ->
     p.N = extent[c];
     p.K = extent[k];
     p.E = p.batched ? extent[entry] : 1;
-    if (p.M < 16 || p.N < 16 || p.K < 16 || p.M * p.K >= (1L << 31) || p.N * p.K >= (1L << 31) || p.M * p.N >= (1L << 31)) return false;
+    // (fewer than 16 rows or columns only with a long contracted range and 64 outputs or more: most of a matrix
+    // instruction is padding then, but memory bounds such a product, and the reduction schedule takes only some of them
+    // (15 x 15 and 8 x 31 outputs over 10^6 terms were left to the generic schedule, which gives the range to single lanes:
+    // 110 ms); where both apply they measure alike (8 x 32 here 181 us, 4 x 32 there 155 us, 16 x 8 there 378 us))
+    const bool longRange = p.K >= 1024 && p.M * p.N >= 64 && std::min(p.M, p.N) >= 2;
+    if (((p.M < 16 || p.N < 16) && !longRange) || p.K < 16 || p.M * p.K >= (1L << 31) || p.N * p.K >= (1L << 31) || p.M * p.N >= (1L << 31)) return false;
     // (smaller matrices per entry have the schedules above; an unbatched product must be worth a launch of its own)
     const long from = envInt("ACRO_HIP_TILED_PRODUCT_FROM", 65);
     if (p.batched && std::max(p.M, p.N) < from && p.K <= 128) return false;
-    if (!p.batched && p.M * p.N < 64 * 64) return false;
+    // (... or have a long contracted range, which the generic schedule would give to single lanes: 32 x 32 outputs over
+    // 10^6 terms 102 ms there, 0.1 % of the HBM peak)
+    if (!p.batched && p.M * p.N < 64 * 64 && p.K < 1024) return false;
     // (one factor small enough for LDS in one piece: that is a dense operator applied to many vectors, "A_e_i = B_i_j X_e_j",
     // which the operator schedule streams at 64 - 86 % of the HBM peak)
     if (!p.batched && std::min(p.M, p.N) * p.K <= envInt("ACRO_HIP_TILED_PRODUCT_OPERATOR", 4096)) return false;

@@ -689,6 +689,13 @@ def test_products_of_large_matrices_run_in_tiles_on_the_matrix_cores(TE, monkeyp
     assert "for (int w = part; w < 191; w += 4) t += scratch[w * 16384L + o];" in src and "result[0L + o] = result[0L + o] + t;" in src
     src = TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(512, 512), at.Tensor(512, 512), at.Tensor(512, 512))
     assert "for (int w = 0; w < 4; ++w) t += scratch[w * 262144L + o];" in src
+    # fewer than 64 x 64 outputs, also fewer than 16 rows or columns, where the contracted range is long (1 024 terms and
+    # more) and there are 64 outputs or more: the generic schedule would give the whole range to single lanes
+    for rows, cols, terms in ((32, 32, 100000), (8, 100, 100000), (100, 8, 100000), (15, 15, 100000), (8, 31, 100000), (3, 300, 5000)):
+        src = TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(rows, cols), at.Tensor(rows, terms), at.Tensor(terms, cols))
+        assert "tiled product schedule" in src and "shares of" in src, (rows, cols, terms)
+    assert "tiled" not in TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(32, 32), at.Tensor(32, 1000), at.Tensor(1000, 32))
+    assert "reduction schedule" in TE.GetImplementation("A_i_j = B_i_k C_k_j", at.Tensor(4, 4), at.Tensor(4, 100000), at.Tensor(100000, 4))
     # 65 to 128 rows or columns per entry, and small matrices with more than 128 terms
     assert "tiled product schedule" in product("A_e_i_j = B_e_i_k C_e_k_j", 72, 72, 72)
     assert "tiled product schedule" in product("A_e_i_j = B_e_i_k C_e_k_j", 32, 48, 200)

@@ -351,6 +351,13 @@ TILED_PRODUCTS = [
     # device idle): a few shares, one lane per output in the second kernel
     ("A_i_j = B_i_k C_k_j", [(256, 256), (256, 256)]),
     ("A_i_j += B_i_k C_k_j", [(300, 520), (520, 200)]),
+    # ... fewer than 16 rows or columns under a long contracted range (most of the matrix instruction is padding; the
+    # generic schedule would give the whole range to single lanes)
+    ("A_i_j = B_i_k C_k_j", [(8, 3000), (3000, 100)]),
+    ("A_i_j -= B_k_i C_j_k", [(5000, 3), (300, 5000)]),
+    ("A_i_j += B_i_k C_j_k", [(15, 4001), (15, 4001)]),
+    ("A_i_j = C_k_j B_i_k", [(2000, 31), (8, 2000)]),
+    ("A_e_i_j = B_e_i_k C_e_k_j", [(3, 8, 1500), (3, 1500, 20)]),
     # ... many shares of few outputs: four and sixteen lanes per output in the second kernel
     ("A_i_j = B_n_i C_n_j", [(20000, 144), (20000, 128)]),
     ("A_i_j -= B_i_k C_k_j", [(64, 60000), (60000, 64)]),
