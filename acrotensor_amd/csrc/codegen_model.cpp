@@ -561,7 +561,9 @@ auto Generator::ProductThenRowSums(int ki, const Sub &orig, std::vector<Sub> &re
 auto Generator::FactoriseKernel(int ki, const Sub &orig, bool alone, std::vector<Sub> &result, int &counter) -> bool
 {
     const int nin = static_cast<int>(orig.in.size());
-    if (batch < 0 || nin < 3 || orig.contr.empty() || !opt.noalias || orig.out.repeated) return false;
+    // (two operands: only where an operand carries a contraction index alone, "A_e = B_e_j C_e_i", and can be summed over
+    // it before the product; the search finds nothing to do otherwise)
+    if (batch < 0 || nin < (envInt("ACRO_HIP_FACTORISE_PAIRS") < 0 ? 3 : 2) || orig.contr.empty() || !opt.noalias || orig.out.repeated) return false;
     if (alone && ReductionServes(orig)) return false;  // the reduction schedule serves it
     for (const auto &r : orig.in)
     {
@@ -585,7 +587,12 @@ auto Generator::FactoriseKernel(int ki, const Sub &orig, bool alone, std::vector
     // ACRO_HIP_FACTORISE=2 (tests): reorder whenever any chain is cheaper at all, however small the kernel.
     const bool eager = envInt("ACRO_HIP_FACTORISE") >= 2;
     if (bestSteps.empty()) return false;
-    if (!eager && (asWritten < kFactoriseMinWork || best * kFactoriseMinGain > asWritten)) return false;
+    // (a product of two operands that can be summed first repeats its loads for every term as written, every lane along
+    // rows of its own: "A_e = B_e_j C_e_i" with 32 and 27 terms took 6.0 ms for 500 MB; such a kernel is taken apart from
+    // 256 multiply-adds per entry on where that leaves an eighth of them)
+    const bool worthIt = nin == 2 ? asWritten >= 256.0 && best * 8.0 <= asWritten
+                                  : asWritten >= kFactoriseMinWork && best * kFactoriseMinGain <= asWritten;
+    if (!eager && !worthIt) return false;
 
     DimensionedKernel *kernel = mk.Kernels[ki];
     auto refText = [&](const std::string &name, const std::vector<int> &ids) {

@@ -1,5 +1,6 @@
 // Kernel code generator, the reduction schedule (few outputs, long contraction) and the kernel-parameter helpers.
 #include "hip_codegen_impl.hpp"
+#include <limits>
 
 namespace acro
 {
@@ -34,6 +35,25 @@ auto Generator::UseReductionSchedule() const -> bool
     const Sub &s = subs[0];
     if (s.out.repeated) return false;
     return ReductionServes(s);
+}
+
+// After the other schedules have declined and the generic plan is known: a kernel with a long contraction whose generic
+// plan leaves each lane hundreds of terms and the device mostly idle (few outputs in any layout: "A_i_j += B_i_e C_j"
+// with 12 x 16 outputs over 2^20 terms took 44 ms, "A_e += B_i C_e_i" with 2 048 rows of 8 192 terms 418 us for 134 MB)
+// shares the contraction range out over workgroups instead.
+auto Generator::UseReductionFallback() const -> bool
+{
+    if (subs.size() != 1 || factorised || NumGatherSlots() > 0 || envInt("ACRO_HIP_RED_FALLBACK") < 0) return false;
+    const Sub &s = subs[0];
+    if (s.out.repeated || s.matrixOp != 0 || s.in.empty() || s.contrCount < kReductionMinContraction) return false;
+    bool anyDims = false;
+    for (const auto &r : s.in) anyDims = anyDims || !r.idx.empty();
+    const long outputs = product(s.outIdx, extent);
+    if (!anyDims || outputs > 65536) return false;
+    const long lanes = E * s.laneCount, each = s.contrCount / std::max(1, s.splitLanes);
+    // (with more lanes than that the generic plan has the parallelism, and which of the two reads the smaller operands in
+    // longer runs depends on their layout: "A_j_k += B_j_k_i C_j_i_e" with 57 344 outputs 3.0 ms as planned, 9.9 ms here)
+    return each >= 256 && lanes <= 32768;
 }
 
 // Expression for the element offset of an occurrence given variables named i_<index> for every loop index.
@@ -99,6 +119,22 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         if (r.size > big->size) big = &r;
     }
     const bool outputsFastest = has(s.outIdx, big->idx.back());
+    // Output entries and contraction terms are numbered in the memory order of the big operand (indices it does not
+    // carry slowest), so that whichever of the two is laid along the lanes walks along its rows.  ("A_i_k = B_j_k_l C_e
+    // D_k_j_e_i" numbered as written puts neighbouring lanes 16 MB apart in D: 2.9 ms for 170 MB.)
+    auto inMemoryOrder = [&](std::vector<int> ids) {
+        auto reach = [&](int id) {
+            long st = 0;
+            for (size_t d = 0; d < big->idx.size(); ++d)
+            {
+                if (big->idx[d] == id) st += big->stride[d];
+            }
+            return st == 0 ? std::numeric_limits<long>::max() : st;
+        };
+        std::stable_sort(ids.begin(), ids.end(), [&](int a, int b) { return reach(a) > reach(b); });
+        return ids;
+    };
+    const std::vector<int> outIds = inMemoryOrder(s.outIdx), contrIds = inMemoryOrder(s.contr);
     // Few output entries that are the fastest dimension of the big operand ("S_i_j = A_n_i_j B_n"): a lane owns
     // whole contraction slices and keeps one accumulator per output entry ("pencil").  It reads the O entries of
     // its slice of A as 16-byte pieces and the slice's entry of B once, i.e. 6 load instructions per 80 bytes;
@@ -130,7 +166,9 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     // and more): a workgroup takes 256 neighbouring outputs, a lane each, and a share of the contraction range; the
     // lanes of a wavefront read 512 consecutive bytes per term.  The finishing kernel has a workgroup per 256 outputs.
     const bool wide = !pencil && !byRows && O > NTr;   // (up to 256 outputs: a lane per output in every workgroup, below)
-    ACROBATIC_ASSERT(!wide || outputsFastest || O <= NTr, "HIP generator: too many outputs for the reduction schedule.");
+    // More outputs than one workgroup's lanes, whichever way they were summed: the finishing kernel has a workgroup per
+    // 256 outputs too.
+    const bool wideFinish = wide || O > 1024;
     const long Sn = pencil ? NTr : (byRows ? 64 : (wide ? 1 : NTr / O));  // contraction slices per workgroup and step
     // (Two neighbouring outputs per lane, read as one 16-byte piece, measured slower: "S_i_j = A_e_i_j" with 32 x 32
     // outputs over 131 072 entries 70 -> 60 % of the HBM peak.)
@@ -151,15 +189,15 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     // measured 16.8 instead of 17.2 us for the pair of launches at n = 2^20), at most 1024.  The one-pass
     // variant finishes with the lanes of the partial kernel.
     int NTf = NTr;
-    const bool twoKernels = envInt("ACRO_HIP_ONE_PASS") <= 0 || wide || O > NTr;
-    if (twoKernels && !wide)
+    const bool twoKernels = envInt("ACRO_HIP_ONE_PASS") <= 0 || wideFinish || O > NTr;
+    if (twoKernels && !wideFinish)
     {
         NTf = kReductionLanes;
         while (NTf < 1024 && (G * O > NTf * 4 || NTf < O)) NTf *= 2;
     }
-    const long S2 = wide ? 1 : NTf / O;
+    const long S2 = wideFinish ? 1 : NTf / O;
     long wideParts = 1;   // lanes per output in the finishing kernel of the wide form
-    while (wide && wideParts < 16 && O * wideParts < 65536 && 8 * wideParts * 4 <= G) wideParts *= 4;
+    while (wideFinish && wideParts < 16 && O * wideParts < 65536 && 8 * wideParts * 4 <= G) wideParts *= 4;
 
     const std::string dimName = mk.GetDimensionedNameString();
     char hex[32];
@@ -221,7 +259,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         out << "    {\n        const long g = " << gExpr << ";\n";
         out << "#pragma unroll " << envInt("ACRO_HIP_RED_UNROLL", 1) << "\n";
         out << "        for (long c = g * " << Sn << " + lane; c < " << Nc << "; c += " << G * Sn << ")\n        {\n";
-        decompose(s.contr, "c", "            ");
+        decompose(contrIds, "c", "            ");
         // operand bases (contraction part of the address) and memoised loads (output part is a literal)
         std::vector<std::string> loads, sums;
         std::map<std::string, std::string> memo;
@@ -239,10 +277,10 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         for (long o = 0; o < O; ++o)
         {
             long rem = o;
-            for (int j = static_cast<int>(s.outIdx.size()) - 1; j >= 0; --j)
+            for (int j = static_cast<int>(outIds.size()) - 1; j >= 0; --j)
             {
-                value[s.outIdx[j]] = static_cast<int>(rem % extent[s.outIdx[j]]);
-                rem /= extent[s.outIdx[j]];
+                value[outIds[j]] = static_cast<int>(rem % extent[outIds[j]]);
+                rem /= extent[outIds[j]];
             }
             std::string prod;
             for (size_t v = 0; v < s.in.size(); ++v)
@@ -285,10 +323,10 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         out << "    const int o = og * " << Ow << " + lane / " << Sn << ", sl = lane % " << Sn << ";\n";
         out << "    double sum = 0.0;\n";
         out << "    if (o < " << O << ")\n    {\n";
-        decompose(s.outIdx, "o", "        ");
+        decompose(outIds, "o", "        ");
         out << "#pragma unroll 4\n";   // (8: 77 -> 71 % of the HBM peak for 64 rows of 2^20 terms)
         out << "        for (long c = (long)gc * " << Sn << " + sl; c < " << Nc << "; c += " << G * Sn << ")\n        {\n";
-        decompose(s.contr, "c", "            ");
+        decompose(contrIds, "c", "            ");
         std::string prod;
         for (const auto &r : s.in)
         {
@@ -311,10 +349,10 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         out << "    const int o = og * " << Ow << " + lane;\n";
         out << "    if (o < " << O << ")\n    {\n";
         out << "        double sum = 0.0;\n";
-        decompose(s.outIdx, "o", "        ");
+        decompose(outIds, "o", "        ");
         out << "#pragma unroll 8\n";
         out << "        for (long c = gc; c < " << Nc << "; c += " << G << ")\n        {\n";
-        decompose(s.contr, "c", "            ");
+        decompose(contrIds, "c", "            ");
         std::string prod;
         for (const auto &r : s.in)
         {
@@ -332,11 +370,11 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
             out << "    const int o = lane / " << Sn << ", sl = lane % " << Sn << ";\n";
         out << "    double sum = 0.0;\n";
         out << "    if (lane < " << Sn * O << ")\n    {\n";
-        decompose(s.outIdx, "o", "        ");
+        decompose(outIds, "o", "        ");
         out << "        const long g = " << gExpr << ";\n";
         out << "#pragma unroll 8\n";   // (4: 71 %, 8: 75 %, 16: 74 % of the HBM peak for 64 column sums over 2^20 rows)
         out << "        for (long c = g * " << Sn << " + sl; c < " << Nc << "; c += " << G * Sn << ")\n        {\n";
-        decompose(s.contr, "c", "            ");
+        decompose(contrIds, "c", "            ");
         std::string prod;
         for (const auto &r : s.in)
         {
@@ -376,7 +414,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         out << "    red[lane] = sum2;\n    __syncthreads();\n";
         out << "    if (lane < " << O << ")\n    {\n        double t = 0.0;\n";
         out << "        for (int k = 0; k < " << S2 << "; ++k) t += red[k * " << O << " + lane];\n";
-        decompose(s.outIdx, "lane", "        ");
+        decompose(outIds, "lane", "        ");
         const std::string dst = (twoKernels ? std::string("result") : PtrName(s.out.uvar)) + "[" + FullOffset(s.out) + "]";
         if (s.op == '=')
             out << "        " << dst << " = t;\n";
@@ -384,7 +422,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
             out << "        " << dst << " = " << dst << (s.op == '+' ? " + t;\n" : " - t;\n");
         out << "    }\n";
     };
-    if (wide)
+    if (wideFinish)
     {
         // a lane per output adds its partials in order; with few outputs and many shares, 4 or 16 lanes per output, each a
         // share of the partials, added through LDS in a fixed order again (1 024 outputs in 256 shares: 16.2 -> 4 us)
@@ -410,7 +448,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
             out << "#pragma unroll 8\n";
             out << "        for (long g = 0; g < " << G << "; ++g) t += scratch[g * " << O << " + o];\n";
         }
-        decompose(s.outIdx, "o", "        ");
+        decompose(outIds, "o", "        ");
         const std::string dst = "result[" + FullOffset(s.out) + "]";
         if (s.op == '=')
             out << "        " << dst << " = t;\n";
@@ -466,7 +504,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     {
         HipLaunch fin;
         fin.function_name = fFinal;
-        fin.grid = wide ? static_cast<unsigned>((O + NTf / wideParts - 1) / (NTf / wideParts)) : 1;
+        fin.grid = wideFinish ? static_cast<unsigned>((O + NTf / wideParts - 1) / (NTf / wideParts)) : 1;
         fin.block = NTf;
         fin.params.push_back(uvars[s.out.uvar].storage);
         fin.params.push_back(-1);

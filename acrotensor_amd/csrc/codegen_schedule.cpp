@@ -392,9 +392,20 @@ auto Generator::ChooseTiles() -> void
             auto perEntry = [&](const VarRef &r) { return has(r.idx, batch) ? r.size / E : r.size; };
             for (const auto &r : s.in)
             {
-                if (perEntry(r) > perEntry(*most)) most = &r;
+                // (of two operands of one size, the one that carries the batch index: "A_e = B_i_j C_e_j_i")
+                if (perEntry(r) > perEntry(*most) || (perEntry(r) == perEntry(*most) && has(r.idx, batch) && !has(most->idx, batch))) most = &r;
             }
-            bool streams = has(most->idx, batch) && most->idx.back() == s.contr.back();
+            // (its fastest dimensions may be the contraction indices in another order than the kernel names them, "A_e =
+            // B_i_j C_e_j_i": the terms are then numbered as they lie in that operand, 13 -> ... % of the HBM peak)
+            std::vector<int> asStored = s.contr;
+            if (s.contr.size() > 1 && most->idx.size() >= s.contr.size() && !most->repeated && envInt("ACRO_HIP_SPLIT_ORDER") >= 0)
+            {
+                const std::vector<int> tail(most->idx.end() - static_cast<long>(s.contr.size()), most->idx.end());
+                bool same = true;
+                for (int id : s.contr) same = same && has(tail, id);
+                if (same) asStored = tail;
+            }
+            bool streams = has(most->idx, batch) && most->idx.back() == asStored.back();
             // ... and a row of its own for every output: where the outputs of an entry all read the same few values
             // ("Y_e_i_j = B_q_i B_r_j D_e_q_r U_e_q_r") the lanes of an entry would only repeat each other's loads
             // (8.7 % of the HBM peak against 55 % with a row of outputs per lane)
@@ -417,6 +428,7 @@ auto Generator::ChooseTiles() -> void
                 if (lanes >= (mid.empty() ? 2 : 4))
                 {
                     s.tile.clear();
+                    s.contr = asStored;
                     SetLanes(s);
                     s.splitLanes = lanes;
                     s.loopMode = true;

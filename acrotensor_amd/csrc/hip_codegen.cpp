@@ -103,6 +103,11 @@ auto Generator::Run() -> HipKernelPlan
             return plan;
         }
     }
+    if (UseReductionFallback())
+    {
+        EmitReduction(plan);
+        return plan;
+    }
     ChooseEntriesFastest();
     Emit(plan);
     return plan;

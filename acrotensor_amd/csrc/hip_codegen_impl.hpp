@@ -368,6 +368,7 @@ class Generator
     static constexpr long kReductionMaxOutputs = 128;
     static constexpr int kReductionLanes = 256;
     bool UseReductionSchedule() const;
+    bool UseReductionFallback() const;
     bool ReductionServes(const Sub &s) const;
     std::string FullOffset(const VarRef &r) const;
     int NumParamStores() const;

@@ -339,7 +339,9 @@ def test_sums_over_a_long_index_take_the_reduction_schedule_whatever_the_number_
     # up to 256 outputs every workgroup has them all; with the summed index fastest a workgroup takes four rows (up to 1 024)
     assert "output entries on adjacent lanes" in TE.GetImplementation("S_i = A_e_i", at.Tensor(200), at.Tensor(50000, 200))
     assert "four outputs per workgroup" in TE.GetImplementation("S_i = A_i_e", at.Tensor(1000), at.Tensor(1000, 50000))
-    assert "reduction schedule" not in TE.GetImplementation("S_i = A_i_e", at.Tensor(1025), at.Tensor(1025, 50000))
+    # ... and beyond, with a finishing workgroup per 256 outputs again
+    src = TE.GetImplementation("S_i = A_i_e", at.Tensor(1025), at.Tensor(1025, 50000))
+    assert "four outputs per workgroup" in src and "const int o = blockIdx.x * 256 + threadIdx.x;" in src
     # short sums are not reductions
     assert "reduction schedule" not in TE.GetImplementation("S_i = A_e_i", at.Tensor(5000), at.Tensor(2000, 5000))
 

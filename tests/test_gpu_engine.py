@@ -1240,6 +1240,38 @@ def test_sums_over_a_long_index_with_many_outputs(at, engine, checker, kernel, s
 
 
 @pytest.mark.parametrize("kernel,shapes,expect", [
+    # more than 128 outputs whose terms do not stream one operand once: every value of B goes into 16 outputs
+    ("A_i_j += B_i_e C_j", [(12, 30011), (16,)], "four outputs per workgroup"),
+    ("A_j_e = B_i_j C_e", [(50021, 9), (20,)], "output entries on adjacent lanes"),
+    # more rows than one finishing workgroup has lanes, summed index fastest: by rows, a finishing workgroup per 256
+    ("A_e -= B_i C_e_i", [(8192,), (2048, 8192)], "four outputs per workgroup"),
+    ("S_i = A_i_e", [(1500, 9000)], "four outputs per workgroup"),
+    # outputs and summed indices interleaved in the big operand, numbered in its memory order
+    ("A_i_k = B_j_k_l C_e D_k_j_e_i", [(6, 9, 5), (700,), (9, 6, 700, 5)], "output entries on adjacent lanes"),
+    ("A_i_j = B_k_i_e C_j_e_k", [(50, 27, 300), (8, 300, 50)], "four outputs per workgroup"),
+    ("A_k_j_i += B_j_e_k C_i_j D_e_i", [(7, 9000, 12), (20, 7), (9000, 20)], "256 outputs per workgroup, a lane each"),
+])
+def test_long_contractions_of_any_layout_are_shared_out_over_workgroups(at, engine, checker, kernel, shapes, expect):
+    # what no other schedule takes and the generic plan would leave to few lanes with hundreds of terms each
+    rng = np.random.default_rng(shapes[0][0])
+    ins = [rng.integers(-3, 4, s).astype(np.float64) for s in shapes]
+    out0 = rng.integers(-3, 4, output_shape(kernel, shapes)).astype(np.float64)
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    src = engine.GetLastImplementation()
+    assert "reduction schedule" in src and expect in src
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert np.array_equal(got, expected)               # small integers: exact in any order
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= 4 * TOL
+    again, _ = run_single(at, engine, checker, kernel, out0, *ins)
+    assert np.array_equal(got, again)                   # fixed order of additions: reproducible
+
+
+@pytest.mark.parametrize("kernel,shapes,expect", [
     ("A_i_e = B_i_e C_i_e", [(16, 5000), (16, 5000)], "lanes(i)=16"),
     ("A_i_j_e -= B_i_k_e C_k_j_e", [(3, 3, 4099), (3, 3, 4099)], "lanes()=1 tile(i,j)=9"),          # ragged last workgroup
     ("A_i_e += B_i_k C_k_e W_e", [(5, 7), (7, 6001), (6001,)], "entry fastest"),
