@@ -487,13 +487,14 @@ auto Generator::StageReusedOperands(int ki, const Sub &asWritten, std::vector<Su
 // then the sums over j, one lane per row (a row stride that is odd spreads the lanes over the banks).
 auto Generator::ProductThenRowSums(int ki, const Sub &orig, std::vector<Sub> &result, int &counter) -> bool
 {
-    if (envInt("ACRO_HIP_ROW_SUMS") < 0 || batch < 0 || orig.in.size() != 2 || orig.contr.empty() || !opt.noalias) return false;
+    if (envInt("ACRO_HIP_ROW_SUMS") < 0 || batch < 0 || orig.in.empty() || orig.in.size() > 3 || orig.contr.empty() || !opt.noalias) return false;
     if (orig.out.repeated || orig.matrixOp != 0) return false;
     {
         ProductShape onMatrixCores;  // (the product schedule takes matrices of up to 128 x 128 with such rows)
         if (ProductPattern(orig, onMatrixCores)) return false;
     }
-    const VarRef *matrix = nullptr, *vec = nullptr;
+    const VarRef *matrix = nullptr;
+    std::vector<const VarRef *> vecs;
     for (const auto &r : orig.in)
     {
         if (r.repeated || r.uvar == orig.out.uvar) return false;
@@ -503,22 +504,42 @@ auto Generator::ProductThenRowSums(int ki, const Sub &orig, std::vector<Sub> &re
         if (all && matrix == nullptr)
             matrix = &r;
         else
-            vec = &r;
+            vecs.push_back(&r);
     }
-    if (matrix == nullptr || vec == nullptr || matrix == vec) return false;
-    // the contraction indices are the matrix's fastest dimensions, the vector carries nothing but them and the batch
+    if (matrix == nullptr) return false;
+    // the contraction indices are the matrix's fastest dimensions, the vectors carry nothing but them and the batch
     const size_t nc = orig.contr.size();
-    if (matrix->idx.size() < nc + 2 || matrix->idx[0] != batch) return false;
+    if (matrix->idx.size() < nc + 1 || matrix->idx[0] != batch) return false;
     for (size_t d = 0; d < nc; ++d)
     {
         if (!has(orig.contr, matrix->idx[matrix->idx.size() - 1 - d])) return false;
     }
-    for (int id : vec->idx)
+    for (const VarRef *vec : vecs)
     {
-        if (id != batch && !has(orig.contr, id)) return false;
+        for (int id : vec->idx)
+        {
+            if (id != batch && !has(orig.contr, id)) return false;
+        }
+        // (factors along part of a row, "A_e = B_e_i_j C_i D_j": no gain from HBM, 67 -> 50 % re-launched)
+        for (int id : orig.contr)
+        {
+            if (vecs.size() > 1 && !has(vec->idx, id)) return false;
+        }
     }
     const long rows = product(orig.outIdx, extent) / extent[batch], row = orig.contrCount;
-    if (row % 4 == 0 || row < 9 || rows < 4 || rows * row > 4096 || row > 512) return false;
+    if (rows * row > 4096 || row > 512) return false;
+    if (rows >= 4)
+    {
+        if (row % 4 == 0 || row < 9 || vecs.size() != 1) return false;
+    }
+    else
+    {
+        // One to three sums per entry ("A_e = B_e_i C_e_i", "A_e = B_e_i", "A_e_k = B_e_k_i C_e_i" with two components), from
+        // HBM: rows of 9 doubles 51 -> 79 % of the HBM peak, 15: 63 -> 77 %, 20: 65 -> 77 %, 27: 57 -> 77 %, 45: 64 -> 75 %,
+        // dot products of rows of 9: 59 -> 77 %, of 27: 62 -> 76 %; rows of 3 and 5 lose (75 -> 56 %, 73 -> 67 %), 6 and
+        // powers of two neither gain nor lose, rows of 100 lose (79 -> 76 %).
+        if (row < 7 || row > 64 || (row & (row - 1)) == 0) return false;
+    }
 
     DimensionedKernel *kernel = mk.Kernels[ki];
     auto refText = [&](const std::string &name, const std::vector<int> &ids) {

@@ -729,9 +729,9 @@ def test_kernels_whose_schedule_follows_the_memory_access_pattern(at, engine, ch
 
 @pytest.mark.parametrize("kernel,shapes", [
     ("A_e = B_e_i C_e_i", [(1003, 16), (1003, 16)]),             # 16 lanes per entry
-    ("A_e += B_e_i C_e_i", [(77, 9), (77, 9)]),                  # 8 lanes, 9 terms: lane 0 takes two
+    ("A_e += B_e_i C_e_i", [(77, 67), (77, 67)]),                # 16 lanes, 67 terms: the first three take five (short odd rows: through LDS)
     ("A_e -= B_e_n", [(301, 1000)]),                             # 64 lanes per entry
-    ("A_e = B_e_i_j C_j_i", [(130, 5, 7), (7, 5)]),              # two contraction indices, one operand transposed
+    ("A_e = B_e_i_j C_j_i", [(130, 5, 13), (13, 5)]),            # two contraction indices, one operand transposed
     ("A_e = B_e_i_j C_e_i_j D_j", [(64, 6, 4), (64, 6, 4), (4,)]),
     ("A_e = B_i_e_j C_e_j", [(3, 50, 11), (50, 11)]),            # batch index in the middle of an operand
     ("A_e_i = B_e_i_j C_e_j", [(203, 16, 16), (203, 16)]),       # element matrix times element vector: 4 lanes per row
@@ -1177,6 +1177,56 @@ def test_element_matrix_times_vector_with_odd_rows(at, engine, checker, kernel, 
     if "-=" in kernel:
         expected = 2.0 * out0 - expected
     assert rel_err(got, expected) <= TOL
+
+
+@pytest.mark.parametrize("kernel,shapes,steps", [
+    ("A_e = B_e_i", [(3001, 9)], True),                                   # row sums
+    ("A_e += B_e_i C_e_i", [(2000, 27), (2000, 27)], True),               # dot products of short rows
+    ("A_e -= B_i C_e_i", [(20,), (1234, 20)], True),                      # a weight vector shared by the entries
+    ("A_e = B_e_i C_i D_e_i", [(500, 45), (45,), (500, 45)], True),       # three factors along the row
+    ("A_e = B_e_i_j C_e_i_j", [(700, 3, 5), (700, 3, 5)], True),          # two contraction indices, rows of 15
+    ("A_e_k = B_e_k_i C_e_i", [(600, 2, 27), (600, 27)], True),           # two sums per entry
+    ("A_e = B_e_i", [(5000, 5)], False),                                  # short rows and powers of two stay as they are
+    ("A_e = B_e_i C_e_i", [(5000, 16), (5000, 16)], False),
+    ("A_e = B_e_i_j C_i D_j", [(900, 7, 9), (7,), (9,)], False),          # factors along part of a row
+])
+def test_short_sums_per_entry_go_through_an_lds_tile(at, engine, checker, kernel, shapes, steps):
+    # the products with the lanes along the operand as it lies in memory, into a tile in LDS, then a lane per sum
+    rng = np.random.default_rng(shapes[0][0])
+    ins = [rng.integers(-3, 4, s).astype(np.float64) for s in shapes]
+    out0 = rng.integers(-3, 4, output_shape(kernel, shapes)).astype(np.float64)
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert ("steps of:" in engine.GetLastImplementation()) == steps
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert np.array_equal(got, expected)
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= TOL
+
+
+@pytest.mark.parametrize("kernel,shapes", [
+    ("A_e = B_e_j C_e_i", [(3000, 32), (3000, 27)]),                         # both operands summed first, then one product
+    ("A_e_l += B_i_l C_e_j_k", [(20, 10), (501, 64, 9)]),                    # the element tensor summed first
+    ("A_e_i_j -= B_e_k C_e_i_j_l", [(333, 27), (333, 12, 20, 9)]),
+    ("A_e_k = B_k_i C_e_j_k", [(12, 32), (2177, 64, 12)]),
+])
+def test_operands_that_carry_a_contraction_index_alone_are_summed_first(at, engine, checker, kernel, shapes):
+    rng = np.random.default_rng(shapes[0][0])
+    ins = [rng.integers(-3, 4, s).astype(np.float64) for s in shapes]
+    out0 = rng.integers(-3, 4, output_shape(kernel, shapes)).astype(np.float64)
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    assert "steps of:" in engine.GetLastImplementation()
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert np.array_equal(got, expected)
+    ins = [rng.uniform(-1, 1, s) for s in shapes]
+    got, expected = run_single(at, engine, checker, kernel, out0, *ins)
+    if "-=" in kernel:
+        expected = 2.0 * out0 - expected
+    assert rel_err(got, expected) <= 4 * TOL            # another order of additions than the oracle's
 
 
 @pytest.mark.parametrize("n,m,op", [(5000, 8, "="), (3001, 4, "+="), (2500, 7, "-="), (2100, 11, "=")])
