@@ -20,9 +20,10 @@ auto Generator::NumGatherSlots() const -> int
 }
 
 // Read of entry `offset` of an operand from device memory.
-auto Generator::GlobalRead(int uvar, const std::string &offset) const -> std::string
+auto Generator::GlobalRead(int uvar, const std::string &offset, bool streamedOnce) const -> std::string
 {
     const int g = GatherSlot(uvar);
+    if (g < 0 && streamedOnce) return "__builtin_nontemporal_load(&" + PtrName(uvar) + "[" + offset + "])";
     if (g < 0) return PtrName(uvar) + "[" + offset + "]";
     return "G" + str(g) + "s[G" + str(g) + "m[" + offset + "]]";
 }
@@ -151,6 +152,36 @@ auto Generator::ScalarBase(const VarRef &r) const -> std::string
     return base;
 }
 
+// Device-memory operand whose values are read once each, by lanes that follow it through memory so that every load
+// instruction of a wavefront takes whole 128-byte lines: requested with the non-temporal hint, which keeps lines that
+// nothing reads again from displacing others (from HBM: "A_e_i = B_e_i C_e_i D_e_i" 345 -> 319 us, "A_e = B_e_n" with
+// rows of 1 024 92 -> 84 us, "A_e_i = B_e_i_n" 182 -> 161 us).  Not where lanes read pieces of lines that a later
+// instruction or a neighbouring workgroup completes: those lines are then fetched twice (the p=3 mass apply 87 -> 106 us,
+// the p=7 diffusion apply 939 -> 1 626 us with every streaming operand read that way).
+auto Generator::StreamedOnce(int k, int v) const -> bool
+{
+    if (envInt("ACRO_HIP_NT_LOADS") < 0 || batch < 0) return false;
+    const Sub &s = subs[k];
+    const VarRef &r = s.in[v];
+    if (SourceOf(k, v) != kFromGlobal || !IsPureInput(r.uvar) || GatherSlot(r.uvar) >= 0 || r.repeated || r.idx.empty() || r.idx[0] != batch) return false;
+    if (s.matrixOp != 0 || !s.tile.empty() || entriesFastest) return false;
+    if (((r.size / E) * NB) % 16 != 0) return false;   // the share of a workgroup: whole lines
+    if (s.splitLanes > 0)
+    {
+        // the lanes of an output walk along the contraction, which is the operand's fastest dimensions in the kernel's order
+        // and long enough for a row of 16 lanes to take a line per step; every output has a row of its own
+        const size_t nc = s.contr.size();
+        if (s.contrCount % 16 != 0 || r.idx.size() < nc + 1 || !std::equal(s.contr.begin(), s.contr.end(), r.idx.end() - static_cast<long>(nc))) return false;
+        for (int id : s.outIdx)
+        {
+            if (!has(r.idx, id)) return false;
+        }
+        return true;
+    }
+    // a kernel without contraction whose operand lies in memory as the result does
+    return s.contr.empty() && !s.out.repeated && r.idx == s.out.idx;
+}
+
 // Device-memory operand that a phase may load long before it is used: never written by the group and
 // addressed through the batch index (the streaming inputs, not small tables).
 auto Generator::Prefetchable(int k, int v) const -> bool
@@ -188,7 +219,7 @@ auto Generator::OperandExpr(int k, int v, const std::vector<int> &value, Body &b
     }
     else
     {
-        const std::string rhs = GlobalRead(r.uvar, base + " + " + Lit(off));
+        const std::string rhs = GlobalRead(r.uvar, base + " + " + Lit(off), StreamedOnce(k, v));
         body.loads.push_back("const double " + name + " = " + rhs + ";");
         if (Prefetchable(k, v)) body.globalLoads.push_back(std::make_pair(key, rhs));
     }
@@ -712,7 +743,9 @@ auto Generator::EmitSplitLanesBody(int k, std::vector<std::string> &lines) -> vo
             // would serve: the index differs from lane to lane here)
             const std::string at = src == kFromConstant ? PtrName(r.uvar) + "[" + ScalarBase(r) + Lit(uvars[r.uvar].viewOffset) + " + " + off + "]"
                                                         : PtrName(r.uvar) + "[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
-            lines.push_back("    const acro_pair p" + str(static_cast<long>(v)) + " = *reinterpret_cast<const acro_pair *>(&" + at + ");");
+            lines.push_back("    const acro_pair p" + str(static_cast<long>(v)) + " = " +
+                            (src == kFromGlobal && StreamedOnce(k, static_cast<int>(v)) ? "__builtin_nontemporal_load(reinterpret_cast<const acro_pair *>(&" + at + "));"
+                                                                                         : "*reinterpret_cast<const acro_pair *>(&" + at + ");"));
             opnd = "p" + str(static_cast<long>(v)) + ".@";
         }
         else if (src == kFromConstant)
@@ -720,7 +753,7 @@ auto Generator::EmitSplitLanesBody(int k, std::vector<std::string> &lines) -> vo
         else if (lds)
             opnd = "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
         else
-            opnd = GlobalRead(r.uvar, "o_k" + str(k) + "v" + str(v) + " + " + off);
+            opnd = GlobalRead(r.uvar, "o_k" + str(k) + "v" + str(v) + " + " + off, StreamedOnce(k, static_cast<int>(v)));
         prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
     }
     if (pairs)
@@ -823,7 +856,7 @@ auto Generator::EmitLoopBody(int k, std::vector<std::string> &lines) -> void
         if (fixed != 0 || off.empty()) off += (off.empty() ? "" : " + ") + (lds ? str(fixed) : Lit(fixed));
         if (src == kFromConstant) return ConstPtrName(r.uvar) + "[" + ScalarBase(r) + Lit(uvars[r.uvar].viewOffset) + " + " + off + "]";
         if (lds) return "lds[o_k" + str(k) + "v" + str(v) + " + " + off + "]";
-        return GlobalRead(r.uvar, "o_k" + str(k) + "v" + str(v) + " + " + off);
+        return GlobalRead(r.uvar, "o_k" + str(k) + "v" + str(v) + " + " + off, StreamedOnce(k, static_cast<int>(v)));
     };
     std::string common;
     for (size_t v = 0; v < s.in.size(); ++v)

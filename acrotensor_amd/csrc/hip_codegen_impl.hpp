@@ -299,7 +299,8 @@ class Generator
     std::string PtrName(int uvar) const { return "T" + str(uvars[uvar].storage); }
     int GatherSlot(int uvar) const;
     int NumGatherSlots() const;
-    std::string GlobalRead(int uvar, const std::string &offset) const;
+    std::string GlobalRead(int uvar, const std::string &offset, bool streamedOnce = false) const;
+    bool StreamedOnce(int k, int v) const;
     std::string ConstPtrName(int uvar) const { return "C" + str(uvars[uvar].storage); }
     const Storage &StoreOf(int uvar) const { return stores[uvars[uvar].storage]; }
     int LdsStride(int uvar, size_t d) const;

@@ -154,13 +154,17 @@ __global__ __launch_bounds__(kMatLanes) void batchMatrixKernel(const double *__r
     const double *src = A + first * MM;
 
     // first * MM * 8 bytes is a multiple of 16 (kMatLanes is even), so pairs of doubles are aligned when A is
-    const double2 *src2 = reinterpret_cast<const double2 *>(src);
     for (int i = threadIdx.x; i < ndbl / 2; i += kMatLanes)
     {
         double2 v;
         if (PAIRS)
         {
-            v = src2[i];
+            // one instruction of the wavefront reads 1 KB of whole lines that nothing reads again: non-temporal (2^22
+            // 3 x 3 matrices from HBM: 108.6 -> 101.1 us; workgroups of 128 or 256 lanes and two matrices per lane
+            // measured slower with either kind of load)
+            const Double2 w = __builtin_nontemporal_load(reinterpret_cast<const Double2 *>(src) + i);
+            v.x = w.x;
+            v.y = w.y;
         }
         else
         {
