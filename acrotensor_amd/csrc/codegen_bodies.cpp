@@ -25,6 +25,7 @@ auto Generator::GlobalRead(int uvar, const std::string &offset, bool streamedOnc
     const int g = GatherSlot(uvar);
     if (g < 0 && streamedOnce) return "__builtin_nontemporal_load(&" + PtrName(uvar) + "[" + offset + "])";
     if (g < 0) return PtrName(uvar) + "[" + offset + "]";
+    // (the map read with the non-temporal hint: scatter + p=3 mass apply in one launch 90.4 -> 92.9 us from HBM, not taken)
     return "G" + str(g) + "s[G" + str(g) + "m[" + offset + "]]";
 }
 
