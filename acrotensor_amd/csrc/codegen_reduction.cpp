@@ -156,6 +156,13 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
     }
     const bool pencil = outputsFastest && (O <= 16 || (O <= 64 && 2 * loadsPerSlice <= O)) && envInt("ACRO_HIP_RED_PENCIL") >= 0;
     const int NTr = kReductionLanes;
+    // The big operand streams through once, its values going into one term each, read by lanes that follow it through
+    // memory in whole 128-byte lines per load instruction: requested with the non-temporal hint (64 column sums over 2^20
+    // rows 75 -> 81 % of the HBM peak, 64 row sums 78 -> 84 %, 32 x 32 sums of element matrices 71 -> 74 %).  Not the
+    // pencil form, whose lanes take 16-byte pieces of lines that their neighbours complete (2^20 slices of 3 x 3: 16.8 ->
+    // 28.5 us), and not operands whose values go into several outputs (192 outputs by rows: 145 -> 238 us).
+    const bool ntBig = envInt("ACRO_HIP_RED_NT") >= 0 && !pencil && !big->repeated && static_cast<double>(O) * static_cast<double>(Nc) <= static_cast<double>(big->size) &&
+                       big->size % 16 == 0 && (outputsFastest ? O % 16 == 0 : big->ext.back() % 16 == 0);
     // Contraction index fastest and more than four outputs ("S_i = A_i_n" with 64 rows): with all outputs in every
     // workgroup only NTr / O lanes would walk along a row (32-byte pieces of 64 different rows per load
     // instruction).  Instead a workgroup takes four outputs, 64 adjacent lanes each, and the workgroups are dealt
@@ -296,7 +303,8 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
                 if (it == memo.end())
                 {
                     const std::string name = "x" + str(static_cast<long>(v)) + "_" + str(static_cast<long>(memo.size()));
-                    loads.push_back("const double " + name + " = " + PtrName(r.uvar) + "[ob" + str(static_cast<long>(v)) + " + " + Lit(lit) + "];");
+                    const std::string at = PtrName(r.uvar) + "[ob" + str(static_cast<long>(v)) + " + " + Lit(lit) + "]";
+                    loads.push_back("const double " + name + " = " + (ntBig && &r == big ? "__builtin_nontemporal_load(&" + at + ")" : at) + ";");
                     it = memo.emplace(key, name).first;
                 }
                 prod = prod.empty() ? it->second : "(" + prod + " * " + it->second + ")";
@@ -330,7 +338,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         std::string prod;
         for (const auto &r : s.in)
         {
-            const std::string opnd = PtrName(r.uvar) + "[" + FullOffset(r) + "]";
+            const std::string opnd = (ntBig && &r == big) ? "__builtin_nontemporal_load(&" + PtrName(r.uvar) + "[" + FullOffset(r) + "])" : PtrName(r.uvar) + "[" + FullOffset(r) + "]";
             prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
         }
         out << "            sum += " << prod << ";\n        }\n    }\n";
@@ -356,7 +364,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         std::string prod;
         for (const auto &r : s.in)
         {
-            const std::string opnd = PtrName(r.uvar) + "[" + FullOffset(r) + "]";
+            const std::string opnd = (ntBig && &r == big) ? "__builtin_nontemporal_load(&" + PtrName(r.uvar) + "[" + FullOffset(r) + "])" : PtrName(r.uvar) + "[" + FullOffset(r) + "]";
             prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
         }
         out << "            sum += " << prod << ";\n        }\n";
@@ -378,7 +386,7 @@ auto Generator::EmitReduction(HipKernelPlan &plan) -> void
         std::string prod;
         for (const auto &r : s.in)
         {
-            const std::string opnd = PtrName(r.uvar) + "[" + FullOffset(r) + "]";
+            const std::string opnd = (ntBig && &r == big) ? "__builtin_nontemporal_load(&" + PtrName(r.uvar) + "[" + FullOffset(r) + "])" : PtrName(r.uvar) + "[" + FullOffset(r) + "]";
             prod = prod.empty() ? opnd : "(" + prod + " * " + opnd + ")";
         }
         out << "            sum += " << prod << ";\n        }\n    }\n";
