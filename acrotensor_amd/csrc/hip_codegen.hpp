@@ -77,8 +77,9 @@
 //                               writes out in whole lines only for a kernel on its own whose lanes each hold a long run of outputs
 //                               (default: also for the last kernel of any group whose store instructions would fill less than
 //                               30 % of the lines they touch).  ACRO_HIP_COPY_OUT_MAX=<doubles per batch entry> (default 2048)
-//   ACRO_HIP_ROW_SUMS=-1        an element matrix times an element vector with rows that are no multiple of four doubles runs as
-//                               written (lanes along the rows) instead of as products into LDS followed by row sums
+//   ACRO_HIP_ROW_SUMS=-1        an element matrix times an element vector with rows that are no multiple of four doubles, and
+//                               one to three short sums per entry (dot products, row sums), run as written (lanes along the
+//                               rows) instead of as products into LDS followed by row sums
 //   ACRO_HIP_PREFETCH_FIRST=-1 / ACRO_HIP_PREFETCH_CLAMP=-1 / ACRO_HIP_PREFETCH_PASSES=-1
 //                               the first phase's operands are not requested ahead of the prefetched ones / prefetch loads of
 //                               partly filled passes stay behind a branch / a first phase of several passes keeps its item loop
@@ -117,6 +118,14 @@
 //                               whose vectors come through scalar loads, whatever the operator's sizes)
 //   ACRO_HIP_RED_PENCIL=-1      split contractions: one lane per (slice, output entry) also when there are few outputs
 //   ACRO_HIP_RED_WIDE=-1        sums over a long index with more than 128 outputs keep the generic schedule
+//   ACRO_HIP_RED_FALLBACK=-1    a long contraction that no schedule takes and that the generic plan leaves to few lanes keeps
+//                               the generic plan instead of being shared out over workgroups
+//   ACRO_HIP_FACTORISE_PAIRS=-1 a kernel of two operands is not taken apart where an operand carries a contraction index alone
+//   ACRO_HIP_SPLIT_ORDER=-1     a contraction shared by lanes is numbered as the kernel names its indices, not as they lie in
+//                               the streaming operand
+//   ACRO_HIP_NT_LOADS=-1 / ACRO_HIP_RED_NT=-1 / ACRO_HIP_GRAM_NT=-1 / ACRO_HIP_PRODUCT_NT=-1
+//                               no non-temporal hint on operands that are read once in whole lines (chain, reduction, Gram
+//                               and product schedules)
 //   ACRO_HIP_RED_ROWS=-1        split contractions of few long rows: all outputs in every workgroup, NT / outputs lanes along a row
 //   ACRO_HIP_ONE_PASS=1         split contractions: the workgroup that finishes last adds the per-workgroup partials
 //                               instead of a second kernel (measured 18.4 against 16.3 us: the device-scope release
