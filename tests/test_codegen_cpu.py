@@ -712,3 +712,69 @@ def test_products_of_large_matrices_run_in_tiles_on_the_matrix_cores(TE, monkeyp
     monkeypatch.setenv("ACRO_HIP_TEST_PRIVATE_BYTES", "8,8")
     src = product("A_e_i_j = B_e_i_k C_e_k_j", 128, 128, 128)
     assert "tiled product schedule" not in src and "was refused" in src
+
+
+def test_operands_read_once_in_whole_lines_take_the_non_temporal_hint(TE, monkeypatch):
+    # the mass apply's element vector: 64 values per entry, the lanes on its two fastest dimensions; the geometric factors,
+    # five doubles per lane at a stride, keep ordinary loads
+    src = chain_source(TE, workloads.config4(E=64), transient=True)
+    assert "__builtin_nontemporal_load(&T2[o_k0v1 + 0])" in src and "__builtin_nontemporal_load(&T6[" not in src
+    assert "= T6[o_k3v0 + 0];" in src
+    # the diffusion apply's element vector is read by two kernels of the group: ordinary loads
+    src = chain_source(TE, workloads.config5(E=8), transient=True)
+    assert "__builtin_nontemporal_load" not in src
+    # kernels without contraction whose operands lie in memory as the result does
+    src = TE.GetImplementation("A_e_i = B_e_i C_e_i", at.Tensor(4096, 16), at.Tensor(4096, 16), at.Tensor(4096, 16))
+    assert src.count("__builtin_nontemporal_load(&T") == 2
+    # ... not an operand whose values go to several work items, not the batch index last
+    assert "__builtin_nontemporal_load" not in TE.GetImplementation("A_e_i_j = B_e_i C_e_j", at.Tensor(4096, 8, 8), at.Tensor(4096, 8), at.Tensor(4096, 8))
+    assert "__builtin_nontemporal_load" not in TE.GetImplementation("A_i_e = B_i_e C_i_e", at.Tensor(16, 4096), at.Tensor(16, 4096), at.Tensor(16, 4096))
+    # a contraction shared by lanes along rows of whole lines; rows of 100 doubles share lines
+    assert "__builtin_nontemporal_load" in TE.GetImplementation("A_e = B_e_n", at.Tensor(4096), at.Tensor(4096, 1024))
+    assert "__builtin_nontemporal_load" not in TE.GetImplementation("A_e = B_e_n", at.Tensor(4096), at.Tensor(4096, 100))
+    # reductions: the streaming forms, not the pencil form
+    assert "__builtin_nontemporal_load" in TE.GetImplementation("S_i = A_n_i", at.Tensor(64), at.Tensor(1 << 16, 64))
+    assert "__builtin_nontemporal_load" not in TE.GetImplementation("S_i_j = A_n_i_j B_n", at.Tensor(3, 3), at.Tensor(1 << 16, 3, 3), at.Tensor(1 << 16))
+    # Gram sums with rows of whole lines, factors of element-matrix products that are whole lines per entry
+    assert "__builtin_nontemporal_load(&b[16 * ti])" in TE.GetImplementation("A_i_j = B_e_i C_e_j", at.Tensor(32, 32), at.Tensor(1 << 16, 32), at.Tensor(1 << 16, 32))
+    assert "__builtin_nontemporal_load" not in TE.GetImplementation("A_i_j = B_e_i C_e_j", at.Tensor(24, 24), at.Tensor(1 << 16, 24), at.Tensor(1 << 16, 24))
+    assert "__builtin_nontemporal_load" in TE.GetImplementation("A_e_i_j = B_e_i_k C_e_k_j", at.Tensor(512, 32, 32), at.Tensor(512, 32, 32), at.Tensor(512, 32, 32))
+    assert "__builtin_nontemporal_load" not in TE.GetImplementation("A_e_i_j = B_e_i_k C_e_k_j", at.Tensor(512, 33, 33), at.Tensor(512, 33, 33), at.Tensor(512, 33, 33))
+    monkeypatch.setenv("ACRO_HIP_NT_LOADS", "-1")
+    assert "__builtin_nontemporal_load" not in chain_source(at.TensorEngine("HIP"), workloads.config4(E=64), transient=True)
+
+
+def test_long_contractions_that_no_schedule_takes_are_shared_out_over_workgroups(TE, monkeypatch):
+    # more than 128 outputs whose big operand does not stream once, few long rows, interleaved layouts: the generic plan
+    # would leave hundreds of terms to each of few lanes
+    src = TE.GetImplementation("A_i_j += B_i_e C_j", at.Tensor(12, 16), at.Tensor(12, 1 << 20), at.Tensor(16))
+    assert "reduction schedule: 192 output entries" in src and "four outputs per workgroup" in src
+    src = TE.GetImplementation("A_e += B_i C_e_i", at.Tensor(2048), at.Tensor(8192), at.Tensor(2048, 8192))
+    assert "reduction schedule: 2048 output entries" in src and "const int o = blockIdx.x * 256 + threadIdx.x;" in src
+    # outputs and terms numbered in the big operand's memory order: D_k_j_e_i has i fastest, then e
+    src = TE.GetImplementation("A_i_k = B_j_k_l C_e D_k_j_e_i", at.Tensor(5, 9), at.Tensor(16, 9, 20), at.Tensor(4096), at.Tensor(9, 16, 4096, 5))
+    assert "const int i_k = (int)(o / 5);" in src and "const int i_i = (int)((o / 1) % 5);" in src
+    assert "const int i_e = (int)((c / 1) % 4096);" in src
+    # many lanes in the generic plan: it keeps the kernel
+    assert "reduction schedule" not in TE.GetImplementation("A_j_k += B_j_k_i C_j_i_e", at.Tensor(7, 8192), at.Tensor(7, 8192, 512), at.Tensor(7, 512, 100))
+    monkeypatch.setenv("ACRO_HIP_RED_FALLBACK", "-1")
+    assert "reduction schedule" not in at.TensorEngine("HIP").GetImplementation("A_i_j += B_i_e C_j", at.Tensor(12, 16), at.Tensor(12, 1 << 20), at.Tensor(16))
+
+
+def test_operands_that_carry_a_contraction_index_alone_are_summed_first(TE):
+    src = TE.GetImplementation("A_e = B_e_j C_e_i", at.Tensor(4096), at.Tensor(4096, 32), at.Tensor(4096, 27))
+    assert "_F1_e = B_e_j" in src and "_F2_e = C_e_i" in src and "A_e = _F1_e _F2_e   (steps of: A_e = B_e_j C_e_i)" in src
+    src = TE.GetImplementation("A_e_l = B_i_l C_e_j_k", at.Tensor(4096, 10), at.Tensor(20, 10), at.Tensor(4096, 64, 9))
+    assert "_F1_e = C_e_j_k" in src and "A_e_l = B_i_l _F1_e" in src
+    # nothing to sum first: both operands carry the contraction index; too little work: as written
+    assert "steps of" not in TE.GetImplementation("A_e_i = B_e_i_j C_e_j", at.Tensor(4096, 8), at.Tensor(4096, 8, 8), at.Tensor(4096, 8))
+    assert "steps of" not in TE.GetImplementation("A_e = B_e_j C_e_i", at.Tensor(4096), at.Tensor(4096, 4), at.Tensor(4096, 4))
+    # short sums per entry: products into an LDS tile with the lanes along memory, then a lane per sum
+    src = TE.GetImplementation("A_e = B_e_i C_e_i", at.Tensor(4096), at.Tensor(4096, 27), at.Tensor(4096, 27))
+    assert "_F1_e_i = B_e_i C_e_i" in src and "A_e = _F1_e_i   (steps of:" in src
+    assert "steps of" in TE.GetImplementation("A_e = B_e_i", at.Tensor(4096), at.Tensor(4096, 9))
+    for row in (3, 5, 16, 100):
+        assert "steps of" not in TE.GetImplementation("A_e = B_e_i", at.Tensor(4096), at.Tensor(4096, row))
+    # a contraction shared by lanes is numbered as the terms lie in the streaming operand
+    src = TE.GetImplementation("A_e = B_i_j C_e_j_i", at.Tensor(4096), at.Tensor(20, 8), at.Tensor(4096, 8, 20))
+    assert "contraction shared by" in src and "lanes()=16" in src
