@@ -292,6 +292,12 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
     // 4 x 4 65 -> 49 %, 4 x 8 82 -> 77 %, 7 x 9 62 -> 57 %, 27 x 3 36 -> 28 %; 20 x 5 a tie.
     // (odd lengths: 9 x 9 47 -> 59 %, 25 x 25 45 -> 68 %, 27 x 27 46 -> 66 %; 5 x 5 63 -> 58 %)
     if (o.comp > 1) return o.rows * o.cols >= envInt("ACRO_HIP_OPERATOR_COMPONENTS_MIN", 256);
+    // Two to four rows applied to vectors of 16 values and more (a gradient at a point, "G_e_d = D_d_i X_e_i"): the generic
+    // schedule has a lane per result read the whole vector (from HBM: 3 x 32 30 %, 4 x 64 25 %, 2 x 64 43 %, 3 x 128 27 % of
+    // the HBM peak); on the matrix cores 73 / 72 / 71 / 67 %, and no worse at 16 columns (2 / 3 / 4 x 16: 56 / 71 / 75 ->
+    // 72 / 75 / 75 %).
+    const long fewRowsFrom = envInt("ACRO_HIP_OPERATOR_FEW_ROWS", 16);
+    if (o.pairs && o.rows >= 2 && o.rows < 5 && fewRowsFrom > 0 && o.cols >= fewRowsFrom) return true;
     return o.pairs ? (o.rows >= 5 && o.cols >= 4) : (o.cols >= 16 || (o.cols >= 9 && o.rows >= 8));
 }
 

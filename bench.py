@@ -257,6 +257,8 @@ KERNEL_SHAPES = [
     ("A_e_i = B_i_j X_e_j", [(81, 8), (1 << 20, 8)], (1 << 20, 81)),
     ("Y_e_i_j = B_q_i B_r_j D_e_q_r U_e_q_r", [(5, 4), (5, 4), (1 << 20, 5, 5), (1 << 20, 5, 5)], (1 << 20, 4, 4)),
     ("U_e_q_r_s = B_q_i B_r_j B_s_k X_e_i_j_k", [(5, 4), (5, 4), (5, 4), (1 << 18, 4, 4, 4)], (1 << 18, 5, 5, 5)),
+    # a gradient at a point: three rows applied to vectors of 32 values
+    ("G_e_d = D_d_i X_e_i", [(3, 32), (1 << 20, 32)], (1 << 20, 3)),
     # short sums per entry (products into an LDS tile, then a lane per sum)
     ("A_e = B_e_i", [(1 << 22, 9)], (1 << 22,)),
     ("A_e = B_e_i C_e_i", [(1 << 20, 27), (1 << 20, 27)], (1 << 20,)),

@@ -269,11 +269,15 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     # very long vectors or very many rows would not fit a lane's registers: not this schedule
     assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 5), at.Tensor(5, 818), at.Tensor(900, 818))
     assert "operator schedule" not in TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(900, 300), at.Tensor(300, 12), at.Tensor(900, 12))
-    # not this schedule: few rows (a register tile with scalar operands serves them), third operand
-    for kernel, shapes in (("A_e_i = B_i_j X_e_j", [(500, 4), (4, 64), (500, 64)]),
+    # not this schedule: few rows of short vectors (a register tile with scalar operands serves them), third operand
+    for kernel, shapes in (("A_e_i = B_i_j X_e_j", [(500, 4), (4, 8), (500, 8)]),
                            ("A_e_i = B_i_j X_e_k_j W_e_k", [(500, 64), (64, 64), (500, 2, 64), (500, 2)])):
         tensors = [at.Tensor(*shp) for shp in shapes]
         assert "operator schedule" not in TE.GetImplementation(kernel, *tensors)
+    # two to four rows applied to vectors of 16 values and more (a gradient at a point) do take it
+    for rows, cols in ((4, 64), (3, 32), (2, 16)):
+        src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(500, rows), at.Tensor(rows, cols), at.Tensor(500, cols))
+        assert "operator schedule on the FP64 matrix cores: %d x %d operator" % (rows, cols) in src
     # without the matrix cores: a lane keeps its row for four entries, whose vectors come through scalar loads
     monkeypatch.setenv("ACRO_HIP_OPERATOR_MFMA", "-1")
     src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 60), at.Tensor(60, 60), at.Tensor(1000, 60))

@@ -840,7 +840,12 @@ def test_small_matrices_per_entry_are_transposed_by_a_lane_per_element(at, engin
     ("A_e_i = B_i_j X_e_j", [(3, 27), (900, 27)]),
     ("A_e_i_k = B_e_i_j C_j_k", [(600, 8, 8), (8, 8)]),                   # entries (e, i), operator stored transposed
     ("A_e_i = B_i_j X_e_j", [(9, 9), (5000, 9)]),
-    ("A_e_i = B_i_j X_e_j", [(4, 8), (5000, 8)]),                         # four rows: not this schedule
+    ("A_e_i = B_i_j X_e_j", [(4, 8), (5000, 8)]),                         # four rows of short vectors: not this schedule
+    # two to four rows applied to vectors of 16 values and more (a gradient at a point)
+    ("A_e_i = B_i_j X_e_j", [(3, 32), (5003, 32)]),
+    ("A_e_i += B_i_j X_e_j", [(4, 64), (1001, 64)]),
+    ("A_e_i -= B_j_i X_e_j", [(16, 2), (2000, 16)]),                      # the operator stored transposed
+    ("A_e_d = D_d_i X_e_i", [(3, 100), (700, 100)]),
     ("A_e_i = B_i_j X_e_j", [(7, 9), (5000, 9)]),                         # odd and short: not this schedule
 ])
 def test_dense_operator_applied_to_every_entry(at, engine, checker, kernel, shapes):
@@ -857,7 +862,7 @@ def test_dense_operator_applied_to_every_entry(at, engine, checker, kernel, shap
         lead = 2 if "_q_" in kernel else 1
         rows = int(np.prod(out0.shape[lead:]))
         cols = operator.size // rows
-    chosen = (rows >= 5 and cols >= 4) if cols % 2 == 0 else (cols >= 16 or (cols >= 9 and rows >= 8))
+    chosen = (rows >= 5 and cols >= 4) or (rows >= 2 and cols >= 16) if cols % 2 == 0 else (cols >= 16 or (cols >= 9 and rows >= 8))
     chosen = chosen and shapes[0] != (1000, 4)           # (there the batch index is i, which the operator carries)
     assert ("operator schedule on the FP64 matrix cores" in engine.GetLastImplementation()) == chosen
     needs_padding = rows % 16 != 0 or cols % (8 if cols % 2 == 0 else 4) != 0
