@@ -167,6 +167,19 @@ auto Generator::StreamedOnce(int k, int v) const -> bool
     if (SourceOf(k, v) != kFromGlobal || !IsPureInput(r.uvar) || GatherSlot(r.uvar) >= 0 || r.repeated || r.idx.empty() || r.idx[0] != batch) return false;
     if (s.matrixOp != 0 || entriesFastest) return false;
     if (((r.size / E) * NB) % 16 != 0) return false;   // the share of a workgroup: whole lines
+    // (a launch that writes more than it reads has few loads to hide behind its stores, and the hinted load takes longer to
+    // come back: "A_e_j_i = B_e_i C_j_i" with 6 values read and 42 written per entry 42 -> 73 us, "A_e_i_j_k = B_i_j_k
+    // C_e_i_k" 89 -> 135 us from HBM)
+    if (WritesDominate()) return false;
+    // (a contraction that runs as a counted loop loads its operands anew in every turn: an operand that does not carry
+    // every contraction index would be asked for again and again, "A_e_j += B_l_k_i C_e_i_j": 1.8 -> 3.3 ms)
+    if (s.loopMode)
+    {
+        for (int id : s.contr)
+        {
+            if (!has(r.idx, id)) return false;
+        }
+    }
     // (read by this kernel only: a second kernel of the group would ask for lines that the hint has let go)
     int readers = 0;
     for (const auto &other : subs)

@@ -539,6 +539,13 @@ auto Generator::ProductThenRowSums(int ki, const Sub &orig, std::vector<Sub> &re
         // dot products of rows of 9: 59 -> 77 %, of 27: 62 -> 76 %; rows of 3 and 5 lose (75 -> 56 %, 73 -> 67 %), 6 and
         // powers of two neither gain nor lose, rows of 100 lose (79 -> 76 %).
         if (row < 7 || row > 64 || (row & (row - 1)) == 0) return false;
+        // (a factor that all entries share is read by every lane of the first step through its own index: with short rows
+        // that costs more than the lanes along the rows lose, from HBM "A_e = B_e_i C_i" with rows of 7 74 -> 58 %, "A_e =
+        // B_i C_i D_e_i" with rows of 12 64 -> 52 %; rows of 20 and 27 gain, 56 -> 59 % and 47 -> 60 %)
+        for (const VarRef *vec : vecs)
+        {
+            if (!has(vec->idx, batch) && row < 20) return false;
+        }
     }
 
     DimensionedKernel *kernel = mk.Kernels[ki];

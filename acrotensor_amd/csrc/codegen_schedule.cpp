@@ -1122,7 +1122,9 @@ auto Generator::ChooseBatching() -> void
         envInt("ACRO_HIP_LIGHT") >= 0)
     {
         bool streaming = subs.back().phase == 0;
-        for (const auto &st : stores) streaming = streaming && !st.wantLds && !st.staged;
+        // (a small invariant operand that every workgroup copies to LDS first does not change that, and more entries per
+        // workgroup share the copy: a 64 x 5 operator, two entries per workgroup, 39 % of the HBM peak)
+        for (const auto &st : stores) streaming = streaming && ((st.staged && envInt("ACRO_HIP_LIGHT_STAGED") >= 0) || (!st.wantLds && !st.staged));
         bool shared = false;   // outputs shared by lanes: their workgroups keep 128 lanes (batched dot product with
                                // 16 entries per workgroup: 76 % in 128 lanes, 66 % in 256)
         for (const auto &s : subs)

@@ -41,7 +41,7 @@ METRIC = "GDOF/s + % HBM peak, p=3 sum-factorised hex mass apply fp64 (1 GPU)"
 # a kernel therefore drops its figure (the line then says null) until the counters are taken again.
 TRAFFIC_BY_KERNEL = {
     ("acro_mk_4ceea56515f0c53c", "5b2c83c4dcb5398d"): 547046884,            # cfg4, intermediates transient
-    ("acro_mk_664cf228dc3d274e", "f303b33e8b931fb8"): 1815949088,           # cfg4, every intermediate stored
+    ("acro_mk_664cf228dc3d274e", "bb5ff2ad54f2a970"): 1815937921,           # cfg4, every intermediate stored
     ("acro_red_35ac69981569e511_partial", "1698cfe138e16625"): 83942685,    # cfg1 (first of its two launches)
     ("batchMatrixKernel<3,inv,det>", "c901ed174aa3fd9b"): 637552436,        # cfg2 (precompiled: hash of hip_ops.hip)
     ("acro_mk_567e3a4d341f4dc2", "663c472f29b65c65"): 210771367,            # cfg3
