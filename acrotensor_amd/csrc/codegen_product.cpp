@@ -99,6 +99,12 @@ auto Generator::ProductPattern(const Sub &s, ProductShape &p) const -> bool
     const bool staged = std::max(p.M, p.N) <= 36 && blocks(p.M) && blocks(p.N) &&
                         !(std::max(p.M, p.N) <= 32 && (byThreeOnly(p.M) || byThreeOnly(p.N))) && !(p.M % 16 == 0 && p.N % 16 == 0);
     if (!vectorForm && staged && envInt("ACRO_HIP_PRODUCT") < 2) return false;
+    // A side of fewer than 16 leaves half and more of the matrix instruction's columns (or rows) empty; where the staged
+    // schedule can hold both factors in LDS it is ahead then (from HBM, % of the HBM peak, here / staged: 64 x 8 by 8 x 8
+    // 57 / 76, 48 x 8 by 8 x 8 58 / 74, 64 x 8 by 8 x 12 60 / 71, 8 x 8 by 8 x 64 78 / 84, 12 x 8 by 8 x 48 77 / 80,
+    // 64 x 32 by 32 x 8 68 / 80, 40 x 16 by 16 x 10 68 / 75; 8 x 32 by 32 x 64 80 / 76).
+    // (measured up to 32 terms)
+    if (!vectorForm && std::min(p.M, p.N) < 16 && p.K <= 32 && (p.M + p.N) * p.K <= 4000 && envInt("ACRO_HIP_PRODUCT") < 2) return false;
     p.TI = (p.M + 15) / 16;
     p.TJ = (p.N + 15) / 16;
     if (p.TI > 8 || p.TJ > 8) return false;
