@@ -237,7 +237,13 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
     {
         // (components between the row indices have no other schedule to fall back on: half as many registers again)
         const long most = 16 * ((o.outMixed ? 24 : 16) / o.comp);
-        if (ComponentsTogether(o) && (o.blockRows > most || (o.blockRows == 0 && o.rows > most))) o.blockRows = most;
+        if (ComponentsTogether(o) && (o.blockRows > most || (o.blockRows == 0 && o.rows > most)))
+        {
+            // (a small operator that only its many components push into blocks of rows, 20 x 9 with nine components: two
+            // launches, 26 us against 10 us on the generic schedule)
+            if (o.rows * o.cols < 1024 && !o.outMixed) return false;
+            o.blockRows = most;
+        }
     }
     // With components: vectors in 8-byte loads, no pointwise factors, and only where the generic schedule (an
     // entry and a row per lane) runs out of scalar registers for the operator or of coalescing for its stores
@@ -296,6 +302,14 @@ auto Generator::OperatorPattern(OperatorShape &o, int k, bool alone) const -> bo
     // schedule has a lane per result read the whole vector (from HBM: 3 x 32 30 %, 4 x 64 25 %, 2 x 64 43 %, 3 x 128 27 % of
     // the HBM peak); on the matrix cores 73 / 72 / 71 / 67 %, and no worse at 16 columns (2 / 3 / 4 x 16: 56 / 71 / 75 ->
     // 72 / 75 / 75 %).
+    // Measured again from HBM with the generic schedule as it is now (results of long runs per lane leave through an LDS
+    // tile, light workgroups take more entries): below 16 rows and 16 columns it is ahead of or level with the matrix
+    // cores, whose 16 x 8 blocks such operators fill in small part (here / generic, % of the HBM peak: 5 x 4 51 / 73,
+    // 8 x 4 61 / 74, 12 x 4 66 / 77, 6 x 6 64 / 75, 10 x 6 69 / 73, 5 x 8 69 / 73, 8 x 8 71 / 71, 5 x 12 65 / 74, 12 x 12
+    // 71 / 70; with a factor per entry 8 x 8 61 / 73).  From 16 rows on the matrix cores stay ahead (32 x 4 81 / 69,
+    // 32 x 8 81 / 68, 56 x 8 75 / 42), and so they do from 16 columns on (5 x 32 74 / 57, 6 x 64 70 / 15).
+    // (a kernel on its own: inside a group the schedule is what joins two operators into one launch)
+    if (alone && o.pairs && o.cols < 16 && o.rows < 16 && envInt("ACRO_HIP_OPERATOR_SMALL") >= 0) return false;
     const long fewRowsFrom = envInt("ACRO_HIP_OPERATOR_FEW_ROWS", 16);
     if (o.pairs && o.rows >= 2 && o.rows < 5 && fewRowsFrom > 0 && o.cols >= fewRowsFrom) return true;
     return o.pairs ? (o.rows >= 5 && o.cols >= 4) : (o.cols >= 16 || (o.cols >= 9 && o.rows >= 8));

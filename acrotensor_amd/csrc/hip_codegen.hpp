@@ -114,6 +114,8 @@
 //   ACRO_HIP_OPERATOR_PAIR=-1   two operator-shaped kernels with a transient intermediate are not joined into one matrix-core kernel
 //   ACRO_HIP_OPERATOR_SEQUENCE=-1  groups of several large operator-shaped kernels run as one fused chain kernel instead of one
 //                               matrix-core launch per kernel
+//   ACRO_HIP_OPERATOR_SMALL=-1  operators below 16 rows and 16 columns applied to vectors of even length take the operator schedule
+//                               from five rows on, as they did before the generic schedule overtook it there
 //   ACRO_HIP_OPERATOR_FEW_ROWS=<n>  operators of two to four rows take the operator schedule from n columns on (default 16; 0: never)
 //   ACRO_HIP_OPERATOR_MFMA=-1   the operator schedule never uses the FP64 matrix cores (a lane keeps its row for four entries,
 //                               whose vectors come through scalar loads, whatever the operator's sizes)

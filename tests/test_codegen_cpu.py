@@ -234,8 +234,13 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1000, 30), at.Tensor(30, 27), at.Tensor(1000, 27))
     assert "(padded to 32 x 28)" in src and "j = 4 * step + (l >> 4);" in src and "xv[q] = 4 * q + g >= 27 ? 0.0 : x[4 * q];" in src
     # pointwise factors: per entry, per output and per row on the result, per element and per column on the vectors
-    src = TE.GetImplementation("A_e_i -= B_i_j X_e_j W_e D_e_j R_i F_e_i C_j", at.Tensor(1000, 10), at.Tensor(10, 12), at.Tensor(1000, 12),
-                               at.Tensor(1000), at.Tensor(1000, 12), at.Tensor(10), at.Tensor(1000, 10), at.Tensor(12))
+    # (an operator below 16 x 16 on its own keeps the generic schedule; the switch brings it here, as a group would)
+    factors = ("A_e_i -= B_i_j X_e_j W_e D_e_j R_i F_e_i C_j", at.Tensor(1000, 10), at.Tensor(10, 12), at.Tensor(1000, 12),
+               at.Tensor(1000), at.Tensor(1000, 12), at.Tensor(10), at.Tensor(1000, 10), at.Tensor(12))
+    assert "operator schedule" not in TE.GetImplementation(*factors)
+    monkeypatch.setenv("ACRO_HIP_OPERATOR_SMALL", "-1")
+    src = at.TensorEngine("HIP").GetImplementation(*factors)
+    monkeypatch.delenv("ACRO_HIP_OPERATOR_SMALL")
     assert "operator schedule on the FP64 matrix cores: 10 x 12 operator" in src and "const double se = T3[0 + en];" in src
     # (10 rows: the results of a trip's 16 entries are collected in LDS in memory order and leave as one contiguous range)
     assert "mid[(4 * r + g) * 10 + 16 * t + c] = acc[t][r] * se * T6[0 + en * 10 + 16 * t + c] * T5[0 + 16 * t + c];" in src

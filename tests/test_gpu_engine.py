@@ -833,7 +833,9 @@ def test_small_matrices_per_entry_are_transposed_by_a_lane_per_element(at, engin
     ("A_e_q_i += B_j_i X_e_q_j", [(24, 32), (100, 7, 24)]),               # 700 entries numbered by two indices
     ("A_e_q_i = B_i_j X_e_q_j", [(30, 20), (100, 7, 20)]),                # padded to 32 x 24
     ("A_e_i = B_j_i X_e_j", [(33, 17), (500, 33)]),                       # odd row length: 8-byte loads, padded to 32 x 36
-    # small operators: with vectors of even length from five rows on, with odd length from 16 columns on
+    # small operators: with vectors of even length from 16 rows or 16 columns on, with odd length from 16 columns on
+    ("A_e_i = B_i_j X_e_j", [(16, 8), (5000, 8)]),
+    ("A_e_i -= B_i_j X_e_j", [(32, 4), (5001, 4)]),
     ("A_e_i = B_i_j X_e_j", [(8, 8), (5000, 8)]),
     ("A_e_i -= B_i_j X_e_j", [(8, 4), (5001, 4)]),
     ("A_e_i += B_i_j X_e_j", [(10, 10), (777, 10)]),
@@ -862,7 +864,9 @@ def test_dense_operator_applied_to_every_entry(at, engine, checker, kernel, shap
         lead = 2 if "_q_" in kernel else 1
         rows = int(np.prod(out0.shape[lead:]))
         cols = operator.size // rows
-    chosen = (rows >= 5 and cols >= 4) or (rows >= 2 and cols >= 16) if cols % 2 == 0 else (cols >= 16 or (cols >= 9 and rows >= 8))
+    # (vectors of even length: from 16 columns on with two rows and more, below that from 16 rows on; below 16 x 16 the
+    # generic schedule is as fast or faster)
+    chosen = ((rows >= 2 and cols >= 16) or (rows >= 16 and cols >= 4)) if cols % 2 == 0 else (cols >= 16 or (cols >= 9 and rows >= 8))
     chosen = chosen and shapes[0] != (1000, 4)           # (there the batch index is i, which the operator carries)
     assert ("operator schedule on the FP64 matrix cores" in engine.GetLastImplementation()) == chosen
     needs_padding = rows % 16 != 0 or cols % (8 if cols % 2 == 0 else 4) != 0
@@ -906,9 +910,10 @@ def test_dense_operators_with_odd_rows_or_too_large_for_lds(at, engine, checker,
     ("A_e_i = B_i_j X_e_j D_e_j C_j W_e", [(20, 17), (777, 17), (777, 17), (17,), (777,)]),   # odd length: 8-byte loads
     ("A_e_q_i = W_e_q B_i_j X_e_q_j", [(601, 3), (16, 8), (601, 3, 8)]),            # the factor first, two entry indices
 ])
-def test_dense_operator_with_pointwise_factors(at, engine, checker, kernel, shapes):
+def test_dense_operator_with_pointwise_factors(at, engine, checker, monkeypatch, kernel, shapes):
     """Factors beside the operator and the vectors: the result is scaled per entry, per output or per row as it is
     stored, the vectors per element or per column as they are loaded (reference semantics: one product per term)."""
+    monkeypatch.setenv("ACRO_HIP_OPERATOR_SMALL", "-1")   # (operators below 16 x 16 on their own: brought here as a group would)
     rng = np.random.default_rng(len(kernel) + shapes[1][0])
     ins = [rng.uniform(-1, 1, s) for s in shapes]
     out0 = rng.uniform(-1, 1, output_shape(kernel, shapes))
@@ -1100,7 +1105,7 @@ def test_batched_matrices_at_odd_offsets(at, engine, checker, m):
 def test_operator_kernels_on_buffers_that_are_only_8_byte_aligned(at, engine, checker):
     # the operator schedule moves the entries' vectors with 16-byte instructions; a caller's device buffer one double
     # into an allocation must work like any other
-    E, n = 300, 12
+    E, n = 300, 20
     rng = np.random.default_rng(77)
     B, X = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (E, n))
     pool = at.Tensor(2 * X.size + 16)

@@ -158,7 +158,7 @@ def test_products_of_element_matrices_beyond_2_31_entries(at, kernel, E, M, N, K
 
 @pytest.mark.parametrize("kernel,E,n,comps", [
     ("A_e_i = B_i_j X_e_j", 34000000, 64, 0),           # results stored from the accumulators
-    ("A_e_i = B_i_j X_e_j", 270000000, 8, 0),           # padded operator, results written out through LDS
+    ("A_e_i = B_i_j X_e_j", 110000000, 20, 0),          # padded operator, results written out through LDS
     ("A_e_i_k = B_i_j X_e_j_k", 12000000, 64, 3),       # three components per vector element
 ])
 def test_operator_on_the_matrix_cores_beyond_2_31_entries(at, kernel, E, n, comps):
