@@ -784,6 +784,11 @@ def test_operands_that_carry_a_contraction_index_alone_are_summed_first(TE):
     assert "steps of" in TE.GetImplementation("A_e = B_e_i", at.Tensor(4096), at.Tensor(4096, 9))
     for row in (3, 5, 16, 100):
         assert "steps of" not in TE.GetImplementation("A_e = B_e_i", at.Tensor(4096), at.Tensor(4096, row))
+    # a vector applied from the left to an element matrix of few columns: the second step adds down the columns of the tile
+    src = TE.GetImplementation("A_e_j = B_e_i_j C_e_i", at.Tensor(4096, 2), at.Tensor(4096, 27, 2), at.Tensor(4096, 27))
+    assert "_F1_e_i_j = B_e_i_j C_e_i" in src and "A_e_j = _F1_e_i_j   (steps of:" in src
+    assert "steps of" not in TE.GetImplementation("A_e_j = B_e_i_j C_i", at.Tensor(4096, 2), at.Tensor(4096, 64, 2), at.Tensor(64))
+    assert "steps of" not in TE.GetImplementation("A_e_j = B_e_i_j C_e_i", at.Tensor(4096, 8), at.Tensor(4096, 27, 8), at.Tensor(4096, 27))
     # a contraction shared by lanes is numbered as the terms lie in the streaming operand
     src = TE.GetImplementation("A_e = B_i_j C_e_j_i", at.Tensor(4096), at.Tensor(20, 8), at.Tensor(4096, 8, 20))
     assert "contraction shared by" in src and "lanes()=16" in src

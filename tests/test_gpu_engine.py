@@ -1196,6 +1196,11 @@ def test_element_matrix_times_vector_with_odd_rows(at, engine, checker, kernel, 
     ("A_e = B_e_i C_i D_e_i", [(500, 45), (45,), (500, 45)], True),       # three factors along the row
     ("A_e = B_e_i_j C_e_i_j", [(700, 3, 5), (700, 3, 5)], True),          # two contraction indices, rows of 15
     ("A_e_k = B_e_k_i C_e_i", [(600, 2, 27), (600, 27)], True),           # two sums per entry
+    ("A_e_j = B_e_i_j C_e_i", [(700, 27, 2), (700, 27)], True),           # a vector applied from the left: sums down the columns
+    ("A_e_j -= B_e_i_j", [(500, 64, 3)], True),                           # column sums
+    ("A_e_j_k = B_e_i_j_k C_e_i", [(300, 20, 2, 2), (300, 20)], True),    # four columns numbered by two indices
+    ("A_e_j = B_e_i_j C_i", [(500, 64, 2), (64,)], False),                # a vector that all entries share: as written
+    ("A_e_j = B_e_i_j C_e_i", [(500, 12, 2), (500, 12)], False),          # few rows: as written
     ("A_e = B_e_i", [(5000, 5)], False),                                  # short rows and powers of two stay as they are
     ("A_e = B_e_i C_e_i", [(5000, 16), (5000, 16)], False),
     ("A_e = B_e_i_j C_i D_j", [(900, 7, 9), (7,), (9,)], False),          # factors along part of a row
