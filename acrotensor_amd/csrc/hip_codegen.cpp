@@ -43,6 +43,18 @@ auto Generator::Run() -> HipKernelPlan
     }
     if (UseTiledProductSchedule())
     {
+        // A shared factor of 4 097 to 8 192 entries with at most 96 columns still does better as an operator in LDS in
+        // blocks of rows, where that schedule takes the kernel (tensors that exceed the memory-side cache, % of the HBM
+        // peak, tiled product -> operator: 125 x 64 39.5 -> 45.5, 128 x 64 47 -> 51, 96 x 48 56 -> 65, 80 x 60 49.5 -> 56,
+        // 72 x 72 41 -> 47.5; but 64 x 125 43 -> 41, 125 x 125 28 -> 20.5, 216 x 64 33 -> 34, 100 x 100 26.5 -> 24).
+        TiledProductShape p;
+        TiledProductPattern(subs[0], p);
+        const long mid = envInt("ACRO_HIP_TILED_PRODUCT_OPERATOR_MID", 8192);
+        if (!p.batched && std::min(p.M, p.N) * p.K <= mid && p.K <= 96 && UseOperatorSchedule())
+        {
+            EmitOperator(plan);
+            return plan;
+        }
         EmitTiledProduct(plan);
         return plan;
     }

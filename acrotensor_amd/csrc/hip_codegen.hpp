@@ -168,7 +168,8 @@
 //   ACRO_HIP_TILED_PRODUCT_XCD=-1  the tiles of an entry are numbered as the hardware deals them (default: an entry's two to four
 //                               tiles on one XCD, so that the strips they share pass through one L2)
 //   ACRO_HIP_TILED_PRODUCT_OPERATOR=<entries>  a product without a batch index one of whose factors has at most this many entries
-//                               is left to the operator schedule (4 096)
+//                               is left to the operator schedule (4 096);  ACRO_HIP_TILED_PRODUCT_OPERATOR_MID=<entries>: up to
+//                               this many entries, with at most 96 columns, the operator schedule goes first where it applies (8 192)
 #ifndef ACRO_HIP_CODEGEN_HPP
 #define ACRO_HIP_CODEGEN_HPP
 

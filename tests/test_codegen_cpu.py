@@ -257,6 +257,13 @@ def test_dense_operator_per_entry_uses_the_operator_schedule(TE, monkeypatch):
     src = TE.GetImplementation("G_e_d_q = D_d_q_i X_e_i", at.Tensor(1000, 3, 64), at.Tensor(3, 64, 64), at.Tensor(1000, 64))
     assert "rows 0 - 127 of the 192 x 64 operator" in src and "rows 128 - 191 of the 192 x 64 operator" in src and src.count("__global__") == 2
     assert "frag[f] = T1[0 + (row + 128) * 64 + j];" in src and "double *a = T0 + 0 + (tile * 16 + g) * 192 + 128 + c;" in src
+    # one shared factor of 4 097 to 8 192 entries and at most 96 columns goes to the operator schedule where that applies,
+    # and stays a tiled product where it does not (vectors stored entries-fastest) or above those sizes
+    src = TE.GetImplementation("A_e_i = B_i_j X_e_j", at.Tensor(1003, 125), at.Tensor(125, 64), at.Tensor(1003, 64))
+    assert "rows 0 - 124 of the 125 x 64 operator in LDS in operand order (padded to 128 x 64)" in src and src.count("__global__") == 1
+    for shapes in [((1003, 125), (125, 125), (1003, 125)), ((1003, 64), (64, 125), (1003, 125))]:
+        assert "tiled product schedule" in TE.GetImplementation("A_e_i = B_i_j X_e_j", *[at.Tensor(*sh) for sh in shapes])
+    assert "tiled product schedule" in TE.GetImplementation("A_e_i = B_i_j X_j_e", at.Tensor(1003, 125), at.Tensor(125, 64), at.Tensor(64, 1003))
     # the operator's dimensions in any order: its copy in LDS is filled through their strides
     src = TE.GetImplementation("J_e_q_n_m = G_q_i_n X_e_i_m", at.Tensor(501, 27, 3, 3), at.Tensor(27, 27, 3), at.Tensor(501, 27, 3))
     assert "81 x 27 operator (dimensions in another order)" in src and "3 components per vector element" in src

@@ -886,6 +886,10 @@ def test_dense_operator_applied_to_every_entry(at, engine, checker, kernel, shap
     ("G_e_d_q = D_d_q_i X_e_i", [(3, 64, 64), (1001, 64)], "rows 128 - 191 of the 192 x 64 operator"),
     ("A_e_i -= B_j_i X_e_j W_e R_i", [(125, 375), (403, 125), (403,), (375,)], "rows 320 - 374 of the 375 x 125 operator (stored transposed)"),
     ("A_e_i += X_e_j B_i_j D_e_j", [(1500, 30), (1000, 30), (1500, 30)], "rows 768 - 999 of the 1000 x 30 operator"),
+    # one shared factor of 4 097 to 8 192 entries and at most 96 columns: the operator schedule before the tiled product
+    ("A_e_i = B_i_j X_e_j", [(125, 64), (1003, 64)], "rows 0 - 124 of the 125 x 64 operator"),
+    ("A_e_i += B_j_i X_e_j", [(48, 96), (777, 48)], "rows 0 - 95 of the 96 x 48 operator (stored transposed)"),
+    ("A_e_i -= B_i_j X_e_j", [(80, 60), (2001, 60)], "rows 0 - 79 of the 80 x 60 operator"),
     # the batch index second among the indices that number the entries
     ("A_i_e_j -= B_i_e_k C_k_j W_i_e", [(8, 501, 16), (16, 12), (8, 501)], "4008 entries"),
 ])
