@@ -217,6 +217,7 @@ KERNEL_SHAPES = [
     ("A_e_i = B_e_i_i", [(1 << 20, 8, 8)], (1 << 20, 8)),
     ("A_e_q_j_k = B_q_i X_e_i_j_k", [(5, 4), (1 << 19, 4, 4, 4)], (1 << 19, 5, 4, 4)),
     ("A_e_i = B_i_j X_e_j", [(64, 64), (1 << 18, 64)], (1 << 18, 64)),
+    ("U_e_q = B_q_i X_e_i", [(125, 64), (1 << 17, 64)], (1 << 17, 125)),
     ("A_e_i_k = B_i_j X_e_j_k", [(64, 64), (1 << 16, 64, 3)], (1 << 16, 64, 3)),
     ("A_e_i_k = B_i_j X_e_j_k", [(16, 16), (1 << 18, 16, 3)], (1 << 18, 16, 3)),
     ("A_e_i = B_i_j X_e_j", [(7, 9), (1 << 21, 9)], (1 << 21, 7)),
